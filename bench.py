@@ -1,0 +1,184 @@
+#!/usr/bin/env python3
+"""Benchmark of the dynamic-k MoE-FFN forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vit_b_50k] [--no-cpu-baseline]
+
+One "step" is one pass of the whole layer (router MLP -> dynamic-k selection -> experts -> bias epilogue) over one
+batch of synthetic tokens that already sit in HBM.  The default workload is the ViT-B-shape layer of the headline
+metric: 256 x 197 = 50432 tokens, D = 768, 128 experts x 24 neurons, ReLU, bf16 storage with float32 accumulation,
+module tau = 0.9 (the layer keeps expert e when norm_e >= (1 - tau) * max norm, the reference's convention).
+The literal reading "norm_e >= 0.9 * max" of the same number is measured too and reported under "literal_rule".
+
+Prints ONE JSON line.  Beyond the common fields it carries
+  roofline      the dominant kernel (the experts kernel) against the MI355X bf16 MFMA peak: achieved = active-expert
+                FLOPs (routed (token, expert) pairs x 4*D*Ed) / the kernel's mean duration, taken with HIP events on
+                the launch stream inside this run
+  cpu_baseline  the CPU restatement of the reference's PyTorch CPU path (router + gate + per-expert loop) timed on
+                this machine's host cores over a bounded sample of the same layer shape
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
+
+WORKLOADS = {
+    # name: (batch, seq, D, E, Ed, W, activation)
+    'vit_b_50k': (256, 197, 768, 128, 24, 128, 'relu'),
+    'vit_b_1576': (8, 197, 768, 128, 24, 128, 'relu'),
+}
+
+
+def make_params(D, E, Ed, W, seed, dtype, device):
+    """Seeded weights with the reference's init (uniform +-1/sqrt(last dim); nn.Linear default for the router)."""
+    g = torch.Generator().manual_seed(seed)
+
+    def uni(*shape, fan):
+        return ((torch.rand(*shape, generator=g) * 2 - 1) / fan ** 0.5).to(dtype).to(device)
+
+    return dict(w1=uni(E, D, Ed, fan=Ed), b1=uni(E, Ed, fan=Ed), w2=uni(E, Ed, D, fan=D),
+                last_bias=torch.zeros(D, dtype=dtype, device=device),
+                router_w1=uni(W, D, fan=D), router_w2=uni(E, W, fan=W))
+
+
+def time_events(fn, steps, warmup):
+    """Mean milliseconds per call of fn, HIP events on torch's current stream (the stream fn launches on)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W):
+    N = x.size(0)
+
+    def layer():
+        return ops.forward(x, p['router_w1'], p['router_w2'], thr_scale, p['w1'], p['b1'], p['w2'], None, p['last_bias'],
+                           act, False, None, False, False, 'auto', packed)
+
+    out, routing, _, _ = layer()
+    torch.cuda.synchronize()
+    per_token = routing.float().sum(-1)
+    pairs = int(per_token.sum().item())
+    mean_k = per_token.mean().item()
+    p99_k = torch.quantile(per_token, 0.99).item()
+    # whole layer, wall clock bracketed by synchronize
+    for _ in range(warmup):
+        layer()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        layer()
+    torch.cuda.synchronize()
+    ms_layer = (time.perf_counter() - t0) * 1e3 / steps
+    # dominant kernel alone (same routing), HIP events on the launch stream
+    ms_experts = time_events(lambda: ops.experts(x, routing, p['w1'], p['b1'], p['w2'], None, p['last_bias'], act, False,
+                                                 'auto', packed), steps, warmup)
+    ms_router = time_events(lambda: ops.router(x, p['router_w1'], p['router_w2']), steps, warmup)
+    active_flops = pairs * 4.0 * D * Ed
+    router_flops = N * (2.0 * D * W + 2.0 * W * E)
+    s = x.element_size()
+    algo_bytes = N * D * s * 2 + N * E * s + (2 * E * D * Ed + E * Ed + D + W * D + E * W) * s
+    return dict(ms_layer=ms_layer, ms_experts=ms_experts, ms_router=ms_router, pairs=pairs, mean_active=mean_k,
+                p99_active=p99_k, active_tflops_layer=active_flops / ms_layer / 1e9,
+                active_tflops_kernel=active_flops / ms_experts / 1e9,
+                total_tflops_layer=(active_flops + router_flops) / ms_layer / 1e9,
+                algo_bytes=algo_bytes, hbm_gbps_layer=algo_bytes / ms_layer / 1e6, tokens_per_s=N / ms_layer * 1e3)
+
+
+def cpu_baseline(D, E, Ed, W, act, tau, budget_s=15.0):
+    """The oracle's restatement of the reference CPU path (router -> dynk_max gate -> per-expert loop), float32,
+    8 x 197 tokens of the same layer shape, repeated until about budget_s seconds have been spent."""
+    from oracle import d2dmoe_oracle as O
+    threads = os.cpu_count() or 1
+    threads = min(threads, 16)   # the box's CPU share for one GPU
+    torch.set_num_threads(threads)
+    p = O.make_layer_params(D, E, Ed, W, seed=0)
+    x = torch.randn(8, 197, D, generator=torch.Generator().manual_seed(1))
+    with torch.no_grad():
+        O.moe_layer_forward(x, p, tau, act, 'naive')
+        times = []
+        t_start = time.perf_counter()
+        while (time.perf_counter() - t_start < budget_s and len(times) < 50) or len(times) < 3:
+            t0 = time.perf_counter()
+            O.moe_layer_forward(x, p, tau, act, 'naive')
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return dict(value=8 * 197 / med, unit='tokens/s', cores=threads, kind='port',
+                sample=f'8x197=1576 tokens of the same layer (D={D}, {E}x{Ed} experts), float32, module tau={tau}, '
+                       f'{len(times)} repetitions, median {med * 1e3:.1f} ms per pass')
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS))
+    ap.add_argument('--tau', type=float, default=0.9, help='module tau (keep expert when norm >= (1 - tau) * max)')
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        print('bench.py: this path is single-GPU (tokens are independent; nothing is exchanged); run with --gpus 1',
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print('bench.py: no GPU visible', file=sys.stderr)
+        sys.exit(1)
+    from d2dmoe_amd import ops
+    dev = torch.device('cuda:0')
+    B, T, D, E, Ed, W, act = WORKLOADS[args.workload]
+    N = B * T
+    dtype = torch.bfloat16
+    p = make_params(D, E, Ed, W, seed=0, dtype=dtype, device=dev)
+    x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
+    shape = ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x), act)
+    packed = ops.pack_weights(shape, p['w1'], p['b1'], p['w2'], None, p['router_w1'], p['router_w2'])
+    with torch.no_grad():
+        main_r = run_regime(ops, x, p, packed, float(1.0 - args.tau), act, args.steps, args.warmup, D, E, Ed, W)
+        lit_r = run_regime(ops, x, p, packed, float(args.tau), act, args.steps, args.warmup, D, E, Ed, W)
+    line = {
+        'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
+        'value': main_r['tokens_per_s'], 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': main_r['ms_layer'], 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'bf16', 'data': 'synthetic',
+        'config': {'workload': f'{args.workload}: {B}x{T}={N} tokens, D={D}, {E} experts x {Ed}, {act}, router {D}->{W}->{E}, '
+                               f'module tau={args.tau} (keep norm >= {1 - args.tau:.2f}*max), whole layer',
+                   'mean_active_experts': main_r['mean_active'], 'p99_active_experts': main_r['p99_active'],
+                   'mfma_kernels': packed is not None},
+        'active_tflops': main_r['active_tflops_layer'], 'hbm_gbps': main_r['hbm_gbps_layer'],
+        'roofline': {'bound': 'mfma', 'kernel': 'experts', 'achieved': main_r['active_tflops_kernel'],
+                     'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s', 'frac': main_r['active_tflops_kernel'] / PEAK_BF16_TFLOPS,
+                     'traffic': None, 'kernel_ms': main_r['ms_experts'], 'router_ms': main_r['ms_router']},
+        'literal_rule': {'rule': f'keep norm >= {args.tau}*max', 'tokens_per_s': lit_r['tokens_per_s'],
+                         'ms_per_step': lit_r['ms_layer'], 'mean_active_experts': lit_r['mean_active'],
+                         'p99_active_experts': lit_r['p99_active'], 'active_tflops': lit_r['active_tflops_layer'],
+                         'roofline': {'bound': 'hbm', 'achieved': lit_r['hbm_gbps_layer'], 'peak': PEAK_HBM_GBPS,
+                                      'unit': 'GB/s', 'frac': lit_r['hbm_gbps_layer'] / PEAK_HBM_GBPS,
+                                      'algorithmic_bytes': lit_r['algo_bytes'], 'kernel_ms': lit_r['ms_experts']}},
+    }
+    if not args.no_cpu_baseline:
+        line['cpu_baseline'] = cpu_baseline(D, E, Ed, W, act, args.tau)
+    print(json.dumps(line))
+
+
+if __name__ == '__main__':
+    main()

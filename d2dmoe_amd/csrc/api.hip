@@ -1,0 +1,212 @@
+// C ABI of the MoE-FFN forward path (declared in include/d2dmoe.h): argument checks and kernel sequencing.
+// Nothing here allocates, synchronises or reads device memory on the host.
+#include <hip/hip_runtime.h>
+
+#include "common.hpp"
+#include "launch.hpp"
+
+using namespace d2dmoe;
+
+namespace {
+
+inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
+inline size_t elem_size(int dtype) { return dtype == D2DMOE_F32 ? 4 : 2; }
+inline bool dtype_ok(int dtype) { return dtype == D2DMOE_F32 || dtype == D2DMOE_BF16; }
+inline bool act_ok(int a) { return a >= D2DMOE_ACT_RELU && a <= D2DMOE_ACT_ABS; }
+inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+
+int check_shape(const d2dmoe_shape* sh) {
+  if (sh == nullptr) return D2DMOE_E_NULL;
+  if (!dtype_ok(sh->dtype)) return D2DMOE_E_DTYPE;
+  if (!act_ok(sh->activation) || !act_ok(sh->router_activation) || !act_ok(sh->router_output_activation))
+    return D2DMOE_E_ACTIVATION;
+  if (sh->n_tokens < 0 || sh->d_model <= 0 || sh->n_experts <= 0 || sh->expert_dim <= 0) return D2DMOE_E_SHAPE;
+  if (sh->n_experts > 1024) return D2DMOE_E_SHAPE;
+  if (sh->n_tokens > (int64_t)1 << 31) return D2DMOE_E_SHAPE;
+  if (sh->n_tokens * (int64_t)sh->n_experts >= ((int64_t)1 << 31)) return D2DMOE_E_SHAPE;  // pair indices are int32
+  return D2DMOE_OK;
+}
+
+struct ForwardWorkspace {
+  size_t hidden_off, norms_off, perm_off, total;
+};
+
+ForwardWorkspace plan_workspace(const d2dmoe_shape& sh) {
+  ForwardWorkspace w;
+  const size_t es = elem_size(sh.dtype);
+  const size_t N = (size_t)sh.n_tokens;
+  size_t off = 0;
+  w.hidden_off = off; off += align_up(N * (size_t)(sh.router_width > 0 ? sh.router_width : 0) * es);
+  w.norms_off = off;  off += align_up(N * (size_t)sh.n_experts * es);
+  w.perm_off = off;   off += align_up(perm_workspace_bytes(sh.n_tokens, sh.n_experts));
+  w.total = off;
+  return w;
+}
+
+}  // namespace
+
+extern "C" {
+
+int d2dmoe_version(void) { return D2DMOE_VERSION; }
+
+const char* d2dmoe_status_string(int status) {
+  switch (status) {
+    case D2DMOE_OK: return "ok";
+    case D2DMOE_E_NULL: return "a required pointer is NULL";
+    case D2DMOE_E_SHAPE: return "size non-positive or outside the supported range";
+    case D2DMOE_E_DTYPE: return "unknown element type";
+    case D2DMOE_E_ACTIVATION: return "unknown activation";
+    case D2DMOE_E_WORKSPACE: return "workspace missing, misaligned or too small";
+    case D2DMOE_E_UNSUPPORTED: return "no kernel for this request in this build";
+    case D2DMOE_E_ALIGN: return "tensor pointer not aligned to 16 bytes";
+    default: break;
+  }
+  if (status > 0) return hipGetErrorString((hipError_t)status);
+  return "unknown status";
+}
+
+size_t d2dmoe_workspace_bytes(const d2dmoe_shape* shape) {
+  if (check_shape(shape) != D2DMOE_OK) return 0;
+  return plan_workspace(*shape).total;
+}
+
+int d2dmoe_router(const void* x, const void* router_w1, const void* router_w2, void* norms, int64_t n_tokens,
+                  int32_t d_model, int32_t router_width, int32_t n_experts, int32_t dtype, int32_t activation,
+                  int32_t output_activation, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !router_w1 || !router_w2 || !norms) return D2DMOE_E_NULL;
+  if (!dtype_ok(dtype)) return D2DMOE_E_DTYPE;
+  if (!act_ok(activation) || !act_ok(output_activation)) return D2DMOE_E_ACTIVATION;
+  if (n_tokens < 0 || d_model <= 0 || router_width <= 0 || n_experts <= 0) return D2DMOE_E_SHAPE;
+  if (n_tokens == 0) return D2DMOE_OK;
+  const size_t need = (size_t)n_tokens * router_width * elem_size(dtype);
+  if (!workspace || workspace_bytes < need || !aligned16(workspace)) return D2DMOE_E_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e;
+  if (dtype == D2DMOE_F32) {
+    e = launch_linear_act<float>(x, router_w1, workspace, n_tokens, d_model, router_width, activation, s);
+    if (e == hipSuccess) e = launch_linear_act<float>(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s);
+  } else {
+    e = launch_linear_act<bf16_t>(x, router_w1, workspace, n_tokens, d_model, router_width, activation, s);
+    if (e == hipSuccess) e = launch_linear_act<bf16_t>(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s);
+  }
+  return (int)e;
+}
+
+int d2dmoe_select(const void* norms, void* routing, int32_t* counts, int64_t n_tokens, int32_t n_experts,
+                  int32_t dtype, float thr_scale, void* stream) {
+  if (!norms || !routing) return D2DMOE_E_NULL;
+  if (!dtype_ok(dtype)) return D2DMOE_E_DTYPE;
+  if (n_tokens < 0 || n_experts <= 0 || n_experts > 1024) return D2DMOE_E_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  if (n_tokens == 0) {
+    if (counts) return (int)launch_fill_i32(counts, n_experts, 0, s);
+    return D2DMOE_OK;
+  }
+  hipError_t e = (dtype == D2DMOE_F32) ? launch_select<float>(norms, routing, counts, n_tokens, n_experts, thr_scale, s)
+                                       : launch_select<bf16_t>(norms, routing, counts, n_tokens, n_experts, thr_scale, s);
+  return (int)e;
+}
+
+int d2dmoe_build_permutation(const void* routing, int64_t n_tokens, int32_t n_experts, int32_t dtype,
+                             int32_t* offsets, int32_t* token_idx, int64_t* sort_indices, int64_t* unsort_indices,
+                             int64_t* bincounts, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!offsets || !token_idx) return D2DMOE_E_NULL;
+  if (!dtype_ok(dtype)) return D2DMOE_E_DTYPE;
+  if (n_tokens < 0 || n_experts <= 0 || n_experts > 1024) return D2DMOE_E_SHAPE;
+  if (n_tokens * (int64_t)n_experts >= ((int64_t)1 << 31)) return D2DMOE_E_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  if (n_tokens == 0) {
+    hipError_t e = launch_fill_i32(offsets, n_experts + 1, 0, s);
+    if (e == hipSuccess && bincounts) e = launch_fill_i32((int32_t*)bincounts, 2 * (int64_t)n_experts, 0, s);
+    return (int)e;
+  }
+  if (!routing) return D2DMOE_E_NULL;
+  if (!workspace || workspace_bytes < perm_workspace_bytes(n_tokens, n_experts) || !aligned16(workspace))
+    return D2DMOE_E_WORKSPACE;
+  hipError_t e = (dtype == D2DMOE_F32)
+                     ? launch_build_permutation<float>(routing, n_tokens, n_experts, offsets, token_idx, sort_indices,
+                                                       unsort_indices, bincounts, workspace, s)
+                     : launch_build_permutation<bf16_t>(routing, n_tokens, n_experts, offsets, token_idx, sort_indices,
+                                                        unsort_indices, bincounts, workspace, s);
+  return (int)e;
+}
+
+size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape) {
+  if (check_shape(shape) != D2DMOE_OK) return 0;
+  if (!mfma_dense_supported(*shape)) return 0;
+  return mfma_packed_bytes(*shape);
+}
+
+int d2dmoe_pack_weights(const d2dmoe_shape* shape, const void* w1, const void* b1, const void* w2, const void* w_up,
+                        const void* router_w1, const void* router_w2, void* packed, size_t packed_bytes, void* stream) {
+  int st = check_shape(shape);
+  if (st != D2DMOE_OK) return st;
+  if (!w1 || !w2 || !packed) return D2DMOE_E_NULL;
+  if (!mfma_dense_supported(*shape)) return D2DMOE_E_UNSUPPORTED;
+  if (packed_bytes < mfma_packed_bytes(*shape) || !aligned16(packed)) return D2DMOE_E_WORKSPACE;
+  return (int)launch_mfma_pack(*shape, w1, b1, w2, w_up, router_w1, router_w2, packed, (hipStream_t)stream);
+}
+
+int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing, const void* w1, const void* b1,
+                   const void* w2, const void* w_up, const void* last_bias, const void* packed, void* out,
+                   int32_t path, void* workspace, size_t workspace_bytes, void* stream) {
+  int st = check_shape(shape);
+  if (st != D2DMOE_OK) return st;
+  const d2dmoe_shape& sh = *shape;
+  if (sh.n_tokens == 0) return D2DMOE_OK;
+  if (!x || !routing || !w1 || !w2 || !out) return D2DMOE_E_NULL;
+  if (sh.gated && !w_up) return D2DMOE_E_NULL;
+  if (sh.gated && b1) return D2DMOE_E_UNSUPPORTED;
+  if (!sh.gated && w_up) return D2DMOE_E_SHAPE;
+  if (!aligned16(x) || !aligned16(out) || !aligned16(routing)) return D2DMOE_E_ALIGN;
+  (void)workspace; (void)workspace_bytes;
+  hipStream_t s = (hipStream_t)stream;
+  if (path == D2DMOE_PATH_AUTO)
+    path = (packed != nullptr && mfma_dense_supported(sh)) ? D2DMOE_PATH_MFMA_DENSE : D2DMOE_PATH_GENERIC;
+  switch (path) {
+    case D2DMOE_PATH_GENERIC: {
+      if (!experts_generic_supported(sh)) return D2DMOE_E_UNSUPPORTED;
+      hipError_t e = (sh.dtype == D2DMOE_F32)
+                         ? launch_experts_generic<float>(sh, x, routing, w1, b1, w2, w_up, last_bias, out, s)
+                         : launch_experts_generic<bf16_t>(sh, x, routing, w1, b1, w2, w_up, last_bias, out, s);
+      return (int)e;
+    }
+    case D2DMOE_PATH_MFMA_DENSE: {
+      if (!mfma_dense_supported(sh)) return D2DMOE_E_UNSUPPORTED;
+      if (!packed) return D2DMOE_E_NULL;
+      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, s);
+    }
+    default: return D2DMOE_E_UNSUPPORTED;
+  }
+}
+
+int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
+                   float thr_scale, const void* w1, const void* b1, const void* w2, const void* w_up,
+                   const void* last_bias, const void* packed, const void* norms_in, void* norms_out, void* routing,
+                   int32_t* counts, void* out, int32_t path, void* workspace, size_t workspace_bytes, void* stream) {
+  int st = check_shape(shape);
+  if (st != D2DMOE_OK) return st;
+  const d2dmoe_shape& sh = *shape;
+  if (!routing || !out) return D2DMOE_E_NULL;
+  if (sh.n_tokens == 0) return counts ? (int)launch_fill_i32(counts, sh.n_experts, 0, (hipStream_t)stream) : D2DMOE_OK;
+  if (!x) return D2DMOE_E_NULL;
+  const ForwardWorkspace plan = plan_workspace(sh);
+  if (!workspace || workspace_bytes < plan.total || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
+  char* ws = (char*)workspace;
+  const void* norms = norms_in;
+  if (norms == nullptr) {
+    if (!router_w1 || !router_w2) return D2DMOE_E_NULL;
+    if (sh.router_width <= 0) return D2DMOE_E_SHAPE;
+    void* nbuf = norms_out ? norms_out : (void*)(ws + plan.norms_off);
+    st = d2dmoe_router(x, router_w1, router_w2, nbuf, sh.n_tokens, sh.d_model, sh.router_width, sh.n_experts, sh.dtype,
+                       sh.router_activation, sh.router_output_activation, ws + plan.hidden_off, plan.norms_off - plan.hidden_off, stream);
+    if (st != D2DMOE_OK) return st;
+    norms = nbuf;
+  }
+  st = d2dmoe_select(norms, routing, counts, sh.n_tokens, sh.n_experts, sh.dtype, thr_scale, stream);
+  if (st != D2DMOE_OK) return st;
+  return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,
+                        plan.total - plan.perm_off, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,467 @@
+// Generic (any-shape) kernels of the MoE-FFN forward path for gfx950: router linear layers, dynamic-k
+// selection, token->expert permutation, and a token-tile-major experts kernel with float32 math.
+// These are the float32 product path and the bf16 fallback for shapes without an MFMA kernel.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace d2dmoe {
+
+// =====================================================================================================
+// Router layer:  C[M, Nout] = round_T(act(round_T(A[M,K] . B[Nout,K]^T)))
+// (moefication.py:328-330: nn.Linear then the activation module, each producing a tensor of dtype T)
+// 64x64 output tile per 256-thread workgroup, K staged through LDS in slabs of 16, 4x4 outputs per thread.
+// =====================================================================================================
+constexpr int LT_M = 64, LT_N = 64, LT_K = 16;
+
+template <typename T>
+__global__ __launch_bounds__(256) void linear_act_kernel(const T* __restrict__ A, const T* __restrict__ B,
+                                                         T* __restrict__ C, int64_t M, int K, int Nout, int act) {
+  __shared__ float As[LT_K][LT_M + 4];
+  __shared__ float Bs[LT_K][LT_N + 4];
+  const int t = threadIdx.x;
+  const int64_t row0 = (int64_t)blockIdx.x * LT_M;
+  const int col0 = blockIdx.y * LT_N;
+  const int lr = t >> 2;        // 0..63: tile row loaded by this thread
+  const int lk = (t & 3) << 2;  // 0,4,8,12: first k of the 4 it loads
+  const int ty = t >> 4, tx = t & 15;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += LT_K) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + lk + i;
+      const int64_t ar = row0 + lr;
+      const int br = col0 + lr;
+      As[lk + i][lr] = (ar < M && k < K) ? Elem<T>::load(A + ar * K + k) : 0.f;
+      Bs[lk + i][lr] = (br < Nout && k < K) ? Elem<T>::load(B + (int64_t)br * K + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < LT_K; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t r = row0 + ty * 4 + i;
+    if (r >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = col0 + tx * 4 + j;
+      if (c < Nout) {
+        float v = Elem<T>::round(acc[i][j]);
+        Elem<T>::store(C + r * Nout + c, apply_act(act, v));
+      }
+    }
+  }
+}
+
+template <typename T>
+hipError_t launch_linear_act(const void* A, const void* B, void* C, int64_t M, int K, int Nout, int act,
+                             hipStream_t s) {
+  dim3 grid((unsigned)cdiv64(M, LT_M), (unsigned)cdiv64(Nout, LT_N));
+  hipLaunchKernelGGL(linear_act_kernel<T>, grid, dim3(256), 0, s, (const T*)A, (const T*)B, (T*)C, M, K, Nout, act);
+  return hipGetLastError();
+}
+template hipError_t launch_linear_act<float>(const void*, const void*, void*, int64_t, int, int, int, hipStream_t);
+template hipError_t launch_linear_act<bf16_t>(const void*, const void*, void*, int64_t, int, int, int, hipStream_t);
+
+// =====================================================================================================
+// small fill kernel (used instead of a memset node so the path stays graph-capture friendly)
+// =====================================================================================================
+__global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
+}
+hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s) {
+  int blocks = (int)(cdiv64(n, 256) < 1024 ? cdiv64(n, 256) : 1024);
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(blocks), dim3(256), 0, s, p, n, v);
+  return hipGetLastError();
+}
+
+// =====================================================================================================
+// Dynamic-k selection (moefication.py:80-85).  One wave per token row; lanes stride over the experts.
+//   m   = max_e norms[n,e]            (NaN-propagating, as torch.max)
+//   thr = round_T(float(m) * thr_scale)
+//   routing[n,e] = norms[n,e] >= thr ? 1 : 0
+// Optional per-expert token counts: accumulated per lane over the wave's rows, then one integer atomic per
+// (wave, expert) -- integer adds, so the result does not depend on the order.
+// =====================================================================================================
+constexpr int SEL_MAX_VPT = 16;  // experts per lane -> E <= 1024
+
+template <typename T>
+__global__ __launch_bounds__(256) void select_kernel(const T* __restrict__ norms, T* __restrict__ routing,
+                                                     int32_t* __restrict__ counts, int64_t N, int E,
+                                                     float thr_scale) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+  const int64_t n_waves = ((int64_t)gridDim.x * blockDim.x) / kWave;
+  const int vpt = (E + kWave - 1) / kWave;
+  int cnt[SEL_MAX_VPT];
+#pragma unroll
+  for (int k = 0; k < SEL_MAX_VPT; ++k) cnt[k] = 0;
+  for (int64_t n = wave; n < N; n += n_waves) {
+    float v[SEL_MAX_VPT];
+    float m = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < SEL_MAX_VPT; ++k) {
+      if (k < vpt) {
+        const int e = lane + k * kWave;
+        v[k] = (e < E) ? Elem<T>::load(norms + n * E + e) : -INFINITY;
+        m = nanmax(m, v[k]);
+      }
+    }
+    m = wave_nanmax(m);
+    const float thr = Elem<T>::round(m * thr_scale);
+#pragma unroll
+    for (int k = 0; k < SEL_MAX_VPT; ++k) {
+      if (k < vpt) {
+        const int e = lane + k * kWave;
+        if (e < E) {
+          const bool on = v[k] >= thr;
+          Elem<T>::store(routing + n * E + e, on ? 1.f : 0.f);
+          cnt[k] += on ? 1 : 0;
+        }
+      }
+    }
+  }
+  if (counts != nullptr) {
+#pragma unroll
+    for (int k = 0; k < SEL_MAX_VPT; ++k) {
+      if (k < vpt) {
+        const int e = lane + k * kWave;
+        if (e < E && cnt[k] != 0) atomicAdd(counts + e, cnt[k]);
+      }
+    }
+  }
+}
+
+template <typename T>
+hipError_t launch_select(const void* norms, void* routing, int32_t* counts, int64_t N, int E, float thr_scale,
+                         hipStream_t s) {
+  if (counts != nullptr) {
+    hipError_t e = launch_fill_i32(counts, E, 0, s);
+    if (e != hipSuccess) return e;
+  }
+  int64_t blocks = cdiv64(N, 4);
+  if (blocks > 2048) blocks = 2048;
+  hipLaunchKernelGGL(select_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, (const T*)norms, (T*)routing, counts,
+                     N, E, thr_scale);
+  return hipGetLastError();
+}
+template hipError_t launch_select<float>(const void*, void*, int32_t*, int64_t, int, float, hipStream_t);
+template hipError_t launch_select<bf16_t>(const void*, void*, int32_t*, int64_t, int, float, hipStream_t);
+
+// =====================================================================================================
+// Token -> expert permutation (moe_layers.py:213-224, 241-249), canonical stable order.
+// Tokens are cut into segments of 64.  Lanes map to experts, so every load of a routing row is coalesced and
+// a per-lane running counter IS the rank of the current token inside its expert's list.
+//   pass 1  perm_count_kernel   seg_counts[seg][e]
+//   pass 2  perm_scan_kernel    seg_offsets[seg][e] = exclusive prefix over segments; totals[e]
+//   pass 3  perm_offsets_kernel offsets[E+1] = exclusive prefix over experts (+ int64 bincounts)
+//   pass 4  perm_scatter_kernel token_idx, optional sort_indices / unsort_indices
+// =====================================================================================================
+constexpr int PERM_SEG = 64;
+constexpr int PERM_MAX_VPT = 16;  // E <= 1024
+
+template <typename T>
+__global__ __launch_bounds__(256) void perm_count_kernel(const T* __restrict__ routing, int32_t* __restrict__ seg_counts,
+                                                         int64_t N, int E, int64_t n_seg) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t seg = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+  if (seg >= n_seg) return;
+  const int vpt = (E + kWave - 1) / kWave;
+  const int64_t t0 = seg * PERM_SEG;
+  const int rows = (int)((N - t0) < PERM_SEG ? (N - t0) : PERM_SEG);
+  int cnt[PERM_MAX_VPT];
+#pragma unroll
+  for (int k = 0; k < PERM_MAX_VPT; ++k) cnt[k] = 0;
+  for (int r = 0; r < rows; ++r) {
+    const T* row = routing + (t0 + r) * E;
+#pragma unroll
+    for (int k = 0; k < PERM_MAX_VPT; ++k) {
+      if (k < vpt) {
+        const int e = lane + k * kWave;
+        if (e < E) cnt[k] += (Elem<T>::load(row + e) > 0.f) ? 1 : 0;
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < PERM_MAX_VPT; ++k) {
+    if (k < vpt) {
+      const int e = lane + k * kWave;
+      if (e < E) seg_counts[seg * E + e] = cnt[k];
+    }
+  }
+}
+
+// One workgroup of 1024 threads (16 waves) per group of 64 experts.  Wave w scans a contiguous range of
+// segments for its 64 experts; the 16 partial sums are combined through LDS.
+__global__ __launch_bounds__(1024) void perm_scan_kernel(const int32_t* __restrict__ seg_counts,
+                                                         int32_t* __restrict__ seg_offsets, int32_t* __restrict__ totals,
+                                                         int E, int64_t n_seg) {
+  __shared__ int32_t part[16][kWave];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int w = threadIdx.x / kWave;
+  const int e = blockIdx.x * kWave + lane;
+  const int64_t per = (n_seg + 15) / 16;
+  const int64_t s0 = w * per;
+  const int64_t s1 = (s0 + per) < n_seg ? (s0 + per) : n_seg;
+  int sum = 0;
+  if (e < E)
+    for (int64_t s = s0; s < s1; ++s) sum += seg_counts[s * E + e];
+  part[w][lane] = sum;
+  __syncthreads();
+  int run = 0;
+  for (int i = 0; i < w; ++i) run += part[i][lane];
+  if (e < E) {
+    for (int64_t s = s0; s < s1; ++s) {
+      const int c = seg_counts[s * E + e];
+      seg_offsets[s * E + e] = run;
+      run += c;
+    }
+    if (w == 15) totals[e] = run;
+  }
+}
+
+// offsets[E+1] from totals[E]; single workgroup, E <= 1024.
+__global__ __launch_bounds__(1024) void perm_offsets_kernel(const int32_t* __restrict__ totals, int32_t* __restrict__ offsets,
+                                                            int64_t* __restrict__ bincounts, int E) {
+  __shared__ int32_t buf[1024];
+  const int t = threadIdx.x;
+  const int c = (t < E) ? totals[t] : 0;
+  buf[t] = c;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {  // Hillis-Steele inclusive scan
+    int v = (t >= off) ? buf[t - off] : 0;
+    __syncthreads();
+    buf[t] += v;
+    __syncthreads();
+  }
+  if (t < E) {
+    offsets[t + 1] = buf[t];
+    if (bincounts != nullptr) bincounts[t] = c;
+  }
+  if (t == 0) offsets[0] = 0;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void perm_scatter_kernel(const T* __restrict__ routing, const int32_t* __restrict__ seg_offsets,
+                                                           const int32_t* __restrict__ offsets, int32_t* __restrict__ token_idx,
+                                                           int64_t* __restrict__ sort_indices, int64_t* __restrict__ unsort_indices,
+                                                           int64_t N, int E, int64_t n_seg) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t seg = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+  if (seg >= n_seg) return;
+  const int vpt = (E + kWave - 1) / kWave;
+  const int64_t t0 = seg * PERM_SEG;
+  const int rows = (int)((N - t0) < PERM_SEG ? (N - t0) : PERM_SEG);
+  int run[PERM_MAX_VPT];   // routed tokens of expert e before the current token
+  int base[PERM_MAX_VPT];  // offsets[e]
+  int total[PERM_MAX_VPT]; // count[e]
+#pragma unroll
+  for (int k = 0; k < PERM_MAX_VPT; ++k) {
+    run[k] = 0; base[k] = 0; total[k] = 0;
+    if (k < vpt) {
+      const int e = lane + k * kWave;
+      if (e < E) {
+        run[k] = seg_offsets[seg * E + e];
+        base[k] = offsets[e];
+        total[k] = offsets[e + 1] - offsets[e];
+      }
+    }
+  }
+  for (int r = 0; r < rows; ++r) {
+    const int64_t tok = t0 + r;
+    const T* row = routing + tok * E;
+#pragma unroll
+    for (int k = 0; k < PERM_MAX_VPT; ++k) {
+      if (k < vpt) {
+        const int e = lane + k * kWave;
+        if (e < E) {
+          const bool on = Elem<T>::load(row + e) > 0.f;
+          // position inside column e of the full (routed first, then the rest) ordering
+          const int64_t pos = on ? (int64_t)run[k] : (int64_t)total[k] + (tok - run[k]);
+          if (on) token_idx[(int64_t)base[k] + run[k]] = (int32_t)tok;
+          if (sort_indices != nullptr) sort_indices[pos * E + e] = tok;
+          if (unsort_indices != nullptr) unsort_indices[tok * E + e] = pos;
+          run[k] += on ? 1 : 0;
+        }
+      }
+    }
+  }
+}
+
+size_t perm_workspace_bytes(int64_t N, int E) {
+  const int64_t n_seg = cdiv64(N, PERM_SEG);
+  // seg_counts + seg_offsets + totals
+  return (size_t)(2 * n_seg * E + E) * sizeof(int32_t);
+}
+
+template <typename T>
+hipError_t launch_build_permutation(const void* routing, int64_t N, int E, int32_t* offsets, int32_t* token_idx,
+                                    int64_t* sort_indices, int64_t* unsort_indices, int64_t* bincounts,
+                                    void* workspace, hipStream_t s) {
+  const int64_t n_seg = cdiv64(N, PERM_SEG);
+  int32_t* seg_counts = (int32_t*)workspace;
+  int32_t* seg_offsets = seg_counts + n_seg * E;
+  int32_t* totals = seg_offsets + n_seg * E;
+  const unsigned seg_blocks = (unsigned)cdiv64(n_seg, 4);
+  hipLaunchKernelGGL(perm_count_kernel<T>, dim3(seg_blocks), dim3(256), 0, s, (const T*)routing, seg_counts, N, E, n_seg);
+  hipLaunchKernelGGL(perm_scan_kernel, dim3((E + kWave - 1) / kWave), dim3(1024), 0, s, seg_counts, seg_offsets, totals, E, n_seg);
+  hipLaunchKernelGGL(perm_offsets_kernel, dim3(1), dim3(1024), 0, s, totals, offsets, bincounts, E);
+  hipLaunchKernelGGL(perm_scatter_kernel<T>, dim3(seg_blocks), dim3(256), 0, s, (const T*)routing, seg_offsets, offsets,
+                     token_idx, sort_indices, unsort_indices, N, E, n_seg);
+  return hipGetLastError();
+}
+template hipError_t launch_build_permutation<float>(const void*, int64_t, int, int32_t*, int32_t*, int64_t*, int64_t*,
+                                                    int64_t*, void*, hipStream_t);
+template hipError_t launch_build_permutation<bf16_t>(const void*, int64_t, int, int32_t*, int32_t*, int64_t*, int64_t*,
+                                                     int64_t*, void*, hipStream_t);
+
+// =====================================================================================================
+// Experts, generic token-tile-major kernel.
+// A workgroup owns BM tokens: their rows of x and routing sit in LDS for the whole kernel, and the output tile
+// [BM, D] lives in registers (thread t owns columns t, t+256, ...).  Experts are visited in ascending order;
+// an expert that no token of the tile routes to is skipped (uniform branch).  For each visited expert:
+//   h[m,j]   = round_T(act(x[m,:] . w1[e,:,j] + b1[e,j]))          (gated: act(x.w1) * (x.w_up))
+//   acc[m,c] += (routing[m,e] * h[m,j]) * w2[e,j,c]
+// so the sum over experts is taken in ascending expert order in float32 and rounded once at the end
+// (the order of moe_merge_results_kernel, moe_impls.py:499-514).  Epilogue: + last_bias, + x (residual).
+// =====================================================================================================
+template <typename T, int BM, int CPT>
+__global__ __launch_bounds__(256) void experts_generic_kernel(
+    const T* __restrict__ x, const T* __restrict__ routing, const T* __restrict__ w1, const T* __restrict__ b1,
+    const T* __restrict__ w2, const T* __restrict__ w_up, const T* __restrict__ last_bias, T* __restrict__ out,
+    int64_t N, int D, int E, int Ed, int act, int add_residual) {
+  extern __shared__ float smem[];
+  float* xs = smem;                 // [BM][D]
+  float* rs = xs + BM * D;          // [BM][E]
+  float* hs = rs + BM * E;          // [BM][Ed]
+  int* active = (int*)(hs + BM * Ed);  // [E]
+  const int t = threadIdx.x;
+  const int64_t tok0 = (int64_t)blockIdx.x * BM;
+
+  for (int i = t; i < BM * D; i += 256) {
+    const int m = i / D, d = i - m * D;
+    const int64_t n = tok0 + m;
+    xs[i] = (n < N) ? Elem<T>::load(x + n * D + d) : 0.f;
+  }
+  for (int i = t; i < BM * E; i += 256) {
+    const int m = i / E, e = i - m * E;
+    const int64_t n = tok0 + m;
+    rs[i] = (n < N) ? Elem<T>::load(routing + n * E + e) : 0.f;
+  }
+  __syncthreads();
+  for (int e = t; e < E; e += 256) {
+    int any = 0;
+    for (int m = 0; m < BM; ++m) any |= (rs[m * E + e] != 0.f) ? 1 : 0;
+    active[e] = any;
+  }
+  __syncthreads();
+
+  float acc[BM][CPT];
+#pragma unroll
+  for (int m = 0; m < BM; ++m)
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) acc[m][c] = 0.f;
+
+  for (int e = 0; e < E; ++e) {
+    if (!active[e]) continue;
+    const T* w1e = w1 + (int64_t)e * D * Ed;
+    const T* wue = (w_up != nullptr) ? (w_up + (int64_t)e * D * Ed) : nullptr;
+    for (int p = t; p < BM * Ed; p += 256) {
+      const int m = p / Ed, j = p - m * Ed;
+      const float* xr = xs + m * D;
+      float a = 0.f, u = 0.f;
+      if (wue == nullptr) {
+        for (int d = 0; d < D; ++d) a = fmaf(xr[d], Elem<T>::load(w1e + (int64_t)d * Ed + j), a);
+        if (b1 != nullptr) a += Elem<T>::load(b1 + (int64_t)e * Ed + j);
+        a = apply_act(act, a);
+      } else {
+        for (int d = 0; d < D; ++d) {
+          a = fmaf(xr[d], Elem<T>::load(w1e + (int64_t)d * Ed + j), a);
+          u = fmaf(xr[d], Elem<T>::load(wue + (int64_t)d * Ed + j), u);
+        }
+        a = apply_act(act, a) * u;
+      }
+      hs[p] = Elem<T>::round(a) * rs[m * E + e];
+    }
+    __syncthreads();
+    const T* w2e = w2 + (int64_t)e * Ed * D;
+    for (int j = 0; j < Ed; ++j) {
+      float w[CPT];
+#pragma unroll
+      for (int c = 0; c < CPT; ++c) {
+        const int col = t + c * 256;
+        w[c] = (col < D) ? Elem<T>::load(w2e + (int64_t)j * D + col) : 0.f;
+      }
+#pragma unroll
+      for (int m = 0; m < BM; ++m) {
+        const float h = hs[m * Ed + j];
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) acc[m][c] = fmaf(h, w[c], acc[m][c]);
+      }
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int c = 0; c < CPT; ++c) {
+    const int col = t + c * 256;
+    if (col >= D) continue;
+    const float lb = (last_bias != nullptr) ? Elem<T>::load(last_bias + col) : 0.f;
+#pragma unroll
+    for (int m = 0; m < BM; ++m) {
+      const int64_t n = tok0 + m;
+      if (n >= N) continue;
+      float v = acc[m][c] + lb;
+      if (add_residual) v += xs[m * D + col];
+      Elem<T>::store(out + n * D + col, v);
+    }
+  }
+}
+
+template <typename T, int BM, int CPT>
+static hipError_t launch_experts_generic_cfg(const d2dmoe_shape& sh, const void* x, const void* routing, const void* w1,
+                                             const void* b1, const void* w2, const void* w_up, const void* last_bias,
+                                             void* out, hipStream_t s) {
+  const size_t lds = (size_t)BM * (sh.d_model + sh.n_experts + sh.expert_dim) * sizeof(float) + sh.n_experts * sizeof(int);
+  if (lds > 160 * 1024) return hipErrorInvalidValue;
+  auto kern = experts_generic_kernel<T, BM, CPT>;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kern, dim3((unsigned)cdiv64(sh.n_tokens, BM)), dim3(256), lds, s, (const T*)x, (const T*)routing,
+                     (const T*)w1, (const T*)b1, (const T*)w2, (const T*)w_up, (const T*)last_bias, (T*)out, sh.n_tokens,
+                     sh.d_model, sh.n_experts, sh.expert_dim, sh.activation, sh.add_residual);
+  return hipGetLastError();
+}
+
+bool experts_generic_supported(const d2dmoe_shape& sh) {
+  if (sh.d_model > 4096) return false;
+  const int bm = sh.d_model <= 768 ? 16 : (sh.d_model <= 2048 ? 8 : 4);
+  const size_t lds = (size_t)bm * (sh.d_model + sh.n_experts + sh.expert_dim) * sizeof(float) + sh.n_experts * sizeof(int);
+  return lds <= 160 * 1024;
+}
+
+template <typename T>
+hipError_t launch_experts_generic(const d2dmoe_shape& sh, const void* x, const void* routing, const void* w1,
+                                  const void* b1, const void* w2, const void* w_up, const void* last_bias, void* out,
+                                  hipStream_t s) {
+  if (sh.d_model <= 768) return launch_experts_generic_cfg<T, 16, 3>(sh, x, routing, w1, b1, w2, w_up, last_bias, out, s);
+  if (sh.d_model <= 2048) return launch_experts_generic_cfg<T, 8, 8>(sh, x, routing, w1, b1, w2, w_up, last_bias, out, s);
+  return launch_experts_generic_cfg<T, 4, 16>(sh, x, routing, w1, b1, w2, w_up, last_bias, out, s);
+}
+template hipError_t launch_experts_generic<float>(const d2dmoe_shape&, const void*, const void*, const void*, const void*,
+                                                  const void*, const void*, const void*, void*, hipStream_t);
+template hipError_t launch_experts_generic<bf16_t>(const d2dmoe_shape&, const void*, const void*, const void*, const void*,
+                                                   const void*, const void*, const void*, void*, hipStream_t);
+
+}  // namespace d2dmoe

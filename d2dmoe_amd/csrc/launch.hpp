@@ -1,0 +1,44 @@
+// Host-side launcher declarations shared between the kernel translation units and the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/d2dmoe.h"
+
+namespace d2dmoe {
+
+// ---- generic kernels (kernels_generic.hip) ----
+template <typename T>
+hipError_t launch_linear_act(const void* A, const void* B, void* C, int64_t M, int K, int Nout, int act, hipStream_t s);
+
+hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s);
+
+template <typename T>
+hipError_t launch_select(const void* norms, void* routing, int32_t* counts, int64_t N, int E, float thr_scale,
+                         hipStream_t s);
+
+size_t perm_workspace_bytes(int64_t N, int E);
+
+template <typename T>
+hipError_t launch_build_permutation(const void* routing, int64_t N, int E, int32_t* offsets, int32_t* token_idx,
+                                    int64_t* sort_indices, int64_t* unsort_indices, int64_t* bincounts,
+                                    void* workspace, hipStream_t s);
+
+bool experts_generic_supported(const d2dmoe_shape& sh);
+
+template <typename T>
+hipError_t launch_experts_generic(const d2dmoe_shape& sh, const void* x, const void* routing, const void* w1,
+                                  const void* b1, const void* w2, const void* w_up, const void* last_bias, void* out,
+                                  hipStream_t s);
+
+// ---- bf16 MFMA kernels (kernels_mfma.hip) ----
+bool mfma_dense_supported(const d2dmoe_shape& sh);
+size_t mfma_packed_bytes(const d2dmoe_shape& sh);
+hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
+                            const void* router_w1, const void* router_w2, void* packed, hipStream_t s);
+hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
+                             const void* last_bias, void* out, hipStream_t s);
+
+}  // namespace d2dmoe

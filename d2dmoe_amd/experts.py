@@ -1,0 +1,267 @@
+"""Experts containers: the plugin boundary of the MoE layer.
+
+Mirrors the reference's experts-container interface (architectures/moe/moe_layers.py):
+``cls(dim, num_experts, depth, expert_dim, bias, activation, intermediate_gating)`` and
+``forward(x[N, D], routing_tensor[N, E]) -> [N, D]``, chosen by name through ``MOE_IMPL_MAP``
+(moe_layers.py:402-407).  Parameter names and shapes equal the reference's so its state_dicts load unchanged.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+from torch import nn
+
+from . import ops
+from .hip_abi import D2DMoEError
+
+# activation module -> kernel activation name (reference: moe_layers.py:11-16, extended for gated experts)
+ACTIVATION_TO_NAME = {
+    nn.GELU: 'gelu',
+    nn.Tanh: 'tanh',
+    nn.ReLU: 'relu',
+    nn.LeakyReLU: 'leaky_relu',
+    nn.SiLU: 'silu',
+    nn.Identity: 'identity',
+}
+
+
+def activation_name(module_or_cls) -> str:
+    """Kernel name of an activation class or instance; GELU(approximate='tanh') maps to 'gelu_tanh'."""
+    cls = module_or_cls if isinstance(module_or_cls, type) else type(module_or_cls)
+    if cls.__name__ in ('PytorchGELUTanh', 'GELUTanh', 'NewGELUActivation'):
+        return 'gelu_tanh'
+    if cls not in ACTIVATION_TO_NAME:
+        raise NotImplementedError(f'{cls} has no HIP kernel activation')
+    if cls is nn.GELU and not isinstance(module_or_cls, type) and getattr(module_or_cls, 'approximate', 'none') == 'tanh':
+        return 'gelu_tanh'
+    return ACTIVATION_TO_NAME[cls]
+
+
+def init_(p: torch.Tensor) -> torch.Tensor:
+    """U(+-1/sqrt(size of last dim)), in place (reference: moe_layers.py:19-24)."""
+    bound = 1.0 / math.sqrt(p.size(-1))
+    with torch.no_grad():
+        p.uniform_(-bound, bound)
+    return p
+
+
+class ExpertsLayer(nn.Module):
+    pass
+
+
+class _IntermediateStub(nn.Module):
+    """Hook point for router training: dense first-layer activations [E,N,Ed] (reference: moe_layers.py:116-124)."""
+
+    def forward(self, x, w1, b1, act):
+        h = torch.einsum('eni,eio->eno', x, w1) + b1.unsqueeze(-2)
+        return act(h)
+
+
+class _OutputStub(nn.Module):
+    """Hook point for router training: dense per-expert outputs [E,N,D] (reference: moe_layers.py:127-133)."""
+
+    def forward(self, h, w2):
+        return torch.einsum('eni,eio->eno', h, w2)
+
+
+class _PackedCache:
+    """Derived MFMA-ordered weight buffer, rebuilt when any source parameter changes (in-place version counter,
+    storage pointer, device or dtype)."""
+
+    def __init__(self):
+        self.key = None
+        self.buf: Optional[torch.Tensor] = None
+
+    def get(self, shape, tensors):
+        key = tuple((t.data_ptr(), t._version, t.dtype, t.device) if t is not None else None for t in tensors)
+        key = key + (shape.d_model, shape.n_experts, shape.expert_dim, shape.gated)
+        if key != self.key:
+            self.buf = ops.pack_weights(shape, *tensors)
+            self.key = key
+        return self.buf
+
+
+class HipKernelExperts(ExpertsLayer):
+    """Two-layer experts with the first-layer bias only, run by the gfx950 HIP kernels.
+
+    Drop-in for the reference's CustomKernelExperts (moe_layers.py:136-264): same constructor, same parameters
+    ``w1 [E,D,Ed]``, ``b1 [E,Ed]``, ``w2 [E,Ed,D]``, same ``forward_mode`` property.  Modes:
+      'masked'  dense PyTorch einsum over all experts, gate-weighted (reference forward_all); keeps the two stub
+                submodules that router training hooks into
+      'naive'   PyTorch per-expert loop (reference forward_naive); the CPU path
+      'hip'     the HIP kernels; 'triton' and 'triton_atomic' are accepted as aliases so reference scripts that
+                select the Triton kernels get this path
+    """
+
+    HIP_MODES = ('hip', 'triton', 'triton_atomic')
+
+    def __init__(self, dim, num_experts, depth=2, expert_dim=None, bias=True, activation=nn.GELU,
+                 intermediate_gating=False):
+        if intermediate_gating:
+            raise NotImplementedError('use HipExecuteAllExperts for gated experts')
+        super().__init__()
+        assert depth == 2, 'only two-layer experts'
+        assert bias == 'without_last', 'bias must be "without_last" (first-layer bias only)'
+        self.activation_str = activation_name(activation)
+        self.num_experts = num_experts
+        self.depth = depth
+        self.expert_dim = dim * 2 if expert_dim is None else expert_dim
+        self.hidden_dim = dim
+        self.bias_mode = bias
+        self.w1 = init_(nn.Parameter(torch.empty(num_experts, dim, self.expert_dim)))
+        self.b1 = init_(nn.Parameter(torch.empty(num_experts, self.expert_dim)))
+        self.w2 = init_(nn.Parameter(torch.empty(num_experts, self.expert_dim, dim)))
+        self.act = activation()
+        self._forward_mode = 'masked'
+        self.kernel_path = 'auto'
+        self.intermediate_activation_extraction_stub = _IntermediateStub()
+        self.output_activation_extraction_stub = _OutputStub()
+        self._packed = _PackedCache()
+
+    @property
+    def forward_mode(self):
+        return self._forward_mode
+
+    @forward_mode.setter
+    def forward_mode(self, value):
+        self._forward_mode = value
+
+    # -- derived buffers --------------------------------------------------------------------
+    def packed_weights(self, router_w1=None, router_w2=None):
+        if not self.w1.is_cuda or self.w1.dtype != torch.bfloat16:
+            return None
+        sh = ops.make_shape(0, self.hidden_dim, self.num_experts, self.expert_dim,
+                            router_w1.size(0) if router_w1 is not None else 0, ops._dtype_code(self.w1),
+                            self.activation_str)
+        return self._packed.get(sh, (self.w1, self.b1, self.w2, None, router_w1, router_w2))
+
+    # -- forward ----------------------------------------------------------------------------
+    def forward(self, x, routing_tensor):
+        assert x.dim() == 2, f'{x.size()=}'
+        mode = self._forward_mode
+        if mode == 'masked':
+            return self.forward_all(x, routing_tensor)
+        if mode == 'naive':
+            return self.forward_naive(x, routing_tensor)
+        if mode in self.HIP_MODES:
+            return self.forward_hip(x, routing_tensor)
+        raise NotImplementedError(f'Unsupported forward_mode: {mode}')
+
+    def forward_all(self, x, routing_tensor):
+        h = self.intermediate_activation_extraction_stub(x.unsqueeze(0), self.w1, self.b1, self.act)
+        y = self.output_activation_extraction_stub(h, self.w2)
+        return torch.einsum('end,ne->nd', y, routing_tensor)
+
+    def forward_naive(self, x, routing_tensor):
+        out = torch.zeros_like(x)
+        for e in range(self.num_experts):
+            mask = routing_tensor[:, e] > 0.0
+            out[mask] += self.act(x[mask] @ self.w1[e] + self.b1[e]) @ self.w2[e]
+        return out
+
+    def forward_hip(self, x, routing_tensor, last_bias=None, add_residual=False):
+        if not x.is_cuda:
+            raise D2DMoEError("forward_mode 'hip' needs a ROCm device; use 'naive' or 'masked' on CPU")
+        if torch.is_grad_enabled() and (x.requires_grad or self.w1.requires_grad):
+            # inference-only, like the reference's kernel wrappers (moe_impls.py:60-64)
+            raise NotImplementedError("the HIP experts path has no backward; wrap the call in torch.no_grad()")
+        return ops.experts(x.contiguous(), routing_tensor.contiguous(), self.w1, self.b1, self.w2, None, last_bias,
+                           self.activation_str, add_residual, self.kernel_path, self.packed_weights())
+
+    # the reference exposes these two as static methods of the container (moe_layers.py:213-224, 241-249)
+    @staticmethod
+    def extract_indices(routing_tensor):
+        if routing_tensor.is_cuda:
+            _, _, s, u, c = ops.build_permutation(routing_tensor.contiguous(), reference_layout=True)
+            return s, u, c
+        r = routing_tensor.to(torch.int32)
+        s = r.argsort(dim=0, descending=True, stable=True)
+        return s, s.argsort(dim=0), r.sum(dim=0)
+
+    @staticmethod
+    def extract_indices_atomic(routing_tensor):
+        s, _, c = HipKernelExperts.extract_indices(routing_tensor)
+        return s, c
+
+
+class _ExecuteAllLayer(nn.Module):
+    """One batched expert layer, parameters ``w [E,in,out]`` and optional ``b [E,1,out]``
+    (reference: moe_layers.py:32-47)."""
+
+    def __init__(self, in_dim, out_dim, num_experts, bias, activation):
+        super().__init__()
+        self.bias = bias
+        self.w = init_(nn.Parameter(torch.empty(num_experts, in_dim, out_dim)))
+        if self.bias:
+            self.b = init_(nn.Parameter(torch.empty(num_experts, 1, out_dim)))
+        self.act = activation()
+
+    def forward(self, x):
+        x = torch.einsum('eni,eio->eno', x, self.w)
+        if self.bias:
+            x = x + self.b
+        return self.act(x)
+
+
+class HipExecuteAllExperts(ExpertsLayer):
+    """Depth-2 experts, optionally with LLaMA/Gemma-style intermediate gating, parameters named as the reference's
+    ExecuteAllExperts (moe_layers.py:50-101): ``layers.0.w`` first/gate projection, ``layers.1.w`` down projection,
+    ``layers.2.w`` up projection (gated only).  ``forward_mode`` 'masked' is the reference's dense einsum; 'hip'
+    runs the HIP kernels, skipping experts that are not routed to."""
+
+    def __init__(self, dim, num_experts, depth=2, expert_dim=None, bias=True, activation=nn.GELU,
+                 intermediate_gating=False):
+        super().__init__()
+        assert depth == 2, 'only two-layer experts'
+        self.num_experts = num_experts
+        self.depth = depth
+        self.dim = dim
+        self.expert_dim = dim * 2 if expert_dim is None else expert_dim
+        self.bias_mode = bias
+        self.activation = activation
+        self.intermediate_gating = intermediate_gating
+        first_bias = True if bias == 'without_last' else bias
+        last_bias = False if bias == 'without_last' else bias
+        self.layers = nn.ModuleList()
+        if intermediate_gating:
+            self.layers.append(_ExecuteAllLayer(dim, self.expert_dim, num_experts, first_bias, activation))
+            self.layers.append(_ExecuteAllLayer(self.expert_dim, dim, num_experts, first_bias, nn.Identity))
+            self.layers.append(_ExecuteAllLayer(dim, self.expert_dim, num_experts, first_bias, nn.Identity))
+        else:
+            self.layers.append(_ExecuteAllLayer(dim, self.expert_dim, num_experts, first_bias, activation))
+            self.layers.append(_ExecuteAllLayer(self.expert_dim, dim, num_experts, last_bias, nn.Identity))
+        self.forward_mode = 'masked'
+        self.kernel_path = 'auto'
+
+    def forward(self, x, routing_tensor):
+        assert x.dim() == 2, f'{x.size()=}'
+        if self.forward_mode == 'hip':
+            return self.forward_hip(x, routing_tensor)
+        x = x.unsqueeze(0)
+        if self.intermediate_gating:
+            x = self.layers[1](self.layers[0](x) * self.layers[2](x))
+        else:
+            for layer in self.layers:
+                x = layer(x)
+        return torch.einsum('end,ne->nd', x, routing_tensor)
+
+    def forward_hip(self, x, routing_tensor, last_bias=None, add_residual=False):
+        if not x.is_cuda:
+            raise D2DMoEError("forward_mode 'hip' needs a ROCm device")
+        if self.layers[1].bias or (self.intermediate_gating and self.layers[0].bias):
+            raise NotImplementedError('the HIP path covers first-layer bias (ungated) or no bias (gated)')
+        b1 = self.layers[0].b.squeeze(1).contiguous() if self.layers[0].bias else None
+        w_up = self.layers[2].w if self.intermediate_gating else None
+        act = activation_name(self.layers[0].act)
+        return ops.experts(x.contiguous(), routing_tensor.contiguous(), self.layers[0].w, b1, self.layers[1].w, w_up,
+                           last_bias, act, add_residual, self.kernel_path, None)
+
+
+MOE_IMPL_MAP = {
+    'hip_kernel': HipKernelExperts,
+    'custom_kernel': HipKernelExperts,     # the reference's name for its Triton-backed container
+    'hip_execute_all': HipExecuteAllExperts,
+    'execute_all': HipExecuteAllExperts,   # the reference's dense container (the one its Gemma runs use)
+}

@@ -1,0 +1,81 @@
+"""ctypes binding of the C ABI in include/d2dmoe.h (libd2dmoe_hip.so, built in-tree by d2dmoe_amd.build).
+
+The library is the only compute path of this package: there is no CPU or eager fallback behind these calls.
+If the shared object is missing or fails to load, every call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
+
+LIB_NAME = 'libd2dmoe_hip.so'
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
+
+# enums of include/d2dmoe.h
+F32, BF16 = 0, 1
+ACT = {'relu': 0, 'gelu': 1, 'tanh': 2, 'leaky_relu': 3, 'gelu_tanh': 4, 'silu': 5, 'identity': 6, 'abs': 7}
+PATH = {'auto': 0, 'generic': 1, 'mfma_dense': 2, 'mfma_sparse': 3}
+
+# every extern "C" symbol the header declares
+EXPORTS = (
+    'd2dmoe_version', 'd2dmoe_status_string', 'd2dmoe_workspace_bytes', 'd2dmoe_router', 'd2dmoe_select',
+    'd2dmoe_build_permutation', 'd2dmoe_experts', 'd2dmoe_packed_bytes', 'd2dmoe_pack_weights', 'd2dmoe_forward',
+)
+
+
+class Shape(Structure):
+    """struct d2dmoe_shape"""
+    _fields_ = [
+        ('n_tokens', c_int64), ('d_model', c_int32), ('n_experts', c_int32), ('expert_dim', c_int32),
+        ('router_width', c_int32), ('dtype', c_int32), ('activation', c_int32), ('gated', c_int32),
+        ('add_residual', c_int32), ('router_activation', c_int32), ('router_output_activation', c_int32),
+    ]
+
+
+class D2DMoEError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads the in-tree shared library (once) and declares the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise D2DMoEError(f'{LIB_PATH} is missing: build it with `python -m d2dmoe_amd.build` '
+                          f'(or __graft_entry__.build()); there is no fallback path')
+    lib = ctypes.CDLL(LIB_PATH)
+    P, I32, I64, SZ = c_void_p, c_int32, c_int64, c_size_t
+    SH = POINTER(Shape)
+    lib.d2dmoe_version.restype = ctypes.c_int
+    lib.d2dmoe_version.argtypes = []
+    lib.d2dmoe_status_string.restype = c_char_p
+    lib.d2dmoe_status_string.argtypes = [ctypes.c_int]
+    lib.d2dmoe_workspace_bytes.restype = SZ
+    lib.d2dmoe_workspace_bytes.argtypes = [SH]
+    lib.d2dmoe_router.restype = ctypes.c_int
+    lib.d2dmoe_router.argtypes = [P, P, P, P, I64, I32, I32, I32, I32, I32, I32, P, SZ, P]
+    lib.d2dmoe_select.restype = ctypes.c_int
+    lib.d2dmoe_select.argtypes = [P, P, P, I64, I32, I32, c_float, P]
+    lib.d2dmoe_build_permutation.restype = ctypes.c_int
+    lib.d2dmoe_build_permutation.argtypes = [P, I64, I32, I32, P, P, P, P, P, P, SZ, P]
+    lib.d2dmoe_experts.restype = ctypes.c_int
+    lib.d2dmoe_experts.argtypes = [SH, P, P, P, P, P, P, P, P, P, I32, P, SZ, P]
+    lib.d2dmoe_packed_bytes.restype = SZ
+    lib.d2dmoe_packed_bytes.argtypes = [SH]
+    lib.d2dmoe_pack_weights.restype = ctypes.c_int
+    lib.d2dmoe_pack_weights.argtypes = [SH, P, P, P, P, P, P, P, SZ, P]
+    lib.d2dmoe_forward.restype = ctypes.c_int
+    lib.d2dmoe_forward.argtypes = [SH, P, P, P, c_float, P, P, P, P, P, P, P, P, P, P, P, I32, P, SZ, P]
+    _lib = lib
+    return lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        msg = load().d2dmoe_status_string(status).decode()
+        raise D2DMoEError(f'{what} failed with status {status}: {msg}')

@@ -1,0 +1,178 @@
+/*
+ * d2dmoe.h -- C ABI of the MI355X (gfx950) dynamic-k MoE-FFN forward path.
+ *
+ * Every entry point
+ *   - takes plain device pointers and sizes (no framework types),
+ *   - enqueues its kernels on the HIP stream passed as `stream` (a hipStream_t cast to void*; NULL = the
+ *     default stream) and returns without synchronising: no hipDeviceSynchronize, no device->host copies,
+ *     no data-dependent launch shapes,
+ *   - allocates and frees no device memory: outputs and the workspace belong to the caller,
+ *   - returns D2DMOE_OK (0), a negative D2DMOE_E_* code for a rejected argument, or a positive hipError_t.
+ *
+ * "Reference" below is the D2DMoE repository; paths are relative to its root.
+ *
+ * Tensor layouts (row-major, contiguous; T = element type selected by `dtype`):
+ *   x          [N, D]      T   tokens (the layer input flattened over batch and sequence)
+ *   router_w1  [W, D]      T   first router Linear weight, [out, in] as nn.Linear stores it
+ *   router_w2  [E, W]      T   second router Linear weight
+ *   norms      [N, E]      T   predicted expert norms = router output
+ *   routing    [N, E]      T   routing tensor; the gate writes exactly 0 or 1
+ *   w1         [E, D, Ed]  T   expert up-projections        (gated experts: the gate projection)
+ *   b1         [E, Ed]     T   expert first-layer biases, or NULL
+ *   w2         [E, Ed, D]  T   expert down-projections
+ *   w_up       [E, D, Ed]  T   gated experts only: the up projection, else NULL
+ *   last_bias  [D]         T   output bias, or NULL
+ *   out        [N, D]      T
+ */
+#ifndef D2DMOE_H
+#define D2DMOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define D2DMOE_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* status codes */
+enum {
+  D2DMOE_OK = 0,
+  D2DMOE_E_NULL = -1,        /* a required pointer is NULL */
+  D2DMOE_E_SHAPE = -2,       /* a size is non-positive or outside what the kernels support */
+  D2DMOE_E_DTYPE = -3,       /* unknown element type */
+  D2DMOE_E_ACTIVATION = -4,  /* unknown activation */
+  D2DMOE_E_WORKSPACE = -5,   /* workspace missing, misaligned or smaller than d2dmoe_workspace_bytes() */
+  D2DMOE_E_UNSUPPORTED = -6, /* valid request that this build has no kernel for */
+  D2DMOE_E_ALIGN = -7        /* a tensor pointer is not aligned to 16 bytes */
+};
+
+/* element types */
+enum { D2DMOE_F32 = 0, D2DMOE_BF16 = 1 };
+
+/* activations.  Reference: utils.py:730-756 (kernel-side definitions), common.py:159-169 (names). */
+enum {
+  D2DMOE_ACT_RELU = 0,       /* x >= 0 ? x : 0 */
+  D2DMOE_ACT_GELU = 1,       /* erf form: x * 0.5 * (1 + erf(x / sqrt 2)) */
+  D2DMOE_ACT_TANH = 2,
+  D2DMOE_ACT_LEAKY_RELU = 3, /* slope 0.01 */
+  D2DMOE_ACT_GELU_TANH = 4,  /* tanh approximation (stock Gemma) */
+  D2DMOE_ACT_SILU = 5,
+  D2DMOE_ACT_IDENTITY = 6,
+  D2DMOE_ACT_ABS = 7
+};
+
+/* which expert kernel family d2dmoe_experts / d2dmoe_forward use */
+enum {
+  D2DMOE_PATH_AUTO = 0,       /* MFMA kernels when the shape and dtype have one, else the generic kernel */
+  D2DMOE_PATH_GENERIC = 1,    /* token-tile-major scalar-FMA kernel: any shape, f32 or bf16 storage, f32 math */
+  D2DMOE_PATH_MFMA_DENSE = 2, /* bf16 MFMA, token-tile-major, masked dense sweep over all experts */
+  D2DMOE_PATH_MFMA_SPARSE = 3 /* bf16 MFMA, expert-major over the permutation, then ordered combine */
+};
+
+/* Shape of one MoE-FFN layer.  Mirrors the constructor arguments of the reference layer
+ * (architectures/moe/moefication.py:30-52) and router (:310-326). */
+typedef struct d2dmoe_shape {
+  int64_t n_tokens;     /* N = batch * sequence */
+  int32_t d_model;      /* D */
+  int32_t n_experts;    /* E */
+  int32_t expert_dim;   /* Ed, neurons per expert */
+  int32_t router_width; /* W */
+  int32_t dtype;        /* D2DMOE_F32 | D2DMOE_BF16 (activations, weights, routing all share it) */
+  int32_t activation;   /* expert activation, D2DMOE_ACT_* */
+  int32_t gated;        /* 0: out = act(x w1 + b1) w2 ; 1: out = (act(x w1) * (x w_up)) w2 */
+  int32_t add_residual; /* 1: out += x  (moefication.py:98-99) */
+  int32_t router_activation;        /* hidden activation of the router MLP (D2DMoE: D2DMOE_ACT_RELU) */
+  int32_t router_output_activation; /* output activation of the router MLP (D2DMoE: D2DMOE_ACT_ABS) */
+} d2dmoe_shape;
+
+/* Library version (D2DMOE_VERSION of the build). */
+int d2dmoe_version(void);
+
+/* Text for a status code returned by this library (negative codes) or by HIP (positive codes). */
+const char* d2dmoe_status_string(int status);
+
+/* Bytes of caller-owned device workspace that d2dmoe_forward / d2dmoe_experts / d2dmoe_build_permutation
+ * need for `shape` (the maximum over the three).  The workspace must be 256-byte aligned.  Replaces the
+ * reference's internal torch.empty/torch.zeros temporaries (moe_impls.py:15, 190, 311). */
+size_t d2dmoe_workspace_bytes(const d2dmoe_shape* shape);
+
+/* Router MLP: norms = out_act(act(x W1^T) W2^T), depth 2, no biases.
+ * Replaces MoeficationRouter.forward (architectures/moe/moefication.py:328-330) for the D2DMoE setting
+ * (depth=2, bias=False; scripts/d2dmoe_vit_wallclock.py:318-325 uses act=relu, out_act=abs).
+ * Intermediate and output are rounded to T after each layer, as eager nn.Linear does.
+ * workspace: at least N*W*sizeof(T) bytes. */
+int d2dmoe_router(const void* x, const void* router_w1, const void* router_w2, void* norms,
+                  int64_t n_tokens, int32_t d_model, int32_t router_width, int32_t n_experts,
+                  int32_t dtype, int32_t activation, int32_t output_activation,
+                  void* workspace, size_t workspace_bytes, void* stream);
+
+/* Dynamic-k selection: routing[n,e] = norms[n,e] >= round_T(max_e norms[n,:] * thr_scale) ? 1 : 0.
+ * Replaces the 'dynk_max' branch of MoeficationMoE.gate (architectures/moe/moefication.py:80-85);
+ * thr_scale is (float)(1.0 - tau).  NaN in a row propagates into its maximum, so that row selects nothing;
+ * an all-zero row selects everything -- both as the reference's tensor ops behave.
+ * counts (optional, int32 [E]) receives the number of tokens routed to each expert (it is zeroed here). */
+int d2dmoe_select(const void* norms, void* routing, int32_t* counts, int64_t n_tokens, int32_t n_experts,
+                  int32_t dtype, float thr_scale, void* stream);
+
+/* Token -> expert permutation from a routing tensor (entry > 0 means routed).
+ * Replaces CustomKernelExperts.extract_indices / extract_indices_atomic
+ * (architectures/moe/moe_layers.py:213-224, 241-249).  The order is canonical and deterministic: within an
+ * expert, tokens ascend (the stable order; the reference's unstable argsort only defines the prefix sets).
+ *   offsets      int32 [E+1]   exclusive prefix sum of the per-expert counts (offsets[E] = number of pairs)
+ *   token_idx    int32 [N*E]   capacity N*E; the first offsets[E] entries are written: expert-major,
+ *                              token-ascending list of routed tokens
+ *   sort_indices   int64 [N,E] optional: column e = routed tokens ascending, then the other tokens ascending
+ *                              (== argsort(routing.int(), dim=0, descending=True, stable=True))
+ *   unsort_indices int64 [N,E] optional: per-column inverse of sort_indices
+ *   bincounts      int64 [E]   optional: per-expert counts
+ * workspace: d2dmoe_workspace_bytes() of a shape with the same N and E. */
+int d2dmoe_build_permutation(const void* routing, int64_t n_tokens, int32_t n_experts, int32_t dtype,
+                             int32_t* offsets, int32_t* token_idx,
+                             int64_t* sort_indices, int64_t* unsort_indices, int64_t* bincounts,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/* Experts: out[n,:] = sum_e routing[n,e] * expert_e(x[n,:]) (+ last_bias) (+ x[n,:]), summed in ascending
+ * expert order in float32 with one final rounding to T; entries with routing == 0 are skipped.
+ * Replaces CustomKernelExperts.forward in its 'triton'/'triton_atomic' modes
+ * (architectures/moe/moe_layers.py:226-264 -> moe_impls.py:8-51, 183-204, 304-363) and, with gated = 1,
+ * ExecuteAllExperts.forward with intermediate gating (moe_layers.py:86-96); last_bias / residual are the
+ * epilogue of MoeficationMoE.forward (moefication.py:96-99).
+ * For 0/1 routing this equals the reference's naive and Triton modes; for weighted routing it equals its
+ * 'masked' mode (forward_all, moe_layers.py:193-198).
+ * packed: optional buffer written by d2dmoe_pack_weights for the same weights (required by the MFMA paths;
+ * D2DMOE_PATH_AUTO without it uses the generic kernel). */
+int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing,
+                   const void* w1, const void* b1, const void* w2, const void* w_up,
+                   const void* last_bias, const void* packed, void* out, int32_t path,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* Bytes of the derived weight buffer for the MFMA kernels (0 when `shape` has no MFMA kernel). */
+size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape);
+
+/* Re-tiles expert (and router) weights into MFMA fragment order.  A derived, cacheable buffer: call once per
+ * weight update.  No counterpart in the reference (Triton re-reads the nn.Parameter layout each call). */
+int d2dmoe_pack_weights(const d2dmoe_shape* shape, const void* w1, const void* b1, const void* w2,
+                        const void* w_up, const void* router_w1, const void* router_w2,
+                        void* packed, size_t packed_bytes, void* stream);
+
+/* Whole layer: router -> dynamic-k select -> experts -> epilogue.
+ * Replaces MoeficationMoE.forward with forward_mode == 'dynk_max'
+ * (architectures/moe/moefication.py:90-101 calling :80-85 and the experts container).
+ *   norms_in   optional [N,E]: when given, the router is skipped and these predicted norms are used -- the
+ *              role of MoeficationRouter(test_override_outputs_p=...) (moefication.py:331-338)
+ *   norms_out  optional [N,E]: receives the router output
+ *   routing    required [N,E]: the routing tensor the layer returns next to its output
+ *   counts     optional int32 [E]: tokens per expert */
+int d2dmoe_forward(const d2dmoe_shape* shape, const void* x,
+                   const void* router_w1, const void* router_w2, float thr_scale,
+                   const void* w1, const void* b1, const void* w2, const void* w_up, const void* last_bias,
+                   const void* packed, const void* norms_in,
+                   void* norms_out, void* routing, int32_t* counts, void* out, int32_t path,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* D2DMOE_H */

@@ -1,0 +1,309 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI (d2dmoe_amd.ops binds include/d2dmoe.h).
+
+Bars:  routing masks, counts and permutations bit-exact given the same predicted norms;
+       layer outputs within 1e-5 (float32) / 2e-2 (bfloat16) relative error, measured as
+       max|got - want| / max|want| against the oracle evaluated in float64 on the same stored inputs.
+"""
+import hashlib
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import d2dmoe_oracle as O
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+DEV = 'cuda:0'
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _ops():
+    from d2dmoe_amd import ops
+    return ops
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+# =================================================================== router ===========================
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('N,D,W,E', [(1, 64, 128, 4), (10, 64, 128, 4), (197, 768, 128, 128), (1576, 768, 128, 128),
+                                     (16, 2048, 256, 256), (70, 100, 37, 19)])
+def test_router_matches_oracle(dtype, N, D, W, E):
+    _say('router', dtype, N, D, W, E)
+    x, _, p = H.random_case(N, D, E, 8, W, seed=N + D, dtype=dtype)
+    got = _ops().router(x.to(DEV), p['router_w1'].to(DEV), p['router_w2'].to(DEV)).cpu()
+    want64 = O.router_forward(x.double(), p['router_w1'].double(), p['router_w2'].double())
+    assert got.dtype == dtype and got.shape == (N, E)
+    assert H.rel_err(got, want64) < H.tol_for(dtype)
+    if dtype == torch.bfloat16:
+        # against the oracle evaluated in bf16 itself: the same values except where the accumulation order moves a
+        # result across a rounding boundary (one bf16 ulp = 2^-8 relative)
+        want = O.router_forward(x, p['router_w1'], p['router_w2']).float()
+        diff = (got.float() - want).abs()
+        assert (diff <= want.abs() * 2 ** -6 + 1e-3).all()
+        assert (diff == 0).float().mean() > 0.9
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_router_other_activations(dtype):
+    x, _, p = H.random_case(33, 96, 12, 8, 40, seed=5, dtype=dtype)
+    for act, oact in [('tanh', 'identity'), ('gelu', 'abs'), ('leaky_relu', 'relu')]:
+        got = _ops().router(x.to(DEV), p['router_w1'].to(DEV), p['router_w2'].to(DEV), act, oact).cpu()
+        want = O.router_forward(x.double(), p['router_w1'].double(), p['router_w2'].double(), act, oact)
+        assert H.rel_err(got, want) < H.tol_for(dtype), (act, oact)
+
+
+# =================================================================== select ===========================
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('N,E', [(1, 1), (7, 5), (197, 128), (1576, 128), (50432, 128), (16, 256), (33, 1000), (64, 64)])
+def test_select_bit_exact(dtype, N, E):
+    _say('select', dtype, N, E)
+    g = torch.Generator().manual_seed(N * 31 + E)
+    norms = torch.randn(N, E, generator=g).abs().to(dtype)
+    if N >= 7:
+        norms[3] = 0.0                  # all-zero row -> everything selected
+        norms[5, E // 2] = float('nan')  # NaN row -> nothing selected
+        norms[6] = norms[6, 0]           # all-equal row
+    for tau in (0.0, 0.1, 0.5, 0.9, 0.99, 1.0):
+        scale = float(1.0 - tau)
+        routing, counts = _ops().select(norms.to(DEV), scale, want_counts=True)
+        want = O.gate_dynk_max(norms, tau)
+        assert routing.dtype == dtype
+        assert torch.equal(routing.cpu(), want), (tau, (routing.cpu() != want).sum().item())
+        assert torch.equal(counts.cpu().long(), want.float().sum(0).long())
+
+
+def test_select_threshold_fraction_convention():
+    """The bench's "threshold fraction f" enters as thr_scale = f; the module's tau enters as 1 - tau."""
+    g = torch.Generator().manual_seed(1)
+    norms = torch.randn(500, 128, generator=g).abs().bfloat16()
+    r, _ = _ops().select(norms.to(DEV), 0.9)
+    assert torch.equal(r.cpu(), O.gate_dynk_max_scaled(norms, 0.9))
+    assert torch.equal(r.cpu(), O.gate_dynk_max(norms, 1.0 - 0.9))
+
+
+# =================================================================== permutation ======================
+def _check_perm(routing_cpu):
+    N, E = routing_cpu.shape
+    off, tok, s, u, c = _ops().build_permutation(routing_cpu.to(DEV), reference_layout=True)
+    so, uo, co = O.extract_indices(routing_cpu)
+    oo, to = O.permutation_csr(routing_cpu)
+    assert torch.equal(off.cpu(), oo)
+    P = int(oo[-1])
+    assert torch.equal(tok.cpu()[:P], to)
+    assert torch.equal(c.cpu(), co)
+    assert torch.equal(s.cpu(), so), 'sort_indices differ from argsort(stable, descending)'
+    assert torch.equal(u.cpu(), uo), 'unsort_indices differ'
+    off2, tok2 = _ops().build_permutation(routing_cpu.to(DEV))
+    assert torch.equal(off2.cpu(), oo) and torch.equal(tok2.cpu()[:P], to)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('N,E,p', [(1, 1, 1.0), (1, 128, 0.5), (63, 4, 0.5), (64, 4, 0.5), (65, 5, 0.5), (197, 128, 0.02),
+                                   (1576, 128, 0.8), (1000, 33, 0.0), (1000, 33, 1.0), (4096, 256, 0.3),
+                                   (1111, 130, 0.6), (50432, 128, 0.79)])
+def test_permutation_bit_exact(dtype, N, E, p):
+    _say('perm', dtype, N, E, p)
+    g = torch.Generator().manual_seed(N + E)
+    routing = (torch.rand(N, E, generator=g) < p).to(dtype)
+    _check_perm(routing)
+
+
+def test_permutation_skewed_and_empty():
+    # Zipf-like expert popularity: a few experts take most tokens
+    g = torch.Generator().manual_seed(3)
+    w = torch.arange(1, 129).float() ** -1.2
+    routing = (torch.rand(5000, 128, generator=g) < (w * 3).clamp(max=1.0)).bfloat16()
+    _check_perm(routing)
+    # no tokens at all
+    off, tok = _ops().build_permutation(torch.empty(0, 16, dtype=torch.float32, device=DEV))
+    assert torch.equal(off.cpu(), torch.zeros(17, dtype=torch.int32))
+
+
+# =================================================================== experts ==========================
+def _experts_want(x, routing, p, act, residual=False):
+    return O.layer_from_routing(x.double(), O.upcast(p), routing.double(), act, 'all', residual)
+
+
+def _experts_got(x, routing, p, act, residual=False, path='generic', packed=None):
+    d = H.to_dev(p, DEV)
+    lb = d['last_bias'].view(-1) if 'last_bias' in d else None
+    if 'w_gate' in d:
+        return _ops().experts(x.to(DEV), routing.to(DEV), d['w_gate'], None, d['w_down'], d['w_up'], lb, act,
+                              residual, path, packed).cpu()
+    return _ops().experts(x.to(DEV), routing.to(DEV), d['w1'], d.get('b1'), d['w2'], None, lb, act, residual, path,
+                          packed).cpu()
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('N,D,E,Ed,density', [(10, 64, 4, 32, 0.5), (1, 64, 4, 32, 1.0), (197, 768, 128, 24, 0.8),
+                                              (197, 768, 128, 24, 0.02), (1576, 768, 128, 24, 0.79),
+                                              (77, 768, 24, 128, 0.5), (50, 100, 7, 5, 0.5), (20, 2048, 16, 64, 0.5)])
+def test_experts_generic_matches_oracle(dtype, N, D, E, Ed, density):
+    _say('experts generic', dtype, N, D, E, Ed, density)
+    x, routing, p = H.random_case(N, D, E, Ed, 8, seed=N + E, dtype=dtype, density=density)
+    got = _experts_got(x, routing, p, 'relu')
+    assert got.dtype == dtype
+    assert H.rel_err(got, _experts_want(x, routing, p, 'relu')) < H.tol_for(dtype)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('act', ['relu', 'gelu', 'tanh', 'leaky_relu'])
+def test_experts_generic_activations_bias_residual(dtype, act):
+    x, routing, p = H.random_case(70, 96, 10, 12, 8, seed=11, dtype=dtype)
+    assert H.rel_err(_experts_got(x, routing, p, act, residual=True), _experts_want(x, routing, p, act, True)) < H.tol_for(dtype)
+    q = {k: v for k, v in p.items() if k not in ('b1', 'last_bias')}
+    assert H.rel_err(_experts_got(x, routing, q, act), _experts_want(x, routing, q, act)) < H.tol_for(dtype)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_experts_generic_special_cases(dtype):
+    x, routing, p = H.random_case(40, 64, 6, 8, 8, seed=12, dtype=dtype)
+    # nothing routed -> last_bias only
+    got = _experts_got(x, torch.zeros_like(routing), p, 'relu')
+    assert torch.equal(got, p['last_bias'].expand(40, -1))
+    # everything routed == dense FFN with the experts concatenated (two library GEMMs)
+    ones = torch.ones_like(routing)
+    E, D, Ed = p['w1'].shape
+    W1 = p['w1'].double().permute(1, 0, 2).reshape(D, E * Ed)
+    dense = torch.relu(x.double() @ W1 + p['b1'].double().reshape(-1)) @ p['w2'].double().reshape(E * Ed, D)
+    dense = dense + p['last_bias'].double()
+    assert H.rel_err(_experts_got(x, ones, p, 'relu'), dense) < H.tol_for(dtype)
+    # weighted routing == the reference's 'masked' formulation
+    g = torch.Generator().manual_seed(1)
+    weights = (routing.float() * torch.rand(40, 6, generator=g)).to(dtype)
+    assert H.rel_err(_experts_got(x, weights, p, 'relu'), _experts_want(x, weights, p, 'relu')) < H.tol_for(dtype)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('act', ['gelu_tanh', 'relu', 'silu'])
+def test_experts_generic_gated(dtype, act):
+    x, routing, p = H.random_case(16, 256, 16, 64, 8, seed=13, dtype=dtype, gated=True, bias=False)
+    assert H.rel_err(_experts_got(x, routing, p, act), _experts_want(x, routing, p, act)) < H.tol_for(dtype)
+
+
+# =================================================================== whole layer ======================
+def _forward(x, p, tau, act='relu', norms_in=None, path='auto', packed=None, residual=False):
+    d = H.to_dev(p, DEV)
+    lb = d['last_bias'].view(-1) if 'last_bias' in d else None
+    x2 = x.reshape(-1, x.size(-1)).to(DEV)
+    nin = None if norms_in is None else norms_in.reshape(-1, norms_in.size(-1)).to(DEV).contiguous()
+    if 'w_gate' in d:
+        return _ops().forward(x2, d['router_w1'], d['router_w2'], float(1.0 - tau), d['w_gate'], None, d['w_down'],
+                              d['w_up'], lb, act, residual, nin, True, True, path, packed)
+    return _ops().forward(x2, d['router_w1'], d['router_w2'], float(1.0 - tau), d['w1'], d.get('b1'), d['w2'], None, lb,
+                          act, residual, nin, True, True, path, packed)
+
+
+@pytest.mark.parametrize('case', ['toy', 'vit197', 'gpt64', 'gated16'])
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_layer_against_golden_fixture(case, dtype):
+    """Parity mode: the oracle's predicted norms go in, so every later stage must reproduce the fixture."""
+    _say('fixture', case, dtype)
+    fx, x, p, c = H.fixture_inputs(case, dtype)
+    dt = 'f32' if dtype == torch.float32 else 'bf16'
+    norms = O.router_forward(x, p['router_w1'], p['router_w2'])
+    for tau in c['taus']:
+        tag = f'{dt}_tau{tau}'
+        out, routing, _, counts = _forward(x, p, tau, c['act'], norms_in=norms)
+        want_r = H.routing_from_bits(fx[f'routing_bits_{tag}'], c['E'])
+        assert torch.equal(routing.cpu().float(), want_r)
+        assert torch.equal(counts.cpu().long(), want_r.sum(0).long())
+        assert H.rel_err(out.cpu()[:32], torch.from_numpy(fx[f'out_{tag}'])) < H.tol_for(dtype)
+        off, tok, s, u, _ = _ops().build_permutation(routing, reference_layout=True)
+        assert np.array_equal(off.cpu().numpy(), fx[f'offsets_{tag}'])
+        assert np.array_equal(tok.cpu().numpy()[:int(off[-1])], fx[f'token_idx_{tag}'])
+        assert hashlib.sha256(s.cpu().numpy().tobytes()).hexdigest() == str(fx[f'sort_crc_{tag}'])
+        assert hashlib.sha256(u.cpu().numpy().tobytes()).hexdigest() == str(fx[f'unsort_crc_{tag}'])
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('tau', [0.1, 0.9])
+def test_layer_end_to_end_vit_shape(dtype, tau):
+    """Full path including the router on the GPU (BASELINE config 1 shape, 8 x 197 tokens).  The mask is a hard
+    compare on router outputs, so a different accumulation order can flip entries that sit within rounding of the
+    threshold; their number is reported and bounded, and outputs are compared on rows whose mask agrees."""
+    _say('e2e', dtype, tau)
+    N, D, E, Ed, W = 1576, 768, 128, 24, 128
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=77, dtype=dtype)
+    out, routing, norms, counts = _forward(x, p, tau)
+    norms_o = O.router_forward(x, p['router_w1'], p['router_w2'])
+    routing_o = O.gate_dynk_max(norms_o, tau)
+    mism = (routing.cpu() != routing_o)
+    frac = mism.float().mean().item()
+    _say(f'  mask mismatches vs oracle router: {int(mism.sum())} of {N * E} ({frac:.2e})')
+    assert frac < (1e-4 if dtype == torch.float32 else 2e-2)
+    # stage-wise: the GPU mask is exactly the oracle's gate applied to the GPU's own norms
+    assert torch.equal(routing.cpu(), O.gate_dynk_max(norms.cpu(), tau))
+    assert torch.equal(counts.cpu().long(), routing.cpu().float().sum(0).long())
+    want = O.layer_from_routing(x.double(), O.upcast(p), routing.cpu().double(), 'relu', 'all')
+    assert H.rel_err(out.cpu(), want) < H.tol_for(dtype)
+    same_rows = ~mism.any(dim=1)
+    want_o = O.layer_from_routing(x.double(), O.upcast(p), routing_o.double(), 'relu', 'all')
+    assert same_rows.float().mean() > 0.5
+    assert H.rel_err(out.cpu()[same_rows], want_o[same_rows]) < H.tol_for(dtype)
+
+
+def test_layer_skewed_norms_override():
+    """BASELINE config 3 in miniature: the router is bypassed by synthetic predicted norms |N(0,1)| x Zipf(1.2)."""
+    N, D, E, Ed = 2048, 768, 128, 24
+    x, _, p = H.random_case(N, D, E, Ed, 128, seed=5, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(9)
+    w = (torch.randperm(E, generator=g) + 1).float() ** -1.2
+    norms = (torch.randn(N, E, generator=g).abs() * (w / w.max())).bfloat16()
+    out, routing, _, counts = _forward(x, p, 1.0 - 0.9, norms_in=norms)
+    want_r = O.gate_dynk_max_scaled(norms, 0.9)
+    assert torch.equal(routing.cpu(), want_r)
+    assert torch.equal(counts.cpu().long(), want_r.float().sum(0).long())
+    want = O.layer_from_routing(x.double(), O.upcast(p), want_r.double(), 'relu', 'all')
+    assert H.rel_err(out.cpu(), want) < H.TOL_BF16
+    _say('  skew: max/mean tokens per expert =', (counts.max() / counts.float().mean()).item())
+
+
+# =================================================================== module drop-in ===================
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('mode', ['naive', 'hip', 'triton_atomic'])
+def test_module_modes_agree_and_do_not_sync(dtype, mode):
+    """The reference's own check (scripts/test_moe_implementations.py:36-85): every forward mode against 'masked'
+    on B=5, T=2, D=64, Ed=32, E=4, ReLU, dynk_max, tau=0.5; the kernel path must not synchronise with the host."""
+    from d2dmoe_amd import MoeficationMoE, MoeficationRouter
+    for rep in range(3):
+        torch.manual_seed(100 + rep)
+        moe = MoeficationMoE('test_moe', 64, 4, True, 32, torch.nn.ReLU, experts_class='custom_kernel')
+        moe.router = MoeficationRouter(64, 4, width=128, depth=2, bias=False, activation='relu', output_activation='abs')
+        moe = moe.to(DEV).to(dtype).eval()
+        moe.forward_mode = 'dynk_max'
+        moe.tau = 0.5
+        x = torch.randn(5, 2, 64, device=DEV, dtype=dtype)
+        with torch.no_grad():
+            want, gating = moe(x)
+            moe.experts.forward_mode = mode
+            moe(x)  # first call builds caches / workspaces
+            if mode != 'naive':
+                torch.cuda.set_sync_debug_mode('error')
+            try:
+                got, gating2 = moe(x)
+            finally:
+                torch.cuda.set_sync_debug_mode('default')
+        assert torch.equal(gating['test_moe'][0], gating2['test_moe'][0])
+        assert H.rel_err(got, want) < H.tol_for(dtype)
+
+
+def test_module_execute_all_gated_hip():
+    from d2dmoe_amd import MoeficationMoE, MoeficationRouter
+    torch.manual_seed(3)
+    moe = MoeficationMoE('g', 256, 16, False, 64, torch.nn.GELU, experts_class='execute_all', add_intermediate_gating=True)
+    moe.router = MoeficationRouter(256, 16, width=32, depth=2, bias=False, activation='relu', output_activation='abs')
+    moe = moe.to(DEV).bfloat16().eval()
+    moe.forward_mode, moe.tau = 'dynk_max', 0.9
+    x = torch.randn(1, 16, 256, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        want, g1 = moe(x)
+        moe.experts.forward_mode = 'hip'
+        got, g2 = moe(x)
+    assert torch.equal(g1['g'][0], g2['g'][0])
+    assert H.rel_err(got, want) < 3e-2   # both sides are bf16 evaluations here
