@@ -186,6 +186,81 @@ def test_experts_generic_gated(dtype, act):
     assert H.rel_err(_experts_got(x, routing, p, act), _experts_want(x, routing, p, act)) < H.tol_for(dtype)
 
 
+# =================================================================== experts, bf16 MFMA ===============
+def _packed_for(p, act='relu'):
+    d = H.to_dev(p, DEV)
+    E, D, Ed = d['w1'].shape
+    sh = _ops().make_shape(0, D, E, Ed, 0, 1, act)
+    packed = _ops().pack_weights(sh, d['w1'], d.get('b1'), d['w2'])
+    assert packed is not None, 'no MFMA kernel for this shape'
+    return packed
+
+
+@pytest.mark.parametrize('N,E,Ed,density', [(197, 128, 24, 0.8), (197, 128, 24, 0.02), (1576, 128, 24, 0.79), (64, 128, 24, 1.0),
+                                            (65, 128, 24, 0.5), (1, 128, 24, 0.5), (300, 24, 128, 0.5), (130, 100, 30, 0.5),
+                                            (100, 7, 5, 0.5)])
+def test_experts_mfma_dense_matches_oracle(N, E, Ed, density):
+    _say('experts mfma', N, E, Ed, density)
+    x, routing, p = H.random_case(N, 768, E, Ed, 8, seed=N + E, dtype=torch.bfloat16, density=density)
+    packed = _packed_for(p)
+    got = _experts_got(x, routing, p, 'relu', path='mfma_dense', packed=packed)
+    assert H.rel_err(got, _experts_want(x, routing, p, 'relu')) < H.TOL_BF16
+    # the two HIP paths share their rounding points (h rounded to bf16, float32 sums, one final rounding)
+    assert H.rel_err(got, _experts_got(x, routing, p, 'relu')) < 1e-2
+
+
+@pytest.mark.parametrize('act', ['relu', 'gelu', 'tanh', 'leaky_relu'])
+def test_experts_mfma_dense_activations_bias_residual_weights(act):
+    x, routing, p = H.random_case(200, 768, 128, 24, 8, seed=21, dtype=torch.bfloat16, density=0.6)
+    packed = _packed_for(p, act)
+    got = _experts_got(x, routing, p, act, residual=True, path='mfma_dense', packed=packed)
+    assert H.rel_err(got, _experts_want(x, routing, p, act, True)) < H.TOL_BF16
+    q = {k: v for k, v in p.items() if k not in ('b1', 'last_bias')}
+    got = _experts_got(x, routing, q, act, path='mfma_dense', packed=_packed_for(q, act))
+    assert H.rel_err(got, _experts_want(x, routing, q, act)) < H.TOL_BF16
+    g = torch.Generator().manual_seed(2)
+    weights = (routing.float() * torch.rand(200, 128, generator=g)).bfloat16()
+    got = _experts_got(x, weights, p, act, path='mfma_dense', packed=packed)
+    assert H.rel_err(got, _experts_want(x, weights, p, act)) < H.TOL_BF16
+    # nothing routed -> last_bias only (every chunk is skipped)
+    got = _experts_got(x, torch.zeros_like(routing), p, act, path='mfma_dense', packed=packed)
+    assert torch.equal(got, p['last_bias'].expand(200, -1))
+
+
+def test_experts_mfma_dense_full_size_properties():
+    """50432 tokens (BASELINE config 2): oracle on a slice of rows, the generic HIP kernel on all rows, and
+    determinism (two runs give identical bits)."""
+    N = 50432
+    x, routing, p = H.random_case(N, 768, 128, 24, 8, seed=31, dtype=torch.bfloat16, density=0.79)
+    packed = _packed_for(p)
+    d = H.to_dev(p, DEV)
+    xg, rg = x.to(DEV), routing.to(DEV)
+    lb = d['last_bias'].view(-1)
+    a = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, 'relu', False, 'mfma_dense', packed)
+    b = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, 'relu', False, 'mfma_dense', packed)
+    assert torch.equal(a, b)
+    gen = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, 'relu', False, 'generic', None)
+    assert H.rel_err(a, gen) < 1e-2
+    rows = torch.cat([torch.arange(0, 128), torch.arange(25000, 25064), torch.arange(N - 64, N)])
+    want = _experts_want(x[rows], routing[rows], p, 'relu')
+    assert H.rel_err(a.cpu()[rows], want) < H.TOL_BF16
+
+
+def test_packed_weights_cache_tracks_parameter_updates():
+    from d2dmoe_amd import HipKernelExperts
+    torch.manual_seed(0)
+    ex = HipKernelExperts(768, 128, 2, 24, 'without_last', torch.nn.ReLU).to(DEV).bfloat16()
+    ex.forward_mode = 'hip'
+    x = torch.randn(70, 768, device=DEV, dtype=torch.bfloat16)
+    r = (torch.rand(70, 128, device=DEV) < 0.5).bfloat16()
+    with torch.no_grad():
+        a = ex(x, r)
+        assert ex._packed.buf is not None
+        ex.w2.mul_(2.0)           # in-place update bumps the version counter -> repack
+        b = ex(x, r)
+    assert H.rel_err(b, 2 * a.float()) < 1e-2
+
+
 # =================================================================== whole layer ======================
 def _forward(x, p, tau, act='relu', norms_in=None, path='auto', packed=None, residual=False):
     d = H.to_dev(p, DEV)
@@ -214,6 +289,11 @@ def test_layer_against_golden_fixture(case, dtype):
         assert torch.equal(routing.cpu().float(), want_r)
         assert torch.equal(counts.cpu().long(), want_r.sum(0).long())
         assert H.rel_err(out.cpu()[:32], torch.from_numpy(fx[f'out_{tag}'])) < H.tol_for(dtype)
+        if dtype == torch.bfloat16 and c['D'] == 768:
+            out_m, routing_m, _, _ = _forward(x, p, tau, c['act'], norms_in=norms, path='mfma_dense',
+                                              packed=_packed_for(p, c['act']))
+            assert torch.equal(routing_m, routing)
+            assert H.rel_err(out_m.cpu()[:32], torch.from_numpy(fx[f'out_{tag}'])) < H.TOL_BF16
         off, tok, s, u, _ = _ops().build_permutation(routing, reference_layout=True)
         assert np.array_equal(off.cpu().numpy(), fx[f'offsets_{tag}'])
         assert np.array_equal(tok.cpu().numpy()[:int(off[-1])], fx[f'token_idx_{tag}'])
@@ -230,7 +310,8 @@ def test_layer_end_to_end_vit_shape(dtype, tau):
     _say('e2e', dtype, tau)
     N, D, E, Ed, W = 1576, 768, 128, 24, 128
     x, _, p = H.random_case(N, D, E, Ed, W, seed=77, dtype=dtype)
-    out, routing, norms, counts = _forward(x, p, tau)
+    packed = _packed_for(p) if dtype == torch.bfloat16 else None
+    out, routing, norms, counts = _forward(x, p, tau, packed=packed)
     norms_o = O.router_forward(x, p['router_w1'], p['router_w2'])
     routing_o = O.gate_dynk_max(norms_o, tau)
     mism = (routing.cpu() != routing_o)
