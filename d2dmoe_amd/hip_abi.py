@@ -10,7 +10,8 @@ import os
 from ctypes import POINTER, Structure, c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
 
 LIB_NAME = 'libd2dmoe_hip.so'
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
+# D2DMOE_LIB names another build of the same library (a full path); default is the in-tree one.
+LIB_PATH = os.environ.get('D2DMOE_LIB') or os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 # enums of include/d2dmoe.h
 F32, BF16 = 0, 1
