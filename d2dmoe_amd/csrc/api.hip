@@ -133,7 +133,7 @@ int d2dmoe_build_permutation(const void* routing, int64_t n_tokens, int32_t n_ex
 
 size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape) {
   if (check_shape(shape) != D2DMOE_OK) return 0;
-  if (!mfma_dense_supported(*shape)) return 0;
+  if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape)) return 0;
   return mfma_packed_bytes(*shape);
 }
 
@@ -142,7 +142,8 @@ int d2dmoe_pack_weights(const d2dmoe_shape* shape, const void* w1, const void* b
   int st = check_shape(shape);
   if (st != D2DMOE_OK) return st;
   if (!w1 || !w2 || !packed) return D2DMOE_E_NULL;
-  if (!mfma_dense_supported(*shape)) return D2DMOE_E_UNSUPPORTED;
+  if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape)) return D2DMOE_E_UNSUPPORTED;
+  if (mfma_router_supported(*shape) && (!router_w1 || !router_w2)) return D2DMOE_E_NULL;
   if (packed_bytes < mfma_packed_bytes(*shape) || !aligned16(packed)) return D2DMOE_E_WORKSPACE;
   return (int)launch_mfma_pack(*shape, w1, b1, w2, w_up, router_w1, router_w2, packed, (hipStream_t)stream);
 }
@@ -194,6 +195,13 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   if (!workspace || workspace_bytes < plan.total || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
   char* ws = (char*)workspace;
   const void* norms = norms_in;
+  if (norms == nullptr && packed != nullptr && mfma_router_supported(sh)) {
+    // fused router + selection on MFMA: no hidden/norms round trip through the workspace
+    hipError_t e = launch_mfma_router_select(sh, x, packed, routing, norms_out, counts, thr_scale, (hipStream_t)stream);
+    if (e != hipSuccess) return (int)e;
+    return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,
+                          plan.total - plan.perm_off, stream);
+  }
   if (norms == nullptr) {
     if (!router_w1 || !router_w2) return D2DMOE_E_NULL;
     if (sh.router_width <= 0) return D2DMOE_E_SHAPE;

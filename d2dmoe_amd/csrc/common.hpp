@@ -47,7 +47,7 @@ template <> struct Elem<bf16_t> {
 // Definitions follow the reference's kernel-side helpers (utils.py:730-756).
 __device__ inline float apply_act(int act, float x) {
   switch (act) {
-    case D2DMOE_ACT_RELU: return x >= 0.f ? x : 0.f;
+    case D2DMOE_ACT_RELU: return fmaxf(x, 0.f);   // == (x >= 0 ? x : 0), NaN -> 0 as well
     case D2DMOE_ACT_GELU: return x * 0.5f * (1.f + erff(x * 0.70710678118654752440f));
     case D2DMOE_ACT_TANH: return tanhf(x);
     case D2DMOE_ACT_LEAKY_RELU: return x >= 0.f ? x : 0.01f * x;

@@ -31,8 +31,36 @@ struct PackedLayout {
   int n_chunks;    // ceil(hidden / MD_HC)
   int hidden_pad;  // n_chunks * MD_HC
   int pieces;      // weight fragments per (wave, chunk): D/16*2 for W1 followed by 16*D/128 for W2
-  size_t w_off, b1_off, eidx_off, total;
+  size_t w_off, b1_off, eidx_off, r1_off, r2_off, total;   // r1/r2: router fragments (present when routed)
+  bool has_dense, has_router;
 };
+
+static size_t dense_lds_bytes(const d2dmoe_shape& sh) {
+  const int hidden = sh.n_experts * sh.expert_dim;
+  const int n_chunks = (hidden + MD_HC - 1) / MD_HC;
+  const int KS1 = sh.d_model / 16;
+  return (size_t)(2 * KS1 * 64 + 2 * MD_KS2 * 64) * 16            // x fragments, h fragments
+         + (size_t)MD_BM * (sh.n_experts + 2) * 2                  // routing tile, rows padded by 2 elements
+         + (size_t)n_chunks * MD_HC * 3                            // b1 (bf16) and expert index (uint8) per neuron
+         + (size_t)(sh.n_experts + n_chunks + 1) * sizeof(int);    // expert-activity flags, active-chunk list
+}
+
+// The fused experts kernel is instantiated for D = 768 (ViT-B, GPT-2 small, BERT-base), ungated experts, bf16.
+bool mfma_dense_supported(const d2dmoe_shape& sh) {
+  if (sh.dtype != D2DMOE_BF16 || sh.gated) return false;
+  if (sh.d_model != 768) return false;
+  if (sh.n_experts > 256) return false;          // expert indices are staged as uint8
+  return dense_lds_bytes(sh) <= 160 * 1024;      // x tile + h tile + routing tile + bias/expert-index tables
+}
+
+// The fused router+select kernel covers the D2DMoE router: bf16, depth 2, ReLU hidden / abs output activation,
+// width and expert count both 128 or both 256, D a multiple of 16.
+bool mfma_router_supported(const d2dmoe_shape& sh) {
+  if (sh.dtype != D2DMOE_BF16 || sh.router_width <= 0) return false;
+  if (sh.router_activation != D2DMOE_ACT_RELU || sh.router_output_activation != D2DMOE_ACT_ABS) return false;
+  if (sh.d_model % 16 != 0) return false;
+  return (sh.router_width == 128 && sh.n_experts == 128) || (sh.router_width == 256 && sh.n_experts == 256);
+}
 
 static PackedLayout packed_layout(const d2dmoe_shape& sh) {
   PackedLayout L;
@@ -41,27 +69,16 @@ static PackedLayout packed_layout(const d2dmoe_shape& sh) {
   L.hidden_pad = L.n_chunks * MD_HC;
   L.pieces = sh.d_model / 16 * 2 + MD_KS2 * (sh.d_model / 128);
   size_t off = 0;
-  L.w_off = off;    off += (size_t)MD_WAVES * L.n_chunks * L.pieces * 64 * 16;
-  L.b1_off = off;   off += (size_t)L.hidden_pad * 2;   // bf16
-  L.eidx_off = off; off += (size_t)L.hidden_pad;       // uint8
+  L.has_dense = mfma_dense_supported(sh);
+  L.w_off = off;    if (L.has_dense) off += (size_t)MD_WAVES * L.n_chunks * L.pieces * 64 * 16;
+  L.b1_off = off;   if (L.has_dense) off += (size_t)L.hidden_pad * 2;   // bf16
+  L.eidx_off = off; if (L.has_dense) off += (size_t)L.hidden_pad;       // uint8
+  off = (off + 255) / 256 * 256;
+  L.has_router = mfma_router_supported(sh);
+  L.r1_off = off;   if (L.has_router) off += (size_t)sh.router_width * sh.d_model * 2;
+  L.r2_off = off;   if (L.has_router) off += (size_t)sh.n_experts * sh.router_width * 2;
   L.total = (off + 255) / 256 * 256;
   return L;
-}
-
-static size_t dense_lds_bytes(const d2dmoe_shape& sh) {
-  const PackedLayout L = packed_layout(sh);
-  const int KS1 = sh.d_model / 16;
-  return (size_t)(2 * KS1 * 64 + 2 * MD_KS2 * 64) * 16            // x fragments, h fragments
-         + (size_t)MD_BM * (sh.n_experts + 2) * 2                  // routing tile, rows padded by 2 elements
-         + (size_t)L.hidden_pad * 3                                // b1 (bf16) and expert index (uint8) per neuron
-         + (size_t)(sh.n_experts + L.n_chunks + 1) * sizeof(int);  // expert-activity flags, active-chunk list
-}
-
-bool mfma_dense_supported(const d2dmoe_shape& sh) {
-  if (sh.dtype != D2DMOE_BF16 || sh.gated) return false;
-  if (sh.d_model != 768) return false;
-  if (sh.n_experts > 256) return false;          // expert indices are staged as uint8
-  return dense_lds_bytes(sh) <= 160 * 1024;      // x tile + h tile + routing tile + bias/expert-index tables
 }
 
 size_t mfma_packed_bytes(const d2dmoe_shape& sh) { return packed_layout(sh).total; }
@@ -119,11 +136,49 @@ __global__ void pack_bias_kernel(const bf16_t* __restrict__ b1, bf16_t* __restri
   eidx[h] = (uint8_t)((h < hidden) ? (h / Ed) : 0);
 }
 
+// Router fragments.
+//   W1 fragments [kstep D/16][row-tile W/32][lane][8]:  row w = rt*32 + c, d = kstep*16 + 8g + i     value W1[w][d]
+//   W2 fragments [kstep2 W/16][row-tile E/32][lane][8]: row e = et*32 + c,
+//       w = (ks2/2)*32 + (ks2%2)*16 + 8*(i/4) + 4g + (i%4)  (the k order in which the first GEMM leaves the hidden
+//       activations in registers)                                                                   value W2[e][w]
+__global__ void pack_router_kernel(const bf16_t* __restrict__ rw1, const bf16_t* __restrict__ rw2, bf16_t* __restrict__ d1,
+                                   bf16_t* __restrict__ d2, int D, int W, int E) {
+  const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t n1 = (int64_t)W * D / 8, n2 = (int64_t)E * W / 8;
+  const int lane = (int)(p % 64);
+  const int g = lane / 32, c = lane % 32;
+  if (p < n1) {
+    const int WT = W / 32;
+    const int64_t q = p / 64;
+    const int rt = (int)(q % WT), ks = (int)(q / WT);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) d1[p * 8 + i] = rw1[(int64_t)(rt * 32 + c) * D + ks * 16 + 8 * g + i];
+  } else if (p < n1 + n2) {
+    const int64_t pp = p - n1;
+    const int ET = E / 32;
+    const int64_t q = pp / 64;
+    const int et = (int)(q % ET), ks2 = (int)(q / ET);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int wi = (ks2 / 2) * 32 + (ks2 % 2) * 16 + 8 * (i / 4) + 4 * g + (i % 4);
+      d2[pp * 8 + i] = rw2[(int64_t)(et * 32 + c) * W + wi];
+    }
+  }
+}
+
 hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                             const void* router_w1, const void* router_w2, void* packed, hipStream_t s) {
-  (void)w_up; (void)router_w1; (void)router_w2;
+  (void)w_up;
   const PackedLayout L = packed_layout(sh);
   char* base = (char*)packed;
+  if (L.has_router) {
+    if (router_w1 == nullptr || router_w2 == nullptr) return hipErrorInvalidValue;
+    const int64_t n = ((int64_t)sh.router_width * sh.d_model + (int64_t)sh.n_experts * sh.router_width) / 8;
+    hipLaunchKernelGGL(pack_router_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const bf16_t*)router_w1,
+                       (const bf16_t*)router_w2, (bf16_t*)(base + L.r1_off), (bf16_t*)(base + L.r2_off), sh.d_model,
+                       sh.router_width, sh.n_experts);
+  }
+  if (!L.has_dense) return hipGetLastError();
   const int64_t n_items = (int64_t)MD_WAVES * L.n_chunks * L.pieces * 64;
   const unsigned blocks = (unsigned)((n_items + 255) / 256);
   hipLaunchKernelGGL(pack_stream_kernel, dim3(blocks), dim3(256), 0, s, (const bf16_t*)w1, (const bf16_t*)w2,
@@ -164,7 +219,7 @@ __device__ inline uint32_t pack2_bf16(float lo, float hi) {
 // LDS-only workgroup barrier: waits for this wave's LDS operations, not for its outstanding global loads.
 __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <int D, int ACT>
+template <int D, int ACT, bool ED8>
 __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ routing, const bf16x8* __restrict__ wp,
     const bf16_t* __restrict__ b1p, const uint8_t* __restrict__ eidx, const bf16_t* __restrict__ last_bias,
@@ -298,21 +353,32 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(
         for (int q = 0; q < 4; ++q) {
           const int hb = chunk * MD_HC + w * 64 + rt * 32 + 8 * q + 4 * g;
           const uint2 bq = *(const uint2*)(b1s + hb);      // 4 bf16
-          const uint32_t eq = *(const uint32_t*)(eis + hb);  // 4 uint8
           bias[q * 4 + 0] = __uint_as_float(bq.x << 16); bias[q * 4 + 1] = __uint_as_float(bq.x & 0xffff0000u);
           bias[q * 4 + 2] = __uint_as_float(bq.y << 16); bias[q * 4 + 3] = __uint_as_float(bq.y & 0xffff0000u);
-          ei[q * 4 + 0] = eq & 0xff; ei[q * 4 + 1] = (eq >> 8) & 0xff;
-          ei[q * 4 + 2] = (eq >> 16) & 0xff; ei[q * 4 + 3] = eq >> 24;
+          if (ED8) {
+            // Ed is a multiple of 8: the aligned block of 8 neurons this q covers belongs to one expert, the same for
+            // every lane, so one routing value per (q, token tile) serves four accumulator rows
+            ei[q * 4] = eis[hb & ~7];
+          } else {
+            const uint32_t eq = *(const uint32_t*)(eis + hb);  // 4 uint8
+            ei[q * 4 + 0] = eq & 0xff; ei[q * 4 + 1] = (eq >> 8) & 0xff;
+            ei[q * 4 + 2] = (eq >> 16) & 0xff; ei[q * 4 + 3] = eq >> 24;
+          }
         }
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt) {
           const bf16_t* rrow = rs + (tt * 32 + c32) * RS;
           float hv[16];
+          float rq[4];
+          if (ED8) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) rq[q] = bf16_to_f32(rrow[ei[q * 4]]);
+          }
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             float v = acc1[rt][tt][r] + bias[r];
             v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(act_rt, v);
-            hv[r] = v * bf16_to_f32(rrow[ei[r]]);
+            hv[r] = v * (ED8 ? rq[r / 4] : bf16_to_f32(rrow[ei[r]]));
           }
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
@@ -375,7 +441,7 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(
   }
 }
 
-template <int D, int ACT>
+template <int D, int ACT, bool ED8>
 static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                                    const void* last_bias, void* out, hipStream_t s) {
   const PackedLayout L = packed_layout(sh);
@@ -384,7 +450,7 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   const size_t lds = dense_lds_bytes(sh);
   if (lds > 160 * 1024) return hipErrorInvalidValue;
   static_assert(KS1 * 16 == D, "D must be a multiple of 16");
-  auto kern = experts_mfma_dense_kernel<D, ACT>;
+  auto kern = experts_mfma_dense_kernel<D, ACT, ED8>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   const unsigned grid = (unsigned)cdiv64(sh.n_tokens, MD_BM);
@@ -395,13 +461,154 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   return hipGetLastError();
 }
 
+template <int D, int ACT>
+static hipError_t launch_dense_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
+                                   const void* last_bias, void* out, hipStream_t s) {
+  if (sh.expert_dim % 8 == 0) return launch_dense_cfg<D, ACT, true>(sh, x, routing, packed, last_bias, out, s);
+  return launch_dense_cfg<D, ACT, false>(sh, x, routing, packed, last_bias, out, s);
+}
+
 hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                              const void* last_bias, void* out, hipStream_t s) {
   switch (sh.activation) {
-    case D2DMOE_ACT_RELU: return launch_dense_cfg<768, D2DMOE_ACT_RELU>(sh, x, routing, packed, last_bias, out, s);
-    case D2DMOE_ACT_GELU: return launch_dense_cfg<768, D2DMOE_ACT_GELU>(sh, x, routing, packed, last_bias, out, s);
-    default: return launch_dense_cfg<768, -1>(sh, x, routing, packed, last_bias, out, s);
+    case D2DMOE_ACT_RELU: return launch_dense_act<768, D2DMOE_ACT_RELU>(sh, x, routing, packed, last_bias, out, s);
+    case D2DMOE_ACT_GELU: return launch_dense_act<768, D2DMOE_ACT_GELU>(sh, x, routing, packed, last_bias, out, s);
+    default: return launch_dense_act<768, -1>(sh, x, routing, packed, last_bias, out, s);
   }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Fused router MLP + dynamic-k selection (moefication.py:328-330 and :80-85).
+// One wave owns 32 tokens end to end; nothing goes through LDS or HBM between the stages:
+//   GEMM1  H1^T[W, 32 tokens] = W1 . X^T          A = W1 fragments, B = x read straight from its rows
+//          relu, round to bf16 -> the accumulators already sit in B-fragment position for the next product
+//   GEMM2  NORMS^T[E, 32 tokens] = W2 . H1^T       A = W2 fragments (k order matched at packing)
+//          abs, round to bf16; per-token maximum = in-lane maximum + one cross-half exchange (NaN-propagating);
+//          thr = bf16(max * thr_scale); routing = norms >= thr ? 1 : 0
+// A lane ends up with one token and 4 consecutive experts per accumulator quad, stored as 8-byte pieces.
+// Optional outputs: the norms, and per-expert token counts (wave ballots + one integer atomic per expert).
+// ---------------------------------------------------------------------------------------------------
+template <int WT, int ET>
+__global__ __launch_bounds__(256) void router_select_mfma_kernel(
+    const bf16_t* __restrict__ x, const bf16x8* __restrict__ w1f, const bf16x8* __restrict__ w2f,
+    bf16_t* __restrict__ routing, bf16_t* __restrict__ norms_out, int32_t* __restrict__ counts, int64_t N, int D,
+    float thr_scale) {
+  constexpr int E = ET * 32;
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 5, c32 = lane & 31;
+  const int64_t tok0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 32;
+  if (tok0 >= N) return;   // whole wave; the kernel has no barriers
+  const int64_t token = tok0 + c32;
+  const bool valid = token < N;
+  const bf16x8* xrow = (const bf16x8*)(x + (valid ? token : (N - 1)) * D);
+  const int KS1 = D / 16;
+
+  f32x16 acc1[WT];
+#pragma unroll
+  for (int a = 0; a < WT; ++a)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc1[a][r] = 0.f;
+  for (int ks = 0; ks < KS1; ++ks) {
+    const bf16x8 b = xrow[2 * ks + g];
+#pragma unroll
+    for (int rt = 0; rt < WT; ++rt) {
+      const bf16x8 a = w1f[(int64_t)(ks * WT + rt) * 64 + lane];
+      acc1[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc1[rt], 0, 0, 0);
+    }
+  }
+  // hidden activations as B fragments of the second product
+  bf16x8 hb[2 * WT];
+#pragma unroll
+  for (int rt = 0; rt < WT; ++rt)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      uint4 pk;
+      pk.x = pack2_bf16(fmaxf(acc1[rt][half * 8 + 0], 0.f), fmaxf(acc1[rt][half * 8 + 1], 0.f));
+      pk.y = pack2_bf16(fmaxf(acc1[rt][half * 8 + 2], 0.f), fmaxf(acc1[rt][half * 8 + 3], 0.f));
+      pk.z = pack2_bf16(fmaxf(acc1[rt][half * 8 + 4], 0.f), fmaxf(acc1[rt][half * 8 + 5], 0.f));
+      pk.w = pack2_bf16(fmaxf(acc1[rt][half * 8 + 6], 0.f), fmaxf(acc1[rt][half * 8 + 7], 0.f));
+      __builtin_memcpy(&hb[rt * 2 + half], &pk, 16);
+    }
+  f32x16 acc2[ET];
+#pragma unroll
+  for (int a = 0; a < ET; ++a)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc2[a][r] = 0.f;
+#pragma unroll
+  for (int ks2 = 0; ks2 < 2 * WT; ++ks2) {
+#pragma unroll
+    for (int et = 0; et < ET; ++et) {
+      const bf16x8 a = w2f[(int64_t)(ks2 * ET + et) * 64 + lane];
+      acc2[et] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, hb[ks2], acc2[et], 0, 0, 0);
+    }
+  }
+  // norms (bf16 values held as float), per-token maximum
+  float m = -INFINITY;
+#pragma unroll
+  for (int et = 0; et < ET; ++et)
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      const uint32_t pk = pack2_bf16(fabsf(acc2[et][r]), fabsf(acc2[et][r + 1]));
+      acc2[et][r] = __uint_as_float(pk << 16);
+      acc2[et][r + 1] = __uint_as_float(pk & 0xffff0000u);
+      m = nanmax(m, nanmax(acc2[et][r], acc2[et][r + 1]));
+    }
+  m = nanmax(m, __shfl_xor(m, 32, kWave));
+  const float thr = __uint_as_float(pack2_bf16(m * thr_scale, 0.f) << 16);
+#pragma unroll
+  for (int et = 0; et < ET; ++et) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e0 = et * 32 + 8 * q + 4 * g;
+      bool on[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) on[s] = acc2[et][q * 4 + s] >= thr;
+      if (valid) {
+        uint2 rv;
+        rv.x = (on[0] ? 0x3F80u : 0u) | (on[1] ? 0x3F800000u : 0u);   // bf16 1.0 = 0x3F80
+        rv.y = (on[2] ? 0x3F80u : 0u) | (on[3] ? 0x3F800000u : 0u);
+        *(uint2*)(routing + token * E + e0) = rv;
+        if (norms_out != nullptr) {
+          uint2 nv;
+          nv.x = (__float_as_uint(acc2[et][q * 4 + 0]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 1]) & 0xffff0000u);
+          nv.y = (__float_as_uint(acc2[et][q * 4 + 2]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 3]) & 0xffff0000u);
+          *(uint2*)(norms_out + token * E + e0) = nv;
+        }
+      }
+      if (counts != nullptr) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const unsigned long long bal = __ballot(on[s] && valid);
+          if (lane == 0) {
+            const int lo = __popcll(bal & 0xffffffffull), hi = __popcll(bal >> 32);
+            if (lo) atomicAdd(counts + et * 32 + 8 * q + s, lo);
+            if (hi) atomicAdd(counts + et * 32 + 8 * q + 4 + s, hi);
+          }
+        }
+      }
+    }
+  }
+}
+
+hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
+                                     void* norms_out, int32_t* counts, float thr_scale, hipStream_t s) {
+  const PackedLayout L = packed_layout(sh);
+  if (!L.has_router) return hipErrorInvalidValue;
+  const char* base = (const char*)packed;
+  if (counts != nullptr) {
+    hipError_t e = launch_fill_i32(counts, sh.n_experts, 0, s);
+    if (e != hipSuccess) return e;
+  }
+  const unsigned grid = (unsigned)cdiv64(sh.n_tokens, 128);
+  if (sh.router_width == 128)
+    hipLaunchKernelGGL((router_select_mfma_kernel<4, 4>), dim3(grid), dim3(256), 0, s, (const bf16_t*)x,
+                       (const bf16x8*)(base + L.r1_off), (const bf16x8*)(base + L.r2_off), (bf16_t*)routing,
+                       (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+  else
+    hipLaunchKernelGGL((router_select_mfma_kernel<8, 8>), dim3(grid), dim3(256), 0, s, (const bf16_t*)x,
+                       (const bf16x8*)(base + L.r1_off), (const bf16x8*)(base + L.r2_off), (bf16_t*)routing,
+                       (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+  return hipGetLastError();
 }
 
 }  // namespace d2dmoe

@@ -35,9 +35,12 @@ hipError_t launch_experts_generic(const d2dmoe_shape& sh, const void* x, const v
 
 // ---- bf16 MFMA kernels (kernels_mfma.hip) ----
 bool mfma_dense_supported(const d2dmoe_shape& sh);
+bool mfma_router_supported(const d2dmoe_shape& sh);
 size_t mfma_packed_bytes(const d2dmoe_shape& sh);
 hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                             const void* router_w1, const void* router_w2, void* packed, hipStream_t s);
+hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
+                                     void* norms_out, int32_t* counts, float thr_scale, hipStream_t s);
 hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                              const void* last_bias, void* out, hipStream_t s);
 

@@ -71,16 +71,18 @@ class _PackedCache:
     storage pointer, device or dtype)."""
 
     def __init__(self):
-        self.key = None
-        self.buf: Optional[torch.Tensor] = None
+        self.slots = {}   # with / without router section -> (key, buffer)
 
     def get(self, shape, tensors):
         key = tuple((t.data_ptr(), t._version, t.dtype, t.device) if t is not None else None for t in tensors)
-        key = key + (shape.d_model, shape.n_experts, shape.expert_dim, shape.gated)
-        if key != self.key:
-            self.buf = ops.pack_weights(shape, *tensors)
-            self.key = key
-        return self.buf
+        key = key + (shape.d_model, shape.n_experts, shape.expert_dim, shape.gated, shape.router_width,
+                     shape.router_activation, shape.router_output_activation)
+        slot = shape.router_width > 0
+        cached = self.slots.get(slot)
+        if cached is None or cached[0] != key:
+            cached = (key, ops.pack_weights(shape, *tensors))
+            self.slots[slot] = cached
+        return cached[1]
 
 
 class HipKernelExperts(ExpertsLayer):
@@ -129,12 +131,13 @@ class HipKernelExperts(ExpertsLayer):
         self._forward_mode = value
 
     # -- derived buffers --------------------------------------------------------------------
-    def packed_weights(self, router_w1=None, router_w2=None):
+    def packed_weights(self, router_w1=None, router_w2=None, router_activation='relu', router_output_activation='abs'):
         if not self.w1.is_cuda or self.w1.dtype != torch.bfloat16:
             return None
         sh = ops.make_shape(0, self.hidden_dim, self.num_experts, self.expert_dim,
                             router_w1.size(0) if router_w1 is not None else 0, ops._dtype_code(self.w1),
-                            self.activation_str)
+                            self.activation_str, router_activation=router_activation,
+                            router_output_activation=router_output_activation)
         return self._packed.get(sh, (self.w1, self.b1, self.w2, None, router_w1, router_w2))
 
     # -- forward ----------------------------------------------------------------------------

@@ -175,12 +175,12 @@ class MoeficationMoE(MoELayer):
             else:
                 norms_in = None
                 rw1, rw2 = router.layers[0].weight, router.layers[2].weight
+            ract = router.activation if router.activation in ACT else 'relu'
+            roact = router.output_activation if router.output_activation in ACT else 'abs'
             out, routing, _, _ = ops.forward(
                 x2, rw1, rw2, float(1.0 - self.tau), ex.w1, ex.b1, ex.w2, None, last_bias, ex.activation_str,
                 self.add_residual_connection, norms_in=norms_in, path=ex.kernel_path,
-                packed=ex.packed_weights(rw1, rw2),
-                router_activation=router.activation if router.activation in ACT else 'relu',
-                router_output_activation=router.output_activation if router.output_activation in ACT else 'abs')
+                packed=ex.packed_weights(rw1, rw2, ract, roact), router_activation=ract, router_output_activation=roact)
             routing_tensor = routing.view(*orig_size[:-1], self.num_experts)
             return out.view(orig_size), {self.name: (routing_tensor,)}
         routing_tensor = self.gate(x)

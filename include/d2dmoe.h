@@ -148,11 +148,15 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
                    const void* last_bias, const void* packed, void* out, int32_t path,
                    void* workspace, size_t workspace_bytes, void* stream);
 
-/* Bytes of the derived weight buffer for the MFMA kernels (0 when `shape` has no MFMA kernel). */
+/* Bytes of the derived weight buffer for the MFMA kernels (0 when `shape` has no MFMA kernel).  The buffer has an
+ * experts section (when the fused experts kernel covers the shape) and a router section (when shape.router_width
+ * > 0 and the fused router+selection kernel covers the router: bf16, ReLU/abs, width = experts = 128 or 256). */
 size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape);
 
-/* Re-tiles expert (and router) weights into MFMA fragment order.  A derived, cacheable buffer: call once per
- * weight update.  No counterpart in the reference (Triton re-reads the nn.Parameter layout each call). */
+/* Re-tiles expert and router weights into MFMA fragment order.  A derived, cacheable buffer: call once per
+ * weight update, with the same `shape` fields (other than n_tokens) that later calls will carry.  router_w1 and
+ * router_w2 are required when the shape has a router section.  No counterpart in the reference (its Triton
+ * kernels re-read the nn.Parameter layout on every call). */
 int d2dmoe_pack_weights(const d2dmoe_shape* shape, const void* w1, const void* b1, const void* w2,
                         const void* w_up, const void* router_w1, const void* router_w2,
                         void* packed, size_t packed_bytes, void* stream);

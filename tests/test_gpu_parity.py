@@ -187,11 +187,13 @@ def test_experts_generic_gated(dtype, act):
 
 
 # =================================================================== experts, bf16 MFMA ===============
-def _packed_for(p, act='relu'):
+def _packed_for(p, act='relu', with_router=False):
     d = H.to_dev(p, DEV)
     E, D, Ed = d['w1'].shape
-    sh = _ops().make_shape(0, D, E, Ed, 0, 1, act)
-    packed = _ops().pack_weights(sh, d['w1'], d.get('b1'), d['w2'])
+    W = d['router_w1'].size(0) if with_router else 0
+    sh = _ops().make_shape(0, D, E, Ed, W, 1, act)
+    packed = _ops().pack_weights(sh, d['w1'], d.get('b1'), d['w2'], None, d['router_w1'] if with_router else None,
+                                 d['router_w2'] if with_router else None)
     assert packed is not None, 'no MFMA kernel for this shape'
     return packed
 
@@ -255,10 +257,42 @@ def test_packed_weights_cache_tracks_parameter_updates():
     r = (torch.rand(70, 128, device=DEV) < 0.5).bfloat16()
     with torch.no_grad():
         a = ex(x, r)
-        assert ex._packed.buf is not None
+        assert ex._packed.slots[False][1] is not None
         ex.w2.mul_(2.0)           # in-place update bumps the version counter -> repack
         b = ex(x, r)
     assert H.rel_err(b, 2 * a.float()) < 1e-2
+
+
+# =================================================================== fused router + select (MFMA) =====
+@pytest.mark.parametrize('N,D,W,E', [(197, 768, 128, 128), (1, 768, 128, 128), (33, 768, 128, 128), (1576, 768, 128, 128),
+                                     (50432, 768, 128, 128), (16, 2048, 256, 256), (300, 2048, 256, 256)])
+@pytest.mark.parametrize('tau', [0.1, 0.9])
+def test_router_select_mfma(N, D, W, E, tau):
+    """Fused router + selection: norms within tolerance of the float64 router, mask bit-exact for the kernel's own
+    norms (stage-wise exactness), counts exact, and few mask flips against the oracle's bf16 router."""
+    _say('router+select mfma', N, D, W, E, tau)
+    Ed = 24 if D == 768 else 8
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=N + D, dtype=torch.bfloat16)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, W, 1, 'relu')
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, d['router_w1'], d['router_w2'])
+    assert packed is not None
+    out, routing, norms, counts = _ops().forward(x.to(DEV), d['router_w1'], d['router_w2'], float(1.0 - tau), d['w1'],
+                                                 d['b1'], d['w2'], None, None, 'relu', False, None, True, True, 'auto', packed)
+    want64 = O.router_forward(x.double(), p['router_w1'].double(), p['router_w2'].double())
+    assert H.rel_err(norms.cpu(), want64) < H.TOL_BF16
+    assert torch.equal(routing.cpu(), O.gate_dynk_max(norms.cpu(), tau))
+    assert torch.equal(counts.cpu().long(), routing.cpu().float().sum(0).long())
+    # the generic (non-MFMA) HIP router rounds at the same points; both masks come from the same rule
+    norms_g = _ops().router(x.to(DEV), d['router_w1'], d['router_w2'])
+    assert (norms_g.float() - norms.float()).abs().max() <= norms_g.float().abs().max() * 2 ** -7
+    flips = (routing.cpu() != O.gate_dynk_max(O.router_forward(x, p['router_w1'], p['router_w2']), tau)).float().mean().item()
+    _say(f'  mask flips vs oracle bf16 router: {flips:.2e}')
+    assert flips < 2e-2
+    if N <= 2000:
+        want = O.layer_from_routing(x.double(), O.upcast({k: v for k, v in p.items() if k != 'last_bias'}),
+                                    routing.cpu().double(), 'relu', 'all')
+        assert H.rel_err(out.cpu(), want) < H.TOL_BF16
 
 
 # =================================================================== whole layer ======================
@@ -310,7 +344,7 @@ def test_layer_end_to_end_vit_shape(dtype, tau):
     _say('e2e', dtype, tau)
     N, D, E, Ed, W = 1576, 768, 128, 24, 128
     x, _, p = H.random_case(N, D, E, Ed, W, seed=77, dtype=dtype)
-    packed = _packed_for(p) if dtype == torch.bfloat16 else None
+    packed = _packed_for(p, with_router=True) if dtype == torch.bfloat16 else None
     out, routing, norms, counts = _forward(x, p, tau, packed=packed)
     norms_o = O.router_forward(x, p['router_w1'], p['router_w2'])
     routing_o = O.gate_dynk_max(norms_o, tau)
