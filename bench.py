@@ -91,7 +91,8 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W):
     # dominant kernel alone (same routing), HIP events on the launch stream
     ms_experts = time_events(lambda: ops.experts(x, routing, p['w1'], p['b1'], p['w2'], None, p['last_bias'], act, False,
                                                  'auto', packed), steps, warmup)
-    ms_router = time_events(lambda: ops.router(x, p['router_w1'], p['router_w2']), steps, warmup)
+    ms_router = time_events(lambda: ops.router_select(x, p['router_w1'], p['router_w2'], thr_scale, packed, E, Ed),
+                            steps, warmup)
     active_flops = pairs * 4.0 * D * Ed
     router_flops = N * (2.0 * D * W + 2.0 * W * E)
     s = x.element_size()
@@ -135,6 +136,8 @@ def main():
     ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS))
     ap.add_argument('--tau', type=float, default=0.9, help='module tau (keep expert when norm >= (1 - tau) * max)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--copy-probe', action='store_true',
+                    help='also run a plain 512 MiB device copy (calibrates FETCH_SIZE / WRITE_SIZE counter units)')
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py: this path is single-GPU (tokens are independent; nothing is exchanged); run with --gpus 1',
@@ -152,6 +155,14 @@ def main():
     x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
     shape = ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x), act)
     packed = ops.pack_weights(shape, p['w1'], p['b1'], p['w2'], None, p['router_w1'], p['router_w2'])
+    if args.copy_probe:
+        # one elementwise kernel that reads 512 MiB and writes 512 MiB
+        src = torch.zeros(128 << 20, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     with torch.no_grad():
         main_r = run_regime(ops, x, p, packed, float(1.0 - args.tau), act, args.steps, args.warmup, D, E, Ed, W)
         lit_r = run_regime(ops, x, p, packed, float(args.tau), act, args.steps, args.warmup, D, E, Ed, W)
@@ -167,7 +178,7 @@ def main():
         'active_tflops': main_r['active_tflops_layer'], 'hbm_gbps': main_r['hbm_gbps_layer'],
         'roofline': {'bound': 'mfma', 'kernel': 'experts', 'achieved': main_r['active_tflops_kernel'],
                      'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s', 'frac': main_r['active_tflops_kernel'] / PEAK_BF16_TFLOPS,
-                     'traffic': None, 'kernel_ms': main_r['ms_experts'], 'router_ms': main_r['ms_router']},
+                     'traffic': None, 'kernel_ms': main_r['ms_experts'], 'router_select_ms': main_r['ms_router']},
         'literal_rule': {'rule': f'keep norm >= {args.tau}*max', 'tokens_per_s': lit_r['tokens_per_s'],
                          'ms_per_step': lit_r['ms_layer'], 'mean_active_experts': lit_r['mean_active'],
                          'p99_active_experts': lit_r['p99_active'], 'active_tflops': lit_r['active_tflops_layer'],

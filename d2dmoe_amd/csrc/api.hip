@@ -181,6 +181,32 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
   }
 }
 
+int d2dmoe_router_select(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
+                         const void* packed, float thr_scale, void* norms_out, void* routing, int32_t* counts,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+  int st = check_shape(shape);
+  if (st != D2DMOE_OK) return st;
+  const d2dmoe_shape& sh = *shape;
+  if (!routing) return D2DMOE_E_NULL;
+  if (sh.router_width <= 0) return D2DMOE_E_SHAPE;
+  if (sh.n_tokens == 0) return counts ? (int)launch_fill_i32(counts, sh.n_experts, 0, (hipStream_t)stream) : D2DMOE_OK;
+  if (!x) return D2DMOE_E_NULL;
+  if (packed != nullptr && mfma_router_supported(sh)) {
+    if (!aligned16(x) || !aligned16(routing) || (norms_out && !aligned16(norms_out))) return D2DMOE_E_ALIGN;
+    return (int)launch_mfma_router_select(sh, x, packed, routing, norms_out, counts, thr_scale, (hipStream_t)stream);
+  }
+  if (!router_w1 || !router_w2) return D2DMOE_E_NULL;
+  const ForwardWorkspace plan = plan_workspace(sh);
+  if (!workspace || workspace_bytes < plan.total || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
+  char* ws = (char*)workspace;
+  void* nbuf = norms_out ? norms_out : (void*)(ws + plan.norms_off);
+  st = d2dmoe_router(x, router_w1, router_w2, nbuf, sh.n_tokens, sh.d_model, sh.router_width, sh.n_experts, sh.dtype,
+                     sh.router_activation, sh.router_output_activation, ws + plan.hidden_off,
+                     plan.norms_off - plan.hidden_off, stream);
+  if (st != D2DMOE_OK) return st;
+  return d2dmoe_select(nbuf, routing, counts, sh.n_tokens, sh.n_experts, sh.dtype, thr_scale, stream);
+}
+
 int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
                    float thr_scale, const void* w1, const void* b1, const void* w2, const void* w_up,
                    const void* last_bias, const void* packed, const void* norms_in, void* norms_out, void* routing,
@@ -194,24 +220,12 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   const ForwardWorkspace plan = plan_workspace(sh);
   if (!workspace || workspace_bytes < plan.total || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
   char* ws = (char*)workspace;
-  const void* norms = norms_in;
-  if (norms == nullptr && packed != nullptr && mfma_router_supported(sh)) {
-    // fused router + selection on MFMA: no hidden/norms round trip through the workspace
-    hipError_t e = launch_mfma_router_select(sh, x, packed, routing, norms_out, counts, thr_scale, (hipStream_t)stream);
-    if (e != hipSuccess) return (int)e;
-    return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,
-                          plan.total - plan.perm_off, stream);
+  if (norms_in == nullptr) {
+    st = d2dmoe_router_select(shape, x, router_w1, router_w2, packed, thr_scale, norms_out, routing, counts, workspace,
+                              workspace_bytes, stream);
+  } else {
+    st = d2dmoe_select(norms_in, routing, counts, sh.n_tokens, sh.n_experts, sh.dtype, thr_scale, stream);
   }
-  if (norms == nullptr) {
-    if (!router_w1 || !router_w2) return D2DMOE_E_NULL;
-    if (sh.router_width <= 0) return D2DMOE_E_SHAPE;
-    void* nbuf = norms_out ? norms_out : (void*)(ws + plan.norms_off);
-    st = d2dmoe_router(x, router_w1, router_w2, nbuf, sh.n_tokens, sh.d_model, sh.router_width, sh.n_experts, sh.dtype,
-                       sh.router_activation, sh.router_output_activation, ws + plan.hidden_off, plan.norms_off - plan.hidden_off, stream);
-    if (st != D2DMOE_OK) return st;
-    norms = nbuf;
-  }
-  st = d2dmoe_select(norms, routing, counts, sh.n_tokens, sh.n_experts, sh.dtype, thr_scale, stream);
   if (st != D2DMOE_OK) return st;
   return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,
                         plan.total - plan.perm_off, stream);

@@ -21,6 +21,7 @@ PATH = {'auto': 0, 'generic': 1, 'mfma_dense': 2, 'mfma_sparse': 3}
 # every extern "C" symbol the header declares
 EXPORTS = (
     'd2dmoe_version', 'd2dmoe_status_string', 'd2dmoe_workspace_bytes', 'd2dmoe_router', 'd2dmoe_select',
+    'd2dmoe_router_select',
     'd2dmoe_build_permutation', 'd2dmoe_experts', 'd2dmoe_packed_bytes', 'd2dmoe_pack_weights', 'd2dmoe_forward',
 )
 
@@ -62,6 +63,8 @@ def load() -> ctypes.CDLL:
     lib.d2dmoe_router.argtypes = [P, P, P, P, I64, I32, I32, I32, I32, I32, I32, P, SZ, P]
     lib.d2dmoe_select.restype = ctypes.c_int
     lib.d2dmoe_select.argtypes = [P, P, P, I64, I32, I32, c_float, P]
+    lib.d2dmoe_router_select.restype = ctypes.c_int
+    lib.d2dmoe_router_select.argtypes = [SH, P, P, P, P, c_float, P, P, P, P, SZ, P]
     lib.d2dmoe_build_permutation.restype = ctypes.c_int
     lib.d2dmoe_build_permutation.argtypes = [P, I64, I32, I32, P, P, P, P, P, P, SZ, P]
     lib.d2dmoe_experts.restype = ctypes.c_int

@@ -97,6 +97,28 @@ def select(norms: torch.Tensor, thr_scale: float, want_counts: bool = False
     return routing, counts
 
 
+def router_select(x: torch.Tensor, router_w1: torch.Tensor, router_w2: torch.Tensor, thr_scale: float,
+                  packed: Optional[torch.Tensor] = None, n_experts: Optional[int] = None, expert_dim: int = 1,
+                  want_norms: bool = False, want_counts: bool = False, activation: str = 'relu',
+                  output_activation: str = 'abs'):
+    """Router MLP + dynamic-k selection through d2dmoe_router_select (one fused MFMA kernel when `packed` carries a
+    router section for this shape).  Returns (routing [N,E], norms or None, counts or None)."""
+    dev = _require_gpu(x, router_w1, router_w2, packed)
+    lib = abi.load()
+    n, d = x.shape
+    w, e = router_w1.size(0), router_w2.size(0)
+    sh = make_shape(n, d, e, expert_dim, w, _dtype_code(x), 'relu', router_activation=activation,
+                    router_output_activation=output_activation)
+    routing = torch.empty(n, e, dtype=x.dtype, device=dev)
+    norms = torch.empty(n, e, dtype=x.dtype, device=dev) if want_norms else None
+    counts = torch.empty(e, dtype=torch.int32, device=dev) if want_counts else None
+    ws = _workspace(dev, max(lib.d2dmoe_workspace_bytes(ctypes.byref(sh)), 256))
+    abi.check(lib.d2dmoe_router_select(ctypes.byref(sh), _ptr(x), _ptr(router_w1), _ptr(router_w2), _ptr(packed),
+                                       ctypes.c_float(thr_scale), _ptr(norms), _ptr(routing), _ptr(counts), _ptr(ws),
+                                       ws.numel(), _stream()), 'd2dmoe_router_select')
+    return routing, norms, counts
+
+
 def build_permutation(routing: torch.Tensor, reference_layout: bool = False):
     """offsets int32 [E+1], token_idx int32 [N*E] (first offsets[E] entries valid); with reference_layout also
     sort_indices / unsort_indices int64 [N,E] and bincounts int64 [E] as the reference's extract_indices returns."""

@@ -116,6 +116,17 @@ int d2dmoe_router(const void* x, const void* router_w1, const void* router_w2, v
 int d2dmoe_select(const void* norms, void* routing, int32_t* counts, int64_t n_tokens, int32_t n_experts,
                   int32_t dtype, float thr_scale, void* stream);
 
+/* Router MLP followed by dynamic-k selection in one call: d2dmoe_router then d2dmoe_select, with the router fixed
+ * to shape->router_activation / router_output_activation.  With `packed` (from d2dmoe_pack_weights, router section
+ * present) and a router the fused MFMA kernel covers, both stages run as ONE kernel and neither the hidden
+ * activations nor the norms touch HBM unless norms_out is given.  Replaces the 'dynk_max' branch of
+ * MoeficationMoE.gate including its router call (architectures/moe/moefication.py:80-85 -> :328-330).
+ *   norms_out optional [N,E]; routing required [N,E]; counts optional int32 [E]
+ * workspace: d2dmoe_workspace_bytes(shape) (only read when the fused kernel does not apply). */
+int d2dmoe_router_select(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
+                         const void* packed, float thr_scale, void* norms_out, void* routing, int32_t* counts,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
 /* Token -> expert permutation from a routing tensor (entry > 0 means routed).
  * Replaces CustomKernelExperts.extract_indices / extract_indices_atomic
  * (architectures/moe/moe_layers.py:213-224, 241-249).  The order is canonical and deterministic: within an

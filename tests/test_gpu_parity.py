@@ -283,6 +283,12 @@ def test_router_select_mfma(N, D, W, E, tau):
     assert H.rel_err(norms.cpu(), want64) < H.TOL_BF16
     assert torch.equal(routing.cpu(), O.gate_dynk_max(norms.cpu(), tau))
     assert torch.equal(counts.cpu().long(), routing.cpu().float().sum(0).long())
+    # the stand-alone entry point runs the same fused kernel
+    r2, n2, c2 = _ops().router_select(x.to(DEV), d['router_w1'], d['router_w2'], float(1.0 - tau), packed, E, Ed, True, True)
+    assert torch.equal(r2, routing) and torch.equal(n2, norms) and torch.equal(c2, counts)
+    # ... and without the packed buffer it composes the generic router and select kernels
+    r3, n3, c3 = _ops().router_select(x.to(DEV), d['router_w1'], d['router_w2'], float(1.0 - tau), None, E, Ed, True, True)
+    assert torch.equal(r3.cpu(), O.gate_dynk_max(n3.cpu(), tau)) and torch.equal(c3.cpu().long(), r3.cpu().float().sum(0).long())
     # the generic (non-MFMA) HIP router rounds at the same points; both masks come from the same rule
     norms_g = _ops().router(x.to(DEV), d['router_w1'], d['router_w2'])
     assert (norms_g.float() - norms.float()).abs().max() <= norms_g.float().abs().max() * 2 ** -7
