@@ -11,6 +11,8 @@
 // registers are already in place: r = 0..7 feed one K=16 step, r = 8..15 the next.  The k-slot -> hidden-neuron
 // map this implies (slot (g, i) of a step <-> neuron 8*(i/4) + 4g + (i%4) of a 16-block) is baked into the
 // packed W2 fragments, so no shuffle is needed between the two GEMMs.
+#include <type_traits>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -40,9 +42,9 @@ static size_t dense_lds_bytes(const d2dmoe_shape& sh) {
   const int n_chunks = (hidden + MD_HC - 1) / MD_HC;
   const int KS1 = sh.d_model / 16;
   return (size_t)(2 * KS1 * 64 + 2 * MD_KS2 * 64) * 16            // x fragments, h fragments
-         + (size_t)MD_BM * (sh.n_experts + 2) * 2                  // routing tile, rows padded by 2 elements
+         + (size_t)MD_BM * (sh.n_experts + 8) * 2                  // routing tile, rows padded by 8 elements
          + (size_t)n_chunks * MD_HC * 3                            // b1 (bf16) and expert index (uint8) per neuron
-         + (size_t)(sh.n_experts + n_chunks + 1) * sizeof(int);    // expert-activity flags, active-chunk list
+         + (size_t)(2 * n_chunks + 1) * sizeof(int);               // chunk-activity flags, active-chunk list
 }
 
 // The fused experts kernel is instantiated for D = 768 (ViT-B, GPT-2 small, BERT-base), ungated experts, bf16.
@@ -50,6 +52,7 @@ bool mfma_dense_supported(const d2dmoe_shape& sh) {
   if (sh.dtype != D2DMOE_BF16 || sh.gated) return false;
   if (sh.d_model != 768) return false;
   if (sh.n_experts > 256) return false;          // expert indices are staged as uint8
+  if (sh.expert_dim > MD_HC) return false;       // an expert spans at most two chunks
   return dense_lds_bytes(sh) <= 160 * 1024;      // x tile + h tile + routing tile + bias/expert-index tables
 }
 
@@ -84,11 +87,12 @@ static PackedLayout packed_layout(const d2dmoe_shape& sh) {
 size_t mfma_packed_bytes(const d2dmoe_shape& sh) { return packed_layout(sh).total; }
 
 // ---------------------------------------------------------------------------------------------------
-// Packing.  Each wave of the fused kernel reads ONE linear stream of 1 KB fragments (16 bytes per lane):
-//   stream[wave][chunk][piece][lane][8 bf16]
-//   pieces 0 .. 2*D/16-1      W1 fragments, piece = kstep*2 + rt:
+// Packing.  Each wave of the fused kernel reads ONE linear stream of 1 KB fragments (16 bytes per lane), in the
+// order the kernel consumes them:
+//   stream[wave][chunk][piece][lane][8 bf16],   KS1 = D/16, CT = D/128
+//   pieces [0, 2 KS1)          W1 fragments, piece = kstep*2 + rt:
 //       neuron h = chunk*256 + wave*64 + rt*32 + c,  d = kstep*16 + 8g + i        value w1[h/Ed][d][h%Ed]
-//   pieces 2*D/16 ..          W2 fragments, piece = 2*D/16 + ks2*(D/128) + ct:
+//   pieces [2 KS1, 2 KS1+16 CT) W2 fragments, piece = 2 KS1 + ks2*CT + ct:
 //       neuron h = chunk*256 + (ks2/2)*32 + (ks2%2)*16 + 8*(i/4) + 4g + (i%4)
 //       column   = wave*(D/4) + ct*32 + c                                         value w2[h/Ed][h%Ed][column]
 // plus b1 as bf16 [hidden_pad] and the expert index of every neuron as uint8 [hidden_pad]; padding neurons
@@ -104,9 +108,9 @@ __global__ void pack_stream_kernel(const bf16_t* __restrict__ w1, const bf16_t* 
   const int chunk = (int)(q % n_chunks);
   const int wave = (int)(q / n_chunks);
   const int g = lane / 32, c = lane % 32;
-  const int n_w1 = D / 16 * 2;
+  const int KS1 = D / 16, CT = D / 128;
   bf16_t v[8];
-  if (piece < n_w1) {
+  if (piece < 2 * KS1) {
     const int ks = piece / 2, rt = piece % 2;
     const int h = chunk * MD_HC + wave * 64 + rt * 32 + c;
 #pragma unroll
@@ -115,8 +119,8 @@ __global__ void pack_stream_kernel(const bf16_t* __restrict__ w1, const bf16_t* 
       v[i] = (h < hidden) ? w1[((int64_t)(h / Ed) * D + d) * Ed + (h % Ed)] : (bf16_t)0;
     }
   } else {
-    const int CT = D / 128;
-    const int ks2 = (piece - n_w1) / CT, ct = (piece - n_w1) % CT;
+    const int r = piece - 2 * KS1;
+    const int ks2 = r / CT, ct = r % CT;
     const int col = wave * (D / 4) + ct * 32 + c;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -190,19 +194,22 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
 
 // ---------------------------------------------------------------------------------------------------
 // Fused experts kernel, token-tile-major ("masked dense sweep").
-// Workgroup = 4 waves, 64 tokens.  LDS: the x tile as B fragments (96 KB at D = 768, resident for the whole
-// kernel), one chunk of h as A fragments (32 KB), the routing tile (64 x E bf16).  Per chunk of 256 neurons:
-//   GEMM1  wave w: H^T[64 neurons of w, 64 tokens] over K = D        A = W1 fragments (global), B = x (LDS)
-//   epilogue      + b1, activation, round to bf16, x routing[token, expert(neuron)], store as A fragments to LDS
-//   GEMM2  wave w: OUT[64 tokens, D/4 columns of w] += H . W2         A = h (LDS), B = W2 fragments (global)
+// Workgroup = 4 waves (one per SIMD), a tile of 64 tokens (or 32: "half tile", used for the last partial round of
+// tiles so the machine does not idle through a mostly empty round).  LDS: the x tile as B fragments (96 KB at
+// D = 768, resident), one chunk of h as A fragments (32 KB), the routing tile, bias / expert-index tables.
+// Per chunk of 256 neurons:
+//   GEMM1  wave w: H^T[64 neurons of w, tokens] over K = D           A = W1 fragments (stream), B = x (LDS)
+//   epilogue      + b1, activation, x routing[token, expert(neuron)], round to bf16, store as A fragments to LDS
+//   GEMM2  wave w: OUT[tokens, D/4 columns of w] += H . W2            A = h (LDS), B = W2 fragments (stream)
 // OUT stays in registers across all chunks (ascending neuron = ascending expert order, float32) and is rounded
 // once in the final epilogue (+ last_bias, + x).  Chunks none of whose experts is routed to by any token of the
 // tile are skipped (uniform branch).
 //
-// Each wave runs at one wave per SIMD, so memory latency is hidden by software: the weight stream is read
-// MD_RING fragments ahead into a register ring (static indices after full unrolling), across phase and chunk
-// boundaries.  The two workgroup barriers per chunk wait on LDS traffic only, so the global loads in flight
-// survive them; GEMM2 of chunk c and GEMM1 of the next chunk run back to back between barriers.
+// Each wave runs at one wave per SIMD, so memory latency is hidden by software: the weight stream is read MD_RING
+// fragments ahead into a register ring (compile-time indices), across phase and chunk boundaries;
+// __builtin_amdgcn_sched_barrier pins every refill where it is written.  The two workgroup barriers per chunk wait
+// on LDS traffic only, so the global loads in flight survive them; GEMM2 of one chunk and GEMM1 of the next run
+// back to back between barriers.
 // ---------------------------------------------------------------------------------------------------
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -219,27 +226,36 @@ __device__ inline uint32_t pack2_bf16(float lo, float hi) {
 // LDS-only workgroup barrier: waits for this wave's LDS operations, not for its outstanding global loads.
 __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <int D, int ACT, bool ED8>
-__global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ routing, const bf16x8* __restrict__ wp,
-    const bf16_t* __restrict__ b1p, const uint8_t* __restrict__ eidx, const bf16_t* __restrict__ last_bias,
-    bf16_t* __restrict__ out, int64_t N, int E, int n_chunks, int hidden, int act_rt, int add_residual) {
+// compile-time loop: f(std::integral_constant<int, I>) for I in [I0, N) -- indices stay constants without relying on
+// the loop unroller
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+struct DenseArgs {
+  const bf16_t* x; const bf16_t* routing; const bf16x8* wp; const bf16_t* b1p; const uint8_t* eidx;
+  const bf16_t* last_bias; bf16_t* out;
+  int64_t N; int E; int expert_dim; int n_chunks; int hidden; int act_rt; int add_residual; int n_full;
+};
+
+template <int D, int ACT, bool ED8, int TT>
+__device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw) {
   constexpr int KS1 = D / 16;          // K steps of GEMM1
   constexpr int CT = D / 128;          // 32-wide column tiles per wave in GEMM2
-  constexpr int NW1 = KS1 * 2;         // W1 fragments per (wave, chunk)
-  constexpr int NW2 = MD_KS2 * CT;     // W2 fragments per (wave, chunk)
-  constexpr int PIECES = NW1 + NW2;
-  constexpr int R = MD_RING;
-  static_assert(NW1 % R == 0 && NW2 % R == 0, "phases must start at ring slot 0");
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  const int E = A.E, n_chunks = A.n_chunks;
+  const int64_t N = A.N;
   bf16x8* xs = (bf16x8*)smem_raw;                              // [2][KS1][64]
   bf16x8* hs = xs + 2 * KS1 * 64;                              // [2][MD_KS2][64]
-  const int RS = E + 2;                                        // padded row stride: tokens land in different banks
+  const int RS = E + 8;                                        // padded row stride (16-byte aligned rows)
   const int HP = n_chunks * MD_HC;
-  bf16_t* rs = (bf16_t*)(hs + 2 * MD_KS2 * 64);                // [64][E+2] routing tile
+  bf16_t* rs = (bf16_t*)(hs + 2 * MD_KS2 * 64);                // [64][E+8] routing tile
   bf16_t* b1s = rs + MD_BM * RS;                               // [HP] first-layer bias
-  int* eact = (int*)(b1s + HP);                                // [E]
-  int* clist = eact + E;                                       // [n_chunks] active chunks, then their number
+  int* cact = (int*)(b1s + HP);                                // [n_chunks] chunk-activity flags
+  int* clist = cact + n_chunks;                                // [n_chunks] active chunks, then their number
   int* n_act_p = clist + n_chunks;
   uint8_t* eis = (uint8_t*)(n_act_p + 1);                      // [HP] expert index of each neuron
 
@@ -247,194 +263,289 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(
   const int lane = t & 63;
   const int w = t >> 6;
   const int g = lane >> 5, c32 = lane & 31;
-  const int64_t tok0 = (int64_t)blockIdx.x * MD_BM;
+  constexpr int NW1 = 2 * KS1;         // W1 fragments per (wave, chunk)
+  constexpr int NW2 = MD_KS2 * CT;     // W2 fragments per (wave, chunk)
+  constexpr int PIECES = NW1 + NW2;
+  constexpr int R = MD_RING;
+  constexpr int BM = 32 * TT;
+  static_assert(NW1 % R == 0 && NW2 % R == 0, "every phase must start at ring slot 0");
 
-  // ---- stage x (as B fragments) and routing
+  // The weight stream of chunk 0 is requested before anything else (almost every tile starts there); if the tile's
+  // first active chunk turns out to be another one the ring is reloaded below.
+  const bf16x8* wbase = A.wp + (int64_t)w * n_chunks * PIECES * 64 + lane;   // this wave's stream
+  bf16x8 ring[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) ring[i] = wbase[i * 64];
+
+  // ---- stage x (as B fragments), routing, bias and expert-index tables; all loads of a kind are issued together
   {
+    for (int i = t; i < n_chunks; i += 256) cact[i] = 0;
     constexpr int PIECES_PER_ROW = D / 8;
+    constexpr int XP = BM * PIECES_PER_ROW / 256;   // 16-byte pieces of x per thread
+    static_assert(BM * PIECES_PER_ROW % 256 == 0, "x tile must divide over the workgroup");
     const uint4 zero4 = {0u, 0u, 0u, 0u};
-    for (int p = t; p < MD_BM * PIECES_PER_ROW; p += 256) {
+    uint4 xv[XP];
+#pragma unroll
+    for (int k = 0; k < XP; ++k) {
+      const int p = t + k * 256;
       const int m = p / PIECES_PER_ROW, kk = p - m * PIECES_PER_ROW;
       const int64_t n = tok0 + m;
-      uint4 v = (n < N) ? *(const uint4*)(x + n * D + kk * 8) : zero4;
+      xv[k] = *(const uint4*)(A.x + (n < N ? n : N - 1) * D + kk * 8);   // clamped address, value zeroed below
+      if (n >= N) xv[k] = zero4;
+    }
+    for (int i = t; i < HP / 8; i += 256) ((uint4*)b1s)[i] = ((const uint4*)A.b1p)[i];
+    for (int i = t; i < HP / 16; i += 256) ((uint4*)eis)[i] = ((const uint4*)A.eidx)[i];
+    __syncthreads();   // cact zeroed before the flags below are raised
+    auto raise_flags = [&](int e) __attribute__((always_inline)) {   // expert e is routed to: mark its chunks active
+      const int h0 = e * A.expert_dim;
+      cact[h0 >> 8] = 1;                                      // benign race: every writer stores 1
+      cact[(h0 + A.expert_dim - 1) >> 8] = 1;
+    };
+    if ((E & 7) == 0) {
+      const int EP = E / 8;   // 16-byte pieces per routing row
+      for (int p = t; p < BM * EP; p += 256) {
+        const int m = p / EP, e0 = (p - m * EP) * 8;
+        const int64_t n = tok0 + m;
+        uint4 rv = *(const uint4*)(A.routing + (n < N ? n : N - 1) * E + e0);
+        if (n >= N) rv = zero4;
+        *(uint4*)(rs + m * RS + e0) = rv;
+        const uint32_t wd[4] = {rv.x, rv.y, rv.z, rv.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (((wd[i >> 1] >> (16 * (i & 1))) & 0x7fffu) != 0) raise_flags(e0 + i);
+      }
+    } else {
+      for (int i = t; i < BM * E; i += 256) {
+        const int m = i / E, e = i - m * E;
+        const int64_t n = tok0 + m;
+        const bf16_t rv = (n < N) ? A.routing[n * E + e] : (bf16_t)0;
+        rs[m * RS + e] = rv;
+        if ((rv & 0x7fff) != 0) raise_flags(e);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < XP; ++k) {
+      const int p = t + k * 256;
+      const int m = p / PIECES_PER_ROW, kk = p - m * PIECES_PER_ROW;
       const int ks = kk >> 1, gg = kk & 1;
-      ((uint4*)xs)[((m >> 5) * KS1 + ks) * 64 + (m & 31) + 32 * gg] = v;
+      ((uint4*)xs)[((m >> 5) * KS1 + ks) * 64 + (m & 31) + 32 * gg] = xv[k];
     }
-    for (int i = t; i < MD_BM * E; i += 256) {
-      const int m = i / E, e = i - m * E;
-      const int64_t n = tok0 + m;
-      rs[m * RS + e] = (n < N) ? routing[n * E + e] : (bf16_t)0;
-    }
-    for (int i = t; i < HP / 8; i += 256) ((uint4*)b1s)[i] = ((const uint4*)b1p)[i];
-    for (int i = t; i < HP / 16; i += 256) ((uint4*)eis)[i] = ((const uint4*)eidx)[i];
-    for (int i = t; i < E; i += 256) eact[i] = 0;
-  }
-  __syncthreads();
-  for (int i = t; i < MD_BM * E; i += 256) {
-    const int m = i / E, e = i - m * E;
-    if ((rs[m * RS + e] & 0x7fff) != 0) eact[e] = 1;   // benign race: every writer stores 1
   }
   __syncthreads();
   if (t == 0) {
     int n_act = 0;
-    for (int ch = 0; ch < n_chunks; ++ch) {
-      const int h_lo = ch * MD_HC;
-      if (h_lo >= hidden) break;
-      const int h_hi = (h_lo + MD_HC - 1 < hidden - 1) ? (h_lo + MD_HC - 1) : (hidden - 1);
-      int any = 0;
-      for (int e = eis[h_lo]; e <= (int)eis[h_hi]; ++e) any |= eact[e];
-      if (any) clist[n_act++] = ch;
-    }
+    for (int ch = 0; ch < n_chunks; ++ch)
+      if (cact[ch]) clist[n_act++] = ch;
     *n_act_p = n_act;
   }
   __syncthreads();
   const int n_act = *n_act_p;
 
-  f32x16 acc2[2][CT];
+  f32x16 acc2[TT][CT];
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < TT; ++a)
 #pragma unroll
     for (int b = 0; b < CT; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc2[a][b][r] = 0.f;
 
   if (n_act > 0) {
-    const bf16x8* wbase = wp + (int64_t)w * n_chunks * PIECES * 64 + lane;   // this wave's stream
-    f32x16 acc1[2][2];
-    bf16x8 ring[R];
-
-    // GEMM1 of one chunk: consumes W1 fragments 0..NW1-1 of `pre`, prefetching R fragments ahead (the stream
-    // continues into the same chunk's W2 fragments).
-    auto gemm1 = [&](const bf16x8* pre) {
-#pragma unroll
-      for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc1[a][b][r] = 0.f;
-      bf16x8 b0 = xs[lane];
-      bf16x8 b1 = xs[KS1 * 64 + lane];
-#pragma unroll
-      for (int ks = 0; ks < KS1; ++ks) {
-        const bf16x8 a0 = ring[(2 * ks) % R];
-        const bf16x8 a1 = ring[(2 * ks + 1) % R];
-        ring[(2 * ks) % R] = pre[(2 * ks + R) * 64];
-        ring[(2 * ks + 1) % R] = pre[(2 * ks + 1 + R) * 64];
-        const int kn = (ks + 1 < KS1) ? ks + 1 : ks;      // x fragments of the next step, read one step ahead
-        const bf16x8 nb0 = xs[(0 * KS1 + kn) * 64 + lane];
-        const bf16x8 nb1 = xs[(1 * KS1 + kn) * 64 + lane];
-        acc1[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc1[0][0], 0, 0, 0);
-        acc1[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc1[0][1], 0, 0, 0);
-        acc1[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc1[1][0], 0, 0, 0);
-        acc1[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc1[1][1], 0, 0, 0);
-        b0 = nb0;
-        b1 = nb1;
-        __builtin_amdgcn_sched_barrier(0);   // keep each refill where it is written: R fragments ahead of its use
-      }
-    };
-
+    f32x16 acc1[2][TT];   // GEMM1 accumulators [row-tile][token tile]
     const bf16x8* cur = wbase + (int64_t)clist[0] * PIECES * 64;
+    if (clist[0] != 0) {
 #pragma unroll
-    for (int i = 0; i < R; ++i) ring[i] = cur[i * 64];
-    gemm1(cur);
+      for (int i = 0; i < R; ++i) ring[i] = cur[i * 64];
+    }
 
     for (int ci = 0; ci < n_act; ++ci) {
       const int chunk = clist[ci];
-      const bool has_next = (ci + 1 < n_act);
-      const bf16x8* nxt = has_next ? (wbase + (int64_t)clist[ci + 1] * PIECES * 64) : cur;
-      // every wave has finished reading the previous h tile
-      lds_barrier();
-      // ---------------------------------------------- epilogue 1: bias, activation, mask -> h fragments in LDS
-#pragma unroll
-      for (int rt = 0; rt < 2; ++rt) {
-        float bias[16];
-        int ei[16];
+      const bf16x8* nxt = (ci + 1 < n_act) ? (wbase + (int64_t)clist[ci + 1] * PIECES * 64) : cur;
+      const int hb0 = chunk * MD_HC + w * 64 + 4 * g;   // first neuron of this lane's accumulator rows, row-tile 0
+
+      // epilogue state, filled and consumed in slices between MFMAs
+      uint2 e_bias[4];     // 4 bf16 biases per accumulator quad
+      uint32_t e_idx[4];   // expert index: one per quad (ED8) or four packed uint8
+      float e_rq[TT][ED8 ? 4 : 16];
+      float e_hv[TT][16];
+      auto epi_load_tables = [&](int rt) __attribute__((always_inline)) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int hb = chunk * MD_HC + w * 64 + rt * 32 + 8 * q + 4 * g;
-          const uint2 bq = *(const uint2*)(b1s + hb);      // 4 bf16
-          bias[q * 4 + 0] = __uint_as_float(bq.x << 16); bias[q * 4 + 1] = __uint_as_float(bq.x & 0xffff0000u);
-          bias[q * 4 + 2] = __uint_as_float(bq.y << 16); bias[q * 4 + 3] = __uint_as_float(bq.y & 0xffff0000u);
-          if (ED8) {
-            // Ed is a multiple of 8: the aligned block of 8 neurons this q covers belongs to one expert, the same for
-            // every lane, so one routing value per (q, token tile) serves four accumulator rows
-            ei[q * 4] = eis[hb & ~7];
-          } else {
-            const uint32_t eq = *(const uint32_t*)(eis + hb);  // 4 uint8
-            ei[q * 4 + 0] = eq & 0xff; ei[q * 4 + 1] = (eq >> 8) & 0xff;
-            ei[q * 4 + 2] = (eq >> 16) & 0xff; ei[q * 4 + 3] = eq >> 24;
+          const int hb = hb0 + rt * 32 + 8 * q;
+          e_bias[q] = *(const uint2*)(b1s + hb);
+          // Ed multiple of 8: the aligned block of 8 neurons a quad pair covers belongs to one expert, the same for
+          // every lane, so one routing value per (quad, token tile) serves four accumulator rows
+          e_idx[q] = ED8 ? (uint32_t)eis[hb & ~7] : *(const uint32_t*)(eis + hb);
+        }
+      };
+      auto epi_load_routing = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+          const bf16_t* rrow = rs + (tt * 32 + c32) * RS;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            if (ED8) {
+              e_rq[tt][q] = bf16_to_f32(rrow[e_idx[q]]);
+            } else {
+#pragma unroll
+              for (int i = 0; i < 4; ++i) e_rq[tt][q * 4 + i] = bf16_to_f32(rrow[(e_idx[q] >> (8 * i)) & 0xff]);
+            }
           }
         }
+      };
+      auto epi_math = [&](int rt, int q) __attribute__((always_inline)) {
+        const float b0 = __uint_as_float(e_bias[q].x << 16), b1 = __uint_as_float(e_bias[q].x & 0xffff0000u);
+        const float b2 = __uint_as_float(e_bias[q].y << 16), b3 = __uint_as_float(e_bias[q].y & 0xffff0000u);
+        const float bias[4] = {b0, b1, b2, b3};
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-          const bf16_t* rrow = rs + (tt * 32 + c32) * RS;
-          float hv[16];
-          float rq[4];
-          if (ED8) {
+        for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) rq[q] = bf16_to_f32(rrow[ei[q * 4]]);
+          for (int i = 0; i < 4; ++i) {
+            const int r = q * 4 + i;
+            float v = acc1[rt][tt][r] + bias[i];
+            v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(A.act_rt, v);
+            e_hv[tt][r] = v * (ED8 ? e_rq[tt][q] : e_rq[tt][r]);
           }
+        }
+      };
+      auto epi_store = [&](int rt) __attribute__((always_inline)) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            float v = acc1[rt][tt][r] + bias[r];
-            v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(act_rt, v);
-            hv[r] = v * (ED8 ? rq[r / 4] : bf16_to_f32(rrow[ei[r]]));
-          }
+        for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             uint4 pk;
-            pk.x = pack2_bf16(hv[half * 8 + 0], hv[half * 8 + 1]);
-            pk.y = pack2_bf16(hv[half * 8 + 2], hv[half * 8 + 3]);
-            pk.z = pack2_bf16(hv[half * 8 + 4], hv[half * 8 + 5]);
-            pk.w = pack2_bf16(hv[half * 8 + 6], hv[half * 8 + 7]);
+            pk.x = pack2_bf16(e_hv[tt][half * 8 + 0], e_hv[tt][half * 8 + 1]);
+            pk.y = pack2_bf16(e_hv[tt][half * 8 + 2], e_hv[tt][half * 8 + 3]);
+            pk.z = pack2_bf16(e_hv[tt][half * 8 + 4], e_hv[tt][half * 8 + 5]);
+            pk.w = pack2_bf16(e_hv[tt][half * 8 + 6], e_hv[tt][half * 8 + 7]);
             const int ks2 = (w * 2 + rt) * 2 + half;
             ((uint4*)hs)[(tt * MD_KS2 + ks2) * 64 + lane] = pk;
           }
         }
-      }
-      lds_barrier();   // h tile complete
-      // ---------------------------------------------- GEMM2: OUT[64 tokens, D/4 columns of this wave] += H . W2
-      {
-        bf16x8 a0 = hs[lane];
-        bf16x8 a1 = hs[MD_KS2 * 64 + lane];
+      };
+      // GEMM1 of the chunk whose stream starts at `pre` (its W1 fragments; the refills run on into its W2 fragments)
+      auto gemm1 = [&](const bf16x8* pre) __attribute__((always_inline)) {
 #pragma unroll
-        for (int ks2 = 0; ks2 < MD_KS2; ++ks2) {
-          const int kn = (ks2 + 1 < MD_KS2) ? ks2 + 1 : ks2;   // h fragments of the next step, read one step ahead
-          const bf16x8 na0 = hs[(0 * MD_KS2 + kn) * 64 + lane];
-          const bf16x8 na1 = hs[(1 * MD_KS2 + kn) * 64 + lane];
+        for (int a = 0; a < 2; ++a)
 #pragma unroll
-          for (int ct = 0; ct < CT; ++ct) {
-            const int s = ks2 * CT + ct;      // position in this phase; refill position s + R
+          for (int b = 0; b < TT; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc1[a][b][r] = 0.f;
+        bf16x8 xb[TT];
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) xb[tt] = xs[tt * KS1 * 64 + lane];
+        static_for<0, KS1>([&](auto ks_c) __attribute__((always_inline)) {
+          constexpr int ks = decltype(ks_c)::value;
+          const bf16x8 a0 = ring[(2 * ks) % R];
+          const bf16x8 a1 = ring[(2 * ks + 1) % R];
+          ring[(2 * ks) % R] = pre[(2 * ks + R) * 64];
+          ring[(2 * ks + 1) % R] = pre[(2 * ks + 1 + R) * 64];
+          constexpr int kn = (ks + 1 < KS1) ? ks + 1 : ks;      // x fragments of the next step, read one step ahead
+          bf16x8 nxb[TT];
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) nxb[tt] = xs[(tt * KS1 + kn) * 64 + lane];
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) {
+            acc1[0][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, xb[tt], acc1[0][tt], 0, 0, 0);
+            acc1[1][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, xb[tt], acc1[1][tt], 0, 0, 0);
+          }
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) xb[tt] = nxb[tt];
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      };
+      // GEMM2 of the current chunk; refills run on into the next chunk's W1 fragments
+      auto gemm2 = [&]() __attribute__((always_inline)) {
+        bf16x8 ha[TT];
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) ha[tt] = hs[tt * MD_KS2 * 64 + lane];
+        static_for<0, MD_KS2>([&](auto j_c) __attribute__((always_inline)) {
+          constexpr int j = decltype(j_c)::value;
+          constexpr int jn = (j + 1 < MD_KS2) ? j + 1 : j;      // h fragments of the next step, read one step ahead
+          bf16x8 nha[TT];
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) nha[tt] = hs[(tt * MD_KS2 + jn) * 64 + lane];
+          static_for<0, CT>([&](auto ct_c) __attribute__((always_inline)) {
+            constexpr int ct = decltype(ct_c)::value;
+            constexpr int s = j * CT + ct;      // position in this phase; refill position s + R
             const bf16x8 b = ring[s % R];
             ring[s % R] = (s + R < NW2) ? cur[(NW1 + s + R) * 64] : nxt[(s + R - NW2) * 64];
-            acc2[0][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b, acc2[0][ct], 0, 0, 0);
-            acc2[1][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b, acc2[1][ct], 0, 0, 0);
-          }
-          a0 = na0;
-          a1 = na1;
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt)
+              acc2[tt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ha[tt], b, acc2[tt][ct], 0, 0, 0);
+          });
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) ha[tt] = nha[tt];
           __builtin_amdgcn_sched_barrier(0);
-        }
+        });
+      };
+
+      if (ci == 0) gemm1(cur);
+      lds_barrier();   // every wave has finished reading the previous h tile
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) {
+        epi_load_tables(rt);
+        epi_load_routing();
+#pragma unroll
+        for (int q = 0; q < 4; ++q) epi_math(rt, q);
+        epi_store(rt);
       }
-      // ---------------------------------------------- GEMM1 of the next active chunk
-      if (has_next) gemm1(nxt);
+      lds_barrier();   // h tile complete
+      gemm2();
+      if (ci + 1 < n_act) gemm1(nxt);
       cur = nxt;
     }
   }
 
-  // ---- final epilogue: + last_bias, + x, one rounding, store
+  // ---- final epilogue: OUT tile -> LDS as float pairs are not needed; the accumulators are rounded to bf16 AFTER
+  // + last_bias (+ x) in float32, so they go through LDS as float in two passes of D/2 columns: write [tokens][D/2]
+  // float, then every thread reads 8 consecutive columns, adds bias / residual, rounds once, stores 16 bytes.
+  {
+    constexpr int HALF = D / 2;
+    constexpr int OS = HALF + 4;                    // row stride in floats (+16 bytes: the two lane halves use
+    float* ot = (float*)smem_raw;                   // different banks); BM * OS * 4 <= x + h regions
+    static_assert((size_t)64 * OS * 4 <= (size_t)(2 * KS1 * 64 + 2 * MD_KS2 * 64) * 16, "out staging fits");
+    constexpr int OP = BM * (HALF / 8) / 256;       // 8-column pieces per thread and pass
+    static_assert(BM * (HALF / 8) % 256 == 0, "out tile must divide over the workgroup");
 #pragma unroll
-  for (int ct = 0; ct < CT; ++ct) {
-    const int col = w * (D / 4) + ct * 32 + c32;
-    const float lb = (last_bias != nullptr) ? bf16_to_f32(last_bias[col]) : 0.f;
+    for (int pass = 0; pass < 2; ++pass) {
+      __syncthreads();                              // previous readers of this LDS region are done
+      if ((w >> 1) == pass) {                       // waves 0,1 own columns [0, D/2), waves 2,3 own [D/2, D)
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
+        for (int ct = 0; ct < CT; ++ct) {
+          const int colh = (w & 1) * (D / 4) + ct * 32 + c32;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t n = tok0 + tt * 32 + 8 * (r / 4) + 4 * g + (r % 4);
+          for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ot[(tt * 32 + 8 * (r / 4) + 4 * g + (r % 4)) * OS + colh] = acc2[tt][ct][r];
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < OP; ++k) {
+        const int p = t + k * 256;
+        const int m = p / (HALF / 8), c8 = (p - m * (HALF / 8)) * 8;
+        const int64_t n = tok0 + m;
         if (n < N) {
-          float v = acc2[tt][ct][r] + lb;
-          if (add_residual) v += bf16_to_f32(x[n * D + col]);
-          out[n * D + col] = (bf16_t)(pack2_bf16(v, 0.f) & 0xffffu);
+          const float4 v0 = *(const float4*)(ot + m * OS + c8);
+          const float4 v1 = *(const float4*)(ot + m * OS + c8 + 4);
+          float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+          const int col = pass * HALF + c8;
+          if (A.last_bias != nullptr) {
+            const uint4 lb = *(const uint4*)(A.last_bias + col);
+            const uint32_t lw[4] = {lb.x, lb.y, lb.z, lb.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] += __uint_as_float((i & 1) ? (lw[i >> 1] & 0xffff0000u) : (lw[i >> 1] << 16));
+          }
+          if (A.add_residual) {
+            const uint4 xr = *(const uint4*)(A.x + n * D + col);
+            const uint32_t xw[4] = {xr.x, xr.y, xr.z, xr.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] += __uint_as_float((i & 1) ? (xw[i >> 1] & 0xffff0000u) : (xw[i >> 1] << 16));
+          }
+          uint4 o;
+          o.x = pack2_bf16(v[0], v[1]); o.y = pack2_bf16(v[2], v[3]);
+          o.z = pack2_bf16(v[4], v[5]); o.w = pack2_bf16(v[6], v[7]);
+          *(uint4*)(A.out + n * D + col) = o;
         }
       }
     }
@@ -442,22 +553,52 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(
 }
 
 template <int D, int ACT, bool ED8>
+__global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  const int b = blockIdx.x;
+  if (b < A.n_full)
+    dense_tile<D, ACT, ED8, 2>(A, (int64_t)b * 64, smem_raw);
+  else
+    dense_tile<D, ACT, ED8, 1>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
+}
+
+static int device_cu_count() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 256;
+    return cus;
+  }();
+  return n;
+}
+
+template <int D, int ACT, bool ED8>
 static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                                    const void* last_bias, void* out, hipStream_t s) {
   const PackedLayout L = packed_layout(sh);
   const char* base = (const char*)packed;
-  constexpr int KS1 = D / 16;
   const size_t lds = dense_lds_bytes(sh);
   if (lds > 160 * 1024) return hipErrorInvalidValue;
-  static_assert(KS1 * 16 == D, "D must be a multiple of 16");
   auto kern = experts_mfma_dense_kernel<D, ACT, ED8>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
-  const unsigned grid = (unsigned)cdiv64(sh.n_tokens, MD_BM);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, s, (const bf16_t*)x, (const bf16_t*)routing,
-                     (const bf16x8*)(base + L.w_off), (const bf16_t*)(base + L.b1_off),
-                     (const uint8_t*)(base + L.eidx_off), (const bf16_t*)last_bias, (bf16_t*)out, sh.n_tokens,
-                     sh.n_experts, L.n_chunks, L.hidden, sh.activation, sh.add_residual);
+  // Tiles of 64 tokens fill whole rounds of one workgroup per CU; when the last round would be at most half full its
+  // tokens go to tiles of 32 instead (twice the workgroups, half the time each).
+  const int cus = device_cu_count();
+  const int64_t t64 = cdiv64(sh.n_tokens, 64);
+  const int64_t leftover = t64 % cus;
+  int64_t n_full = t64, n_half = 0;
+  if (leftover > 0 && leftover * 2 <= cus) {
+    n_full = t64 - leftover;
+    n_half = cdiv64(sh.n_tokens - n_full * 64, 32);
+  }
+  DenseArgs A;
+  A.x = (const bf16_t*)x; A.routing = (const bf16_t*)routing; A.wp = (const bf16x8*)(base + L.w_off);
+  A.b1p = (const bf16_t*)(base + L.b1_off); A.eidx = (const uint8_t*)(base + L.eidx_off);
+  A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.N = sh.n_tokens; A.E = sh.n_experts; A.expert_dim = sh.expert_dim;
+  A.n_chunks = L.n_chunks; A.hidden = L.hidden; A.act_rt = sh.activation; A.add_residual = sh.add_residual;
+  A.n_full = (int)n_full;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(n_full + n_half)), dim3(256), lds, s, A);
   return hipGetLastError();
 }
 
