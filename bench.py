@@ -66,12 +66,12 @@ def time_events(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
-def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W):
+def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, path='auto'):
     N = x.size(0)
 
     def layer():
         return ops.forward(x, p['router_w1'], p['router_w2'], thr_scale, p['w1'], p['b1'], p['w2'], None, p['last_bias'],
-                           act, False, None, False, False, 'auto', packed)
+                           act, False, None, False, False, path, packed)
 
     out, routing, _, _ = layer()
     torch.cuda.synchronize()
@@ -90,7 +90,8 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W):
     ms_layer = (time.perf_counter() - t0) * 1e3 / steps
     # dominant kernel alone (same routing), HIP events on the launch stream
     ms_experts = time_events(lambda: ops.experts(x, routing, p['w1'], p['b1'], p['w2'], None, p['last_bias'], act, False,
-                                                 'auto', packed), steps, warmup)
+                                                 path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 else 'auto'),
+                                                 packed), steps, warmup)
     ms_router = time_events(lambda: ops.router_select(x, p['router_w1'], p['router_w2'], thr_scale, packed, E, Ed),
                             steps, warmup)
     active_flops = pairs * 4.0 * D * Ed

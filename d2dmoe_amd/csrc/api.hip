@@ -38,7 +38,10 @@ ForwardWorkspace plan_workspace(const d2dmoe_shape& sh) {
   size_t off = 0;
   w.hidden_off = off; off += align_up(N * (size_t)(sh.router_width > 0 ? sh.router_width : 0) * es);
   w.norms_off = off;  off += align_up(N * (size_t)sh.n_experts * es);
-  w.perm_off = off;   off += align_up(perm_workspace_bytes(sh.n_tokens, sh.n_experts));
+  size_t scratch = perm_workspace_bytes(sh.n_tokens, sh.n_experts);
+  const size_t sparse = mfma_sparse_workspace_bytes(sh);   // plan + result rows of the expert-major path
+  if (sparse > scratch) scratch = sparse;
+  w.perm_off = off;   off += align_up(scratch);
   w.total = off;
   return w;
 }
@@ -160,7 +163,6 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
   if (sh.gated && b1) return D2DMOE_E_UNSUPPORTED;
   if (!sh.gated && w_up) return D2DMOE_E_SHAPE;
   if (!aligned16(x) || !aligned16(out) || !aligned16(routing)) return D2DMOE_E_ALIGN;
-  (void)workspace; (void)workspace_bytes;
   hipStream_t s = (hipStream_t)stream;
   if (path == D2DMOE_PATH_AUTO)
     path = (packed != nullptr && mfma_dense_supported(sh)) ? D2DMOE_PATH_MFMA_DENSE : D2DMOE_PATH_GENERIC;
@@ -175,7 +177,18 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
     case D2DMOE_PATH_MFMA_DENSE: {
       if (!mfma_dense_supported(sh)) return D2DMOE_E_UNSUPPORTED;
       if (!packed) return D2DMOE_E_NULL;
-      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, s);
+      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, nullptr, s);
+    }
+    case D2DMOE_PATH_MFMA_SPARSE: {
+      // expert-major when the routed pairs fit the provisioned capacity, else the dense sweep: decided on the device
+      if (!mfma_sparse_supported(sh) || !mfma_dense_supported(sh)) return D2DMOE_E_UNSUPPORTED;
+      if (!packed) return D2DMOE_E_NULL;
+      const size_t need = mfma_sparse_workspace_bytes(sh);
+      if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
+      const int* flag = nullptr;
+      hipError_t e = launch_mfma_sparse(sh, x, routing, packed, last_bias, out, workspace, 8, &flag, s);
+      if (e != hipSuccess) return (int)e;
+      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, s);
     }
     default: return D2DMOE_E_UNSUPPORTED;
   }
@@ -227,6 +240,11 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
     st = d2dmoe_select(norms_in, routing, counts, sh.n_tokens, sh.n_experts, sh.dtype, thr_scale, stream);
   }
   if (st != D2DMOE_OK) return st;
+  // A high threshold fraction keeps few experts per token: take the expert-major path (it falls back to the dense
+  // sweep on the device if the routing turns out dense after all).
+  if (path == D2DMOE_PATH_AUTO && packed != nullptr && thr_scale >= 0.75f && mfma_sparse_supported(sh) &&
+      mfma_dense_supported(sh))
+    path = D2DMOE_PATH_MFMA_SPARSE;
   return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,
                         plan.total - plan.perm_off, stream);
 }

@@ -299,6 +299,10 @@ __global__ __launch_bounds__(256) void perm_scatter_kernel(const T* __restrict__
   }
 }
 
+void launch_perm_scan(const int32_t* seg_counts, int32_t* seg_offsets, int32_t* totals, int E, int64_t n_seg, hipStream_t s) {
+  hipLaunchKernelGGL(perm_scan_kernel, dim3((E + kWave - 1) / kWave), dim3(1024), 0, s, seg_counts, seg_offsets, totals, E, n_seg);
+}
+
 size_t perm_workspace_bytes(int64_t N, int E) {
   const int64_t n_seg = cdiv64(N, PERM_SEG);
   // seg_counts + seg_offsets + totals

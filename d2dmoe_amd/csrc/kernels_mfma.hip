@@ -11,31 +11,9 @@
 // registers are already in place: r = 0..7 feed one K=16 step, r = 8..15 the next.  The k-slot -> hidden-neuron
 // map this implies (slot (g, i) of a step <-> neuron 8*(i/4) + 4g + (i%4) of a 16-block) is baked into the
 // packed W2 fragments, so no shuffle is needed between the two GEMMs.
-#include <type_traits>
-
-#include "common.hpp"
-#include "launch.hpp"
+#include "mfma_common.hpp"
 
 namespace d2dmoe {
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-constexpr int MD_BM = 64;       // tokens per workgroup
-constexpr int MD_HC = 256;      // hidden neurons per chunk (4 waves x 64)
-constexpr int MD_WAVES = 4;
-constexpr int MD_KS2 = MD_HC / 16;  // K=16 steps of the second GEMM per chunk
-
-constexpr int MD_RING = 32;     // weight fragments kept in flight per wave (16 bytes per lane each)
-
-struct PackedLayout {
-  int hidden;      // E * Ed
-  int n_chunks;    // ceil(hidden / MD_HC)
-  int hidden_pad;  // n_chunks * MD_HC
-  int pieces;      // weight fragments per (wave, chunk): D/16*2 for W1 followed by 16*D/128 for W2
-  size_t w_off, b1_off, eidx_off, r1_off, r2_off, total;   // r1/r2: router fragments (present when routed)
-  bool has_dense, has_router;
-};
 
 static size_t dense_lds_bytes(const d2dmoe_shape& sh) {
   const int hidden = sh.n_experts * sh.expert_dim;
@@ -65,7 +43,14 @@ bool mfma_router_supported(const d2dmoe_shape& sh) {
   return (sh.router_width == 128 && sh.n_experts == 128) || (sh.router_width == 256 && sh.n_experts == 256);
 }
 
-static PackedLayout packed_layout(const d2dmoe_shape& sh) {
+// The expert-major kernel covers the same layers as the dense sweep with experts of at most 128 neurons.
+bool mfma_sparse_supported(const d2dmoe_shape& sh) {
+  if (sh.dtype != D2DMOE_BF16 || sh.gated) return false;
+  if (sh.d_model != 768) return false;
+  return sh.expert_dim <= 128 && sh.n_experts <= 1024;
+}
+
+PackedLayout packed_layout(const d2dmoe_shape& sh) {
   PackedLayout L;
   L.hidden = sh.n_experts * sh.expert_dim;
   L.n_chunks = (L.hidden + MD_HC - 1) / MD_HC;
@@ -77,6 +62,16 @@ static PackedLayout packed_layout(const d2dmoe_shape& sh) {
   L.b1_off = off;   if (L.has_dense) off += (size_t)L.hidden_pad * 2;   // bf16
   L.eidx_off = off; if (L.has_dense) off += (size_t)L.hidden_pad;       // uint8
   off = (off + 255) / 256 * 256;
+  L.has_sparse = mfma_sparse_supported(sh);
+  const int nt = (sh.expert_dim + 31) / 32;
+  L.nt = (nt <= 1) ? 1 : (nt == 2 ? 2 : 4);   // kernels are instantiated for 1, 2 and 4 row tiles
+  const size_t frag_bytes = (size_t)sh.n_experts * L.nt * 32 * sh.d_model * 2;
+  L.s1_off = off;   if (L.has_sparse) off += frag_bytes;
+  L.s2_off = off;   if (L.has_sparse) off += frag_bytes;
+  L.sb_off = off;   if (L.has_sparse) off += (size_t)sh.n_experts * L.nt * 32 * 2;
+  off = (off + 255) / 256 * 256;
+  // the router section comes last, so the expert sections sit at the same offsets whether or not the shape handed
+  // to a later call names the router
   L.has_router = mfma_router_supported(sh);
   L.r1_off = off;   if (L.has_router) off += (size_t)sh.router_width * sh.d_model * 2;
   L.r2_off = off;   if (L.has_router) off += (size_t)sh.n_experts * sh.router_width * 2;
@@ -182,6 +177,10 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
                        (const bf16_t*)router_w2, (bf16_t*)(base + L.r1_off), (bf16_t*)(base + L.r2_off), sh.d_model,
                        sh.router_width, sh.n_experts);
   }
+  if (L.has_sparse) {
+    hipError_t e = launch_sparse_pack(sh, L, w1, b1, w2, packed, s);
+    if (e != hipSuccess) return e;
+  }
   if (!L.has_dense) return hipGetLastError();
   const int64_t n_items = (int64_t)MD_WAVES * L.n_chunks * L.pieces * 64;
   const unsigned blocks = (unsigned)((n_items + 255) / 256);
@@ -211,34 +210,10 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
 // on LDS traffic only, so the global loads in flight survive them; GEMM2 of one chunk and GEMM1 of the next run
 // back to back between barriers.
 // ---------------------------------------------------------------------------------------------------
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-
-// two float32 -> packed bf16 pair, round-to-nearest-even (one v_cvt_pk_bf16_f32 on gfx950)
-__device__ inline uint32_t pack2_bf16(float lo, float hi) {
-  const f32x2 v = {lo, hi};
-  const bf16x2 b = __builtin_convertvector(v, bf16x2);
-  uint32_t u;
-  __builtin_memcpy(&u, &b, 4);
-  return u;
-}
-
-// LDS-only workgroup barrier: waits for this wave's LDS operations, not for its outstanding global loads.
-__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
-// compile-time loop: f(std::integral_constant<int, I>) for I in [I0, N) -- indices stay constants without relying on
-// the loop unroller
-template <int I, int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (I < N) {
-    f(std::integral_constant<int, I>{});
-    static_for<I + 1, N>(f);
-  }
-}
-
 struct DenseArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* wp; const bf16_t* b1p; const uint8_t* eidx;
   const bf16_t* last_bias; bf16_t* out;
+  const int* skip_flag;   // optional device flag: non-zero = the expert-major path handles this call
   int64_t N; int E; int expert_dim; int n_chunks; int hidden; int act_rt; int add_residual; int n_full;
 };
 
@@ -555,6 +530,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
 template <int D, int ACT, bool ED8>
 __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
   const int b = blockIdx.x;
   if (b < A.n_full)
     dense_tile<D, ACT, ED8, 2>(A, (int64_t)b * 64, smem_raw);
@@ -562,7 +538,7 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(const DenseA
     dense_tile<D, ACT, ED8, 1>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
 }
 
-static int device_cu_count() {
+int device_cu_count() {
   static const int n = [] {
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 256;
@@ -574,7 +550,7 @@ static int device_cu_count() {
 
 template <int D, int ACT, bool ED8>
 static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
-                                   const void* last_bias, void* out, hipStream_t s) {
+                                   const void* last_bias, void* out, const int* skip_flag, hipStream_t s) {
   const PackedLayout L = packed_layout(sh);
   const char* base = (const char*)packed;
   const size_t lds = dense_lds_bytes(sh);
@@ -597,24 +573,24 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   A.b1p = (const bf16_t*)(base + L.b1_off); A.eidx = (const uint8_t*)(base + L.eidx_off);
   A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.N = sh.n_tokens; A.E = sh.n_experts; A.expert_dim = sh.expert_dim;
   A.n_chunks = L.n_chunks; A.hidden = L.hidden; A.act_rt = sh.activation; A.add_residual = sh.add_residual;
-  A.n_full = (int)n_full;
+  A.n_full = (int)n_full; A.skip_flag = skip_flag;
   hipLaunchKernelGGL(kern, dim3((unsigned)(n_full + n_half)), dim3(256), lds, s, A);
   return hipGetLastError();
 }
 
 template <int D, int ACT>
 static hipError_t launch_dense_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
-                                   const void* last_bias, void* out, hipStream_t s) {
-  if (sh.expert_dim % 8 == 0) return launch_dense_cfg<D, ACT, true>(sh, x, routing, packed, last_bias, out, s);
-  return launch_dense_cfg<D, ACT, false>(sh, x, routing, packed, last_bias, out, s);
+                                   const void* last_bias, void* out, const int* skip_flag, hipStream_t s) {
+  if (sh.expert_dim % 8 == 0) return launch_dense_cfg<D, ACT, true>(sh, x, routing, packed, last_bias, out, skip_flag, s);
+  return launch_dense_cfg<D, ACT, false>(sh, x, routing, packed, last_bias, out, skip_flag, s);
 }
 
 hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
-                             const void* last_bias, void* out, hipStream_t s) {
+                             const void* last_bias, void* out, const int* skip_flag, hipStream_t s) {
   switch (sh.activation) {
-    case D2DMOE_ACT_RELU: return launch_dense_act<768, D2DMOE_ACT_RELU>(sh, x, routing, packed, last_bias, out, s);
-    case D2DMOE_ACT_GELU: return launch_dense_act<768, D2DMOE_ACT_GELU>(sh, x, routing, packed, last_bias, out, s);
-    default: return launch_dense_act<768, -1>(sh, x, routing, packed, last_bias, out, s);
+    case D2DMOE_ACT_RELU: return launch_dense_act<768, D2DMOE_ACT_RELU>(sh, x, routing, packed, last_bias, out, skip_flag, s);
+    case D2DMOE_ACT_GELU: return launch_dense_act<768, D2DMOE_ACT_GELU>(sh, x, routing, packed, last_bias, out, skip_flag, s);
+    default: return launch_dense_act<768, -1>(sh, x, routing, packed, last_bias, out, skip_flag, s);
   }
 }
 

@@ -1,0 +1,467 @@
+// Expert-major bf16 MFMA path for sparse routing (few experts per token): device-side plan (permutation, tiles,
+// path flag), grouped per-expert fused up-projection + activation + down-projection, and the ordered combine.
+//
+//   plan     routing [N,E]  ->  offsets[E+1], token_idx[P] (expert-major, tokens ascending: the canonical permutation),
+//                               tok_off[N+1] (token-major offsets), pair_dst[P] (expert-major pair -> token-major
+//                               slot, experts ascending inside a token), tile_off[E+1] (tiles of 32 pairs), flag
+//   experts  one workgroup per tile of 32 (token, expert) pairs of ONE expert: gather the 32 x rows, GEMM1 against
+//            that expert's W1 fragments, bias + activation + routing weight, GEMM2 against its W2^T fragments, store
+//            the 32 result rows (bf16, as the reference's per-expert intermediate is) at their token-major slots
+//   combine  out[n] = sum over the token's slots in ascending expert order, float32, one rounding, + last_bias (+ x)
+//            -- the order of the reference's merge kernel (moe_impls.py:499-514), no atomics.
+// Nothing is decided on the host: when the routed pairs exceed the provisioned capacity the flag stays 0, these
+// kernels return at once and the dense sweep (launched after them with the same flag) does the work.
+#include "mfma_common.hpp"
+
+namespace d2dmoe {
+
+constexpr int SP_BT = 32;        // pairs per tile
+constexpr int SP_SEG = 64;       // tokens per plan segment (one wave)
+constexpr int SP_MAX_VPT = 16;   // experts per lane -> E <= 1024
+
+struct SparseWorkspace {
+  int64_t n_seg, cap;
+  size_t seg_counts, seg_offsets, totals, seg_pairs, seg_pairbase, offsets, tile_off, flag, tok_off, token_idx, pair_dst, y,
+      total;
+};
+
+static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) {
+  SparseWorkspace W;
+  const int64_t N = sh.n_tokens;
+  const int E = sh.n_experts;
+  W.n_seg = cdiv64(N, SP_SEG);
+  W.cap = N * max_mean_k;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off += (bytes + 255) / 256 * 256; return o; };
+  W.seg_counts = take((size_t)W.n_seg * E * 4);
+  W.seg_offsets = take((size_t)W.n_seg * E * 4);
+  W.totals = take((size_t)E * 4);
+  W.seg_pairs = take((size_t)W.n_seg * 4);
+  W.seg_pairbase = take((size_t)W.n_seg * 4);
+  W.offsets = take((size_t)(E + 1) * 4);
+  W.tile_off = take((size_t)(E + 1) * 4);
+  W.flag = take(16);
+  W.tok_off = take((size_t)(N + 1) * 4);
+  W.token_idx = take((size_t)W.cap * 4);
+  W.pair_dst = take((size_t)W.cap * 4);
+  W.y = take((size_t)W.cap * sh.d_model * 2);
+  W.total = off;
+  return W;
+}
+
+size_t mfma_sparse_workspace_bytes(const d2dmoe_shape& sh) {
+  if (!mfma_sparse_supported(sh)) return 0;
+  return sparse_workspace(sh, SP_MAX_MEAN_K).total;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Packing of the expert-major section.  nt = row tiles of 32 neurons per expert (Ed padded to nt*32 with zeros).
+//   W1 fragments   [E][kstep D/16][nt][lane][8]:  neuron j = t*32 + c, d = kstep*16 + 8g + i          w1[e][d][j]
+//   W2^T fragments [E][col-tile D/32][kstep2 2 nt][lane][8]:  column = ct*32 + c,
+//                  neuron j = (ks2/2)*32 + (ks2%2)*16 + 8*(i/4) + 4g + (i%4)                           w2[e][j][column]
+//   bias           [E][nt*32] bf16
+// ---------------------------------------------------------------------------------------------------
+__global__ void pack_sparse_kernel(const bf16_t* __restrict__ w1, const bf16_t* __restrict__ b1, const bf16_t* __restrict__ w2,
+                                   bf16_t* __restrict__ d1, bf16_t* __restrict__ d2, bf16_t* __restrict__ db, int D, int E,
+                                   int Ed, int nt) {
+  const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t per_expert = (int64_t)nt * 32 * D / 8;   // 16-byte pieces per expert in either fragment array
+  const int64_t n = (int64_t)E * per_expert;
+  const int lane = (int)(p % 64);
+  const int g = lane / 32, c = lane % 32;
+  if (p < n) {
+    const int e = (int)(p / per_expert);
+    int64_t q = (p % per_expert) / 64;
+    const int t = (int)(q % nt);
+    const int ks = (int)(q / nt);
+    const int j = t * 32 + c;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int d = ks * 16 + 8 * g + i;
+      d1[p * 8 + i] = (j < Ed) ? w1[((int64_t)e * D + d) * Ed + j] : (bf16_t)0;
+    }
+  } else if (p < 2 * n) {
+    const int64_t pp = p - n;
+    const int e = (int)(pp / per_expert);
+    int64_t q = (pp % per_expert) / 64;
+    const int ks2 = (int)(q % (2 * nt));
+    const int ct = (int)(q / (2 * nt));
+    const int col = ct * 32 + c;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int j = (ks2 / 2) * 32 + (ks2 % 2) * 16 + 8 * (i / 4) + 4 * g + (i % 4);
+      d2[pp * 8 + i] = (j < Ed) ? w2[((int64_t)e * Ed + j) * D + col] : (bf16_t)0;
+    }
+  } else if (p < 2 * n + (int64_t)E * nt * 32) {
+    const int64_t pp = p - 2 * n;
+    const int e = (int)(pp / (nt * 32)), j = (int)(pp % (nt * 32));
+    db[pp] = (j < Ed && b1 != nullptr) ? b1[(int64_t)e * Ed + j] : (bf16_t)0;
+  }
+}
+
+hipError_t launch_sparse_pack(const d2dmoe_shape& sh, const PackedLayout& L, const void* w1, const void* b1, const void* w2,
+                              void* packed, hipStream_t s) {
+  char* base = (char*)packed;
+  const int64_t n = 2 * (int64_t)sh.n_experts * L.nt * 32 * sh.d_model / 8 + (int64_t)sh.n_experts * L.nt * 32;
+  hipLaunchKernelGGL(pack_sparse_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const bf16_t*)w1,
+                     (const bf16_t*)b1, (const bf16_t*)w2, (bf16_t*)(base + L.s1_off), (bf16_t*)(base + L.s2_off),
+                     (bf16_t*)(base + L.sb_off), sh.d_model, sh.n_experts, sh.expert_dim, L.nt);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Plan, pass 1: per segment of 64 tokens (one wave, lanes = experts) the number of routed tokens per expert and the
+// segment's number of pairs.
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void plan_count_kernel(const bf16_t* __restrict__ routing, int32_t* __restrict__ seg_counts,
+                                                         int32_t* __restrict__ seg_pairs, int64_t N, int E, int64_t n_seg) {
+  const int lane = threadIdx.x & 63;
+  const int64_t seg = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / 64;
+  if (seg >= n_seg) return;
+  const int vpt = (E + 63) / 64;
+  const int64_t t0 = seg * SP_SEG;
+  const int rows = (int)((N - t0) < SP_SEG ? (N - t0) : SP_SEG);
+  int cnt[SP_MAX_VPT];
+#pragma unroll
+  for (int k = 0; k < SP_MAX_VPT; ++k) cnt[k] = 0;
+  for (int r = 0; r < rows; ++r) {
+    const bf16_t* row = routing + (t0 + r) * E;
+#pragma unroll
+    for (int k = 0; k < SP_MAX_VPT; ++k)
+      if (k < vpt) {
+        const int e = lane + k * 64;
+        if (e < E) cnt[k] += ((row[e] & 0x7fff) != 0) ? 1 : 0;   // non-zero routing weight
+      }
+  }
+  int tot = 0;
+#pragma unroll
+  for (int k = 0; k < SP_MAX_VPT; ++k)
+    if (k < vpt) {
+      const int e = lane + k * 64;
+      if (e < E) seg_counts[seg * E + e] = cnt[k];
+      tot += cnt[k];
+    }
+  tot = wave_sum_i32(tot);
+  if (lane == 0) seg_pairs[seg] = tot;
+}
+
+// Plan, pass 3 (after the per-expert scan over segments): expert offsets, tile offsets, segment pair bases, the
+// path flag and tok_off[N].  One workgroup of 1024 threads.
+__global__ __launch_bounds__(1024) void plan_finish_kernel(const int32_t* __restrict__ totals, const int32_t* __restrict__ seg_pairs,
+                                                           int32_t* __restrict__ seg_pairbase, int32_t* __restrict__ offsets,
+                                                           int32_t* __restrict__ tile_off, int32_t* __restrict__ flag,
+                                                           int32_t* __restrict__ tok_off, int E, int64_t n_seg, int64_t N,
+                                                           int64_t cap) {
+  __shared__ int32_t a[1024];
+  __shared__ int32_t b[1024];
+  const int t = threadIdx.x;
+  const int c = (t < E) ? totals[t] : 0;
+  a[t] = c;
+  b[t] = (c + SP_BT - 1) / SP_BT;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {   // inclusive scans of counts and of tile counts
+    const int va = (t >= off) ? a[t - off] : 0;
+    const int vb = (t >= off) ? b[t - off] : 0;
+    __syncthreads();
+    a[t] += va;
+    b[t] += vb;
+    __syncthreads();
+  }
+  if (t < E) {
+    offsets[t + 1] = a[t];
+    tile_off[t + 1] = b[t];
+  }
+  if (t == 0) {
+    offsets[0] = 0;
+    tile_off[0] = 0;
+  }
+  const int64_t P = a[E - 1];
+  if (t == 0) {
+    flag[0] = (P <= cap) ? 1 : 0;
+    tok_off[N] = (int32_t)P;
+  }
+  __syncthreads();
+  // exclusive scan of the segments' pair counts: each thread owns a contiguous run of segments
+  const int64_t per = (n_seg + 1023) / 1024;
+  const int64_t s0 = (int64_t)t * per, s1 = (s0 + per < n_seg) ? (s0 + per) : n_seg;
+  int sum = 0;
+  for (int64_t s = s0; s < s1; ++s) sum += seg_pairs[s];
+  a[t] = sum;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const int v = (t >= off) ? a[t - off] : 0;
+    __syncthreads();
+    a[t] += v;
+    __syncthreads();
+  }
+  int run = a[t] - sum;
+  for (int64_t s = s0; s < s1; ++s) {
+    seg_pairbase[s] = run;
+    run += seg_pairs[s];
+  }
+}
+
+// Plan, pass 4: scatter.  A wave walks its 64 tokens in order; lanes = experts, so a lane's running counter is the
+// token's rank inside the expert's list (expert-major position) and a prefix count over the lanes is the expert's
+// rank inside the token's list (token-major position).
+__global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restrict__ routing, const int32_t* __restrict__ seg_offsets,
+                                                           const int32_t* __restrict__ seg_pairbase, const int32_t* __restrict__ offsets,
+                                                           const int32_t* __restrict__ flag, int32_t* __restrict__ tok_off,
+                                                           int32_t* __restrict__ token_idx, int32_t* __restrict__ pair_dst,
+                                                           int64_t N, int E, int64_t n_seg) {
+  if (flag[0] == 0) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t seg = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / 64;
+  if (seg >= n_seg) return;
+  const int vpt = (E + 63) / 64;
+  const int64_t t0 = seg * SP_SEG;
+  const int rows = (int)((N - t0) < SP_SEG ? (N - t0) : SP_SEG);
+  int pos[SP_MAX_VPT];   // next expert-major position of expert e
+#pragma unroll
+  for (int k = 0; k < SP_MAX_VPT; ++k) {
+    pos[k] = 0;
+    if (k < vpt) {
+      const int e = lane + k * 64;
+      if (e < E) pos[k] = offsets[e] + seg_offsets[seg * E + e];
+    }
+  }
+  int tokbase = seg_pairbase[seg];
+  const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int r = 0; r < rows; ++r) {
+    const int64_t tok = t0 + r;
+    const bf16_t* row = routing + tok * E;
+    int before = 0;   // routed experts of this token with a smaller index, over the previous lane groups
+#pragma unroll
+    for (int k = 0; k < SP_MAX_VPT; ++k) {
+      if (k < vpt) {
+        const int e = lane + k * 64;
+        const bool on = (e < E) && ((row[e] & 0x7fff) != 0);
+        const unsigned long long bal = __ballot(on);
+        if (on) {
+          const int rank_in_token = before + __popcll(bal & lt_mask);
+          token_idx[pos[k]] = (int32_t)tok;
+          pair_dst[pos[k]] = tokbase + rank_in_token;
+          pos[k] += 1;
+        }
+        before += __popcll(bal);
+      }
+    }
+    if (lane == 0) tok_off[tok] = tokbase;
+    tokbase += before;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Expert-major fused experts kernel.  256 threads = 4 waves per tile of 32 pairs of one expert.  Every wave computes
+// the tile's hidden activations itself (GEMM1 transposed, x rows read straight from their gathered positions as B
+// fragments), then owns D/4 output columns of the second product (also transposed, so a lane ends with ONE token and
+// 4 consecutive columns per accumulator quad: 8-byte stores into the token-major slot of the pair).
+// A fixed grid loops over the tiles listed by tile_off; the expert of a tile is found by bisection.
+// ---------------------------------------------------------------------------------------------------
+struct SparseArgs {
+  const bf16_t* x; const bf16_t* routing; const bf16x8* w1s; const bf16x8* w2s; const bf16_t* b1s;
+  const int32_t* offsets; const int32_t* tile_off; const int32_t* token_idx; const int32_t* pair_dst; const int32_t* flag;
+  bf16_t* y; int E; int act_rt;
+};
+
+template <int D, int NT, int ACT>
+__global__ __launch_bounds__(256) void experts_mfma_sparse_kernel(const SparseArgs A) {
+  constexpr int KS1 = D / 16;
+  constexpr int CTW = D / 128;   // column tiles per wave
+  __shared__ int32_t s_tile_off[1025];
+  if (A.flag[0] == 0) return;
+  const int E = A.E;
+  for (int i = threadIdx.x; i <= E; i += 256) s_tile_off[i] = A.tile_off[i];
+  __syncthreads();
+  const int n_tiles = s_tile_off[E];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int g = lane >> 5, c32 = lane & 31;
+  for (int T = blockIdx.x; T < n_tiles; T += gridDim.x) {
+    int lo = 0, hi = E;   // largest e with tile_off[e] <= T (experts without tiles share their successor's offset)
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (s_tile_off[mid] <= T) lo = mid; else hi = mid;
+    }
+    const int e = lo;
+    const int base = A.offsets[e];
+    const int cnt = A.offsets[e + 1] - base;
+    const int j0 = (T - s_tile_off[e]) * SP_BT;
+    const int rows = (cnt - j0 < SP_BT) ? (cnt - j0) : SP_BT;
+    const bool valid = c32 < rows;
+    const int pj = base + j0 + (valid ? c32 : rows - 1);
+    const int tok = A.token_idx[pj];
+    const int dst = A.pair_dst[pj];
+    const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)tok * D);
+    const float rw = bf16_to_f32(A.routing[(int64_t)tok * E + e]);
+
+    // GEMM1: H^T[NT*32 neurons, 32 pairs]
+    f32x16 acc1[NT];
+#pragma unroll
+    for (int a = 0; a < NT; ++a)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc1[a][r] = 0.f;
+    const bf16x8* w1f = A.w1s + ((int64_t)e * KS1 * NT) * 64 + lane;
+#pragma unroll 8
+    for (int ks = 0; ks < KS1; ++ks) {
+      const bf16x8 b = xrow[2 * ks + g];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const bf16x8 a = w1f[(ks * NT + t) * 64];
+        acc1[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc1[t], 0, 0, 0);
+      }
+    }
+    // bias, activation, routing weight, round to bf16 -> B fragments of the second product
+    bf16x8 hb[2 * NT];
+    const bf16_t* bias_e = A.b1s + (int64_t)e * NT * 32;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      float hv[16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint2 bq = *(const uint2*)(bias_e + t * 32 + 8 * q + 4 * g);
+        const float bias[4] = {__uint_as_float(bq.x << 16), __uint_as_float(bq.x & 0xffff0000u),
+                               __uint_as_float(bq.y << 16), __uint_as_float(bq.y & 0xffff0000u)};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v = acc1[t][q * 4 + i] + bias[i];
+          v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(A.act_rt, v);
+          hv[q * 4 + i] = v * rw;
+        }
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        uint4 pk;
+        pk.x = pack2_bf16(hv[half * 8 + 0], hv[half * 8 + 1]);
+        pk.y = pack2_bf16(hv[half * 8 + 2], hv[half * 8 + 3]);
+        pk.z = pack2_bf16(hv[half * 8 + 4], hv[half * 8 + 5]);
+        pk.w = pack2_bf16(hv[half * 8 + 6], hv[half * 8 + 7]);
+        __builtin_memcpy(&hb[t * 2 + half], &pk, 16);
+      }
+    }
+    // GEMM2 (transposed): OUT^T[D/4 columns of this wave, 32 pairs]
+    f32x16 acc2[CTW];
+#pragma unroll
+    for (int a = 0; a < CTW; ++a)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc2[a][r] = 0.f;
+    const bf16x8* w2f = A.w2s + ((int64_t)e * (D / 32) + w * CTW) * (2 * NT) * 64 + lane;
+#pragma unroll
+    for (int ct = 0; ct < CTW; ++ct)
+#pragma unroll
+      for (int ks2 = 0; ks2 < 2 * NT; ++ks2) {
+        const bf16x8 a = w2f[(ct * 2 * NT + ks2) * 64];
+        acc2[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, hb[ks2], acc2[ct], 0, 0, 0);
+      }
+    if (valid) {
+      bf16_t* yrow = A.y + (int64_t)dst * D + w * (D / 4) + 4 * g;
+#pragma unroll
+      for (int ct = 0; ct < CTW; ++ct)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint2 o;
+          o.x = pack2_bf16(acc2[ct][q * 4 + 0], acc2[ct][q * 4 + 1]);
+          o.y = pack2_bf16(acc2[ct][q * 4 + 2], acc2[ct][q * 4 + 3]);
+          *(uint2*)(yrow + ct * 32 + 8 * q) = o;
+        }
+    }
+  }
+}
+
+// Ordered combine: thread = (token, 8 columns); the token's result rows are contiguous, experts ascending.
+__global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__ y, const int32_t* __restrict__ tok_off,
+                                                      const int32_t* __restrict__ flag, const bf16_t* __restrict__ x,
+                                                      const bf16_t* __restrict__ last_bias, bf16_t* __restrict__ out, int64_t N,
+                                                      int D, int add_residual) {
+  if (flag[0] == 0) return;
+  const int ppr = D / 8;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t n = idx / ppr;
+  if (n >= N) return;
+  const int col = (int)(idx - n * ppr) * 8;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  const int q0 = tok_off[n], q1 = tok_off[n + 1];
+  for (int q = q0; q < q1; ++q) {
+    const uint4 v = *(const uint4*)(y + (int64_t)q * D + col);
+    const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+  }
+  if (last_bias != nullptr) {
+    const uint4 v = *(const uint4*)(last_bias + col);
+    const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+  }
+  if (add_residual) {
+    const uint4 v = *(const uint4*)(x + n * D + col);
+    const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+  }
+  uint4 o;
+  o.x = pack2_bf16(acc[0], acc[1]); o.y = pack2_bf16(acc[2], acc[3]);
+  o.z = pack2_bf16(acc[4], acc[5]); o.w = pack2_bf16(acc[6], acc[7]);
+  *(uint4*)(out + n * D + col) = o;
+}
+
+template <int NT>
+static void launch_sparse_experts(const SparseArgs& A, int act, unsigned grid, hipStream_t s) {
+  switch (act) {
+    case D2DMOE_ACT_RELU:
+      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, D2DMOE_ACT_RELU>), dim3(grid), dim3(256), 0, s, A); break;
+    case D2DMOE_ACT_GELU:
+      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, D2DMOE_ACT_GELU>), dim3(grid), dim3(256), 0, s, A); break;
+    default:
+      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, -1>), dim3(grid), dim3(256), 0, s, A); break;
+  }
+}
+
+hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
+                              const void* last_bias, void* out, void* workspace, int max_mean_k, const int** flag_out,
+                              hipStream_t s) {
+  if (max_mean_k > SP_MAX_MEAN_K) max_mean_k = SP_MAX_MEAN_K;
+  const SparseWorkspace W = sparse_workspace(sh, SP_MAX_MEAN_K);   // sized for the maximum; the flag uses max_mean_k
+  const PackedLayout L = packed_layout(sh);
+  char* ws = (char*)workspace;
+  const char* pk = (const char*)packed;
+  const int64_t N = sh.n_tokens;
+  const int E = sh.n_experts;
+  int32_t* seg_counts = (int32_t*)(ws + W.seg_counts);
+  int32_t* seg_offsets = (int32_t*)(ws + W.seg_offsets);
+  int32_t* totals = (int32_t*)(ws + W.totals);
+  int32_t* seg_pairs = (int32_t*)(ws + W.seg_pairs);
+  int32_t* seg_pairbase = (int32_t*)(ws + W.seg_pairbase);
+  int32_t* offsets = (int32_t*)(ws + W.offsets);
+  int32_t* tile_off = (int32_t*)(ws + W.tile_off);
+  int32_t* flag = (int32_t*)(ws + W.flag);
+  int32_t* tok_off = (int32_t*)(ws + W.tok_off);
+  int32_t* token_idx = (int32_t*)(ws + W.token_idx);
+  int32_t* pair_dst = (int32_t*)(ws + W.pair_dst);
+  bf16_t* y = (bf16_t*)(ws + W.y);
+  const unsigned seg_blocks = (unsigned)cdiv64(W.n_seg, 4);
+  hipLaunchKernelGGL(plan_count_kernel, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_counts, seg_pairs, N, E,
+                     W.n_seg);
+  launch_perm_scan(seg_counts, seg_offsets, totals, E, W.n_seg, s);
+  hipLaunchKernelGGL(plan_finish_kernel, dim3(1), dim3(1024), 0, s, totals, seg_pairs, seg_pairbase, offsets, tile_off, flag,
+                     tok_off, E, W.n_seg, N, N * (int64_t)max_mean_k);
+  hipLaunchKernelGGL(plan_scatter_kernel, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_offsets, seg_pairbase,
+                     offsets, flag, tok_off, token_idx, pair_dst, N, E, W.n_seg);
+  SparseArgs A;
+  A.x = (const bf16_t*)x; A.routing = (const bf16_t*)routing; A.w1s = (const bf16x8*)(pk + L.s1_off);
+  A.w2s = (const bf16x8*)(pk + L.s2_off); A.b1s = (const bf16_t*)(pk + L.sb_off); A.offsets = offsets;
+  A.tile_off = tile_off; A.token_idx = token_idx; A.pair_dst = pair_dst; A.flag = flag; A.y = y; A.E = E;
+  A.act_rt = sh.activation;
+  const unsigned grid = (unsigned)(4 * device_cu_count());
+  if (L.nt == 1) launch_sparse_experts<1>(A, sh.activation, grid, s);
+  else if (L.nt == 2) launch_sparse_experts<2>(A, sh.activation, grid, s);
+  else launch_sparse_experts<4>(A, sh.activation, grid, s);
+  const int64_t n_threads = N * (sh.d_model / 8);
+  hipLaunchKernelGGL(combine_kernel, dim3((unsigned)cdiv64(n_threads, 256)), dim3(256), 0, s, y, tok_off, flag, (const bf16_t*)x,
+                     (const bf16_t*)last_bias, (bf16_t*)out, N, sh.d_model, sh.add_residual);
+  *flag_out = flag;
+  return hipGetLastError();
+}
+
+}  // namespace d2dmoe

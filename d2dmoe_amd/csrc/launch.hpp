@@ -42,6 +42,17 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
 hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
                                      void* norms_out, int32_t* counts, float thr_scale, hipStream_t s);
 hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
-                             const void* last_bias, void* out, hipStream_t s);
+                             const void* last_bias, void* out, const int* skip_flag, hipStream_t s);
+
+// ---- bf16 MFMA expert-major path (kernels_sparse.hip) ----
+bool mfma_sparse_supported(const d2dmoe_shape& sh);
+size_t mfma_sparse_workspace_bytes(const d2dmoe_shape& sh);
+// Plans the call on the device (permutation, tiles, path flag), runs the expert-major kernels when the number of routed
+// pairs is at most n_tokens * max_mean_k, and leaves *flag == 0 otherwise so that the dense sweep (launched by the
+// caller with skip_flag = the returned pointer) does the work instead.
+hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
+                              const void* last_bias, void* out, void* workspace, int max_mean_k, const int** flag_out,
+                              hipStream_t s);
+void launch_perm_scan(const int32_t* seg_counts, int32_t* seg_offsets, int32_t* totals, int E, int64_t n_seg, hipStream_t s);
 
 }  // namespace d2dmoe

@@ -1,0 +1,64 @@
+// Shared pieces of the bf16 MFMA kernels (gfx950): vector types, tile constants, the packed-weight layout, small
+// device helpers.
+#pragma once
+
+#include <type_traits>
+
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace d2dmoe {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int MD_BM = 64;       // tokens per workgroup of the dense sweep
+constexpr int MD_HC = 256;      // hidden neurons per chunk (4 waves x 64)
+constexpr int MD_WAVES = 4;
+constexpr int MD_KS2 = MD_HC / 16;  // K=16 steps of the second GEMM per chunk
+constexpr int MD_RING = 32;     // weight fragments kept in flight per wave (16 bytes per lane each)
+constexpr int SP_MAX_MEAN_K = 8;    // the expert-major path is provisioned for at most N * 8 routed pairs
+
+// Sections of the buffer d2dmoe_pack_weights writes.  A section is present when its kernel covers the shape.
+struct PackedLayout {
+  int hidden;      // E * Ed
+  int n_chunks;    // ceil(hidden / MD_HC)
+  int hidden_pad;  // n_chunks * MD_HC
+  int pieces;      // weight fragments per (wave, chunk) of the dense stream
+  int nt;          // 32-neuron row tiles per expert in the expert-major section: ceil(Ed / 32)
+  size_t w_off, b1_off, eidx_off;        // dense sweep: weight stream, bias (bf16), expert index per neuron (uint8)
+  size_t r1_off, r2_off;                 // router fragments
+  size_t s1_off, s2_off, sb_off;         // expert-major: W1 fragments, W2^T fragments, bias (bf16, padded to nt*32)
+  size_t total;
+  bool has_dense, has_router, has_sparse;
+};
+PackedLayout packed_layout(const d2dmoe_shape& sh);
+int device_cu_count();
+hipError_t launch_sparse_pack(const d2dmoe_shape& sh, const PackedLayout& L, const void* w1, const void* b1, const void* w2,
+                              void* packed, hipStream_t s);
+
+// two float32 -> packed bf16 pair, round-to-nearest-even (one v_cvt_pk_bf16_f32 on gfx950)
+__device__ inline uint32_t pack2_bf16(float lo, float hi) {
+  const f32x2 v = {lo, hi};
+  const bf16x2 b = __builtin_convertvector(v, bf16x2);
+  uint32_t u;
+  __builtin_memcpy(&u, &b, 4);
+  return u;
+}
+
+// LDS-only workgroup barrier: waits for this wave's LDS operations, not for its outstanding global loads.
+__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// compile-time loop: f(std::integral_constant<int, I>) for I in [I0, N) -- indices stay constants without relying on
+// the loop unroller
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+}  // namespace d2dmoe

@@ -248,6 +248,63 @@ def test_experts_mfma_dense_full_size_properties():
     assert H.rel_err(a.cpu()[rows], want) < H.TOL_BF16
 
 
+@pytest.mark.parametrize('N,E,Ed,density', [(197, 128, 24, 0.02), (1576, 128, 24, 0.0165), (65, 128, 24, 0.05), (1, 128, 24, 0.05),
+                                            (300, 24, 128, 0.1), (130, 100, 30, 0.05), (333, 16, 64, 0.2), (100, 7, 5, 0.3),
+                                            (1576, 128, 24, 0.5)])
+def test_experts_mfma_sparse_matches_oracle(N, E, Ed, density):
+    """Expert-major path: plan -> grouped per-expert kernel -> ordered combine.  The last case routes 64 experts per
+    token, more than the path is provisioned for, so the device-side flag hands the call to the dense sweep."""
+    _say('experts sparse', N, E, Ed, density)
+    x, routing, p = H.random_case(N, 768, E, Ed, 8, seed=N + E + 1, dtype=torch.bfloat16, density=density)
+    packed = _packed_for(p)
+    got = _experts_got(x, routing, p, 'relu', path='mfma_sparse', packed=packed)
+    assert H.rel_err(got, _experts_want(x, routing, p, 'relu')) < H.TOL_BF16
+    assert H.rel_err(got, _experts_got(x, routing, p, 'relu', path='mfma_dense', packed=packed)) < 1e-2
+    assert torch.equal(got, _experts_got(x, routing, p, 'relu', path='mfma_sparse', packed=packed))   # deterministic
+
+
+@pytest.mark.parametrize('act', ['relu', 'gelu', 'tanh'])
+def test_experts_mfma_sparse_activations_weights_edges(act):
+    x, routing, p = H.random_case(500, 768, 128, 24, 8, seed=41, dtype=torch.bfloat16, density=0.03)
+    packed = _packed_for(p, act)
+    got = _experts_got(x, routing, p, act, residual=True, path='mfma_sparse', packed=packed)
+    assert H.rel_err(got, _experts_want(x, routing, p, act, True)) < H.TOL_BF16
+    g = torch.Generator().manual_seed(2)
+    weights = (routing.float() * (torch.rand(500, 128, generator=g) + 0.5)).bfloat16()
+    got = _experts_got(x, weights, p, act, path='mfma_sparse', packed=packed)
+    assert H.rel_err(got, _experts_want(x, weights, p, act)) < H.TOL_BF16
+    # nothing routed -> last_bias only; a single expert taking every token (maximal skew)
+    got = _experts_got(x, torch.zeros_like(routing), p, act, path='mfma_sparse', packed=packed)
+    assert torch.equal(got, p['last_bias'].expand(500, -1))
+    one = torch.zeros_like(routing)
+    one[:, 77] = 1
+    got = _experts_got(x, one, p, act, path='mfma_sparse', packed=packed)
+    assert H.rel_err(got, _experts_want(x, one, p, act)) < H.TOL_BF16
+
+
+def test_experts_mfma_sparse_full_size_and_auto_switch():
+    """50432 tokens with ~2 experts per token: the oracle on slices of rows, the dense sweep on all rows; and the
+    whole-layer call picks the expert-major path by itself for a high threshold fraction."""
+    N = 50432
+    x, routing, p = H.random_case(N, 768, 128, 24, 128, seed=51, dtype=torch.bfloat16, density=0.0165)
+    packed = _packed_for(p, with_router=True)
+    d = H.to_dev(p, DEV)
+    xg, rg = x.to(DEV), routing.to(DEV)
+    lb = d['last_bias'].view(-1)
+    a = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, 'relu', False, 'mfma_sparse', packed)
+    b = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, 'relu', False, 'mfma_dense', packed)
+    assert H.rel_err(a, b) < 1e-2
+    rows = torch.cat([torch.arange(0, 128), torch.arange(25000, 25064), torch.arange(N - 64, N)])
+    assert H.rel_err(a.cpu()[rows], _experts_want(x[rows], routing[rows], p, 'relu')) < H.TOL_BF16
+    out_auto, r_auto, _, _ = _ops().forward(xg, d['router_w1'], d['router_w2'], 0.9, d['w1'], d['b1'], d['w2'], None, lb,
+                                            'relu', False, None, False, False, 'auto', packed)
+    out_dense, r_dense, _, _ = _ops().forward(xg, d['router_w1'], d['router_w2'], 0.9, d['w1'], d['b1'], d['w2'], None, lb,
+                                              'relu', False, None, False, False, 'mfma_dense', packed)
+    assert torch.equal(r_auto, r_dense) and H.rel_err(out_auto, out_dense) < 1e-2
+    want = O.layer_from_routing(x[rows].double(), O.upcast(p), r_auto.cpu()[rows].double(), 'relu', 'all')
+    assert H.rel_err(out_auto.cpu()[rows], want) < H.TOL_BF16
+
+
 def test_packed_weights_cache_tracks_parameter_updates():
     from d2dmoe_amd import HipKernelExperts
     torch.manual_seed(0)
