@@ -215,13 +215,16 @@ __global__ __launch_bounds__(1024) void perm_scan_kernel(const int32_t* __restri
   const int64_t s0 = w * per;
   const int64_t s1 = (s0 + per) < n_seg ? (s0 + per) : n_seg;
   int sum = 0;
-  if (e < E)
+  if (e < E) {
+#pragma unroll 32
     for (int64_t s = s0; s < s1; ++s) sum += seg_counts[s * E + e];
+  }
   part[w][lane] = sum;
   __syncthreads();
   int run = 0;
   for (int i = 0; i < w; ++i) run += part[i][lane];
   if (e < E) {
+#pragma unroll 32
     for (int64_t s = s0; s < s1; ++s) {
       const int c = seg_counts[s * E + e];
       seg_offsets[s * E + e] = run;

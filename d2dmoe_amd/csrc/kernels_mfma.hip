@@ -35,11 +35,11 @@ bool mfma_dense_supported(const d2dmoe_shape& sh) {
 }
 
 // The fused router+select kernel covers the D2DMoE router: bf16, depth 2, ReLU hidden / abs output activation,
-// width and expert count both 128 or both 256, D a multiple of 16.
+// width and expert count both 128 or both 256, D a multiple of 64.
 bool mfma_router_supported(const d2dmoe_shape& sh) {
   if (sh.dtype != D2DMOE_BF16 || sh.router_width <= 0) return false;
   if (sh.router_activation != D2DMOE_ACT_RELU || sh.router_output_activation != D2DMOE_ACT_ABS) return false;
-  if (sh.d_model % 16 != 0) return false;
+  if (sh.d_model % 64 != 0) return false;
   return (sh.router_width == 128 && sh.n_experts == 128) || (sh.router_width == 256 && sh.n_experts == 256);
 }
 
@@ -618,20 +618,24 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
   const int64_t token = tok0 + c32;
   const bool valid = token < N;
   const bf16x8* xrow = (const bf16x8*)(x + (valid ? token : (N - 1)) * D);
-  const int KS1 = D / 16;
+  const int KS1 = D / 16;   // a multiple of 4 (checked by the launcher's support test)
 
   f32x16 acc1[WT];
 #pragma unroll
   for (int a = 0; a < WT; ++a)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc1[a][r] = 0.f;
-  for (int ks = 0; ks < KS1; ++ks) {
-    const bf16x8 b = xrow[2 * ks + g];
+  for (int ks0 = 0; ks0 < KS1; ks0 += 4) {
+    bf16x8 b[4];   // four K steps of x fetched together
 #pragma unroll
-    for (int rt = 0; rt < WT; ++rt) {
-      const bf16x8 a = w1f[(int64_t)(ks * WT + rt) * 64 + lane];
-      acc1[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc1[rt], 0, 0, 0);
-    }
+    for (int i = 0; i < 4; ++i) b[i] = xrow[2 * (ks0 + i) + g];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int rt = 0; rt < WT; ++rt) {
+        const bf16x8 a = w1f[(int64_t)((ks0 + i) * WT + rt) * 64 + lane];
+        acc1[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[i], acc1[rt], 0, 0, 0);
+      }
   }
   // hidden activations as B fragments of the second product
   bf16x8 hb[2 * WT];

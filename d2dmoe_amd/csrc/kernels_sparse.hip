@@ -16,8 +16,7 @@
 namespace d2dmoe {
 
 constexpr int SP_BT = 32;        // pairs per tile
-constexpr int SP_SEG = 64;       // tokens per plan segment (one wave)
-constexpr int SP_MAX_VPT = 16;   // experts per lane -> E <= 1024
+constexpr int SP_SEG = 16;       // tokens per plan segment (one wave); small, so a pass is one round trip to memory
 
 struct SparseWorkspace {
   int64_t n_seg, cap;
@@ -113,6 +112,7 @@ hipError_t launch_sparse_pack(const d2dmoe_shape& sh, const PackedLayout& L, con
 // Plan, pass 1: per segment of 64 tokens (one wave, lanes = experts) the number of routed tokens per expert and the
 // segment's number of pairs.
 // ---------------------------------------------------------------------------------------------------
+template <int VPT>
 __global__ __launch_bounds__(256) void plan_count_kernel(const bf16_t* __restrict__ routing, int32_t* __restrict__ seg_counts,
                                                          int32_t* __restrict__ seg_pairs, int64_t N, int E, int64_t n_seg) {
   const int lane = threadIdx.x & 63;
@@ -121,21 +121,27 @@ __global__ __launch_bounds__(256) void plan_count_kernel(const bf16_t* __restric
   const int vpt = (E + 63) / 64;
   const int64_t t0 = seg * SP_SEG;
   const int rows = (int)((N - t0) < SP_SEG ? (N - t0) : SP_SEG);
-  int cnt[SP_MAX_VPT];
+  int cnt[VPT];
 #pragma unroll
-  for (int k = 0; k < SP_MAX_VPT; ++k) cnt[k] = 0;
-  for (int r = 0; r < rows; ++r) {
-    const bf16_t* row = routing + (t0 + r) * E;
+  for (int k = 0; k < VPT; ++k) cnt[k] = 0;
 #pragma unroll
-    for (int k = 0; k < SP_MAX_VPT; ++k)
-      if (k < vpt) {
-        const int e = lane + k * 64;
-        if (e < E) cnt[k] += ((row[e] & 0x7fff) != 0) ? 1 : 0;   // non-zero routing weight
+  for (int k = 0; k < VPT; ++k) {
+    if (k < vpt) {   // uniform
+      const int e = lane + k * 64;
+      bf16_t v[SP_SEG];   // the segment's rows for this lane group, fetched together
+#pragma unroll
+      for (int i = 0; i < SP_SEG; ++i) {
+        const int r = (i < rows) ? i : (rows - 1);
+        v[i] = (e < E) ? routing[(t0 + r) * E + e] : (bf16_t)0;
       }
+#pragma unroll
+      for (int i = 0; i < SP_SEG; ++i)
+        if (i < rows) cnt[k] += ((v[i] & 0x7fff) != 0) ? 1 : 0;   // non-zero routing weight
+    }
   }
   int tot = 0;
 #pragma unroll
-  for (int k = 0; k < SP_MAX_VPT; ++k)
+  for (int k = 0; k < VPT; ++k)
     if (k < vpt) {
       const int e = lane + k * 64;
       if (e < E) seg_counts[seg * E + e] = cnt[k];
@@ -204,6 +210,7 @@ __global__ __launch_bounds__(1024) void plan_finish_kernel(const int32_t* __rest
 // Plan, pass 4: scatter.  A wave walks its 64 tokens in order; lanes = experts, so a lane's running counter is the
 // token's rank inside the expert's list (expert-major position) and a prefix count over the lanes is the expert's
 // rank inside the token's list (token-major position).
+template <int VPT>
 __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restrict__ routing, const int32_t* __restrict__ seg_offsets,
                                                            const int32_t* __restrict__ seg_pairbase, const int32_t* __restrict__ offsets,
                                                            const int32_t* __restrict__ flag, int32_t* __restrict__ tok_off,
@@ -216,9 +223,9 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restr
   const int vpt = (E + 63) / 64;
   const int64_t t0 = seg * SP_SEG;
   const int rows = (int)((N - t0) < SP_SEG ? (N - t0) : SP_SEG);
-  int pos[SP_MAX_VPT];   // next expert-major position of expert e
+  int pos[VPT];   // next expert-major position of expert e
 #pragma unroll
-  for (int k = 0; k < SP_MAX_VPT; ++k) {
+  for (int k = 0; k < VPT; ++k) {
     pos[k] = 0;
     if (k < vpt) {
       const int e = lane + k * 64;
@@ -227,35 +234,53 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restr
   }
   int tokbase = seg_pairbase[seg];
   const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-  for (int r = 0; r < rows; ++r) {
-    const int64_t tok = t0 + r;
-    const bf16_t* row = routing + tok * E;
-    int before = 0;   // routed experts of this token with a smaller index, over the previous lane groups
+  for (int r0 = 0; r0 < rows; r0 += 4) {
+    bf16_t v[4][VPT];   // four rows fetched together, then walked in order
 #pragma unroll
-    for (int k = 0; k < SP_MAX_VPT; ++k) {
-      if (k < vpt) {
-        const int e = lane + k * 64;
-        const bool on = (e < E) && ((row[e] & 0x7fff) != 0);
-        const unsigned long long bal = __ballot(on);
-        if (on) {
-          const int rank_in_token = before + __popcll(bal & lt_mask);
-          token_idx[pos[k]] = (int32_t)tok;
-          pair_dst[pos[k]] = tokbase + rank_in_token;
-          pos[k] += 1;
+    for (int i = 0; i < 4; ++i) {
+      const int r = (r0 + i < rows) ? (r0 + i) : (rows - 1);
+      const bf16_t* row = routing + (t0 + r) * E;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k)
+        if (k < vpt) {
+          const int e = lane + k * 64;
+          v[i][k] = (e < E) ? row[e] : (bf16_t)0;
         }
-        before += __popcll(bal);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (r0 + i < rows) {   // uniform
+        const int64_t tok = t0 + r0 + i;
+        int before = 0;   // routed experts of this token with a smaller index, over the previous lane groups
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+          if (k < vpt) {
+            const bool on = (v[i][k] & 0x7fff) != 0;
+            const unsigned long long bal = __ballot(on);
+            if (on) {
+              const int rank_in_token = before + __popcll(bal & lt_mask);
+              token_idx[pos[k]] = (int32_t)tok;
+              pair_dst[pos[k]] = tokbase + rank_in_token;
+              pos[k] += 1;
+            }
+            before += __popcll(bal);
+          }
+        }
+        if (lane == 0) tok_off[tok] = tokbase;
+        tokbase += before;
       }
     }
-    if (lane == 0) tok_off[tok] = tokbase;
-    tokbase += before;
   }
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Expert-major fused experts kernel.  256 threads = 4 waves per tile of 32 pairs of one expert.  Every wave computes
-// the tile's hidden activations itself (GEMM1 transposed, x rows read straight from their gathered positions as B
-// fragments), then owns D/4 output columns of the second product (also transposed, so a lane ends with ONE token and
-// 4 consecutive columns per accumulator quad: 8-byte stores into the token-major slot of the pair).
+// Expert-major fused experts kernel.  256 threads = 4 waves per tile of 32 pairs of one expert.
+//   GEMM1 (transposed, H^T = W1^T . X^T) is split over K: wave w multiplies its quarter of the model dimension, reading
+//   the x rows straight from their gathered positions as B fragments; the four partial tiles are summed through LDS
+//   in wave order, so every wave ends up with the same complete H^T.
+//   Bias, activation, routing weight and the rounding to bf16 happen in registers, which already sit in B-fragment
+//   position for GEMM2 (also transposed: OUT^T = W2^T . H^T), of which wave w owns D/4 output columns.  A lane ends
+//   with ONE pair and 4 consecutive columns per accumulator quad: 8-byte stores into the pair's token-major slot.
 // A fixed grid loops over the tiles listed by tile_off; the expert of a tile is found by bisection.
 // ---------------------------------------------------------------------------------------------------
 struct SparseArgs {
@@ -265,10 +290,13 @@ struct SparseArgs {
 };
 
 template <int D, int NT, int ACT>
-__global__ __launch_bounds__(256) void experts_mfma_sparse_kernel(const SparseArgs A) {
+__global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const SparseArgs A) {
   constexpr int KS1 = D / 16;
+  constexpr int KQ = KS1 / 4;    // K steps per wave
   constexpr int CTW = D / 128;   // column tiles per wave
+  static_assert(KS1 % 4 == 0, "the model dimension must split over four waves");
   __shared__ int32_t s_tile_off[1025];
+  __shared__ float part[4][NT * 16][64];
   if (A.flag[0] == 0) return;
   const int E = A.E;
   for (int i = threadIdx.x; i <= E; i += 256) s_tile_off[i] = A.tile_off[i];
@@ -291,25 +319,34 @@ __global__ __launch_bounds__(256) void experts_mfma_sparse_kernel(const SparseAr
     const int pj = base + j0 + (valid ? c32 : rows - 1);
     const int tok = A.token_idx[pj];
     const int dst = A.pair_dst[pj];
-    const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)tok * D);
+    const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)tok * D) + 2 * w * KQ + g;
     const float rw = bf16_to_f32(A.routing[(int64_t)tok * E + e]);
 
-    // GEMM1: H^T[NT*32 neurons, 32 pairs]
+    // GEMM1, this wave's quarter of K: all loads are issued before the first MFMA
+    const bf16x8* w1f = A.w1s + ((int64_t)e * KS1 + w * KQ) * NT * 64 + lane;
+    bf16x8 xb[KQ];
+#pragma unroll
+    for (int ks = 0; ks < KQ; ++ks) xb[ks] = xrow[2 * ks];
     f32x16 acc1[NT];
 #pragma unroll
     for (int a = 0; a < NT; ++a)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc1[a][r] = 0.f;
-    const bf16x8* w1f = A.w1s + ((int64_t)e * KS1 * NT) * 64 + lane;
-#pragma unroll 8
-    for (int ks = 0; ks < KS1; ++ks) {
-      const bf16x8 b = xrow[2 * ks + g];
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const bf16x8 a = w1f[(ks * NT + t) * 64];
-        acc1[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc1[t], 0, 0, 0);
-      }
-    }
+    for (int ks = 0; ks < KQ; ++ks)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc1[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1f[(ks * NT + t) * 64], xb[ks], acc1[t], 0, 0, 0);
+    // W2^T fragments of this wave's columns: requested now, used after the reduction
+    const bf16x8* w2f = A.w2s + ((int64_t)e * (D / 32) + w * CTW) * (2 * NT) * 64 + lane;
+    bf16x8 w2r[CTW * 2 * NT];
+#pragma unroll
+    for (int i = 0; i < CTW * 2 * NT; ++i) w2r[i] = w2f[i * 64];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) part[w][t * 16 + r][lane] = acc1[t][r];
+    __syncthreads();
     // bias, activation, routing weight, round to bf16 -> B fragments of the second product
     bf16x8 hb[2 * NT];
     const bf16_t* bias_e = A.b1s + (int64_t)e * NT * 32;
@@ -323,9 +360,12 @@ __global__ __launch_bounds__(256) void experts_mfma_sparse_kernel(const SparseAr
                                __uint_as_float(bq.y << 16), __uint_as_float(bq.y & 0xffff0000u)};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          float v = acc1[t][q * 4 + i] + bias[i];
+          const int r = q * 4 + i;
+          float v = ((part[0][t * 16 + r][lane] + part[1][t * 16 + r][lane]) + part[2][t * 16 + r][lane]) +
+                    part[3][t * 16 + r][lane];
+          v += bias[i];
           v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(A.act_rt, v);
-          hv[q * 4 + i] = v * rw;
+          hv[r] = v * rw;
         }
       }
 #pragma unroll
@@ -338,20 +378,18 @@ __global__ __launch_bounds__(256) void experts_mfma_sparse_kernel(const SparseAr
         __builtin_memcpy(&hb[t * 2 + half], &pk, 16);
       }
     }
+    __syncthreads();   // partial tiles are rewritten by the next tile
     // GEMM2 (transposed): OUT^T[D/4 columns of this wave, 32 pairs]
     f32x16 acc2[CTW];
 #pragma unroll
     for (int a = 0; a < CTW; ++a)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc2[a][r] = 0.f;
-    const bf16x8* w2f = A.w2s + ((int64_t)e * (D / 32) + w * CTW) * (2 * NT) * 64 + lane;
 #pragma unroll
     for (int ct = 0; ct < CTW; ++ct)
 #pragma unroll
-      for (int ks2 = 0; ks2 < 2 * NT; ++ks2) {
-        const bf16x8 a = w2f[(ct * 2 * NT + ks2) * 64];
-        acc2[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, hb[ks2], acc2[ct], 0, 0, 0);
-      }
+      for (int ks2 = 0; ks2 < 2 * NT; ++ks2)
+        acc2[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w2r[ct * 2 * NT + ks2], hb[ks2], acc2[ct], 0, 0, 0);
     if (valid) {
       bf16_t* yrow = A.y + (int64_t)dst * D + w * (D / 4) + 4 * g;
 #pragma unroll
@@ -441,19 +479,28 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   int32_t* pair_dst = (int32_t*)(ws + W.pair_dst);
   bf16_t* y = (bf16_t*)(ws + W.y);
   const unsigned seg_blocks = (unsigned)cdiv64(W.n_seg, 4);
-  hipLaunchKernelGGL(plan_count_kernel, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_counts, seg_pairs, N, E,
-                     W.n_seg);
+  const int vpt = (E + 63) / 64;
+#define D2DMOE_PLAN_DISPATCH(V)                                                                                          \
+  hipLaunchKernelGGL(plan_count_kernel<V>, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_counts, seg_pairs, N, \
+                     E, W.n_seg)
+  if (vpt <= 1) D2DMOE_PLAN_DISPATCH(1); else if (vpt <= 2) D2DMOE_PLAN_DISPATCH(2); else if (vpt <= 4) D2DMOE_PLAN_DISPATCH(4);
+  else if (vpt <= 8) D2DMOE_PLAN_DISPATCH(8); else D2DMOE_PLAN_DISPATCH(16);
+#undef D2DMOE_PLAN_DISPATCH
   launch_perm_scan(seg_counts, seg_offsets, totals, E, W.n_seg, s);
   hipLaunchKernelGGL(plan_finish_kernel, dim3(1), dim3(1024), 0, s, totals, seg_pairs, seg_pairbase, offsets, tile_off, flag,
                      tok_off, E, W.n_seg, N, N * (int64_t)max_mean_k);
-  hipLaunchKernelGGL(plan_scatter_kernel, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_offsets, seg_pairbase,
-                     offsets, flag, tok_off, token_idx, pair_dst, N, E, W.n_seg);
+#define D2DMOE_PLAN_DISPATCH(V)                                                                                          \
+  hipLaunchKernelGGL(plan_scatter_kernel<V>, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_offsets,    \
+                     seg_pairbase, offsets, flag, tok_off, token_idx, pair_dst, N, E, W.n_seg)
+  if (vpt <= 1) D2DMOE_PLAN_DISPATCH(1); else if (vpt <= 2) D2DMOE_PLAN_DISPATCH(2); else if (vpt <= 4) D2DMOE_PLAN_DISPATCH(4);
+  else if (vpt <= 8) D2DMOE_PLAN_DISPATCH(8); else D2DMOE_PLAN_DISPATCH(16);
+#undef D2DMOE_PLAN_DISPATCH
   SparseArgs A;
   A.x = (const bf16_t*)x; A.routing = (const bf16_t*)routing; A.w1s = (const bf16x8*)(pk + L.s1_off);
   A.w2s = (const bf16x8*)(pk + L.s2_off); A.b1s = (const bf16_t*)(pk + L.sb_off); A.offsets = offsets;
   A.tile_off = tile_off; A.token_idx = token_idx; A.pair_dst = pair_dst; A.flag = flag; A.y = y; A.E = E;
   A.act_rt = sh.activation;
-  const unsigned grid = (unsigned)(4 * device_cu_count());
+  const unsigned grid = (unsigned)(8 * device_cu_count());
   if (L.nt == 1) launch_sparse_experts<1>(A, sh.activation, grid, s);
   else if (L.nt == 2) launch_sparse_experts<2>(A, sh.activation, grid, s);
   else launch_sparse_experts<4>(A, sh.activation, grid, s);
