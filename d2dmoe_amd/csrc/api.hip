@@ -41,6 +41,8 @@ ForwardWorkspace plan_workspace(const d2dmoe_shape& sh) {
   size_t scratch = perm_workspace_bytes(sh.n_tokens, sh.n_experts);
   const size_t sparse = mfma_sparse_workspace_bytes(sh);   // plan + result rows of the expert-major path
   if (sparse > scratch) scratch = sparse;
+  const size_t decode = mfma_decode_workspace_bytes(sh);   // per-expert result rows of the small-batch path
+  if (decode > scratch) scratch = decode;
   w.perm_off = off;   off += align_up(scratch);
   w.total = off;
   return w;
@@ -85,7 +87,11 @@ int d2dmoe_router(const void* x, const void* router_w1, const void* router_w2, v
   if (!workspace || workspace_bytes < need || !aligned16(workspace)) return D2DMOE_E_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   hipError_t e;
-  if (dtype == D2DMOE_F32) {
+  if (linear_skinny_supported(n_tokens, d_model, dtype) && linear_skinny_supported(n_tokens, router_width, dtype)) {
+    // a handful of tokens: MFMA kernels that spread the output features over the machine
+    e = launch_linear_skinny(x, router_w1, workspace, (int)n_tokens, d_model, router_width, activation, s);
+    if (e == hipSuccess) e = launch_linear_skinny(workspace, router_w2, norms, (int)n_tokens, router_width, n_experts, output_activation, s);
+  } else if (dtype == D2DMOE_F32) {
     e = launch_linear_act<float>(x, router_w1, workspace, n_tokens, d_model, router_width, activation, s);
     if (e == hipSuccess) e = launch_linear_act<float>(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s);
   } else {
@@ -136,7 +142,7 @@ int d2dmoe_build_permutation(const void* routing, int64_t n_tokens, int32_t n_ex
 
 size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape) {
   if (check_shape(shape) != D2DMOE_OK) return 0;
-  if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape)) return 0;
+  if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape) && !mfma_decode_supported(*shape)) return 0;
   return mfma_packed_bytes(*shape);
 }
 
@@ -145,7 +151,9 @@ int d2dmoe_pack_weights(const d2dmoe_shape* shape, const void* w1, const void* b
   int st = check_shape(shape);
   if (st != D2DMOE_OK) return st;
   if (!w1 || !w2 || !packed) return D2DMOE_E_NULL;
-  if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape)) return D2DMOE_E_UNSUPPORTED;
+  if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape) && !mfma_decode_supported(*shape))
+    return D2DMOE_E_UNSUPPORTED;
+  if (shape->gated && !w_up) return D2DMOE_E_NULL;
   if (mfma_router_supported(*shape) && (!router_w1 || !router_w2)) return D2DMOE_E_NULL;
   if (packed_bytes < mfma_packed_bytes(*shape) || !aligned16(packed)) return D2DMOE_E_WORKSPACE;
   return (int)launch_mfma_pack(*shape, w1, b1, w2, w_up, router_w1, router_w2, packed, (hipStream_t)stream);
@@ -164,8 +172,10 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
   if (!sh.gated && w_up) return D2DMOE_E_SHAPE;
   if (!aligned16(x) || !aligned16(out) || !aligned16(routing)) return D2DMOE_E_ALIGN;
   hipStream_t s = (hipStream_t)stream;
-  if (path == D2DMOE_PATH_AUTO)
-    path = (packed != nullptr && mfma_dense_supported(sh)) ? D2DMOE_PATH_MFMA_DENSE : D2DMOE_PATH_GENERIC;
+  if (path == D2DMOE_PATH_AUTO) {
+    if (packed != nullptr && sh.n_tokens <= 16 && mfma_decode_supported(sh)) path = D2DMOE_PATH_MFMA_DECODE;
+    else path = (packed != nullptr && mfma_dense_supported(sh)) ? D2DMOE_PATH_MFMA_DENSE : D2DMOE_PATH_GENERIC;
+  }
   switch (path) {
     case D2DMOE_PATH_GENERIC: {
       if (!experts_generic_supported(sh)) return D2DMOE_E_UNSUPPORTED;
@@ -190,6 +200,14 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
       if (e != hipSuccess) return (int)e;
       return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, s);
     }
+    case D2DMOE_PATH_MFMA_DECODE: {
+      if (!mfma_decode_supported(sh) || sh.n_tokens > 16) return D2DMOE_E_UNSUPPORTED;
+      if (!packed) return D2DMOE_E_NULL;
+      const size_t need = mfma_decode_workspace_bytes(sh);
+      if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
+      return (int)launch_mfma_decode(sh, x, routing, (const char*)packed + mfma_decode_section_offset(sh), last_bias, out,
+                                     workspace, s);
+    }
     default: return D2DMOE_E_UNSUPPORTED;
   }
 }
@@ -204,7 +222,7 @@ int d2dmoe_router_select(const d2dmoe_shape* shape, const void* x, const void* r
   if (sh.router_width <= 0) return D2DMOE_E_SHAPE;
   if (sh.n_tokens == 0) return counts ? (int)launch_fill_i32(counts, sh.n_experts, 0, (hipStream_t)stream) : D2DMOE_OK;
   if (!x) return D2DMOE_E_NULL;
-  if (packed != nullptr && mfma_router_supported(sh)) {
+  if (packed != nullptr && mfma_router_supported(sh) && sh.n_tokens > 16) {
     if (!aligned16(x) || !aligned16(routing) || (norms_out && !aligned16(norms_out))) return D2DMOE_E_ALIGN;
     return (int)launch_mfma_router_select(sh, x, packed, routing, norms_out, counts, thr_scale, (hipStream_t)stream);
   }
@@ -242,7 +260,7 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   if (st != D2DMOE_OK) return st;
   // A high threshold fraction keeps few experts per token: take the expert-major path (it falls back to the dense
   // sweep on the device if the routing turns out dense after all).
-  if (path == D2DMOE_PATH_AUTO && packed != nullptr && thr_scale >= 0.75f && mfma_sparse_supported(sh) &&
+  if (path == D2DMOE_PATH_AUTO && sh.n_tokens > 16 && packed != nullptr && thr_scale >= 0.75f && mfma_sparse_supported(sh) &&
       mfma_dense_supported(sh))
     path = D2DMOE_PATH_MFMA_SPARSE;
   return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,

@@ -70,6 +70,8 @@ PackedLayout packed_layout(const d2dmoe_shape& sh) {
   L.s2_off = off;   if (L.has_sparse) off += frag_bytes;
   L.sb_off = off;   if (L.has_sparse) off += (size_t)sh.n_experts * L.nt * 32 * 2;
   off = (off + 255) / 256 * 256;
+  L.has_decode = mfma_decode_supported(sh);
+  L.dc_off = off;   if (L.has_decode) off += mfma_decode_packed_bytes(sh);
   // the router section comes last, so the expert sections sit at the same offsets whether or not the shape handed
   // to a later call names the router
   L.has_router = mfma_router_supported(sh);
@@ -80,6 +82,7 @@ PackedLayout packed_layout(const d2dmoe_shape& sh) {
 }
 
 size_t mfma_packed_bytes(const d2dmoe_shape& sh) { return packed_layout(sh).total; }
+size_t mfma_decode_section_offset(const d2dmoe_shape& sh) { return packed_layout(sh).dc_off; }
 
 // ---------------------------------------------------------------------------------------------------
 // Packing.  Each wave of the fused kernel reads ONE linear stream of 1 KB fragments (16 bytes per lane), in the
@@ -167,7 +170,6 @@ __global__ void pack_router_kernel(const bf16_t* __restrict__ rw1, const bf16_t*
 
 hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                             const void* router_w1, const void* router_w2, void* packed, hipStream_t s) {
-  (void)w_up;
   const PackedLayout L = packed_layout(sh);
   char* base = (char*)packed;
   if (L.has_router) {
@@ -179,6 +181,10 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
   }
   if (L.has_sparse) {
     hipError_t e = launch_sparse_pack(sh, L, w1, b1, w2, packed, s);
+    if (e != hipSuccess) return e;
+  }
+  if (L.has_decode) {
+    hipError_t e = launch_decode_pack(sh, w1, b1, w2, w_up, base + L.dc_off, s);
     if (e != hipSuccess) return e;
   }
   if (!L.has_dense) return hipGetLastError();

@@ -53,6 +53,14 @@ size_t mfma_sparse_workspace_bytes(const d2dmoe_shape& sh);
 hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                               const void* last_bias, void* out, void* workspace, int max_mean_k, const int** flag_out,
                               hipStream_t s);
+// ---- small-batch (<= 16 tokens) bf16 MFMA path (kernels_decode.hip) ----
+bool mfma_decode_supported(const d2dmoe_shape& sh);
+size_t mfma_decode_workspace_bytes(const d2dmoe_shape& sh);
+hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
+                              const void* last_bias, void* out, void* workspace, hipStream_t s);
+size_t mfma_decode_section_offset(const d2dmoe_shape& sh);
+bool linear_skinny_supported(int64_t N, int K, int dtype);
+hipError_t launch_linear_skinny(const void* A, const void* B, void* C, int N, int K, int Nout, int act, hipStream_t s);
 void launch_perm_scan(const int32_t* seg_counts, int32_t* seg_offsets, int32_t* totals, int E, int64_t n_seg, hipStream_t s);
 
 }  // namespace d2dmoe

@@ -68,9 +68,11 @@ enum {
   D2DMOE_PATH_AUTO = 0,       /* MFMA kernels when the shape and dtype have one, else the generic kernel */
   D2DMOE_PATH_GENERIC = 1,    /* token-tile-major scalar-FMA kernel: any shape, f32 or bf16 storage, f32 math */
   D2DMOE_PATH_MFMA_DENSE = 2, /* bf16 MFMA, token-tile-major, masked dense sweep over all experts */
-  D2DMOE_PATH_MFMA_SPARSE = 3 /* bf16 MFMA, expert-major over the permutation, then ordered combine; taken when at most
+  D2DMOE_PATH_MFMA_SPARSE = 3, /* bf16 MFMA, expert-major over the permutation, then ordered combine; taken when at most
                                  8 experts per token are routed on average (checked on the device), else the dense
                                  sweep runs.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 */
+  D2DMOE_PATH_MFMA_DECODE = 4 /* bf16 MFMA for at most 16 tokens: one workgroup per expert streams that expert's packed
+                                 weights once (gated or ungated experts); AUTO picks it when it applies */
 };
 
 /* Shape of one MoE-FFN layer.  Mirrors the constructor arguments of the reference layer

@@ -358,6 +358,43 @@ def test_router_select_mfma(N, D, W, E, tau):
         assert H.rel_err(out.cpu(), want) < H.TOL_BF16
 
 
+# =================================================================== small-batch (decode) path ========
+@pytest.mark.parametrize('N', [1, 5, 16])
+@pytest.mark.parametrize('D,E,Ed,W,gated,act', [(2048, 256, 64, 256, True, 'gelu_tanh'), (2048, 256, 64, 256, True, 'relu'),
+                                               (768, 128, 24, 128, False, 'relu'), (768, 24, 128, 128, False, 'gelu'),
+                                               (1024, 16, 32, 128, True, 'silu')])
+def test_decode_path_matches_oracle(N, D, E, Ed, W, gated, act):
+    """At most 16 tokens: one workgroup per expert streams its packed weights; BASELINE config 5 is the first shape."""
+    _say('decode', N, D, E, Ed, gated, act)
+    x, routing, p = H.random_case(N, D, E, Ed, W, seed=N + E, dtype=torch.bfloat16, gated=gated, bias=not gated, density=0.7)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, W, 1, act, gated=gated)
+    if gated:
+        packed = _ops().pack_weights(sh, d['w_gate'], None, d['w_down'], d['w_up'], d['router_w1'], d['router_w2'])
+    else:
+        packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, d['router_w1'], d['router_w2'])
+    assert packed is not None
+    got = _experts_got(x, routing, p, act, path='mfma_decode', packed=packed)
+    assert H.rel_err(got, _experts_want(x, routing, p, act)) < H.TOL_BF16
+    assert H.rel_err(got, _experts_got(x, routing, p, act, path='generic')) < 1e-2
+    assert torch.equal(got, _experts_got(x, routing, p, act, path='auto', packed=packed))   # AUTO picks it for N <= 16
+    # nothing routed / one expert for everybody / weighted routing
+    zero = _experts_got(x, torch.zeros_like(routing), p, act, path='mfma_decode', packed=packed)
+    lbias = p['last_bias'].expand(N, -1).float() if 'last_bias' in p else torch.zeros(N, D)
+    assert torch.equal(zero.float(), lbias)
+    g = torch.Generator().manual_seed(3)
+    weights = (routing.float() * (torch.rand(N, E, generator=g) + 0.5)).bfloat16()
+    got = _experts_got(x, weights, p, act, residual=True, path='mfma_decode', packed=packed)
+    assert H.rel_err(got, _experts_want(x, weights, p, act, True)) < H.TOL_BF16
+    # whole layer: skinny router kernels + select + decode experts
+    out, r, norms, counts = _forward(x, p, 0.9, act, packed=packed)
+    want64 = O.router_forward(x.double(), p['router_w1'].double(), p['router_w2'].double())
+    assert H.rel_err(norms.cpu(), want64) < H.TOL_BF16
+    assert torch.equal(r.cpu(), O.gate_dynk_max(norms.cpu(), 0.9))
+    want = O.layer_from_routing(x.double(), O.upcast(p), r.cpu().double(), act, 'all')
+    assert H.rel_err(out.cpu(), want) < H.TOL_BF16
+
+
 # =================================================================== whole layer ======================
 def _forward(x, p, tau, act='relu', norms_in=None, path='auto', packed=None, residual=False):
     d = H.to_dev(p, DEV)
