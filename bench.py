@@ -37,6 +37,12 @@ WORKLOADS = {
     'vit_b_50k': (256, 197, 768, 128, 24, 128, 'relu'),
     'vit_b_1576': (8, 197, 768, 128, 24, 128, 'relu'),
 }
+# Gemma-2B-shape gated layer (BASELINE config 5): (tokens, D, E, Ed, W, activation)
+GATED_WORKLOADS = {
+    'gemma_1': (1, 2048, 256, 64, 256, 'gelu_tanh'),
+    'gemma_16': (16, 2048, 256, 64, 256, 'gelu_tanh'),
+    'gemma_4096': (4096, 2048, 256, 64, 256, 'gelu_tanh'),
+}
 
 
 def make_params(D, E, Ed, W, seed, dtype, device):
@@ -105,6 +111,53 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, pa
                 algo_bytes=algo_bytes, hbm_gbps_layer=algo_bytes / ms_layer / 1e6, tokens_per_s=N / ms_layer * 1e3)
 
 
+def run_gated(args, ops, dev):
+    """Gemma-shape gated layer: whole-layer time and the HBM rate over the bytes that have to move (router weights,
+    the weights of every expert some token routes to, token input/output)."""
+    N, D, E, Ed, W, act = GATED_WORKLOADS[args.workload]
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(0)
+
+    def uni(*shape, fan):
+        return ((torch.rand(*shape, generator=g) * 2 - 1) / fan ** 0.5).to(dtype).to(dev)
+
+    wg, wd, wu = uni(E, D, Ed, fan=Ed), uni(E, Ed, D, fan=D), uni(E, D, Ed, fan=Ed)
+    rw1, rw2 = uni(W, D, fan=D), uni(E, W, fan=W)
+    x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
+    shape = ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x), act, gated=True)
+    packed = ops.pack_weights(shape, wg, None, wd, wu, rw1, rw2)
+    thr_scale = float(1.0 - args.tau)
+
+    def layer():
+        return ops.forward(x, rw1, rw2, thr_scale, wg, None, wd, wu, None, act, False, None, False, False, 'auto', packed)
+
+    out, routing, _, _ = layer()
+    torch.cuda.synchronize()
+    union = int((routing.float().sum(0) > 0).sum().item())
+    pairs = int(routing.float().sum().item())
+    ms_layer = time_events(layer, args.steps, args.warmup)
+    ms_experts = time_events(lambda: ops.experts(x, routing, wg, None, wd, wu, None, act, False, 'auto', packed),
+                             args.steps, args.warmup)
+    s = x.element_size()
+    algo_bytes = (W * D + E * W) * s + union * 3 * D * Ed * s + 2 * N * D * s + N * E * s
+    line = {
+        'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
+        'value': N / ms_layer * 1e3, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': ms_layer, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16',
+        'data': 'synthetic',
+        'config': {'workload': f'{args.workload}: {N} tokens, D={D}, {E} gated experts x {Ed}, {act}, router {D}->{W}->{E}, '
+                               f'module tau={args.tau}, whole layer', 'experts_routed_to': union,
+                   'mean_active_experts': pairs / N, 'mfma_kernels': packed is not None},
+        'active_tflops': pairs * 6.0 * D * Ed / ms_layer / 1e9, 'hbm_gbps': algo_bytes / ms_layer / 1e6,
+        'roofline': {'bound': 'hbm', 'kernel': 'experts', 'achieved': (union * 3 * D * Ed * s + 2 * N * D * s) / ms_experts / 1e6,
+                     'peak': PEAK_HBM_GBPS, 'unit': 'GB/s',
+                     'frac': (union * 3 * D * Ed * s + 2 * N * D * s) / ms_experts / 1e6 / PEAK_HBM_GBPS, 'traffic': None,
+                     'kernel_ms': ms_experts, 'algorithmic_bytes_layer': algo_bytes,
+                     'layer_frac': algo_bytes / ms_layer / 1e6 / PEAK_HBM_GBPS},
+    }
+    print(json.dumps(line))
+
+
 def cpu_baseline(D, E, Ed, W, act, tau, budget_s=15.0):
     """The oracle's restatement of the reference CPU path (router -> dynk_max gate -> per-expert loop), float32,
     8 x 197 tokens of the same layer shape, repeated until about budget_s seconds have been spent."""
@@ -134,7 +187,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS))
+    ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS) + sorted(GATED_WORKLOADS))
     ap.add_argument('--tau', type=float, default=0.9, help='module tau (keep expert when norm >= (1 - tau) * max)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--copy-probe', action='store_true',
@@ -149,6 +202,10 @@ def main():
         sys.exit(1)
     from d2dmoe_amd import ops
     dev = torch.device('cuda:0')
+    if args.workload in GATED_WORKLOADS:
+        with torch.no_grad():
+            run_gated(args, ops, dev)
+        return
     B, T, D, E, Ed, W, act = WORKLOADS[args.workload]
     N = B * T
     dtype = torch.bfloat16

@@ -127,7 +127,7 @@ struct DecodeArgs {
   bf16_t* y; int N; int D; int E; int act; int gated;
 };
 
-template <int NT16, bool GATED>
+template <int NT16, bool GATED, int U1, int U2>
 __global__ __launch_bounds__(256) void decode_experts_kernel(const DecodeArgs A) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int D = A.D, N = A.N, E = A.E;
@@ -164,10 +164,10 @@ __global__ __launch_bounds__(256) void decode_experts_kernel(const DecodeArgs A)
   const int64_t mat_frags = (int64_t)KS * NT16 * 64;
   const bf16x8* wgf = A.wg + (int64_t)e * mat_frags + (int64_t)w * KQ * NT16 * 64 + lane;
   const bf16x8* wuf = GATED ? (A.wu + (int64_t)e * mat_frags + (int64_t)w * KQ * NT16 * 64 + lane) : nullptr;
-  for (int ks0 = 0; ks0 < KQ; ks0 += 2) {   // two K steps per trip: their weight fragments are in flight together
-    bf16x8 b[2], ag[2][NT16], au[2][NT16];
+  for (int ks0 = 0; ks0 < KQ; ks0 += U1) {   // U1 K steps per trip: their weight fragments are in flight together
+    bf16x8 b[U1], ag[U1][NT16], au[U1][NT16];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < U1; ++u) {
       b[u] = xs[(w * KQ + ks0 + u) * 64 + lane];
 #pragma unroll
       for (int a = 0; a < NT16; ++a) {
@@ -176,16 +176,21 @@ __global__ __launch_bounds__(256) void decode_experts_kernel(const DecodeArgs A)
       }
     }
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+    for (int u = 0; u < U1; ++u)
 #pragma unroll
       for (int a = 0; a < NT16; ++a) {
         acc1[0][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ag[u][a], b[u], acc1[0][a], 0, 0, 0);
         if (GATED) acc1[NM - 1][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(au[u][a], b[u], acc1[NM - 1][a], 0, 0, 0);
       }
   }
-  // W2^T fragments of this wave's columns: the first batch is requested before the reduction
+  // W2^T fragments of this wave's columns: the first batch is requested before the reduction below
   const int CTW = D / 64;   // 16-column tiles per wave
   const bf16x8* wdf = A.wd + ((int64_t)e * (D / 16) + (int64_t)w * CTW) * KS2 * 64 + lane;
+  bf16x8 a2[U2][KS2];
+#pragma unroll
+  for (int j = 0; j < U2; ++j)
+#pragma unroll
+    for (int k2 = 0; k2 < KS2; ++k2) a2[j][k2] = wdf[(j * KS2 + k2) * 64];
 #pragma unroll
   for (int m = 0; m < NM; ++m)
 #pragma unroll
@@ -222,16 +227,21 @@ __global__ __launch_bounds__(256) void decode_experts_kernel(const DecodeArgs A)
     pk.z = pack2_bf16(hv[4], hv[5]); pk.w = pack2_bf16(hv[6], hv[7]);
     __builtin_memcpy(&hb[k2], &pk, 16);
   }
-  // ---- GEMM2 (transposed), 4 column tiles at a time
+  // ---- GEMM2 (transposed), U2 column tiles at a time, double-buffered in registers
   bf16_t* yrow = A.y + ((int64_t)e * DC_MAX_TOKENS + c16) * D + (int64_t)w * (D / 4) + 4 * gq;
-  for (int ct0 = 0; ct0 < CTW; ct0 += 4) {
-    bf16x8 a[4][KS2];
+  for (int ct0 = 0; ct0 < CTW; ct0 += U2) {
+    bf16x8 a[U2][KS2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < U2; ++j)
 #pragma unroll
-      for (int k2 = 0; k2 < KS2; ++k2) a[j][k2] = wdf[((ct0 + j) * KS2 + k2) * 64];
+      for (int k2 = 0; k2 < KS2; ++k2) {
+        a[j][k2] = a2[j][k2];
+        // request the next batch while this one is multiplied (the last trip re-reads its own batch: in bounds)
+        const int ctn = (ct0 + U2 < CTW) ? (ct0 + U2) : ct0;
+        a2[j][k2] = wdf[((ctn + j) * KS2 + k2) * 64];
+      }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < U2; ++j) {
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int k2 = 0; k2 < KS2; ++k2) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][k2], hb[k2], acc, 0, 0, 0);
@@ -245,26 +255,32 @@ __global__ __launch_bounds__(256) void decode_experts_kernel(const DecodeArgs A)
   }
 }
 
-// Ordered combine for the decode path: thread = (token, 8 columns); experts ascending, float32, one rounding.
+// Combine for the decode path.  A workgroup owns one token and 128 output columns: 16 column pieces (8 columns, 16
+// bytes) x 16 expert groups.  Thread (piece, group) adds its group's routed experts in ascending order; the 16 group
+// sums are then added in ascending group order.  The summation order is fixed, so results are reproducible.
 __global__ __launch_bounds__(256) void decode_combine_kernel(const bf16_t* __restrict__ y, const bf16_t* __restrict__ routing,
                                                              const bf16_t* __restrict__ x, const bf16_t* __restrict__ last_bias,
                                                              bf16_t* __restrict__ out, int N, int D, int E, int add_residual) {
-  const int ppr = D / 8;
-  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-  const int n = idx / ppr;
-  if (n >= N) return;
-  const int col = (idx - n * ppr) * 8;
+  __shared__ float part[16][16][9];   // [group][piece][8 columns + pad]
+  const int t = threadIdx.x;
+  const int piece = t & 15, grp = t >> 4;
+  const int blocks_per_token = D / 128;
+  const int n = blockIdx.x / blocks_per_token;
+  const int col = (blockIdx.x % blocks_per_token) * 128 + piece * 8;
+  const int per = (E + 15) / 16;            // experts per group
+  const int e_lo = grp * per, e_hi = (e_lo + per < E) ? (e_lo + per) : E;
+  const bf16_t* rrow = routing + (int64_t)n * E;
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-  const bf16_t* rrow = routing + (int64_t)n * E;
-  for (int e0 = 0; e0 < E; e0 += 8) {
+  for (int e0 = e_lo; e0 < e_hi; e0 += 8) {
     uint4 v[8];
     bool on[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      on[j] = (e0 + j < E) && ((rrow[e0 + j] & 0x7fff) != 0);
-      v[j] = on[j] ? *(const uint4*)(y + ((int64_t)(e0 + j) * DC_MAX_TOKENS + n) * D + col) : uint4{0u, 0u, 0u, 0u};
+      on[j] = (e0 + j < e_hi) && ((rrow[e0 + j] & 0x7fff) != 0);
+      v[j] = uint4{0u, 0u, 0u, 0u};
+      if (on[j]) v[j] = *(const uint4*)(y + ((int64_t)(e0 + j) * DC_MAX_TOKENS + n) * D + col);
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -275,38 +291,54 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const bf16_t* __res
       }
     }
   }
-  if (last_bias != nullptr) {
-    const uint4 v = *(const uint4*)(last_bias + col);
-    const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
-  }
-  if (add_residual) {
-    const uint4 v = *(const uint4*)(x + (int64_t)n * D + col);
-    const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
+  for (int i = 0; i < 8; ++i) part[grp][piece][i] = acc[i];
+  __syncthreads();
+  if (grp == 0) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+    for (int i = 0; i < 8; ++i) {
+      float s = part[0][piece][i];
+      for (int gi = 1; gi < 16; ++gi) s += part[gi][piece][i];
+      acc[i] = s;
+    }
+    if (last_bias != nullptr) {
+      const uint4 v = *(const uint4*)(last_bias + col);
+      const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+    }
+    if (add_residual) {
+      const uint4 v = *(const uint4*)(x + (int64_t)n * D + col);
+      const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+    }
+    uint4 o;
+    o.x = pack2_bf16(acc[0], acc[1]); o.y = pack2_bf16(acc[2], acc[3]);
+    o.z = pack2_bf16(acc[4], acc[5]); o.w = pack2_bf16(acc[6], acc[7]);
+    *(uint4*)(out + (int64_t)n * D + col) = o;
   }
-  uint4 o;
-  o.x = pack2_bf16(acc[0], acc[1]); o.y = pack2_bf16(acc[2], acc[3]);
-  o.z = pack2_bf16(acc[4], acc[5]); o.w = pack2_bf16(acc[6], acc[7]);
-  *(uint4*)(out + (int64_t)n * D + col) = o;
+}
+
+template <int NT16, bool GATED, int U1, int U2>
+static hipError_t launch_decode_cfg(const DecodeArgs& A, size_t lds, hipStream_t s) {
+  auto k = decode_experts_kernel<NT16, GATED, U1, U2>;
+  hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(k, dim3(A.E), dim3(256), lds, s, A);
+  return hipGetLastError();
 }
 
 template <int NT16>
 static hipError_t launch_decode_nt(const DecodeArgs& A, size_t lds, hipStream_t s) {
+  // deeper batches when the per-wave trip counts divide: K steps per wave = D/128, column tiles per wave = D/64
+  const bool deep = (A.D % 512 == 0);
   if (A.gated) {
-    auto k = decode_experts_kernel<NT16, true>;
-    hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(k, dim3(A.E), dim3(256), lds, s, A);
-  } else {
-    auto k = decode_experts_kernel<NT16, false>;
-    hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(k, dim3(A.E), dim3(256), lds, s, A);
+    if (deep && NT16 <= 4) return launch_decode_cfg<NT16, true, 4, 8>(A, lds, s);
+    return launch_decode_cfg<NT16, true, 2, 4>(A, lds, s);
   }
-  return hipGetLastError();
+  if (deep && NT16 <= 4) return launch_decode_cfg<NT16, false, 4, 8>(A, lds, s);
+  return launch_decode_cfg<NT16, false, 2, 4>(A, lds, s);
 }
 
 hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
@@ -325,8 +357,7 @@ hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void*
   else if (L.nt16 == 4) e = launch_decode_nt<4>(A, lds, s);
   else e = launch_decode_nt<8>(A, lds, s);
   if (e != hipSuccess) return e;
-  const int n_threads = (int)sh.n_tokens * (sh.d_model / 8);
-  hipLaunchKernelGGL(decode_combine_kernel, dim3((n_threads + 255) / 256), dim3(256), 0, s, (const bf16_t*)workspace,
+  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)sh.n_tokens * (sh.d_model / 128)), dim3(256), 0, s, (const bf16_t*)workspace,
                      (const bf16_t*)routing, (const bf16_t*)x, (const bf16_t*)last_bias, (bf16_t*)out, (int)sh.n_tokens,
                      sh.d_model, sh.n_experts, sh.add_residual);
   return hipGetLastError();
