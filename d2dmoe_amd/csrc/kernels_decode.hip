@@ -1,7 +1,8 @@
 // Small-batch ("decode") bf16 MFMA path: at most 16 tokens, so the layer is bound by streaming the weights of the
-// routed experts once.  One workgroup per expert pulls that expert's packed weights (gate/up and down projections)
-// through v_mfma_f32_16x16x32_bf16 with all tokens resident in LDS; per-expert results are summed afterwards in
-// ascending expert order.  Also here: a skinny Linear kernel (router layers for <= 16 tokens) that needs no packing.
+// routed experts once.  One workgroup per expert pulls that expert's packed gate/up weights through
+// v_mfma_f32_16x16x32_bf16 with all tokens resident in LDS and leaves the hidden activations (256 KB for 256 experts
+// of 32 neurons) in memory; a second kernel owns 16 output columns per workgroup and sums the down projections of the
+// routed experts in ascending order.  Also here: a skinny Linear kernel (router layers for <= 16 tokens) that needs no packing.
 //
 // Fragment layouts of the 16x16x32 bf16 MFMA on a 64-lane wave (gq = lane / 16, c = lane % 16):
 //   A (16 x 32): lane holds row c,    k = 8 gq .. 8 gq + 7
@@ -22,7 +23,7 @@ constexpr int DC_MAX_TOKENS = 16;
 struct DecodeLayout {
   int edp;      // neurons per expert padded to a multiple of 32
   int nt16;     // 16-neuron tiles per expert
-  size_t g_off, u_off, d_off, b_off, total;   // gate (or w1), up, down^T fragments, bias (bf16, padded)
+  size_t gu_off, d_off, b_off, total;   // gate(/up) fragment stream, down^T fragments, bias (bf16, padded)
 };
 
 static DecodeLayout decode_layout(const d2dmoe_shape& sh) {
@@ -31,8 +32,7 @@ static DecodeLayout decode_layout(const d2dmoe_shape& sh) {
   L.nt16 = L.edp / 16;
   const size_t mat = (size_t)sh.n_experts * L.edp * sh.d_model * 2;
   size_t off = 0;
-  L.g_off = off; off += mat;
-  L.u_off = off; if (sh.gated) off += mat;
+  L.gu_off = off; off += mat * (sh.gated ? 2 : 1);
   L.d_off = off; off += mat;
   L.b_off = off; off += (size_t)sh.n_experts * L.edp * 2;
   L.total = (off + 255) / 256 * 256;
@@ -41,7 +41,7 @@ static DecodeLayout decode_layout(const d2dmoe_shape& sh) {
 
 bool mfma_decode_supported(const d2dmoe_shape& sh) {
   if (sh.dtype != D2DMOE_BF16) return false;
-  if (sh.d_model % 256 != 0 || sh.d_model > 4096) return false;   // K quarters of whole 32-steps, column tiles in fours
+  if (sh.d_model % 256 != 0 || sh.d_model > 4096) return false;   // an even number of whole 32-steps per wave
   const int edp = (sh.expert_dim + 31) / 32 * 32;
   return edp == 32 || edp == 64 || edp == 128;
 }
@@ -50,54 +50,59 @@ size_t mfma_decode_packed_bytes(const d2dmoe_shape& sh) { return mfma_decode_sup
 
 size_t mfma_decode_workspace_bytes(const d2dmoe_shape& sh) {
   if (!mfma_decode_supported(sh)) return 0;
-  return (size_t)sh.n_experts * DC_MAX_TOKENS * sh.d_model * 2;   // per-expert result rows, bf16
+  // hidden activations as bf16 fragments, then one "some token routes here" flag per expert
+  return (size_t)sh.n_experts * decode_layout(sh).edp * DC_MAX_TOKENS * 2 + (size_t)sh.n_experts * 4;
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Packing.  KS = D/32 K steps, nt16 neuron tiles, EdP padded neurons.
-//   gate / up fragments [E][kstep KS][nt16][lane][8]:  neuron j = t*16 + c, d = kstep*32 + 8 gq + i     w[e][d][j]
-//   down^T fragments    [E][col-tile D/16][kstep2 EdP/32][lane][8]:  column = ct*16 + c,
-//                       neuron j = ks2*32 + 16*(i/4) + 4 gq + (i%4)                                       w2[e][j][column]
-//   bias                [E][EdP] bf16
+// Packing.  KS = D/32 K steps, EdP padded neurons, NB = EdP/32 neuron blocks, NM = 2 if gated else 1.  Every workgroup of
+// the two kernels below reads ONE contiguous stream.
+//   gate(/up) stream [E][block NB][kstep KS][matrix NM][tile 2][lane 64][8]:
+//                    neuron j = block*32 + tile*16 + c, d = kstep*32 + 8 gq + i                          w[e][d][j]
+//   down^T stream    [column block D/8][E][kstep2 NB][gq 4][c8 8][8]:  column = cb*8 + c8,
+//                    neuron j = ks2*32 + 16*(i/4) + 4 gq + (i%4)                                         w2[e][j][column]
+//   bias             [E][EdP] bf16
 // ---------------------------------------------------------------------------------------------------
 __global__ void pack_decode_kernel(const bf16_t* __restrict__ w1, const bf16_t* __restrict__ b1, const bf16_t* __restrict__ w2,
-                                   const bf16_t* __restrict__ w_up, bf16_t* __restrict__ dg, bf16_t* __restrict__ du,
-                                   bf16_t* __restrict__ dd, bf16_t* __restrict__ db, int D, int E, int Ed, int edp) {
+                                   const bf16_t* __restrict__ w_up, bf16_t* __restrict__ dgu, bf16_t* __restrict__ dd,
+                                   bf16_t* __restrict__ db, int D, int E, int Ed, int edp) {
   const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t per_expert = (int64_t)edp * D / 8;   // 16-byte pieces per expert and matrix
-  const int64_t n = (int64_t)E * per_expert;
-  const int lane = (int)(p % 64);
-  const int gq = lane / 16, c = lane % 16;
-  const int nt16 = edp / 16;
-  if (p < 2 * n) {   // gate, then up
-    const bool is_up = p >= n;
-    const int64_t pp = is_up ? p - n : p;
-    if (is_up && w_up == nullptr) return;
-    const bf16_t* src = is_up ? w_up : w1;
-    bf16_t* dst = is_up ? du : dg;
-    const int e = (int)(pp / per_expert);
-    const int64_t q = (pp % per_expert) / 64;
-    const int t = (int)(q % nt16), ks = (int)(q / nt16);
-    const int j = t * 16 + c;
+  const int nm = (w_up != nullptr) ? 2 : 1;
+  const int KS = D / 32, NB = edp / 32;
+  const int64_t n_gu = (int64_t)E * NB * KS * nm * 2 * 64;   // 16-byte pieces
+  const int64_t n_d = (int64_t)(D / 8) * E * NB * 32;
+  if (p < n_gu) {
+    int64_t q = p;
+    const int lane = (int)(q % 64); q /= 64;
+    const int tile = (int)(q % 2); q /= 2;
+    const int m = (int)(q % nm); q /= nm;
+    const int ks = (int)(q % KS); q /= KS;
+    const int blk = (int)(q % NB);
+    const int e = (int)(q / NB);
+    const int gq = lane / 16, c = lane % 16;
+    const bf16_t* src = m ? w_up : w1;
+    const int j = blk * 32 + tile * 16 + c;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int d = ks * 32 + 8 * gq + i;
-      dst[pp * 8 + i] = (j < Ed) ? src[((int64_t)e * D + d) * Ed + j] : (bf16_t)0;
+      dgu[p * 8 + i] = (j < Ed) ? src[((int64_t)e * D + d) * Ed + j] : (bf16_t)0;
     }
-  } else if (p < 3 * n) {
-    const int64_t pp = p - 2 * n;
-    const int e = (int)(pp / per_expert);
-    const int64_t q = (pp % per_expert) / 64;
-    const int nks2 = edp / 32;
-    const int ks2 = (int)(q % nks2), ct = (int)(q / nks2);
-    const int col = ct * 16 + c;
+  } else if (p < n_gu + n_d) {
+    const int64_t pp = p - n_gu;
+    int64_t q = pp;
+    const int c8 = (int)(q % 8); q /= 8;
+    const int gq = (int)(q % 4); q /= 4;
+    const int ks2 = (int)(q % NB); q /= NB;
+    const int e = (int)(q % E);
+    const int cb = (int)(q / E);
+    const int col = cb * 8 + c8;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int j = ks2 * 32 + 16 * (i / 4) + 4 * gq + (i % 4);
       dd[pp * 8 + i] = (j < Ed) ? w2[((int64_t)e * Ed + j) * D + col] : (bf16_t)0;
     }
-  } else if (p < 3 * n + (int64_t)E * edp) {
-    const int64_t pp = p - 3 * n;
+  } else if (p < n_gu + n_d + (int64_t)E * edp) {
+    const int64_t pp = p - n_gu - n_d;
     const int e = (int)(pp / edp), j = (int)(pp % edp);
     db[pp] = (j < Ed && b1 != nullptr) ? b1[(int64_t)e * Ed + j] : (bf16_t)0;
   }
@@ -107,238 +112,235 @@ hipError_t launch_decode_pack(const d2dmoe_shape& sh, const void* w1, const void
                               void* packed_section, hipStream_t s) {
   const DecodeLayout L = decode_layout(sh);
   char* base = (char*)packed_section;
-  const int64_t n = 3 * (int64_t)sh.n_experts * L.edp * sh.d_model / 8 + (int64_t)sh.n_experts * L.edp;
+  const int nm = sh.gated ? 2 : 1;
+  const int64_t n = (int64_t)(nm + 1) * sh.n_experts * L.edp * sh.d_model / 8 + (int64_t)sh.n_experts * L.edp;
   hipLaunchKernelGGL(pack_decode_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const bf16_t*)w1, (const bf16_t*)b1,
-                     (const bf16_t*)w2, (const bf16_t*)w_up, (bf16_t*)(base + L.g_off), (bf16_t*)(base + L.u_off),
+                     (const bf16_t*)w2, sh.gated ? (const bf16_t*)w_up : (const bf16_t*)nullptr, (bf16_t*)(base + L.gu_off),
                      (bf16_t*)(base + L.d_off), (bf16_t*)(base + L.b_off), sh.d_model, sh.n_experts, sh.expert_dim, L.edp);
   return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Decode experts kernel: workgroup = expert, 4 waves.
-//   stage   x [N <= 16, D] as B fragments in LDS (rows beyond N are zero); leave at once if no token routes here
-//   GEMM1   wave w: its quarter of K for all neuron tiles, gate and (if gated) up; partial tiles summed through LDS
-//           in wave order
-//   hidden  gated: act(g) * u, else act(g + b1); times the routing weight; rounded to bf16 -> B fragments
-//   GEMM2   wave w: D/4 output columns, OUT^T = W2^T . H^T; the lane's token row of y[e] gets 8-byte stores
+// Two kernels, no per-expert output rows in memory:
+//
+// decode_hidden_kernel: workgroup = (expert, block of 32 neurons), 4 waves.
+//   leave at once if no token routes to the expert
+//   GEMM1   wave w: its quarter of K for the block's two neuron tiles, gate and (if gated) up.  Weight fragments and
+//           the x fragments (straight from the row-major x, which stays in L2) go through two register buffers so the
+//           stream never drains; the four partial tiles are summed through LDS in wave order
+//   hidden  gated: act(g) * u, else act(g + b1); times the routing weight; rounded to bf16 and stored as one B
+//           fragment of the second product: hfrag[e][block][lane]
+//
+// decode_out_kernel: workgroup = 8 output columns, 8 waves.
+//   the routed experts are listed in ascending order and cut into 8 consecutive runs, one per wave; a wave chains
+//   OUT^T += W2[e]^T . H[e]^T over its run in one float32 accumulator (rows 8..15 of the 16-row MFMA tile are zero
+//   and dropped); the 8 partial tiles are added in wave order, then last_bias and the residual, one
+//   rounding.  The summation order depends on the routing only.
 // ---------------------------------------------------------------------------------------------------
 struct DecodeArgs {
-  const bf16_t* x; const bf16_t* routing; const bf16x8* wg; const bf16x8* wu; const bf16x8* wd; const bf16_t* bias;
-  bf16_t* y; int N; int D; int E; int act; int gated;
+  const bf16_t* x; const bf16_t* routing; const bf16x8* wgu; const bf16x8* wd; const bf16_t* bias;
+  bf16x8* hfrag; int* active; const bf16_t* last_bias; bf16_t* out; int N; int D; int E; int nt16; int act; int add_residual;
 };
 
-template <int NT16, bool GATED, int U1, int U2>
-__global__ __launch_bounds__(256) void decode_experts_kernel(const DecodeArgs A) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  const int D = A.D, N = A.N, E = A.E;
+template <bool GATED, int U1>
+__global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) {
+  __shared__ float part[4][(GATED ? 2 : 1) * 8][64];
+  const int D = A.D, N = A.N, E = A.E, NT16 = A.nt16;
   const int KS = D / 32;          // K steps of GEMM1
   const int KQ = KS / 4;          // per wave
   constexpr int NM = GATED ? 2 : 1;
-  constexpr int KS2 = NT16 / 2;   // K steps of GEMM2
-  bf16x8* xs = (bf16x8*)smem_raw;                                   // [KS][64]
-  float* part = (float*)(xs + (size_t)KS * 64);                     // [4][NM*NT16*4][64]
-  int* s_any = (int*)(part + 4 * NM * NT16 * 4 * 64);
-  const int e = blockIdx.x;
+  constexpr int FPS = NM * 2;     // fragments per K step
+  const int KS2 = NT16 / 2;
+  const int e = blockIdx.x / KS2, k2 = blockIdx.x % KS2;
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
   const int gq = lane >> 4, c16 = lane & 15;
-  if (t == 0) *s_any = 0;
-  __syncthreads();
-  if (t < N && (A.routing[(int64_t)t * E + e] & 0x7fff) != 0) *s_any = 1;
-  // x tile -> B fragments: fragment (ks, lane) = x[token c16][ks*32 + 8 gq .. +7]
-  for (int p = t; p < KS * 64; p += 256) {
-    const int ks = p >> 6, l = p & 63;
-    const int tok = l & 15, g4 = l >> 4;
-    uint4 v = {0u, 0u, 0u, 0u};
-    if (tok < N) v = *(const uint4*)(A.x + (int64_t)tok * D + ks * 32 + 8 * g4);
-    ((uint4*)xs)[p] = v;
-  }
-  __syncthreads();
-  if (*s_any == 0) return;   // nobody routes to this expert: its rows of y are never read
+  const int tc = (c16 < N) ? c16 : (N - 1);
+  const bf16_t rbits = A.routing[(int64_t)tc * E + e];
+  const bool any = __ballot((rbits & 0x7fff) != 0) != 0ull;
+  if (k2 == 0 && t == 0) A.active[e] = any ? 1 : 0;
+  if (!any) return;   // nobody routes to this expert: its fragments are never read
 
-  // ---- GEMM1, this wave's quarter of K
-  f32x4 acc1[NM][NT16];
+  f32x4 acc1[NM][2];
 #pragma unroll
   for (int m = 0; m < NM; ++m)
 #pragma unroll
-    for (int a = 0; a < NT16; ++a) acc1[m][a] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int64_t mat_frags = (int64_t)KS * NT16 * 64;
-  const bf16x8* wgf = A.wg + (int64_t)e * mat_frags + (int64_t)w * KQ * NT16 * 64 + lane;
-  const bf16x8* wuf = GATED ? (A.wu + (int64_t)e * mat_frags + (int64_t)w * KQ * NT16 * 64 + lane) : nullptr;
-  for (int ks0 = 0; ks0 < KQ; ks0 += U1) {   // U1 K steps per trip: their weight fragments are in flight together
-    bf16x8 b[U1], ag[U1][NT16], au[U1][NT16];
+    for (int a = 0; a < 2; ++a) acc1[m][a] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // this workgroup's stream is contiguous: KS steps of FPS fragments; wave w takes steps [w*KQ, (w+1)*KQ)
+  const bf16x8* wf = A.wgu + ((int64_t)blockIdx.x * KS + (int64_t)w * KQ) * FPS * 64 + lane;
+  const bf16x8* xf = (const bf16x8*)(A.x + (int64_t)tc * D + (int64_t)w * KQ * 32) + gq;   // + 4 per K step
+  // Two register buffers of U1 K steps each: while one is multiplied the other is being filled.  KQ is a multiple of
+  // 2*U1 (the launcher picks U1 that way).
+  bf16x8 wA[U1][FPS], xA[U1], wB[U1][FPS], xB[U1];
+  auto fill = [&](bf16x8 (&wr)[U1][FPS], bf16x8 (&xb)[U1], int ks0) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < U1; ++u) {
-      b[u] = xs[(w * KQ + ks0 + u) * 64 + lane];
+      xb[u] = xf[(ks0 + u) * 4];
 #pragma unroll
-      for (int a = 0; a < NT16; ++a) {
-        ag[u][a] = wgf[((ks0 + u) * NT16 + a) * 64];
-        if (GATED) au[u][a] = wuf[((ks0 + u) * NT16 + a) * 64];
-      }
+      for (int f = 0; f < FPS; ++f) wr[u][f] = wf[((ks0 + u) * FPS + f) * 64];
     }
+  };
+  auto multiply = [&](bf16x8 (&wr)[U1][FPS], bf16x8 (&xb)[U1]) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < U1; ++u)
 #pragma unroll
-      for (int a = 0; a < NT16; ++a) {
-        acc1[0][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ag[u][a], b[u], acc1[0][a], 0, 0, 0);
-        if (GATED) acc1[NM - 1][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(au[u][a], b[u], acc1[NM - 1][a], 0, 0, 0);
-      }
+      for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+          acc1[m][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wr[u][m * 2 + a], xb[u], acc1[m][a], 0, 0, 0);
+  };
+  fill(wA, xA, 0);
+  for (int ks0 = 0; ks0 < KQ; ks0 += 2 * U1) {
+    fill(wB, xB, ks0 + U1);
+    multiply(wA, xA);
+    fill(wA, xA, (ks0 + 2 * U1 < KQ) ? (ks0 + 2 * U1) : ks0);   // the last trip re-reads its own steps: in bounds, unused
+    multiply(wB, xB);
   }
-  // W2^T fragments of this wave's columns: the first batch is requested before the reduction below
-  const int CTW = D / 64;   // 16-column tiles per wave
-  const bf16x8* wdf = A.wd + ((int64_t)e * (D / 16) + (int64_t)w * CTW) * KS2 * 64 + lane;
-  bf16x8 a2[U2][KS2];
-#pragma unroll
-  for (int j = 0; j < U2; ++j)
-#pragma unroll
-    for (int k2 = 0; k2 < KS2; ++k2) a2[j][k2] = wdf[(j * KS2 + k2) * 64];
 #pragma unroll
   for (int m = 0; m < NM; ++m)
 #pragma unroll
-    for (int a = 0; a < NT16; ++a)
+    for (int a = 0; a < 2; ++a)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) part[((w * NM + m) * NT16 * 4 + a * 4 + r) * 64 + lane] = acc1[m][a][r];
+      for (int r = 0; r < 4; ++r) part[w][m * 8 + a * 4 + r][lane] = acc1[m][a][r];
   __syncthreads();
-  // ---- hidden activations -> B fragments of GEMM2
-  const float rw = (c16 < N) ? bf16_to_f32(A.routing[(int64_t)c16 * E + e]) : 0.f;
-  const bf16_t* bias_e = A.bias + (int64_t)e * NT16 * 16;
-  bf16x8 hb[KS2];
+  if (w != 0) return;
+  // ---- hidden activations -> the block's B fragment of GEMM2.  Rows of x beyond N were copies of row N-1; their
+  // columns are zeroed here and never stored by the output kernel.
+  const float rw = (c16 < N) ? bf16_to_f32(rbits) : 0.f;
+  const bf16_t* bias_e = A.bias + (int64_t)e * NT16 * 16 + k2 * 32;
+  float hv[8];
 #pragma unroll
-  for (int k2 = 0; k2 < KS2; ++k2) {
-    float hv[8];
+  for (int i = 0; i < 8; ++i) {
+    const int a = i >> 2, r = i & 3;
+    float gsum = 0.f, usum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int a = 2 * k2 + (i >> 2), r = i & 3;
-      float gsum = 0.f, usum = 0.f;
-#pragma unroll
-      for (int ww = 0; ww < 4; ++ww) {
-        gsum += part[((ww * NM + 0) * NT16 * 4 + a * 4 + r) * 64 + lane];
-        if (GATED) usum += part[((ww * NM + NM - 1) * NT16 * 4 + a * 4 + r) * 64 + lane];
-      }
-      float v;
-      if (GATED) {
-        v = apply_act(A.act, gsum) * usum;
-      } else {
-        v = apply_act(A.act, gsum + bf16_to_f32(bias_e[a * 16 + 4 * gq + r]));
-      }
-      hv[i] = v * rw;
+    for (int ww = 0; ww < 4; ++ww) {
+      gsum += part[ww][a * 4 + r][lane];
+      if (GATED) usum += part[ww][(NM - 1) * 8 + a * 4 + r][lane];
     }
-    uint4 pk;
-    pk.x = pack2_bf16(hv[0], hv[1]); pk.y = pack2_bf16(hv[2], hv[3]);
-    pk.z = pack2_bf16(hv[4], hv[5]); pk.w = pack2_bf16(hv[6], hv[7]);
-    __builtin_memcpy(&hb[k2], &pk, 16);
+    float v;
+    if (GATED) {
+      v = apply_act(A.act, gsum) * usum;
+    } else {
+      v = apply_act(A.act, gsum + bf16_to_f32(bias_e[a * 16 + 4 * gq + r]));
+    }
+    hv[i] = (c16 < N) ? v * rw : 0.f;
   }
-  // ---- GEMM2 (transposed), U2 column tiles at a time, double-buffered in registers
-  bf16_t* yrow = A.y + ((int64_t)e * DC_MAX_TOKENS + c16) * D + (int64_t)w * (D / 4) + 4 * gq;
-  for (int ct0 = 0; ct0 < CTW; ct0 += U2) {
-    bf16x8 a[U2][KS2];
+  uint4 pk;
+  pk.x = pack2_bf16(hv[0], hv[1]); pk.y = pack2_bf16(hv[2], hv[3]);
+  pk.z = pack2_bf16(hv[4], hv[5]); pk.w = pack2_bf16(hv[6], hv[7]);
+  ((uint4*)A.hfrag)[((int64_t)e * KS2 + k2) * 64 + lane] = pk;
+}
+
+constexpr int DO_WAVES = 8;
+
+// Workgroup = 8 output columns, 8 waves; wave w owns experts [w*EW, (w+1)*EW) with EW = ceil(E/8) rounded up to 64 at
+// most per pass, and walks the routed ones among them in ascending order.
+template <int KS2>
+__global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeArgs A) {
+  constexpr int UB = 8 / KS2;                  // experts per load batch (8 fragments of each operand)
+  __shared__ float part[DO_WAVES][4][64];
+  const int D = A.D, N = A.N, E = A.E;
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  const int gq = lane >> 4, c16 = lane & 15;
+  const int cb = blockIdx.x;                   // 8-column block
+  const int EW = (E + DO_WAVES - 1) / DO_WAVES;
+  const int e_lo = w * EW, e_hi = (e_lo + EW < E) ? (e_lo + EW) : E;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  // A fragment rows 0..7 only (lanes c16 < 8); result rows 8..15 are dropped
+  const bf16x8* wdf = A.wd + (int64_t)cb * E * KS2 * 32 + gq * 8 + (c16 & 7);
+  const bf16x8* hf = A.hfrag + lane;
+  bf16x8 aA[UB][KS2], bA[UB][KS2], aB[UB][KS2], bB[UB][KS2];
+  for (int e0 = e_lo; e0 < e_hi; e0 += 64) {   // 64 experts per pass: one flag per lane
+    const bool on = (e0 + lane < e_hi) && (A.active[e0 + lane] != 0);
+    unsigned long long mask = __ballot(on);
+    int cntA = 0, cntB = 0;
+    // take the next up to UB routed experts off the mask and request their fragments; unused slots repeat the last one
+    auto fill = [&](bf16x8 (&a)[UB][KS2], bf16x8 (&b)[UB][KS2], int& cnt) __attribute__((always_inline)) {
+      cnt = 0;
+      int e = e0;
+      int es[UB];
 #pragma unroll
-    for (int j = 0; j < U2; ++j)
+      for (int j = 0; j < UB; ++j)
 #pragma unroll
-      for (int k2 = 0; k2 < KS2; ++k2) {
-        a[j][k2] = a2[j][k2];
-        // request the next batch while this one is multiplied (the last trip re-reads its own batch: in bounds)
-        const int ctn = (ct0 + U2 < CTW) ? (ct0 + U2) : ct0;
-        a2[j][k2] = wdf[((ctn + j) * KS2 + k2) * 64];
+        for (int k2 = 0; k2 < KS2; ++k2) a[j][k2] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < UB; ++j) {
+        if (mask != 0ull) {
+          e = e0 + (int)__builtin_ctzll(mask);
+          mask &= mask - 1ull;
+          ++cnt;
+        }
+#pragma unroll
+        for (int k2 = 0; k2 < KS2; ++k2) b[j][k2] = hf[((int64_t)e * KS2 + k2) * 64];
+        es[j] = e;
       }
+      // rows 8..15 of the A tile are not needed: those lanes request nothing and multiply zeros
+      if (c16 < 8) {
 #pragma unroll
-    for (int j = 0; j < U2; ++j) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < UB; ++j)
 #pragma unroll
-      for (int k2 = 0; k2 < KS2; ++k2) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][k2], hb[k2], acc, 0, 0, 0);
-      if (c16 < N) {
-        uint2 o;
-        o.x = pack2_bf16(acc[0], acc[1]);
-        o.y = pack2_bf16(acc[2], acc[3]);
-        *(uint2*)(yrow + (ct0 + j) * 16) = o;
+          for (int k2 = 0; k2 < KS2; ++k2) a[j][k2] = wdf[((int64_t)es[j] * KS2 + k2) * 32];
+      }
+    };
+    auto multiply = [&](bf16x8 (&a)[UB][KS2], bf16x8 (&b)[UB][KS2], int cnt) __attribute__((always_inline)) {
+#pragma unroll
+      for (int j = 0; j < UB; ++j) {
+        if (j < cnt) {
+#pragma unroll
+          for (int k2 = 0; k2 < KS2; ++k2) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][k2], b[j][k2], acc, 0, 0, 0);
+        }
+      }
+    };
+    if (mask != 0ull) {
+      fill(aA, bA, cntA);
+      while (cntA > 0) {
+        cntB = 0;
+        if (mask != 0ull) fill(aB, bB, cntB);
+        multiply(aA, bA, cntA);
+        cntA = 0;
+        if (mask != 0ull) fill(aA, bA, cntA);
+        multiply(aB, bB, cntB);
       }
     }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) part[w][r][lane] = acc[r];
+  __syncthreads();
+  if (w == 0 && c16 < N && gq < 2) {
+    // C layout (transposed product): lane holds token c16, rows 4 gq + r = columns cb*8 + 4 gq + r
+    float o[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float sacc = part[0][r][lane];
+#pragma unroll
+      for (int ww = 1; ww < DO_WAVES; ++ww) sacc += part[ww][r][lane];
+      o[r] = sacc;
+    }
+    const int col = cb * 8 + 4 * gq;
+    if (A.last_bias != nullptr) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[r] += bf16_to_f32(A.last_bias[col + r]);
+    }
+    if (A.add_residual) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[r] += bf16_to_f32(A.x[(int64_t)c16 * D + col + r]);
+    }
+    uint2 ov;
+    ov.x = pack2_bf16(o[0], o[1]);
+    ov.y = pack2_bf16(o[2], o[3]);
+    *(uint2*)(A.out + (int64_t)c16 * D + col) = ov;
   }
 }
 
-// Combine for the decode path.  A workgroup owns one token and 128 output columns: 16 column pieces (8 columns, 16
-// bytes) x 16 expert groups.  Thread (piece, group) adds its group's routed experts in ascending order; the 16 group
-// sums are then added in ascending group order.  The summation order is fixed, so results are reproducible.
-__global__ __launch_bounds__(256) void decode_combine_kernel(const bf16_t* __restrict__ y, const bf16_t* __restrict__ routing,
-                                                             const bf16_t* __restrict__ x, const bf16_t* __restrict__ last_bias,
-                                                             bf16_t* __restrict__ out, int N, int D, int E, int add_residual) {
-  __shared__ float part[16][16][9];   // [group][piece][8 columns + pad]
-  const int t = threadIdx.x;
-  const int piece = t & 15, grp = t >> 4;
-  const int blocks_per_token = D / 128;
-  const int n = blockIdx.x / blocks_per_token;
-  const int col = (blockIdx.x % blocks_per_token) * 128 + piece * 8;
-  const int per = (E + 15) / 16;            // experts per group
-  const int e_lo = grp * per, e_hi = (e_lo + per < E) ? (e_lo + per) : E;
-  const bf16_t* rrow = routing + (int64_t)n * E;
-  float acc[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-  for (int e0 = e_lo; e0 < e_hi; e0 += 8) {
-    uint4 v[8];
-    bool on[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      on[j] = (e0 + j < e_hi) && ((rrow[e0 + j] & 0x7fff) != 0);
-      v[j] = uint4{0u, 0u, 0u, 0u};
-      if (on[j]) v[j] = *(const uint4*)(y + ((int64_t)(e0 + j) * DC_MAX_TOKENS + n) * D + col);
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      if (on[j]) {
-        const uint32_t wd[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
-      }
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < 8; ++i) part[grp][piece][i] = acc[i];
-  __syncthreads();
-  if (grp == 0) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float s = part[0][piece][i];
-      for (int gi = 1; gi < 16; ++gi) s += part[gi][piece][i];
-      acc[i] = s;
-    }
-    if (last_bias != nullptr) {
-      const uint4 v = *(const uint4*)(last_bias + col);
-      const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
-    }
-    if (add_residual) {
-      const uint4 v = *(const uint4*)(x + (int64_t)n * D + col);
-      const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
-    }
-    uint4 o;
-    o.x = pack2_bf16(acc[0], acc[1]); o.y = pack2_bf16(acc[2], acc[3]);
-    o.z = pack2_bf16(acc[4], acc[5]); o.w = pack2_bf16(acc[6], acc[7]);
-    *(uint4*)(out + (int64_t)n * D + col) = o;
-  }
-}
-
-template <int NT16, bool GATED, int U1, int U2>
-static hipError_t launch_decode_cfg(const DecodeArgs& A, size_t lds, hipStream_t s) {
-  auto k = decode_experts_kernel<NT16, GATED, U1, U2>;
-  hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(k, dim3(A.E), dim3(256), lds, s, A);
+template <bool GATED>
+static hipError_t launch_hidden(const DecodeArgs& A, hipStream_t s) {
+  // K steps per wave (D/128) must be a multiple of 2*U1; D is a multiple of 256, so U1 = 1 always fits.
+  const int KQ = A.D / 128;
+  const dim3 grid((unsigned)(A.E * (A.nt16 / 2)));
+  if (KQ % 8 == 0) hipLaunchKernelGGL((decode_hidden_kernel<GATED, 4>), grid, dim3(256), 0, s, A);
+  else if (KQ % 4 == 0) hipLaunchKernelGGL((decode_hidden_kernel<GATED, 2>), grid, dim3(256), 0, s, A);
+  else hipLaunchKernelGGL((decode_hidden_kernel<GATED, 1>), grid, dim3(256), 0, s, A);
   return hipGetLastError();
-}
-
-template <int NT16>
-static hipError_t launch_decode_nt(const DecodeArgs& A, size_t lds, hipStream_t s) {
-  // deeper batches when the per-wave trip counts divide: K steps per wave = D/128, column tiles per wave = D/64
-  const bool deep = (A.D % 512 == 0);
-  if (A.gated) {
-    if (deep && NT16 <= 4) return launch_decode_cfg<NT16, true, 4, 8>(A, lds, s);
-    return launch_decode_cfg<NT16, true, 2, 4>(A, lds, s);
-  }
-  if (deep && NT16 <= 4) return launch_decode_cfg<NT16, false, 4, 8>(A, lds, s);
-  return launch_decode_cfg<NT16, false, 2, 4>(A, lds, s);
 }
 
 hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
@@ -346,41 +348,52 @@ hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void*
   const DecodeLayout L = decode_layout(sh);
   const char* pk = (const char*)packed_section;
   DecodeArgs A;
-  A.x = (const bf16_t*)x; A.routing = (const bf16_t*)routing; A.wg = (const bf16x8*)(pk + L.g_off);
-  A.wu = (const bf16x8*)(pk + L.u_off); A.wd = (const bf16x8*)(pk + L.d_off); A.bias = (const bf16_t*)(pk + L.b_off);
-  A.y = (bf16_t*)workspace; A.N = (int)sh.n_tokens; A.D = sh.d_model; A.E = sh.n_experts; A.act = sh.activation;
-  A.gated = sh.gated;
-  const int nm = sh.gated ? 2 : 1;
-  const size_t lds = (size_t)(sh.d_model / 32) * 64 * 16 + (size_t)4 * nm * L.nt16 * 4 * 64 * 4 + 16;
-  hipError_t e;
-  if (L.nt16 == 2) e = launch_decode_nt<2>(A, lds, s);
-  else if (L.nt16 == 4) e = launch_decode_nt<4>(A, lds, s);
-  else e = launch_decode_nt<8>(A, lds, s);
+  A.x = (const bf16_t*)x; A.routing = (const bf16_t*)routing; A.wgu = (const bf16x8*)(pk + L.gu_off);
+  A.wd = (const bf16x8*)(pk + L.d_off); A.bias = (const bf16_t*)(pk + L.b_off);
+  A.hfrag = (bf16x8*)workspace;
+  A.active = (int*)((char*)workspace + (size_t)sh.n_experts * L.edp * DC_MAX_TOKENS * 2);
+  A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out;
+  A.N = (int)sh.n_tokens; A.D = sh.d_model; A.E = sh.n_experts; A.nt16 = L.nt16; A.act = sh.activation;
+  A.add_residual = sh.add_residual;
+  const hipError_t e = sh.gated ? launch_hidden<true>(A, s) : launch_hidden<false>(A, s);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)sh.n_tokens * (sh.d_model / 128)), dim3(256), 0, s, (const bf16_t*)workspace,
-                     (const bf16_t*)routing, (const bf16_t*)x, (const bf16_t*)last_bias, (bf16_t*)out, (int)sh.n_tokens,
-                     sh.d_model, sh.n_experts, sh.add_residual);
+  const dim3 grid((unsigned)(sh.d_model / 8));
+  if (L.nt16 == 2) hipLaunchKernelGGL(decode_out_kernel<1>, grid, dim3(DO_WAVES * 64), 0, s, A);
+  else if (L.nt16 == 4) hipLaunchKernelGGL(decode_out_kernel<2>, grid, dim3(DO_WAVES * 64), 0, s, A);
+  else hipLaunchKernelGGL(decode_out_kernel<4>, grid, dim3(DO_WAVES * 64), 0, s, A);
   return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------------------------------
 // Skinny Linear for <= 16 rows: C[N, Nout] = round(act(round(A[N,K] . B[Nout,K]^T))), bf16.
-// Both operands are read straight from their row-major layouts (K contiguous in each): a wave owns 16 output features
-// and a quarter of K; partial tiles are summed through LDS in wave order.  Used for the router layers at small N.
+// Both operands are read straight from their row-major layouts (K contiguous in each): a workgroup owns 16 output features,
+// its 4 or 16 waves share K; partial tiles are summed through LDS in wave order.  Used for the router layers at small N.
 // ---------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void linear_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
-                                                            bf16_t* __restrict__ C, int N, int K, int Nout, int act) {
-  __shared__ float part[4][4][64];
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
+                                                               bf16_t* __restrict__ C, int N, int K, int Nout, int act) {
+  __shared__ float part[NW][4][64];
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
   const int gq = lane >> 4, c16 = lane & 15;
   const int f0 = blockIdx.x * 16;                 // first output feature of this workgroup
-  const int KQ = K / 4;                           // per wave, a multiple of 32
+  const int KQ = K / NW;                          // per wave, a multiple of 32
   const int frow = (f0 + c16 < Nout) ? (f0 + c16) : (Nout - 1);
   const int trow = (c16 < N) ? c16 : (N - 1);
   const bf16x8* bp = (const bf16x8*)(B + (int64_t)frow * K + w * KQ) + gq;
   const bf16x8* ap = (const bf16x8*)(A + (int64_t)trow * K + w * KQ) + gq;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int ks = 0; ks < KQ / 32; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bp[ks * 4], ap[ks * 4], acc, 0, 0, 0);
+  for (int ks0 = 0; ks0 < KQ / 32; ks0 += 4) {   // four K steps requested together, then multiplied
+    bf16x8 bv[4], av[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int ks = (ks0 + u < KQ / 32) ? (ks0 + u) : ks0;
+      bv[u] = bp[ks * 4];
+      av[u] = ap[ks * 4];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (ks0 + u < KQ / 32) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv[u], av[u], acc, 0, 0, 0);
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) part[w][r][lane] = acc[r];
   __syncthreads();
@@ -388,7 +401,9 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(const bf16_t* __rest
     // C layout: lane holds token (column) c16, features 4 gq + r
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const float v = ((part[0][r][lane] + part[1][r][lane]) + part[2][r][lane]) + part[3][r][lane];
+      float v = part[0][r][lane];
+#pragma unroll
+      for (int ww = 1; ww < NW; ++ww) v += part[ww][r][lane];
       const int f = f0 + 4 * gq + r;
       if (c16 < N && f < Nout) {
         const float vr = bf16_to_f32(f32_to_bf16(v));
@@ -401,8 +416,12 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(const bf16_t* __rest
 bool linear_skinny_supported(int64_t N, int K, int dtype) { return dtype == D2DMOE_BF16 && N >= 1 && N <= 16 && K % 128 == 0; }
 
 hipError_t launch_linear_skinny(const void* A, const void* B, void* C, int N, int K, int Nout, int act, hipStream_t s) {
-  hipLaunchKernelGGL(linear_skinny_kernel, dim3((Nout + 15) / 16), dim3(256), 0, s, (const bf16_t*)A, (const bf16_t*)B,
-                     (bf16_t*)C, N, K, Nout, act);
+  if (K % 512 == 0 && K >= 1024)   // long rows: 16 waves share K so that each requests its part in one go
+    hipLaunchKernelGGL(linear_skinny_kernel<16>, dim3((Nout + 15) / 16), dim3(1024), 0, s, (const bf16_t*)A, (const bf16_t*)B,
+                       (bf16_t*)C, N, K, Nout, act);
+  else
+    hipLaunchKernelGGL(linear_skinny_kernel<4>, dim3((Nout + 15) / 16), dim3(256), 0, s, (const bf16_t*)A, (const bf16_t*)B,
+                       (bf16_t*)C, N, K, Nout, act);
   return hipGetLastError();
 }
 
