@@ -43,6 +43,8 @@ ForwardWorkspace plan_workspace(const d2dmoe_shape& sh) {
   if (sparse > scratch) scratch = sparse;
   const size_t decode = mfma_decode_workspace_bytes(sh);   // per-expert result rows of the small-batch path
   if (decode > scratch) scratch = decode;
+  const size_t gemm = (sh.n_tokens > 16) ? mfma_gemm_workspace_bytes(sh) : 0;   // H fragments + partial sums of the gated path
+  if (gemm > scratch) scratch = gemm;
   w.perm_off = off;   off += align_up(scratch);
   w.total = off;
   return w;
@@ -142,7 +144,8 @@ int d2dmoe_build_permutation(const void* routing, int64_t n_tokens, int32_t n_ex
 
 size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape) {
   if (check_shape(shape) != D2DMOE_OK) return 0;
-  if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape) && !mfma_decode_supported(*shape)) return 0;
+  if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape) && !mfma_decode_supported(*shape) &&
+      !mfma_gemm_supported(*shape)) return 0;
   return mfma_packed_bytes(*shape);
 }
 
@@ -151,7 +154,8 @@ int d2dmoe_pack_weights(const d2dmoe_shape* shape, const void* w1, const void* b
   int st = check_shape(shape);
   if (st != D2DMOE_OK) return st;
   if (!w1 || !w2 || !packed) return D2DMOE_E_NULL;
-  if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape) && !mfma_decode_supported(*shape))
+  if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape) && !mfma_decode_supported(*shape) &&
+      !mfma_gemm_supported(*shape))
     return D2DMOE_E_UNSUPPORTED;
   if (shape->gated && !w_up) return D2DMOE_E_NULL;
   if (mfma_router_supported(*shape) && (!router_w1 || !router_w2)) return D2DMOE_E_NULL;
@@ -174,7 +178,9 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
   hipStream_t s = (hipStream_t)stream;
   if (path == D2DMOE_PATH_AUTO) {
     if (packed != nullptr && sh.n_tokens <= 16 && mfma_decode_supported(sh)) path = D2DMOE_PATH_MFMA_DECODE;
-    else path = (packed != nullptr && mfma_dense_supported(sh)) ? D2DMOE_PATH_MFMA_DENSE : D2DMOE_PATH_GENERIC;
+    else if (packed != nullptr && mfma_dense_supported(sh)) path = D2DMOE_PATH_MFMA_DENSE;
+    else if (packed != nullptr && mfma_gemm_supported(sh)) path = D2DMOE_PATH_MFMA_GEMM;
+    else path = D2DMOE_PATH_GENERIC;
   }
   switch (path) {
     case D2DMOE_PATH_GENERIC: {
@@ -207,6 +213,14 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
       if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
       return (int)launch_mfma_decode(sh, x, routing, (const char*)packed + mfma_decode_section_offset(sh), last_bias, out,
                                      workspace, s);
+    }
+    case D2DMOE_PATH_MFMA_GEMM: {
+      if (!mfma_gemm_supported(sh)) return D2DMOE_E_UNSUPPORTED;
+      if (!packed) return D2DMOE_E_NULL;
+      const size_t need = mfma_gemm_workspace_bytes(sh);
+      if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
+      return (int)launch_mfma_gemm(sh, x, routing, (const char*)packed + mfma_gemm_section_offset(sh), last_bias, out,
+                                   workspace, s);
     }
     default: return D2DMOE_E_UNSUPPORTED;
   }

@@ -52,10 +52,12 @@ __device__ inline float apply_act(int act, float x) {
     case D2DMOE_ACT_TANH: return tanhf(x);
     case D2DMOE_ACT_LEAKY_RELU: return x >= 0.f ? x : 0.01f * x;
     case D2DMOE_ACT_GELU_TANH: {
-      const float k = 0.79788456080286535588f;  // sqrt(2/pi)
-      return 0.5f * x * (1.f + tanhf(k * (x + 0.044715f * x * x * x)));
+      // 0.5 x (1 + tanh(u)) == x * sigmoid(2u),  u = sqrt(2/pi) (x + 0.044715 x^3): one exp and one reciprocal
+      const float k2 = 2.f * 0.79788456080286535588f;
+      const float u2 = k2 * (x + 0.044715f * x * x * x);
+      return x * __builtin_amdgcn_rcpf(1.f + __expf(-u2));
     }
-    case D2DMOE_ACT_SILU: return x / (1.f + __expf(-x));
+    case D2DMOE_ACT_SILU: return x * __builtin_amdgcn_rcpf(1.f + __expf(-x));
     case D2DMOE_ACT_ABS: return fabsf(x);
     default: return x;
   }

@@ -1,0 +1,396 @@
+// Large-batch gated experts (Gemma shape) on bf16 MFMA as two tiled products with the hidden activations kept in
+// memory between them:
+//
+//   up    H^T[hidden, token] = act(Wg^T . X^T) * (Wu^T . X^T) * routing[token, expert(hidden)]      (ExecuteAllExperts
+//         with intermediate gating, moe_layers.py:71-78, 91-96, restricted to the routed pairs by the routing factor)
+//   down  OUT[token, :] = sum over hidden of H[token, hidden] . Wd[hidden, :]  (+ last_bias, + x)
+//
+// With D = 2048 neither a token tile's x rows nor its output accumulators fit next to each other on a CU, and the
+// expert weights (201 MB) dwarf the activations, so the fused token-stationary sweep of the ViT shape does not carry
+// over; under the dynk_max rule most experts are active for most tokens, so computing whole tiles and multiplying by
+// the routing value wastes little.  The sum over hidden units runs in ascending order inside one float32 accumulator
+// (per K split), which is the ascending-expert order of the reference's merge kernel (moe_impls.py:485-514).
+//
+// One kernel template serves both products.  Workgroup = 4 waves (2 x 2), tile = 256 tokens x 256 rows/columns of the
+// weight operand, wave tile 128 x 128 = 16 accumulator tiles of v_mfma_f32_32x32x16_bf16 (256 AGPRs).  The token
+// operand (x, or H) goes through LDS in fragment order, double-buffered, 64 K values per stage; the weight operand is
+// read straight from its packed fragment stream into two register buffers (one stage ahead).  One LDS-only barrier
+// per stage (64 MFMAs per wave).
+//
+// The up product is computed transposed so that each lane ends up with ONE token and 16 hidden units per tile; the 8
+// values of accumulator rows r = 8k .. 8k+7 are exactly one A fragment of the down product (32 tokens x 16 hidden
+// units, k order: slot (g, i) <-> hidden 16*kstep + 8*(i/4) + 4g + i%4, baked into the packed Wd fragments).  H is
+// therefore written as 1 KB fragments, fully coalesced, and staged into LDS by the down product with straight copies.
+#include "mfma_common.hpp"
+
+namespace d2dmoe {
+
+constexpr int GM_BT = 256;         // tokens per workgroup tile
+constexpr int GM_SLAB = 8192;      // tokens per pass: bounds the workspace (H fragments + float32 partial sums)
+constexpr int GM_MAX_SPLIT = 8;
+
+struct GemmLayout {
+  int edp;   // neurons per expert padded to a multiple of 32: every 32-row MFMA tile belongs to one expert
+  int hp;    // padded hidden size, a multiple of 128
+  size_t up_off, dn_off, total;
+};
+
+static GemmLayout gemm_layout(const d2dmoe_shape& sh) {
+  GemmLayout L;
+  L.edp = (sh.expert_dim + 31) / 32 * 32;
+  L.hp = (sh.n_experts * L.edp + 127) / 128 * 128;
+  L.up_off = 0;
+  L.dn_off = (size_t)L.hp * 2 * sh.d_model * 2;
+  L.total = (L.dn_off + (size_t)L.hp * sh.d_model * 2 + 255) / 256 * 256;
+  return L;
+}
+
+bool mfma_gemm_supported(const d2dmoe_shape& sh) {
+  return sh.dtype == D2DMOE_BF16 && sh.gated && sh.d_model % 256 == 0 && sh.d_model >= 256;
+}
+
+size_t mfma_gemm_packed_bytes(const d2dmoe_shape& sh) { return mfma_gemm_supported(sh) ? gemm_layout(sh).total : 0; }
+
+struct GemmPlan {
+  int slab;      // tokens per pass
+  int n_ttiles;  // 256-token tiles per (full) pass
+  int ksplit;    // K splits of the down product
+  size_t h_bytes, partial_bytes;
+};
+
+static GemmPlan gemm_plan(const d2dmoe_shape& sh) {
+  const GemmLayout L = gemm_layout(sh);
+  GemmPlan P;
+  P.slab = (int)(sh.n_tokens < GM_SLAB ? sh.n_tokens : GM_SLAB);
+  P.n_ttiles = (P.slab + GM_BT - 1) / GM_BT;
+  // the down product has n_ttiles * D/256 tiles; split K until the machine is covered (the K steps of every split
+  // must still be whole stages of 4)
+  const int tiles = P.n_ttiles * (sh.d_model / 256);
+  const int ks2 = L.hp / 16;
+  P.ksplit = 1;
+  while (P.ksplit < GM_MAX_SPLIT && tiles * P.ksplit < device_cu_count() && (ks2 / (P.ksplit * 2)) % 4 == 0) P.ksplit *= 2;
+  P.h_bytes = ((size_t)P.n_ttiles * GM_BT * L.hp * 2 + 255) / 256 * 256;
+  P.partial_bytes = ((size_t)P.ksplit * P.slab * sh.d_model * 4 + 255) / 256 * 256;
+  return P;
+}
+
+size_t mfma_gemm_workspace_bytes(const d2dmoe_shape& sh) {
+  if (!mfma_gemm_supported(sh) || sh.n_tokens <= 0) return 0;
+  const GemmPlan P = gemm_plan(sh);
+  return P.h_bytes + P.partial_bytes;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Packing (lane = 32 g + c).  KS = D/16, KS2 = HP/16; hidden index h = e*EdP + j, zero beyond Ed and beyond E.
+//   up stream   [hidden block HP/64][kstep KS][tile 4: gate 0,1, up 0,1][lane][8]   A fragment:
+//               row h = 64*block + 32*(tile%2) + c,  d = 16*kstep + 8g + i             value w[e][d][j]
+//   down stream [column block D/128][kstep2 KS2][tile 4][lane][8]                   B fragment:
+//               column = 128*block + 32*tile + c,  h = 16*kstep2 + 8*(i/4) + 4g + i%4   value w2[e][j][column]
+// ---------------------------------------------------------------------------------------------------
+__global__ void pack_gemm_kernel(const bf16_t* __restrict__ wg, const bf16_t* __restrict__ wu, const bf16_t* __restrict__ wd,
+                                 bf16_t* __restrict__ dup, bf16_t* __restrict__ ddn, int D, int E, int Ed, int edp, int hp) {
+  const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int KS = D / 16, KS2 = hp / 16;
+  const int64_t n_up = (int64_t)(hp / 64) * KS * 4 * 64;
+  const int64_t n_dn = (int64_t)(D / 128) * KS2 * 4 * 64;
+  if (p < n_up) {
+    int64_t q = p;
+    const int lane = (int)(q % 64); q /= 64;
+    const int tile = (int)(q % 4); q /= 4;
+    const int ks = (int)(q % KS);
+    const int blk = (int)(q / KS);
+    const int g = lane >> 5, c = lane & 31;
+    const int h = 64 * blk + 32 * (tile & 1) + c;
+    const int e = h / edp, j = h % edp;
+    const bf16_t* src = (tile < 2) ? wg : wu;
+    const bool ok = e < E && j < Ed;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int d = 16 * ks + 8 * g + i;
+      dup[p * 8 + i] = ok ? src[((int64_t)e * D + d) * Ed + j] : (bf16_t)0;
+    }
+  } else if (p < n_up + n_dn) {
+    const int64_t pp = p - n_up;
+    int64_t q = pp;
+    const int lane = (int)(q % 64); q /= 64;
+    const int tile = (int)(q % 4); q /= 4;
+    const int ks2 = (int)(q % KS2);
+    const int blk = (int)(q / KS2);
+    const int g = lane >> 5, c = lane & 31;
+    const int col = 128 * blk + 32 * tile + c;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int h = 16 * ks2 + 8 * (i / 4) + 4 * g + (i % 4);
+      const int e = h / edp, j = h % edp;
+      ddn[pp * 8 + i] = (e < E && j < Ed) ? wd[((int64_t)e * Ed + j) * D + col] : (bf16_t)0;
+    }
+  }
+}
+
+hipError_t launch_gemm_pack(const d2dmoe_shape& sh, const void* w_gate, const void* w_down, const void* w_up,
+                            void* packed_section, hipStream_t s) {
+  const GemmLayout L = gemm_layout(sh);
+  char* base = (char*)packed_section;
+  const int64_t n = (int64_t)(L.hp / 64) * (sh.d_model / 16) * 256 + (int64_t)(sh.d_model / 128) * (L.hp / 16) * 256;
+  hipLaunchKernelGGL(pack_gemm_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const bf16_t*)w_gate,
+                     (const bf16_t*)w_up, (const bf16_t*)w_down, (bf16_t*)(base + L.up_off), (bf16_t*)(base + L.dn_off),
+                     sh.d_model, sh.n_experts, sh.expert_dim, L.edp, L.hp);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------------
+struct GemmArgs {
+  const bf16_t* x;         // [N, D] rows of this pass
+  const bf16_t* routing;   // [N, E]
+  const bf16x8* w;         // packed weight stream of this product
+  bf16x8* hfrag;           // [token tile N/32][kstep2 HP/16][lane] hidden activations as A fragments
+  float* partial;          // [ksplit][N][D] float32 sums of the down product
+  int N; int D; int E; int edp; int hp; int act;
+  int n_ttiles;            // 256-token tiles
+  int tpx;                 // token tiles per XCD: ceil(n_ttiles / 8)
+  int ksplit;
+};
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// MODE 0: up product (weights = A operand, x = B operand through LDS); MODE 1: down product (H = A operand through
+// LDS, weights = B operand).
+template <int MODE, int ACT>
+__global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16x8* lds0 = (bf16x8*)smem_raw;          // [8 token tiles][4 ksteps][64 lanes]
+  bf16x8* lds1 = lds0 + 8 * 4 * 64;
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  const int wm = w >> 1, wn = w & 1;         // half of the weight rows/columns, half of the tokens
+  const int g = lane >> 5, c32 = lane & 31;
+  // Workgroups are dealt to the 8 XCDs round-robin.  An XCD keeps "its" token tiles (tpx of them) and walks the weight
+  // blocks, so at any time its L2 holds a few token tiles and one set of weight blocks shared by all of its CUs.
+  const int xcd = blockIdx.x & 7, kk = blockIdx.x >> 3;
+  const int tt = xcd + 8 * (kk % A.tpx);
+  int nb = kk / A.tpx;
+  if (tt >= A.n_ttiles) return;
+  int split = 0;
+  if (MODE == 1) { split = nb % A.ksplit; nb /= A.ksplit; }
+  const int N = A.N, D = A.D;
+  const int KS2T = A.hp / 16;                                    // K steps of the whole down product
+  const int n_ks = (MODE == 0) ? (D / 16) : (KS2T / A.ksplit);   // K steps of this workgroup
+  const int ks_begin = (MODE == 0) ? 0 : split * n_ks;
+  const int S = n_ks / 4;                                        // stages
+  const int KST = (MODE == 0) ? (D / 16) : KS2T;
+  const bf16x8* wbase = A.w + ((int64_t)(nb * 2 + wm) * KST + ks_begin) * 256 + lane;
+
+  f32x16 acc[4][4];   // [weight tile][token tile]
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // ---- token operand: global -> registers -> LDS, 8 pieces of 16 bytes per thread and stage
+  u32x4 xv[8];
+  const int xrow = t >> 3, xpc = t & 7;   // MODE 0: row within a 32-token tile, 16-byte piece of the 64-wide K slice
+  auto load_x = [&](int s) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (MODE == 0) {
+        int64_t tok = (int64_t)tt * GM_BT + i * 32 + xrow;
+        tok = tok < N ? tok : (N - 1);   // rows beyond N repeat the last row; their H is forced to zero below
+        xv[i] = *(const u32x4*)(A.x + tok * D + s * 64 + xpc * 8);
+      } else {
+        xv[i] = *(const u32x4*)(A.hfrag + (((int64_t)tt * 8 + i) * KS2T + ks_begin + s * 4 + w) * 64 + lane);
+      }
+    }
+  };
+  auto store_x = [&](bf16x8* buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (MODE == 0) ((u32x4*)buf)[(i * 4 + (xpc >> 1)) * 64 + xrow + 32 * (xpc & 1)] = xv[i];
+      else ((u32x4*)buf)[i * 256 + t] = xv[i];
+    }
+  };
+  // ---- weight operand: a register ring of 16 fragments (one stage); a slot is refilled with the fragment one stage
+  // ahead as soon as it has been handed to the MFMAs
+  bf16x8 ring[4][4];   // [kstep][tile]
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ring[ks][i] = wbase[(ks * 4 + i) * 64];
+  auto compute = [&](const bf16x8* buf, int s_next) __attribute__((always_inline)) {
+    const bf16x8* xl = buf + (wn * 4) * 4 * 64 + lane;
+    const bf16x8* wn_ = wbase + (int64_t)s_next * 16 * 64;
+    bf16x8 xb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xb[j] = xl[(j * 4 + 0) * 64];
+    static_for<0, 4>([&](auto ks_c) __attribute__((always_inline)) {
+      constexpr int ks = decltype(ks_c)::value;
+      constexpr int kn = (ks + 1 < 4) ? ks + 1 : ks;
+      bf16x8 wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        wv[i] = ring[ks][i];
+        ring[ks][i] = wn_[(ks * 4 + i) * 64];
+      }
+      bf16x8 nxb[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) nxb[j] = xl[(j * 4 + kn) * 64];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (MODE == 0) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv[i], xb[j], acc[i][j], 0, 0, 0);
+          else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xb[j], wv[i], acc[i][j], 0, 0, 0);
+        }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xb[j] = nxb[j];
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  load_x(0);
+  store_x(lds0);
+  __syncthreads();
+  for (int s = 0; s < S; ++s) {
+    bf16x8* cur = (s & 1) ? lds1 : lds0;
+    bf16x8* nxt = (s & 1) ? lds0 : lds1;
+    const bool more = s + 1 < S;
+    if (more) load_x(s + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(cur, more ? s + 1 : s);   // the last stage re-reads its own fragments: in bounds, unused
+    if (more) store_x(nxt);
+    lds_barrier();
+  }
+
+  if (MODE == 0) {
+    // weight tiles 0,1 = gate rows, 2,3 = up rows of the same 64 hidden units; lane = token c32 of token tile j
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int tl = wn * 4 + j;
+      const int64_t tok = (int64_t)tt * GM_BT + tl * 32 + c32;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int h0 = (nb * 2 + wm) * 64 + 32 * i;
+        const int e = h0 / A.edp;
+        const bool live = tok < N && e < A.E;
+        const float rw = live ? bf16_to_f32(A.routing[tok * A.E + e]) : 0.f;
+        float hv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float gv = (ACT >= 0) ? act_fn<ACT>(acc[i][j][r]) : apply_act(A.act, acc[i][j][r]);
+          const float v = gv * acc[2 + i][j][r] * rw;
+          hv[r] = (live && rw != 0.f) ? v : 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          u32x4 pk;
+          pk.x = pack2_bf16(hv[8 * k + 0], hv[8 * k + 1]); pk.y = pack2_bf16(hv[8 * k + 2], hv[8 * k + 3]);
+          pk.z = pack2_bf16(hv[8 * k + 4], hv[8 * k + 5]); pk.w = pack2_bf16(hv[8 * k + 6], hv[8 * k + 7]);
+          const int ks2 = h0 / 16 + k;
+          *(u32x4*)(A.hfrag + (((int64_t)tt * 8 + tl) * KS2T + ks2) * 64 + lane) = pk;
+        }
+      }
+    }
+  } else {
+    // lane = column c32 of weight tile i; accumulator row r = token 8*(r/4) + 4g + r%4 of token tile j
+    float* pbase = A.partial + (int64_t)split * N * D;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = (nb * 2 + wm) * 128 + 32 * i + c32;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t tok0 = (int64_t)tt * GM_BT + (wn * 4 + j) * 32 + 4 * g;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t tok = tok0 + 8 * (r / 4) + (r % 4);
+          if (tok < N) pbase[tok * D + col] = acc[i][j][r];
+        }
+      }
+    }
+  }
+}
+
+// out[n, :] = round(sum over splits (ascending) + last_bias + x), 8 columns per thread
+__global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restrict__ partial, const bf16_t* __restrict__ last_bias,
+                                                          const bf16_t* __restrict__ x, bf16_t* __restrict__ out, int64_t N, int D,
+                                                          int ksplit, int add_residual) {
+  const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int per_row = D / 8;
+  if (p >= N * per_row) return;
+  const int64_t n = p / per_row;
+  const int col = (int)(p % per_row) * 8;
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = 0.f;
+  for (int s = 0; s < ksplit; ++s) {
+    const float4 a = *(const float4*)(partial + ((int64_t)s * N + n) * D + col);
+    const float4 b = *(const float4*)(partial + ((int64_t)s * N + n) * D + col + 4);
+    v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w; v[4] += b.x; v[5] += b.y; v[6] += b.z; v[7] += b.w;
+  }
+  if (last_bias != nullptr) {
+    const uint4 lb = *(const uint4*)(last_bias + col);
+    const uint32_t lw[4] = {lb.x, lb.y, lb.z, lb.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] += __uint_as_float((i & 1) ? (lw[i >> 1] & 0xffff0000u) : (lw[i >> 1] << 16));
+  }
+  if (add_residual) {
+    const uint4 xr = *(const uint4*)(x + n * D + col);
+    const uint32_t xw[4] = {xr.x, xr.y, xr.z, xr.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] += __uint_as_float((i & 1) ? (xw[i >> 1] & 0xffff0000u) : (xw[i >> 1] << 16));
+  }
+  uint4 o;
+  o.x = pack2_bf16(v[0], v[1]); o.y = pack2_bf16(v[2], v[3]);
+  o.z = pack2_bf16(v[4], v[5]); o.w = pack2_bf16(v[6], v[7]);
+  *(uint4*)(out + n * D + col) = o;
+}
+
+template <int ACT>
+static hipError_t launch_gemm_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
+                                  const void* last_bias, void* out, void* workspace, hipStream_t s) {
+  const GemmLayout L = gemm_layout(sh);
+  const GemmPlan P = gemm_plan(sh);
+  const char* pk = (const char*)packed_section;
+  const size_t lds = 2 * 8 * 4 * 64 * 16;
+  auto k_up = gated_gemm_kernel<0, ACT>;
+  auto k_dn = gated_gemm_kernel<1, -1>;
+  hipError_t e = hipFuncSetAttribute((const void*)k_up, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return e;
+  e = hipFuncSetAttribute((const void*)k_dn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return e;
+  for (int64_t t0 = 0; t0 < sh.n_tokens; t0 += P.slab) {
+    const int n = (int)((sh.n_tokens - t0) < P.slab ? (sh.n_tokens - t0) : P.slab);
+    GemmArgs A;
+    A.x = (const bf16_t*)x + t0 * sh.d_model;
+    A.routing = (const bf16_t*)routing + t0 * sh.n_experts;
+    A.hfrag = (bf16x8*)workspace;
+    A.partial = (float*)((char*)workspace + P.h_bytes);
+    A.N = n; A.D = sh.d_model; A.E = sh.n_experts; A.edp = L.edp; A.hp = L.hp; A.act = sh.activation;
+    A.n_ttiles = (n + GM_BT - 1) / GM_BT;
+    A.tpx = (A.n_ttiles + 7) / 8;
+    A.ksplit = P.ksplit;
+    A.w = (const bf16x8*)(pk + L.up_off);
+    hipLaunchKernelGGL(k_up, dim3((unsigned)(8 * A.tpx * (L.hp / 128))), dim3(256), lds, s, A);
+    A.w = (const bf16x8*)(pk + L.dn_off);
+    hipLaunchKernelGGL(k_dn, dim3((unsigned)(8 * A.tpx * (sh.d_model / 256) * P.ksplit)), dim3(256), lds, s, A);
+    const int64_t items = (int64_t)n * (sh.d_model / 8);
+    hipLaunchKernelGGL(gemm_finish_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, (const float*)A.partial,
+                       (const bf16_t*)last_bias, A.x, (bf16_t*)out + t0 * sh.d_model, (int64_t)n, sh.d_model, P.ksplit,
+                       sh.add_residual);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+hipError_t launch_mfma_gemm(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
+                            const void* last_bias, void* out, void* workspace, hipStream_t s) {
+  switch (sh.activation) {
+    case D2DMOE_ACT_RELU: return launch_gemm_act<D2DMOE_ACT_RELU>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_GELU: return launch_gemm_act<D2DMOE_ACT_GELU>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_GELU_TANH: return launch_gemm_act<D2DMOE_ACT_GELU_TANH>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_SILU: return launch_gemm_act<D2DMOE_ACT_SILU>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    default: return launch_gemm_act<-1>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+  }
+}
+
+}  // namespace d2dmoe

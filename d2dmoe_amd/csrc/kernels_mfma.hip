@@ -72,6 +72,8 @@ PackedLayout packed_layout(const d2dmoe_shape& sh) {
   off = (off + 255) / 256 * 256;
   L.has_decode = mfma_decode_supported(sh);
   L.dc_off = off;   if (L.has_decode) off += mfma_decode_packed_bytes(sh);
+  L.has_gemm = mfma_gemm_supported(sh);
+  L.gm_off = off;   if (L.has_gemm) off += mfma_gemm_packed_bytes(sh);
   // the router section comes last, so the expert sections sit at the same offsets whether or not the shape handed
   // to a later call names the router
   L.has_router = mfma_router_supported(sh);
@@ -83,6 +85,7 @@ PackedLayout packed_layout(const d2dmoe_shape& sh) {
 
 size_t mfma_packed_bytes(const d2dmoe_shape& sh) { return packed_layout(sh).total; }
 size_t mfma_decode_section_offset(const d2dmoe_shape& sh) { return packed_layout(sh).dc_off; }
+size_t mfma_gemm_section_offset(const d2dmoe_shape& sh) { return packed_layout(sh).gm_off; }
 
 // ---------------------------------------------------------------------------------------------------
 // Packing.  Each wave of the fused kernel reads ONE linear stream of 1 KB fragments (16 bytes per lane), in the
@@ -185,6 +188,10 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
   }
   if (L.has_decode) {
     hipError_t e = launch_decode_pack(sh, w1, b1, w2, w_up, base + L.dc_off, s);
+    if (e != hipSuccess) return e;
+  }
+  if (L.has_gemm) {
+    hipError_t e = launch_gemm_pack(sh, w1, w2, w_up, base + L.gm_off, s);
     if (e != hipSuccess) return e;
   }
   if (!L.has_dense) return hipGetLastError();
@@ -717,6 +724,141 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
   }
 }
 
+// The same computation for launches that would leave most of the machine idle with one wave per 32 tokens (few tokens,
+// long rows): a workgroup owns 32 tokens and its 4 waves share the OUTPUT features of each layer -- wave w computes
+// hidden tiles [w*TW, (w+1)*TW) over all of K, the hidden activations are exchanged through LDS as B fragments, then
+// wave w computes expert tiles [w*TE, (w+1)*TE); the per-token maximum is completed through LDS.  No partial sums are
+// exchanged, so every value is bit-identical to the one-wave kernel's.  Loads run U K steps ahead in two register
+// buffers.
+template <int TW, int TE, int U>
+__global__ __launch_bounds__(256) void router_select_split_kernel(
+    const bf16_t* __restrict__ x, const bf16x8* __restrict__ w1f, const bf16x8* __restrict__ w2f,
+    bf16_t* __restrict__ routing, bf16_t* __restrict__ norms_out, int32_t* __restrict__ counts, int64_t N, int D,
+    float thr_scale) {
+  constexpr int WT = 4 * TW, ET = 4 * TE, E = ET * 32;
+  __shared__ bf16x8 hs[2 * WT][64];
+  __shared__ float smax[4][32];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int g = lane >> 5, c32 = lane & 31;
+  const int64_t tok0 = (int64_t)blockIdx.x * 32;
+  const int64_t token = tok0 + c32;
+  const bool valid = token < N;
+  const bf16x8* xrow = (const bf16x8*)(x + (valid ? token : (N - 1)) * D) + g;   // + 2 per K step
+  const bf16x8* w1w = w1f + (int64_t)(w * TW) * 64 + lane;                       // + WT*64 per K step, + 64 per tile
+  const int KS1 = D / 16;   // a multiple of 2*U (checked by the launcher)
+
+  f32x16 acc1[TW];
+#pragma unroll
+  for (int a = 0; a < TW; ++a)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc1[a][r] = 0.f;
+  bf16x8 xA[U], wA[U][TW], xB[U], wB[U][TW];
+  auto fill = [&](bf16x8 (&xb)[U], bf16x8 (&wr)[U][TW], int ks0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      xb[u] = xrow[2 * (ks0 + u)];
+#pragma unroll
+      for (int a = 0; a < TW; ++a) wr[u][a] = w1w[((int64_t)(ks0 + u) * WT + a) * 64];
+    }
+  };
+  auto multiply = [&](bf16x8 (&xb)[U], bf16x8 (&wr)[U][TW]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int a = 0; a < TW; ++a) acc1[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wr[u][a], xb[u], acc1[a], 0, 0, 0);
+  };
+  fill(xA, wA, 0);
+  for (int ks0 = 0; ks0 < KS1; ks0 += 2 * U) {
+    fill(xB, wB, ks0 + U);
+    multiply(xA, wA);
+    fill(xA, wA, (ks0 + 2 * U < KS1) ? (ks0 + 2 * U) : ks0);   // the last trip re-reads its own steps: in bounds, unused
+    multiply(xB, wB);
+  }
+  // the first TE expert-tile fragments of the second layer are requested before the exchange
+  const bf16x8* w2w = w2f + (int64_t)(w * TE) * 64 + lane;   // + ET*64 per K step, + 64 per tile
+  // hidden activations -> LDS as B fragments of the second product
+#pragma unroll
+  for (int a = 0; a < TW; ++a)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      uint4 pk;
+      pk.x = pack2_bf16(fmaxf(acc1[a][half * 8 + 0], 0.f), fmaxf(acc1[a][half * 8 + 1], 0.f));
+      pk.y = pack2_bf16(fmaxf(acc1[a][half * 8 + 2], 0.f), fmaxf(acc1[a][half * 8 + 3], 0.f));
+      pk.z = pack2_bf16(fmaxf(acc1[a][half * 8 + 4], 0.f), fmaxf(acc1[a][half * 8 + 5], 0.f));
+      pk.w = pack2_bf16(fmaxf(acc1[a][half * 8 + 6], 0.f), fmaxf(acc1[a][half * 8 + 7], 0.f));
+      ((uint4*)hs)[((w * TW + a) * 2 + half) * 64 + lane] = pk;
+    }
+  __syncthreads();
+  f32x16 acc2[TE];
+#pragma unroll
+  for (int a = 0; a < TE; ++a)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc2[a][r] = 0.f;
+  for (int k0 = 0; k0 < 2 * WT; k0 += 8) {   // 2*WT is a multiple of 8
+    bf16x8 a2[8][TE];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+#pragma unroll
+      for (int et = 0; et < TE; ++et) a2[k][et] = w2w[((int64_t)(k0 + k) * ET + et) * 64];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const bf16x8 hb = hs[k0 + k][lane];
+#pragma unroll
+      for (int et = 0; et < TE; ++et) acc2[et] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2[k][et], hb, acc2[et], 0, 0, 0);
+    }
+  }
+  // norms (bf16 values held as float), per-token maximum over this wave's experts, then over the four waves
+  float m = -INFINITY;
+#pragma unroll
+  for (int et = 0; et < TE; ++et)
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      const uint32_t pk = pack2_bf16(fabsf(acc2[et][r]), fabsf(acc2[et][r + 1]));
+      acc2[et][r] = __uint_as_float(pk << 16);
+      acc2[et][r + 1] = __uint_as_float(pk & 0xffff0000u);
+      m = nanmax(m, nanmax(acc2[et][r], acc2[et][r + 1]));
+    }
+  m = nanmax(m, __shfl_xor(m, 32, kWave));
+  if (g == 0) smax[w][c32] = m;
+  __syncthreads();
+  m = nanmax(nanmax(smax[0][c32], smax[1][c32]), nanmax(smax[2][c32], smax[3][c32]));
+  const float thr = __uint_as_float(pack2_bf16(m * thr_scale, 0.f) << 16);
+#pragma unroll
+  for (int et = 0; et < TE; ++et) {
+    const int etg = w * TE + et;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e0 = etg * 32 + 8 * q + 4 * g;
+      bool on[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) on[s] = acc2[et][q * 4 + s] >= thr;
+      if (valid) {
+        uint2 rv;
+        rv.x = (on[0] ? 0x3F80u : 0u) | (on[1] ? 0x3F800000u : 0u);   // bf16 1.0 = 0x3F80
+        rv.y = (on[2] ? 0x3F80u : 0u) | (on[3] ? 0x3F800000u : 0u);
+        *(uint2*)(routing + token * E + e0) = rv;
+        if (norms_out != nullptr) {
+          uint2 nv;
+          nv.x = (__float_as_uint(acc2[et][q * 4 + 0]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 1]) & 0xffff0000u);
+          nv.y = (__float_as_uint(acc2[et][q * 4 + 2]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 3]) & 0xffff0000u);
+          *(uint2*)(norms_out + token * E + e0) = nv;
+        }
+      }
+      if (counts != nullptr) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const unsigned long long bal = __ballot(on[s] && valid);
+          if (lane == 0) {
+            const int lo = __popcll(bal & 0xffffffffull), hi = __popcll(bal >> 32);
+            if (lo) atomicAdd(counts + etg * 32 + 8 * q + s, lo);
+            if (hi) atomicAdd(counts + etg * 32 + 8 * q + 4 + s, hi);
+          }
+        }
+      }
+    }
+  }
+}
+
 hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
                                      void* norms_out, int32_t* counts, float thr_scale, hipStream_t s) {
   const PackedLayout L = packed_layout(sh);
@@ -726,14 +868,34 @@ hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, cons
     hipError_t e = launch_fill_i32(counts, sh.n_experts, 0, s);
     if (e != hipSuccess) return e;
   }
+  const bf16_t* xp = (const bf16_t*)x;
+  const bf16x8* r1 = (const bf16x8*)(base + L.r1_off);
+  const bf16x8* r2 = (const bf16x8*)(base + L.r2_off);
+  // One wave per 32 tokens fills the machine from about 4 * 32 * CUs tokens on; below that (or with long rows, where a
+  // wave's K loop is the critical path) a workgroup per 32 tokens shares the output features among its waves.
+  const bool split = (sh.n_tokens < (int64_t)128 * device_cu_count() || sh.d_model >= 2048) && (sh.d_model / 16) % 4 == 0;
+  if (split) {
+    const unsigned grid = (unsigned)cdiv64(sh.n_tokens, 32);
+    const bool deep = (sh.d_model / 16) % 8 == 0;
+    if (sh.router_width == 128) {
+      if (deep) hipLaunchKernelGGL((router_select_split_kernel<1, 1, 4>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+                                   (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+      else hipLaunchKernelGGL((router_select_split_kernel<1, 1, 2>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+                              (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+    } else {
+      if (deep) hipLaunchKernelGGL((router_select_split_kernel<2, 2, 4>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+                                   (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+      else hipLaunchKernelGGL((router_select_split_kernel<2, 2, 2>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+                              (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+    }
+    return hipGetLastError();
+  }
   const unsigned grid = (unsigned)cdiv64(sh.n_tokens, 128);
   if (sh.router_width == 128)
-    hipLaunchKernelGGL((router_select_mfma_kernel<4, 4>), dim3(grid), dim3(256), 0, s, (const bf16_t*)x,
-                       (const bf16x8*)(base + L.r1_off), (const bf16x8*)(base + L.r2_off), (bf16_t*)routing,
+    hipLaunchKernelGGL((router_select_mfma_kernel<4, 4>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
                        (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
   else
-    hipLaunchKernelGGL((router_select_mfma_kernel<8, 8>), dim3(grid), dim3(256), 0, s, (const bf16_t*)x,
-                       (const bf16x8*)(base + L.r1_off), (const bf16x8*)(base + L.r2_off), (bf16_t*)routing,
+    hipLaunchKernelGGL((router_select_mfma_kernel<8, 8>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
                        (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
   return hipGetLastError();
 }

@@ -32,8 +32,9 @@ struct PackedLayout {
   size_t r1_off, r2_off;                 // router fragments
   size_t s1_off, s2_off, sb_off;         // expert-major: W1 fragments, W2^T fragments, bias (bf16, padded to nt*32)
   size_t dc_off;                         // small-batch (decode) section
+  size_t gm_off;                         // large-batch gated section (tiled products)
   size_t total;
-  bool has_dense, has_router, has_sparse, has_decode;
+  bool has_dense, has_router, has_sparse, has_decode, has_gemm;
 };
 PackedLayout packed_layout(const d2dmoe_shape& sh);
 int device_cu_count();

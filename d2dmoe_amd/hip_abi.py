@@ -16,7 +16,7 @@ LIB_PATH = os.environ.get('D2DMOE_LIB') or os.path.join(os.path.dirname(os.path.
 # enums of include/d2dmoe.h
 F32, BF16 = 0, 1
 ACT = {'relu': 0, 'gelu': 1, 'tanh': 2, 'leaky_relu': 3, 'gelu_tanh': 4, 'silu': 5, 'identity': 6, 'abs': 7}
-PATH = {'auto': 0, 'generic': 1, 'mfma_dense': 2, 'mfma_sparse': 3, 'mfma_decode': 4}
+PATH = {'auto': 0, 'generic': 1, 'mfma_dense': 2, 'mfma_sparse': 3, 'mfma_decode': 4, 'mfma_gemm': 5}
 
 # every extern "C" symbol the header declares
 EXPORTS = (
