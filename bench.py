@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the dynamic-k MoE-FFN forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vit_b_50k] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vit_b_50k] [--no-cpu-baseline] [--no-sweep]
 
 One "step" is one pass of the whole layer (router MLP -> dynamic-k selection -> experts -> bias epilogue) over one
 batch of synthetic tokens that already sit in HBM.  The default workload is the ViT-B-shape layer of the headline
@@ -13,6 +13,10 @@ Prints ONE JSON line.  Beyond the common fields it carries
   roofline      the dominant kernel (the experts kernel) against the MI355X bf16 MFMA peak: achieved = active-expert
                 FLOPs (routed (token, expert) pairs x 4*D*Ed) / the kernel's mean duration, taken with HIP events on
                 the launch stream inside this run
+  sweep         the threshold number v in {0.5, 0.8, 0.9, 0.95, 0.99} under both readings (module tau: keep norm >=
+                (1 - v) * max; literal: keep norm >= v * max) with mean / p99 experts per token
+  dense_mlp_ms, measured_ceilings   the dense FFN of the same size on library GEMMs, and what this GPU sustains on
+                a large library GEMM and a streaming copy
   cpu_baseline  the CPU restatement of the reference's PyTorch CPU path (router + gate + per-expert loop) timed on
                 this machine's host cores over a bounded sample of the same layer shape
 """
@@ -36,6 +40,16 @@ WORKLOADS = {
     # name: (batch, seq, D, E, Ed, W, activation)
     'vit_b_50k': (256, 197, 768, 128, 24, 128, 'relu'),
     'vit_b_1576': (8, 197, 768, 128, 24, 128, 'relu'),
+    # BASELINE config 3: router bypassed, norms = |randn| * w_e with w_e = rank_e^-1.2 (a few experts draw most tokens)
+    'vit_b_skew': (256, 197, 768, 128, 24, 128, 'relu'),
+}
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (profiles/), scaled by
+# the factors a plain copy kernel of known size gives for the same counters (2.0 and 1.0); None = not measured
+MEASURED_TRAFFIC = {
+    'vit_b_50k': 472.8e6,     # experts_mfma_dense_kernel
+    'gemma_16': 207.1e6,      # decode_hidden_kernel + decode_out_kernel
+    'gemma_1': 163.7e6,
+    'gemma_4096': 2169.8e6,   # up product + down product + finish
 }
 # Gemma-2B-shape gated layer (BASELINE config 5): (tokens, D, E, Ed, W, activation)
 GATED_WORKLOADS = {
@@ -72,12 +86,58 @@ def time_events(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
-def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, path='auto'):
+def time_quantiles(fn, iters, warmup):
+    """Per-call durations of fn from one HIP event pair per call on the launch stream: median, 2.5 % and 97.5 %
+    quantiles in milliseconds (the reference's own bench reports the same three, test_moe_implementations.py:171-175)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    t = sorted(a.elapsed_time(b) for a, b in evs)
+    return {'median_ms': t[len(t) // 2], 'q025_ms': t[int(0.025 * (len(t) - 1))], 'q975_ms': t[int(0.975 * (len(t) - 1))],
+            'iters': iters}
+
+
+def measured_ceilings(dev):
+    """What this very GPU sustains on plain library work: a large bf16 GEMM (hipBLASLt through torch.matmul) and a
+    streaming copy.  Printed next to the published peaks; the roofline fractions stay relative to the published ones."""
+    a = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+    b = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+    ms = time_events(lambda: torch.matmul(a, b), 10, 3)
+    gemm = 2 * 8192 ** 3 / ms / 1e9
+    del a, b
+    src = torch.zeros(64 << 20, dtype=torch.float32, device=dev)   # 256 MiB read + 256 MiB written per call
+    dst = torch.empty_like(src)
+    ms = time_events(lambda: dst.copy_(src), 10, 3)
+    copy = 2 * src.numel() * 4 / ms / 1e6
+    del src, dst
+    return {'library_gemm_bf16_8192_tflops': gemm, 'copy_gbps': copy}
+
+
+def dense_mlp_ms(x, D, hidden, act, steps, warmup):
+    """The dense FFN the MoE layer was split from (Linear(D, hidden) + activation + Linear(hidden, D), bf16, library
+    GEMMs), timed on the same tokens; the reference times a compiled MLP alongside its kernels the same way
+    (test_moe_implementations.py:128-131, 172-176)."""
+    g = torch.Generator().manual_seed(7)
+    fc1 = ((torch.rand(hidden, D, generator=g) * 2 - 1) / D ** 0.5).to(x.dtype).to(x.device)
+    b1 = torch.zeros(hidden, dtype=x.dtype, device=x.device)
+    fc2 = ((torch.rand(D, hidden, generator=g) * 2 - 1) / hidden ** 0.5).to(x.dtype).to(x.device)
+    b2 = torch.zeros(D, dtype=x.dtype, device=x.device)
+    fn_act = {'relu': torch.relu, 'gelu': torch.nn.functional.gelu}[act]
+    return time_events(lambda: torch.nn.functional.linear(fn_act(torch.nn.functional.linear(x, fc1, b1)), fc2, b2), steps, warmup)
+
+
+def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, path='auto', quantile_iters=0, norms_in=None):
     N = x.size(0)
 
     def layer():
         return ops.forward(x, p['router_w1'], p['router_w2'], thr_scale, p['w1'], p['b1'], p['w2'], None, p['last_bias'],
-                           act, False, None, False, False, path, packed)
+                           act, False, norms_in, False, False, path, packed)
 
     out, routing, _, _ = layer()
     torch.cuda.synchronize()
@@ -98,8 +158,14 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, pa
     ms_experts = time_events(lambda: ops.experts(x, routing, p['w1'], p['b1'], p['w2'], None, p['last_bias'], act, False,
                                                  path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 else 'auto'),
                                                  packed), steps, warmup)
+    experts_path = path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 else 'auto')
+    quant = None
+    if quantile_iters:
+        quant = time_quantiles(lambda: ops.experts(x, routing, p['w1'], p['b1'], p['w2'], None, p['last_bias'], act, False,
+                                                   experts_path, packed), quantile_iters, 20)
     ms_router = time_events(lambda: ops.router_select(x, p['router_w1'], p['router_w2'], thr_scale, packed, E, Ed),
                             steps, warmup)
+    tokens_per_expert = routing.float().sum(0)
     active_flops = pairs * 4.0 * D * Ed
     router_flops = N * (2.0 * D * W + 2.0 * W * E)
     s = x.element_size()
@@ -108,7 +174,9 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, pa
                 p99_active=p99_k, active_tflops_layer=active_flops / ms_layer / 1e9,
                 active_tflops_kernel=active_flops / ms_experts / 1e9,
                 total_tflops_layer=(active_flops + router_flops) / ms_layer / 1e9,
-                algo_bytes=algo_bytes, hbm_gbps_layer=algo_bytes / ms_layer / 1e6, tokens_per_s=N / ms_layer * 1e3)
+                algo_bytes=algo_bytes, hbm_gbps_layer=algo_bytes / ms_layer / 1e6, tokens_per_s=N / ms_layer * 1e3,
+                experts_quantiles=quant,
+                expert_load_max_over_mean=(tokens_per_expert.max() / tokens_per_expert.mean().clamp_min(1e-9)).item())
 
 
 def run_gated(args, ops, dev):
@@ -149,12 +217,24 @@ def run_gated(args, ops, dev):
                                f'module tau={args.tau}, whole layer', 'experts_routed_to': union,
                    'mean_active_experts': pairs / N, 'mfma_kernels': packed is not None},
         'active_tflops': pairs * 6.0 * D * Ed / ms_layer / 1e9, 'hbm_gbps': algo_bytes / ms_layer / 1e6,
-        'roofline': {'bound': 'hbm', 'kernel': 'experts', 'achieved': (union * 3 * D * Ed * s + 2 * N * D * s) / ms_experts / 1e6,
+        'roofline': {'bound': 'hbm', 'kernel': 'experts (hidden + out kernels)',
+                     'achieved': (union * 3 * D * Ed * s + 2 * N * D * s) / ms_experts / 1e6,
                      'peak': PEAK_HBM_GBPS, 'unit': 'GB/s',
-                     'frac': (union * 3 * D * Ed * s + 2 * N * D * s) / ms_experts / 1e6 / PEAK_HBM_GBPS, 'traffic': None,
+                     'frac': (union * 3 * D * Ed * s + 2 * N * D * s) / ms_experts / 1e6 / PEAK_HBM_GBPS,
+                     'traffic': MEASURED_TRAFFIC.get(args.workload),
                      'kernel_ms': ms_experts, 'algorithmic_bytes_layer': algo_bytes,
                      'layer_frac': algo_bytes / ms_layer / 1e6 / PEAK_HBM_GBPS},
     }
+    if N > 16:
+        # enough tokens per expert to be compute-bound: active-pair FLOPs against the MFMA peak; the tiled products
+        # execute every (token, expert) pair, so the executed rate is reported as well
+        active = pairs * 6.0 * D * Ed
+        executed = N * E * 6.0 * D * Ed
+        line['roofline'] = {'bound': 'mfma', 'kernel': 'experts (up + down products + finish)',
+                            'achieved': active / ms_experts / 1e9, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
+                            'frac': active / ms_experts / 1e9 / PEAK_BF16_TFLOPS,
+                            'traffic': MEASURED_TRAFFIC.get(args.workload), 'kernel_ms': ms_experts,
+                            'executed_tflops': executed / ms_experts / 1e9}
     print(json.dumps(line))
 
 
@@ -190,6 +270,9 @@ def main():
     ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS) + sorted(GATED_WORKLOADS))
     ap.add_argument('--tau', type=float, default=0.9, help='module tau (keep expert when norm >= (1 - tau) * max)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--no-sweep', action='store_true', help='skip the threshold sweep (5 values x 2 readings)')
+    ap.add_argument('--quantile-iters', type=int, default=200,
+                    help='per-call timed launches of the experts kernel for median / 2.5 % / 97.5 % (0 = skip)')
     ap.add_argument('--copy-probe', action='store_true',
                     help='also run a plain 512 MiB device copy (calibrates FETCH_SIZE / WRITE_SIZE counter units)')
     args = ap.parse_args()
@@ -202,6 +285,14 @@ def main():
         sys.exit(1)
     from d2dmoe_amd import ops
     dev = torch.device('cuda:0')
+    if args.copy_probe:
+        # one elementwise kernel that reads 512 MiB and writes 512 MiB
+        src = torch.zeros(128 << 20, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     if args.workload in GATED_WORKLOADS:
         with torch.no_grad():
             run_gated(args, ops, dev)
@@ -213,17 +304,27 @@ def main():
     x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
     shape = ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x), act)
     packed = ops.pack_weights(shape, p['w1'], p['b1'], p['w2'], None, p['router_w1'], p['router_w2'])
-    if args.copy_probe:
-        # one elementwise kernel that reads 512 MiB and writes 512 MiB
-        src = torch.zeros(128 << 20, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            torch.add(src, 1.0, out=dst)
-        torch.cuda.synchronize()
-        del src, dst
+    norms_in = None
+    if args.workload == 'vit_b_skew':
+        g = torch.Generator().manual_seed(2)
+        ranks = torch.randperm(E, generator=g).float() + 1.0
+        wts = ranks ** -1.2
+        norms_in = (torch.randn(N, E, generator=g).abs() * (wts / wts.max())).to(dtype).to(dev)
     with torch.no_grad():
-        main_r = run_regime(ops, x, p, packed, float(1.0 - args.tau), act, args.steps, args.warmup, D, E, Ed, W)
-        lit_r = run_regime(ops, x, p, packed, float(args.tau), act, args.steps, args.warmup, D, E, Ed, W)
+        main_r = run_regime(ops, x, p, packed, float(1.0 - args.tau), act, args.steps, args.warmup, D, E, Ed, W,
+                            quantile_iters=args.quantile_iters, norms_in=norms_in)
+        lit_r = run_regime(ops, x, p, packed, float(args.tau), act, args.steps, args.warmup, D, E, Ed, W, norms_in=norms_in)
+        sweep = []
+        if not args.no_sweep:
+            # BASELINE config 2: the threshold number under both readings
+            for v in (0.5, 0.8, 0.9, 0.95, 0.99):
+                for rule, thr in (('module_tau', 1.0 - v), ('literal', v)):
+                    r = run_regime(ops, x, p, packed, float(thr), act, max(args.steps // 5, 5), 3, D, E, Ed, W, norms_in=norms_in)
+                    sweep.append({'v': v, 'rule': rule, 'keep_norm_ge_frac_of_max': round(thr, 4), 'ms_per_step': r['ms_layer'],
+                                  'tokens_per_s': r['tokens_per_s'], 'mean_active_experts': r['mean_active'],
+                                  'p99_active_experts': r['p99_active'], 'active_tflops': r['active_tflops_layer']})
+        dense_ms = dense_mlp_ms(x, D, E * Ed, act, args.steps, args.warmup)
+        ceil = measured_ceilings(dev)
     line = {
         'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
         'value': main_r['tokens_per_s'], 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
@@ -236,13 +337,19 @@ def main():
         'active_tflops': main_r['active_tflops_layer'], 'hbm_gbps': main_r['hbm_gbps_layer'],
         'roofline': {'bound': 'mfma', 'kernel': 'experts', 'achieved': main_r['active_tflops_kernel'],
                      'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s', 'frac': main_r['active_tflops_kernel'] / PEAK_BF16_TFLOPS,
-                     'traffic': None, 'kernel_ms': main_r['ms_experts'], 'router_select_ms': main_r['ms_router']},
+                     'traffic': MEASURED_TRAFFIC.get(args.workload), 'kernel_ms': main_r['ms_experts'],
+                     'kernel_quantiles': main_r['experts_quantiles'], 'router_select_ms': main_r['ms_router'],
+                     'frac_of_library_gemm': main_r['active_tflops_kernel'] / ceil['library_gemm_bf16_8192_tflops']},
+        'measured_ceilings': ceil,
+        'dense_mlp_ms': dense_ms,
+        'expert_load_max_over_mean': main_r['expert_load_max_over_mean'],
         'literal_rule': {'rule': f'keep norm >= {args.tau}*max', 'tokens_per_s': lit_r['tokens_per_s'],
                          'ms_per_step': lit_r['ms_layer'], 'mean_active_experts': lit_r['mean_active'],
                          'p99_active_experts': lit_r['p99_active'], 'active_tflops': lit_r['active_tflops_layer'],
                          'roofline': {'bound': 'hbm', 'achieved': lit_r['hbm_gbps_layer'], 'peak': PEAK_HBM_GBPS,
                                       'unit': 'GB/s', 'frac': lit_r['hbm_gbps_layer'] / PEAK_HBM_GBPS,
                                       'algorithmic_bytes': lit_r['algo_bytes'], 'kernel_ms': lit_r['ms_experts']}},
+        'sweep': sweep,
     }
     if not args.no_cpu_baseline:
         line['cpu_baseline'] = cpu_baseline(D, E, Ed, W, act, args.tau)

@@ -202,35 +202,52 @@ __global__ __launch_bounds__(256) void perm_count_kernel(const T* __restrict__ r
   }
 }
 
-// One workgroup of 1024 threads (16 waves) per group of 64 experts.  Wave w scans a contiguous range of
-// segments for its 64 experts; the 16 partial sums are combined through LDS.
+// Exclusive prefix over segments, per expert.  Grid = (groups of 64 experts) x (PERM_SCAN_BLOCKS blocks of consecutive
+// segments); a workgroup has 16 waves, lanes = experts.  A workgroup first adds up everything before its block (its
+// waves share that range), then wave w scans its own slice of the block; partial sums meet in LDS.  Integer sums, so
+// the result does not depend on the split.
+constexpr int PERM_SCAN_BLOCKS = 16;
+
 __global__ __launch_bounds__(1024) void perm_scan_kernel(const int32_t* __restrict__ seg_counts,
                                                          int32_t* __restrict__ seg_offsets, int32_t* __restrict__ totals,
                                                          int E, int64_t n_seg) {
+  __shared__ int32_t before[16][kWave];
   __shared__ int32_t part[16][kWave];
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x / kWave;
   const int e = blockIdx.x * kWave + lane;
-  const int64_t per = (n_seg + 15) / 16;
-  const int64_t s0 = w * per;
-  const int64_t s1 = (s0 + per) < n_seg ? (s0 + per) : n_seg;
-  int sum = 0;
+  const int64_t per_block = (n_seg + PERM_SCAN_BLOCKS - 1) / PERM_SCAN_BLOCKS;
+  const int64_t b0 = ((int64_t)blockIdx.y * per_block) < n_seg ? ((int64_t)blockIdx.y * per_block) : n_seg;
+  const int64_t b1 = (b0 + per_block) < n_seg ? (b0 + per_block) : n_seg;
+  // segments [0, b0) split over the waves
+  const int64_t pa = (b0 + 15) / 16;
+  const int64_t a0 = (w * pa) < b0 ? (w * pa) : b0;
+  const int64_t a1 = (a0 + pa) < b0 ? (a0 + pa) : b0;
+  // this wave's slice of [b0, b1)
+  const int64_t per = (b1 > b0) ? ((b1 - b0 + 15) / 16) : 0;
+  const int64_t s0 = (b0 + w * per) < b1 ? (b0 + w * per) : b1;
+  const int64_t s1 = (s0 + per) < b1 ? (s0 + per) : b1;
+  int pre = 0, sum = 0;
   if (e < E) {
-#pragma unroll 32
+#pragma unroll 16
+    for (int64_t s = a0; s < a1; ++s) pre += seg_counts[s * E + e];
+#pragma unroll 16
     for (int64_t s = s0; s < s1; ++s) sum += seg_counts[s * E + e];
   }
+  before[w][lane] = pre;
   part[w][lane] = sum;
   __syncthreads();
   int run = 0;
+  for (int i = 0; i < 16; ++i) run += before[i][lane];
   for (int i = 0; i < w; ++i) run += part[i][lane];
   if (e < E) {
-#pragma unroll 32
+#pragma unroll 16
     for (int64_t s = s0; s < s1; ++s) {
       const int c = seg_counts[s * E + e];
       seg_offsets[s * E + e] = run;
       run += c;
     }
-    if (w == 15) totals[e] = run;
+    if (w == 15 && blockIdx.y == PERM_SCAN_BLOCKS - 1) totals[e] = run;
   }
 }
 
@@ -303,7 +320,7 @@ __global__ __launch_bounds__(256) void perm_scatter_kernel(const T* __restrict__
 }
 
 void launch_perm_scan(const int32_t* seg_counts, int32_t* seg_offsets, int32_t* totals, int E, int64_t n_seg, hipStream_t s) {
-  hipLaunchKernelGGL(perm_scan_kernel, dim3((E + kWave - 1) / kWave), dim3(1024), 0, s, seg_counts, seg_offsets, totals, E, n_seg);
+  hipLaunchKernelGGL(perm_scan_kernel, dim3((E + kWave - 1) / kWave, PERM_SCAN_BLOCKS), dim3(1024), 0, s, seg_counts, seg_offsets, totals, E, n_seg);
 }
 
 size_t perm_workspace_bytes(int64_t N, int E) {
@@ -322,7 +339,7 @@ hipError_t launch_build_permutation(const void* routing, int64_t N, int E, int32
   int32_t* totals = seg_offsets + n_seg * E;
   const unsigned seg_blocks = (unsigned)cdiv64(n_seg, 4);
   hipLaunchKernelGGL(perm_count_kernel<T>, dim3(seg_blocks), dim3(256), 0, s, (const T*)routing, seg_counts, N, E, n_seg);
-  hipLaunchKernelGGL(perm_scan_kernel, dim3((E + kWave - 1) / kWave), dim3(1024), 0, s, seg_counts, seg_offsets, totals, E, n_seg);
+  hipLaunchKernelGGL(perm_scan_kernel, dim3((E + kWave - 1) / kWave, PERM_SCAN_BLOCKS), dim3(1024), 0, s, seg_counts, seg_offsets, totals, E, n_seg);
   hipLaunchKernelGGL(perm_offsets_kernel, dim3(1), dim3(1024), 0, s, totals, offsets, bincounts, E);
   hipLaunchKernelGGL(perm_scatter_kernel<T>, dim3(seg_blocks), dim3(256), 0, s, (const T*)routing, seg_offsets, offsets,
                      token_idx, sort_indices, unsort_indices, N, E, n_seg);

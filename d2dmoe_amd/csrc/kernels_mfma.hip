@@ -227,7 +227,7 @@ struct DenseArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* wp; const bf16_t* b1p; const uint8_t* eidx;
   const bf16_t* last_bias; bf16_t* out;
   const int* skip_flag;   // optional device flag: non-zero = the expert-major path handles this call
-  int64_t N; int E; int expert_dim; int n_chunks; int hidden; int act_rt; int add_residual; int n_full;
+  int64_t N; int E; int expert_dim; int n_chunks; int hidden; int act_rt; int add_residual; int n_full; int n_tiles;
 };
 
 template <int D, int ACT, bool ED8, int TT>
@@ -540,6 +540,28 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   }
 }
 
+// Out-of-line copy of the tile routine for the variant below (keeps its register allocation apart from the loop).
+template <int D, int ACT, bool ED8, int TT>
+__device__ __attribute__((noinline)) void dense_tile_call(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw) {
+  dense_tile<D, ACT, ED8, TT>(A, tok0, smem_raw);
+}
+
+// The same sweep launched as one workgroup per CU that walks the tiles in launch order.  Used where the launch is
+// usually a no-op (the fall-back behind the expert-major path): a skipped call then retires after one round of empty
+// workgroups instead of one per tile.
+template <int D, int ACT, bool ED8>
+__global__ __launch_bounds__(256, 1) void experts_mfma_dense_walk_kernel(const DenseArgs A) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
+  for (int b = blockIdx.x; b < A.n_tiles; b += gridDim.x) {
+    if (b < A.n_full)
+      dense_tile_call<D, ACT, ED8, 2>(A, (int64_t)b * 64, smem_raw);
+    else
+      dense_tile_call<D, ACT, ED8, 1>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
+    __syncthreads();   // the next tile's staging overwrites the LDS the final epilogue just read
+  }
+}
+
 template <int D, int ACT, bool ED8>
 __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -568,7 +590,7 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   const char* base = (const char*)packed;
   const size_t lds = dense_lds_bytes(sh);
   if (lds > 160 * 1024) return hipErrorInvalidValue;
-  auto kern = experts_mfma_dense_kernel<D, ACT, ED8>;
+  auto kern = (skip_flag != nullptr) ? experts_mfma_dense_walk_kernel<D, ACT, ED8> : experts_mfma_dense_kernel<D, ACT, ED8>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   // Tiles of 64 tokens fill whole rounds of one workgroup per CU; when the last round would be at most half full its
@@ -586,8 +608,9 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   A.b1p = (const bf16_t*)(base + L.b1_off); A.eidx = (const uint8_t*)(base + L.eidx_off);
   A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.N = sh.n_tokens; A.E = sh.n_experts; A.expert_dim = sh.expert_dim;
   A.n_chunks = L.n_chunks; A.hidden = L.hidden; A.act_rt = sh.activation; A.add_residual = sh.add_residual;
-  A.n_full = (int)n_full; A.skip_flag = skip_flag;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(n_full + n_half)), dim3(256), lds, s, A);
+  A.n_full = (int)n_full; A.n_tiles = (int)(n_full + n_half); A.skip_flag = skip_flag;
+  const int64_t grid = (skip_flag != nullptr && A.n_tiles > cus) ? cus : A.n_tiles;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, s, A);
   return hipGetLastError();
 }
 
