@@ -238,6 +238,67 @@ def run_gated(args, ops, dev):
     print(json.dumps(line))
 
 
+def run_gpt2(args, dev):
+    """BASELINE config 4: GPT-2-small (12 blocks, D = 768, 12 heads, vocab 50257) with every FFN replaced by a MoE layer
+    of 128 experts x 24 neurons (GELU-erf, biases) and a 768 -> 128 -> 128 router; 16 x 1024 token ids; bf16; random
+    weights.  Attention, LayerNorm, embeddings and the LM head are stock PyTorch; the MoE layers are this library."""
+    from d2dmoe_amd import add_routers, gpt2, ops
+    torch.manual_seed(0)
+    cfg = gpt2.GPTConfig(block_size=1024, vocab_size=50257, n_layer=12, n_head=12, n_embd=768)
+    dense = gpt2.GPT(cfg).eval().to(dev).to(torch.bfloat16)
+    moe, names = gpt2.replace_with_moes(dense, num_experts=128, experts_class='hip_kernel')
+    gpt2.split_original_parameters(dense, moe, names)
+    add_routers(moe, dict(width=128, depth=2, bias=False, activation='relu', output_activation='abs'))
+    moe = moe.to(dev).to(torch.bfloat16)
+    layers = [gpt2.get_module_by_name(moe, n) for n in names]
+    for layer in layers:
+        layer.forward_mode, layer.tau = 'dynk_max', args.tau
+        layer.experts.forward_mode = 'hip'
+    B, T = 16, 1024
+    idx = torch.randint(0, cfg.vocab_size, (B, T), generator=torch.Generator().manual_seed(1)).to(dev)
+    captured = {}
+    hooks = [layer.register_forward_hook(lambda m, inp, out, n=n: captured.__setitem__(n, (inp[0].detach(), out[1][n][0])))
+             for n, layer in zip(names, layers)]
+    moe(idx)
+    for h in hooks:
+        h.remove()
+    torch.cuda.synchronize()
+    ms_moe_model = time_events(lambda: moe(idx), args.steps, args.warmup)
+    ms_dense_model = time_events(lambda: dense(idx), args.steps, args.warmup)
+    per_layer = []
+    for n, layer in zip(names, layers):
+        x, routing = captured[n]
+        ms = time_events(lambda: layer(x), args.steps, args.warmup)
+        per_layer.append({'layer': n, 'ms': ms, 'mean_active_experts': routing.float().sum(-1).mean().item()})
+    ms_moe_layers = sum(r['ms'] for r in per_layer)
+    ms_dense_ffn = time_events(lambda: dense.transformer.h[0].mlp(captured[names[0]][0]), args.steps, args.warmup)
+    # dominant kernel: the experts kernel of the first MoE layer on its real input and routing
+    x0, r0 = captured[names[0]]
+    ex = layers[0].experts
+    x0 = x0.reshape(-1, 768).contiguous()
+    r0 = r0.reshape(-1, 128).contiguous()
+    packed = ex.packed_weights(layers[0].router.layers[0].weight, layers[0].router.layers[2].weight, 'relu', 'abs')
+    lb = layers[0].last_bias.view(-1)
+    ms_experts = time_events(lambda: ops.experts(x0, r0, ex.w1, ex.b1, ex.w2, None, lb, 'gelu', False, 'auto', packed),
+                             args.steps, args.warmup)
+    active = r0.float().sum().item() * 4.0 * 768 * 24
+    N = B * T
+    line = {
+        'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
+        'value': N / ms_moe_model * 1e3, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': ms_moe_model, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16',
+        'data': 'synthetic',
+        'config': {'workload': f'gpt2_small: whole model forward, 12 blocks, {B}x{T}={N} token ids, MoE FFN 128 experts x 24 '
+                               f'(gelu, biases), router 768->128->128, module tau={args.tau}; one step = one model forward'},
+        'moe_layers_ms': ms_moe_layers, 'moe_share_of_model': ms_moe_layers / ms_moe_model,
+        'dense_model_ms': ms_dense_model, 'dense_ffn_layer_ms': ms_dense_ffn, 'per_layer': per_layer,
+        'roofline': {'bound': 'mfma', 'kernel': 'experts (first MoE layer, its real input and routing)',
+                     'achieved': active / ms_experts / 1e9, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': active / ms_experts / 1e9 / PEAK_BF16_TFLOPS, 'traffic': None, 'kernel_ms': ms_experts},
+    }
+    print(json.dumps(line))
+
+
 def cpu_baseline(D, E, Ed, W, act, tau, budget_s=15.0):
     """The oracle's restatement of the reference CPU path (router -> dynk_max gate -> per-expert loop), float32,
     8 x 197 tokens of the same layer shape, repeated until about budget_s seconds have been spent."""
@@ -267,7 +328,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS) + sorted(GATED_WORKLOADS))
+    ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS) + sorted(GATED_WORKLOADS) + ['gpt2_small'])
     ap.add_argument('--tau', type=float, default=0.9, help='module tau (keep expert when norm >= (1 - tau) * max)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-sweep', action='store_true', help='skip the threshold sweep (5 values x 2 readings)')
@@ -296,6 +357,10 @@ def main():
     if args.workload in GATED_WORKLOADS:
         with torch.no_grad():
             run_gated(args, ops, dev)
+        return
+    if args.workload == 'gpt2_small':
+        with torch.no_grad():
+            run_gpt2(args, dev)
         return
     B, T, D, E, Ed, W, act = WORKLOADS[args.workload]
     N = B * T

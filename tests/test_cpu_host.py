@@ -186,3 +186,72 @@ def test_extract_indices_cpu_matches_oracle():
     s, u, c = HipKernelExperts.extract_indices(routing)
     so, uo, co = O.extract_indices(routing)
     assert torch.equal(s, so) and torch.equal(u, uo) and torch.equal(c.long(), co)
+
+
+# ------------------------------------------------------------------------------------- GPT-2 model surgery
+def _tiny_gpt(seed=0, activation='gelu'):
+    from d2dmoe_amd import gpt2
+    torch.manual_seed(seed)
+    cfg = gpt2.GPTConfig(block_size=32, vocab_size=96, n_layer=2, n_head=2, n_embd=64, activation=activation)
+    model = gpt2.GPT(cfg).eval()
+    with torch.no_grad():   # make the zero-initialised biases matter
+        for n, p in model.named_parameters():
+            if n.endswith('bias'):
+                p.normal_(0.0, 0.05)
+    return gpt2, model
+
+
+@pytest.mark.parametrize('labelling', ['contiguous', 'shuffled'])
+def test_gpt_surgery_all_experts_reproduces_the_dense_model(labelling):
+    """replace_with_moes + split_original_parameters: with every expert running ('all'), the MoE model is the dense
+    model, whatever balanced labelling moved the neurons (reference: moefication.py:157-202, 205-306)."""
+    gpt2, model = _tiny_gpt()
+    moe, names = gpt2.replace_with_moes(model, expert_size=16, experts_class='hip_kernel')
+    assert names == ['transformer.h.0.mlp', 'transformer.h.1.mlp']
+    labels = None
+    if labelling == 'shuffled':
+        g = torch.Generator().manual_seed(5)
+        labels = {n: (torch.arange(256) // 16)[torch.randperm(256, generator=g)] for n in names}
+    gpt2.split_original_parameters(model, moe, names, labels)
+    for n in names:
+        layer = gpt2.get_module_by_name(moe, n)
+        assert layer.num_experts == 16 and layer.expert_dim == 16 and isinstance(layer.dropout, nn.Dropout)
+        layer.forward_mode = 'all'
+        layer.experts.forward_mode = 'masked'
+    idx = torch.randint(0, 96, (3, 20), generator=torch.Generator().manual_seed(1))
+    with torch.no_grad():
+        want = model(idx)
+        got, gating = moe(idx, return_gating_data=True)
+        assert torch.equal(moe(idx), got)
+    assert set(gating) == set(names) and gating[names[0]][0].shape == (3, 20, 16)
+    assert H.rel_err(got, want) < 1e-5
+    # state_dict keys of a MoE block follow the reference layer's
+    keys = [k for k in moe.state_dict() if k.startswith('transformer.h.0.mlp')]
+    assert keys == ['transformer.h.0.mlp.last_bias', 'transformer.h.0.mlp.experts.w1', 'transformer.h.0.mlp.experts.b1',
+                    'transformer.h.0.mlp.experts.w2']
+
+
+def test_gpt_dynk_max_on_cpu_matches_oracle_layer():
+    from d2dmoe_amd import add_routers
+    gpt2, model = _tiny_gpt(activation='relu')
+    moe, names = gpt2.replace_with_moes(model, num_experts=8)
+    gpt2.split_original_parameters(model, moe, names)
+    add_routers(moe, dict(width=16, depth=2, bias=False, activation='relu', output_activation='abs'))
+    for n in names:
+        layer = gpt2.get_module_by_name(moe, n)
+        layer.forward_mode, layer.tau = 'dynk_max', 0.6
+        layer.experts.forward_mode = 'masked'
+    idx = torch.randint(0, 96, (2, 16), generator=torch.Generator().manual_seed(2))
+    captured = {}
+    layer0 = gpt2.get_module_by_name(moe, names[0])
+    hook = layer0.register_forward_hook(lambda m, inp, out: captured.update(x=inp[0], out=out[0], routing=out[1][names[0]][0]))
+    with torch.no_grad():
+        moe(idx)
+    hook.remove()
+    p = dict(w1=layer0.experts.w1.detach(), b1=layer0.experts.b1.detach(), w2=layer0.experts.w2.detach(),
+             last_bias=layer0.last_bias.detach(), router_w1=layer0.router.layers[0].weight.detach(),
+             router_w2=layer0.router.layers[2].weight.detach())
+    want_out, want_routing, _ = O.moe_layer_forward(captured["x"], p, 0.6, "relu", "all")
+    assert torch.equal(captured['routing'], want_routing.view_as(captured['routing']))
+    assert H.rel_err(captured['out'], want_out.view_as(captured['out'])) < 1e-5
+    assert 0 < captured['routing'].mean().item() < 1

@@ -553,3 +553,56 @@ def test_module_execute_all_gated_hip():
         got, g2 = moe(x)
     assert torch.equal(g1['g'][0], g2['g'][0])
     assert H.rel_err(got, want) < 3e-2   # both sides are bf16 evaluations here
+
+
+# =================================================================== GPT-2 model-level drop-in ========
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', ['tiny', 'gpt2_width'])
+def test_gpt_with_hip_moe_layers(shape, dtype):
+    """Model surgery on the GPU: with every expert running, the MoE model (HIP experts) reproduces the dense model's
+    logits; under dynk_max the fused layer returns the gating data of every block without a host synchronisation."""
+    from d2dmoe_amd import add_routers, gpt2
+    _say('gpt', shape, dtype)
+    torch.manual_seed(0)
+    if shape == 'tiny':
+        cfg = gpt2.GPTConfig(block_size=32, vocab_size=96, n_layer=2, n_head=2, n_embd=64)
+        kw, width = dict(expert_size=16), 16
+    else:   # GPT-2-small width, MFMA kernels in bf16: 128 experts x 24 neurons, GELU, biases
+        cfg = gpt2.GPTConfig(block_size=128, vocab_size=512, n_layer=2, n_head=12, n_embd=768)
+        kw, width = dict(num_experts=128), 128
+    model = gpt2.GPT(cfg).eval()
+    with torch.no_grad():
+        for n, prm in model.named_parameters():
+            if n.endswith('bias'):
+                prm.normal_(0.0, 0.05)
+    model = model.to(DEV).to(dtype)
+    moe, names = gpt2.replace_with_moes(model, experts_class='hip_kernel', **kw)
+    gpt2.split_original_parameters(model, moe, names)
+    for n in names:
+        layer = gpt2.get_module_by_name(moe, n)
+        layer.forward_mode = 'all'
+        layer.experts.forward_mode = 'hip'
+    idx = torch.randint(0, cfg.vocab_size, (4, cfg.block_size), generator=torch.Generator().manual_seed(1)).to(DEV)
+    with torch.no_grad():
+        want = model.float()(idx) if dtype == torch.float32 else model(idx)
+        got, gating = moe(idx, return_gating_data=True)
+    tol = 2e-4 if dtype == torch.float32 else H.TOL_BF16
+    assert H.rel_err(got.float().cpu(), want.float().cpu()) < tol
+    assert set(gating) == set(names)
+    # dynamic-k mode through the fused layer call
+    add_routers(moe, dict(width=width, depth=2, bias=False, activation='relu', output_activation='abs'))
+    moe = moe.to(DEV).to(dtype)
+    for n in names:
+        layer = gpt2.get_module_by_name(moe, n)
+        layer.forward_mode, layer.tau = 'dynk_max', 0.5
+    with torch.no_grad():
+        moe(idx)
+        torch.cuda.synchronize()
+        torch.cuda.set_sync_debug_mode('error')
+        try:
+            out, gating = moe(idx, return_gating_data=True)
+        finally:
+            torch.cuda.set_sync_debug_mode('default')
+    frac = gating[names[-1]][0].float().mean().item()
+    assert out.shape == (4, cfg.block_size, cfg.vocab_size) and 0.0 < frac < 1.0
+    assert torch.isfinite(out.float()).all()
