@@ -40,7 +40,7 @@ WORKLOADS = {
     # name: (batch, seq, D, E, Ed, W, activation)
     'vit_b_50k': (256, 197, 768, 128, 24, 128, 'relu'),
     'vit_b_1576': (8, 197, 768, 128, 24, 128, 'relu'),
-    # BASELINE config 3: router bypassed, norms = |randn| * w_e with w_e = rank_e^-1.2 (a few experts draw most tokens)
+    # skewed routing: router bypassed, norms = |randn| * w_e with w_e = rank_e^-1.2 (a few experts draw most tokens)
     'vit_b_skew': (256, 197, 768, 128, 24, 128, 'relu'),
 }
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (profiles/), scaled by
@@ -51,7 +51,7 @@ MEASURED_TRAFFIC = {
     'gemma_1': 163.7e6,
     'gemma_4096': 2169.8e6,   # up product + down product + finish
 }
-# Gemma-2B-shape gated layer (BASELINE config 5): (tokens, D, E, Ed, W, activation)
+# Gemma-2B-shape gated layer: (tokens, D, E, Ed, W, activation)
 GATED_WORKLOADS = {
     'gemma_1': (1, 2048, 256, 64, 256, 'gelu_tanh'),
     'gemma_16': (16, 2048, 256, 64, 256, 'gelu_tanh'),
@@ -239,7 +239,7 @@ def run_gated(args, ops, dev):
 
 
 def run_gpt2(args, dev):
-    """BASELINE config 4: GPT-2-small (12 blocks, D = 768, 12 heads, vocab 50257) with every FFN replaced by a MoE layer
+    """Whole-model workload: GPT-2-small (12 blocks, D = 768, 12 heads, vocab 50257) with every FFN replaced by a MoE layer
     of 128 experts x 24 neurons (GELU-erf, biases) and a 768 -> 128 -> 128 router; 16 x 1024 token ids; bf16; random
     weights.  Attention, LayerNorm, embeddings and the LM head are stock PyTorch; the MoE layers are this library."""
     from d2dmoe_amd import add_routers, gpt2, ops
@@ -381,7 +381,7 @@ def main():
         lit_r = run_regime(ops, x, p, packed, float(args.tau), act, args.steps, args.warmup, D, E, Ed, W, norms_in=norms_in)
         sweep = []
         if not args.no_sweep:
-            # BASELINE config 2: the threshold number under both readings
+            # the threshold number under both readings
             for v in (0.5, 0.8, 0.9, 0.95, 0.99):
                 for rule, thr in (('module_tau', 1.0 - v), ('literal', v)):
                     r = run_regime(ops, x, p, packed, float(thr), act, max(args.steps // 5, 5), 3, D, E, Ed, W, norms_in=norms_in)

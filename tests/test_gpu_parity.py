@@ -230,7 +230,7 @@ def test_experts_mfma_dense_activations_bias_residual_weights(act):
 
 
 def test_experts_mfma_dense_full_size_properties():
-    """50432 tokens (BASELINE config 2): oracle on a slice of rows, the generic HIP kernel on all rows, and
+    """50432 tokens (the headline workload): oracle on a slice of rows, the generic HIP kernel on all rows, and
     determinism (two runs give identical bits)."""
     N = 50432
     x, routing, p = H.random_case(N, 768, 128, 24, 8, seed=31, dtype=torch.bfloat16, density=0.79)
@@ -364,7 +364,7 @@ def test_router_select_mfma(N, D, W, E, tau):
                                                (768, 128, 24, 128, False, 'relu'), (768, 24, 128, 128, False, 'gelu'),
                                                (1024, 16, 32, 128, True, 'silu')])
 def test_decode_path_matches_oracle(N, D, E, Ed, W, gated, act):
-    """At most 16 tokens: one workgroup per expert streams its packed weights; BASELINE config 5 is the first shape."""
+    """At most 16 tokens: one workgroup per expert streams its packed weights; the Gemma-2B FFN is the first shape."""
     _say('decode', N, D, E, Ed, gated, act)
     x, routing, p = H.random_case(N, D, E, Ed, W, seed=N + E, dtype=torch.bfloat16, gated=gated, bias=not gated, density=0.7)
     d = H.to_dev(p, DEV)
@@ -401,7 +401,7 @@ def test_decode_path_matches_oracle(N, D, E, Ed, W, gated, act):
                                             (1030, 2048, 256, 64, 256, 'gelu_tanh')])
 def test_gated_gemm_path_matches_oracle(N, D, E, Ed, W, act):
     """Gated experts, more than 16 tokens: up product with the routing value as a factor, hidden activations kept as
-    fragments, down product with K splits; BASELINE config 5 at N = 4096 has the last shape.  9000 tokens take two
+    fragments, down product with K splits; the last shape is the Gemma-2B FFN.  9000 tokens take two
     passes of the token slab."""
     _say('gated gemm', N, D, E, Ed, act)
     x, routing, p = H.random_case(N, D, E, Ed, W, seed=N + E, dtype=torch.bfloat16, gated=True, bias=False, density=0.7)
@@ -469,7 +469,7 @@ def test_layer_against_golden_fixture(case, dtype):
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('tau', [0.1, 0.9])
 def test_layer_end_to_end_vit_shape(dtype, tau):
-    """Full path including the router on the GPU (BASELINE config 1 shape, 8 x 197 tokens).  The mask is a hard
+    """Full path including the router on the GPU (the ViT-B shape the CPU baseline runs, 8 x 197 tokens).  The mask is a hard
     compare on router outputs, so a different accumulation order can flip entries that sit within rounding of the
     threshold; their number is reported and bounded, and outputs are compared on rows whose mask agrees."""
     _say('e2e', dtype, tau)
@@ -495,7 +495,7 @@ def test_layer_end_to_end_vit_shape(dtype, tau):
 
 
 def test_layer_skewed_norms_override():
-    """BASELINE config 3 in miniature: the router is bypassed by synthetic predicted norms |N(0,1)| x Zipf(1.2)."""
+    """The skewed-routing workload in miniature: the router is bypassed by synthetic predicted norms |N(0,1)| x Zipf(1.2)."""
     N, D, E, Ed = 2048, 768, 128, 24
     x, _, p = H.random_case(N, D, E, Ed, 128, seed=5, dtype=torch.bfloat16)
     g = torch.Generator().manual_seed(9)
