@@ -14,7 +14,7 @@
 // One kernel template serves both products.  Workgroup = 4 waves (2 x 2), tile = 256 tokens x 256 rows/columns of the
 // weight operand, wave tile 128 x 128 = 16 accumulator tiles of v_mfma_f32_32x32x16_bf16 (256 AGPRs).  The token
 // operand (x, or H) goes through LDS in fragment order, double-buffered, 64 K values per stage; the weight operand is
-// read straight from its packed fragment stream into two register buffers (one stage ahead).  One LDS-only barrier
+// read straight from its packed fragment stream through a register ring refilled one stage ahead.  One LDS-only barrier
 // per stage (64 MFMAs per wave).
 //
 // The up product is computed transposed so that each lane ends up with ONE token and 16 hidden units per tile; the 8
@@ -190,6 +190,13 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
   // ---- token operand: global -> registers -> LDS, 8 pieces of 16 bytes per thread and stage
   u32x4 xv[8];
   const int xrow = t >> 3, xpc = t & 7;   // MODE 0: row within a 32-token tile, 16-byte piece of the 64-wide K slice
+  // MODE 0 stores 8 pieces of one row per 8 lanes; inside a fragment the row slot is XORed with the piece index (and
+  // bit 3 with the row's parity) so that those stores spread over all LDS banks.  A read of fragment (kstep, half)
+  // applies the same XOR, which only permutes its 32 consecutive slots.
+  int xoff[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks)
+    xoff[ks] = (MODE == 0) ? (32 * g + (c32 ^ (2 * ks + g) ^ ((c32 & 1) << 3))) : lane;
   auto load_x = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -205,7 +212,7 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
   auto store_x = [&](bf16x8* buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      if (MODE == 0) ((u32x4*)buf)[(i * 4 + (xpc >> 1)) * 64 + xrow + 32 * (xpc & 1)] = xv[i];
+      if (MODE == 0) ((u32x4*)buf)[(i * 4 + (xpc >> 1)) * 64 + 32 * (xpc & 1) + (xrow ^ xpc ^ ((xrow & 1) << 3))] = xv[i];
       else ((u32x4*)buf)[i * 256 + t] = xv[i];
     }
   };
@@ -217,11 +224,11 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) ring[ks][i] = wbase[(ks * 4 + i) * 64];
   auto compute = [&](const bf16x8* buf, int s_next) __attribute__((always_inline)) {
-    const bf16x8* xl = buf + (wn * 4) * 4 * 64 + lane;
+    const bf16x8* xl = buf + (wn * 4) * 4 * 64;
     const bf16x8* wn_ = wbase + (int64_t)s_next * 16 * 64;
     bf16x8 xb[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) xb[j] = xl[(j * 4 + 0) * 64];
+    for (int j = 0; j < 4; ++j) xb[j] = xl[(j * 4 + 0) * 64 + xoff[0]];
     static_for<0, 4>([&](auto ks_c) __attribute__((always_inline)) {
       constexpr int ks = decltype(ks_c)::value;
       constexpr int kn = (ks + 1 < 4) ? ks + 1 : ks;
@@ -233,7 +240,7 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
       }
       bf16x8 nxb[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) nxb[j] = xl[(j * 4 + kn) * 64];
+      for (int j = 0; j < 4; ++j) nxb[j] = xl[(j * 4 + kn) * 64 + xoff[kn]];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
