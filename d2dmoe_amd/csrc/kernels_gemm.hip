@@ -1,9 +1,12 @@
-// Large-batch gated experts (Gemma shape) on bf16 MFMA as two tiled products with the hidden activations kept in
-// memory between them:
+// Experts on bf16 MFMA as two tiled products with the hidden activations kept in memory between them.  Serves gated
+// experts (Gemma shape) at more than 16 tokens, and ungated experts whose width the fused sweep is not built for:
 //
-//   up    H^T[hidden, token] = act(Wg^T . X^T) * (Wu^T . X^T) * routing[token, expert(hidden)]      (ExecuteAllExperts
-//         with intermediate gating, moe_layers.py:71-78, 91-96, restricted to the routed pairs by the routing factor)
-//   down  OUT[token, :] = sum over hidden of H[token, hidden] . Wd[hidden, :]  (+ last_bias, + x)
+//   up    gated:   H^T[hidden, token] = act(Wg^T . X^T) * (Wu^T . X^T) * routing[token, expert(hidden)]
+//                  (ExecuteAllExperts with intermediate gating, moe_layers.py:71-78, 91-96)
+//         ungated: H^T[hidden, token] = act(W1^T . X^T + b1) * routing[token, expert(hidden)]
+//                  (CustomKernelExperts.forward_all, moe_layers.py:116-133)
+//         -- in both cases restricted to the routed pairs by the routing factor
+//   down  OUT[token, :] = sum over hidden of H[token, hidden] . W2[hidden, :]  (+ last_bias, + x)
 //
 // With D = 2048 neither a token tile's x rows nor its output accumulators fit next to each other on a CU, and the
 // expert weights (201 MB) dwarf the activations, so the fused token-stationary sweep of the ViT shape does not carry
@@ -14,12 +17,12 @@
 // One kernel template serves both products.  Workgroup = 4 waves (2 x 2), tile = 256 tokens x 256 rows/columns of the
 // weight operand, wave tile 128 x 128 = 16 accumulator tiles of v_mfma_f32_32x32x16_bf16 (256 AGPRs).  The token
 // operand (x, or H) goes through LDS in fragment order, double-buffered, 64 K values per stage; the weight operand is
-// read straight from its packed fragment stream through a register ring refilled one stage ahead.  One LDS-only barrier
-// per stage (64 MFMAs per wave).
+// read straight from its packed fragment stream through a register ring refilled one stage ahead.  One LDS-only
+// barrier per stage (64 MFMAs per wave).
 //
 // The up product is computed transposed so that each lane ends up with ONE token and 16 hidden units per tile; the 8
 // values of accumulator rows r = 8k .. 8k+7 are exactly one A fragment of the down product (32 tokens x 16 hidden
-// units, k order: slot (g, i) <-> hidden 16*kstep + 8*(i/4) + 4g + i%4, baked into the packed Wd fragments).  H is
+// units, k order: slot (g, i) <-> hidden 16*kstep + 8*(i/4) + 4g + i%4, baked into the packed W2 fragments).  H is
 // therefore written as 1 KB fragments, fully coalesced, and staged into LDS by the down product with straight copies.
 #include "mfma_common.hpp"
 
@@ -31,22 +34,24 @@ constexpr int GM_MAX_SPLIT = 8;
 
 struct GemmLayout {
   int edp;   // neurons per expert padded to a multiple of 32: every 32-row MFMA tile belongs to one expert
-  int hp;    // padded hidden size, a multiple of 128
-  size_t up_off, dn_off, total;
+  int hp;    // padded hidden size: a multiple of 128 (gated) or 256 (ungated), the hidden units one workgroup covers
+  size_t up_off, dn_off, b_off, total;
 };
 
 static GemmLayout gemm_layout(const d2dmoe_shape& sh) {
   GemmLayout L;
   L.edp = (sh.expert_dim + 31) / 32 * 32;
-  L.hp = (sh.n_experts * L.edp + 127) / 128 * 128;
+  const int quantum = sh.gated ? 128 : 256;
+  L.hp = (sh.n_experts * L.edp + quantum - 1) / quantum * quantum;
   L.up_off = 0;
-  L.dn_off = (size_t)L.hp * 2 * sh.d_model * 2;
-  L.total = (L.dn_off + (size_t)L.hp * sh.d_model * 2 + 255) / 256 * 256;
+  L.dn_off = (size_t)L.hp * (sh.gated ? 2 : 1) * sh.d_model * 2;
+  L.b_off = L.dn_off + (size_t)L.hp * sh.d_model * 2;
+  L.total = (L.b_off + (size_t)L.hp * 2 + 255) / 256 * 256;
   return L;
 }
 
 bool mfma_gemm_supported(const d2dmoe_shape& sh) {
-  return sh.dtype == D2DMOE_BF16 && sh.gated && sh.d_model % 256 == 0 && sh.d_model >= 256;
+  return sh.dtype == D2DMOE_BF16 && sh.d_model % 256 == 0 && sh.d_model >= 256;
 }
 
 size_t mfma_gemm_packed_bytes(const d2dmoe_shape& sh) { return mfma_gemm_supported(sh) ? gemm_layout(sh).total : 0; }
@@ -82,16 +87,20 @@ size_t mfma_gemm_workspace_bytes(const d2dmoe_shape& sh) {
 
 // ---------------------------------------------------------------------------------------------------
 // Packing (lane = 32 g + c).  KS = D/16, KS2 = HP/16; hidden index h = e*EdP + j, zero beyond Ed and beyond E.
-//   up stream   [hidden block HP/64][kstep KS][tile 4: gate 0,1, up 0,1][lane][8]   A fragment:
-//               row h = 64*block + 32*(tile%2) + c,  d = 16*kstep + 8g + i             value w[e][d][j]
+//   up stream   gated:   [hidden block HP/64][kstep KS][tile 4: gate 0,1, up 0,1][lane][8]   A fragment:
+//                        row h = 64*block + 32*(tile%2) + c,  d = 16*kstep + 8g + i            value w[e][d][j]
+//               ungated: [hidden block HP/128][kstep KS][tile 4][lane][8]:  row h = 128*block + 32*tile + c
 //   down stream [column block D/128][kstep2 KS2][tile 4][lane][8]                   B fragment:
 //               column = 128*block + 32*tile + c,  h = 16*kstep2 + 8*(i/4) + 4g + i%4   value w2[e][j][column]
+//   bias        [HP] bf16 (ungated; zeros when the experts have none)
 // ---------------------------------------------------------------------------------------------------
 __global__ void pack_gemm_kernel(const bf16_t* __restrict__ wg, const bf16_t* __restrict__ wu, const bf16_t* __restrict__ wd,
-                                 bf16_t* __restrict__ dup, bf16_t* __restrict__ ddn, int D, int E, int Ed, int edp, int hp) {
+                                 const bf16_t* __restrict__ b1, bf16_t* __restrict__ dup, bf16_t* __restrict__ ddn,
+                                 bf16_t* __restrict__ db, int D, int E, int Ed, int edp, int hp, int gated) {
   const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int KS = D / 16, KS2 = hp / 16;
-  const int64_t n_up = (int64_t)(hp / 64) * KS * 4 * 64;
+  const int hb = gated ? 64 : 128;   // hidden units per block of the up stream
+  const int64_t n_up = (int64_t)(hp / hb) * KS * 4 * 64;
   const int64_t n_dn = (int64_t)(D / 128) * KS2 * 4 * 64;
   if (p < n_up) {
     int64_t q = p;
@@ -100,9 +109,9 @@ __global__ void pack_gemm_kernel(const bf16_t* __restrict__ wg, const bf16_t* __
     const int ks = (int)(q % KS);
     const int blk = (int)(q / KS);
     const int g = lane >> 5, c = lane & 31;
-    const int h = 64 * blk + 32 * (tile & 1) + c;
+    const int h = gated ? (64 * blk + 32 * (tile & 1) + c) : (128 * blk + 32 * tile + c);
     const int e = h / edp, j = h % edp;
-    const bf16_t* src = (tile < 2) ? wg : wu;
+    const bf16_t* src = (gated && tile >= 2) ? wu : wg;
     const bool ok = e < E && j < Ed;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -124,17 +133,23 @@ __global__ void pack_gemm_kernel(const bf16_t* __restrict__ wg, const bf16_t* __
       const int e = h / edp, j = h % edp;
       ddn[pp * 8 + i] = (e < E && j < Ed) ? wd[((int64_t)e * Ed + j) * D + col] : (bf16_t)0;
     }
+  } else if (p < n_up + n_dn + hp) {
+    const int h = (int)(p - n_up - n_dn);
+    const int e = h / edp, j = h % edp;
+    db[h] = (b1 != nullptr && e < E && j < Ed) ? b1[(int64_t)e * Ed + j] : (bf16_t)0;
   }
 }
 
-hipError_t launch_gemm_pack(const d2dmoe_shape& sh, const void* w_gate, const void* w_down, const void* w_up,
+hipError_t launch_gemm_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                             void* packed_section, hipStream_t s) {
   const GemmLayout L = gemm_layout(sh);
   char* base = (char*)packed_section;
-  const int64_t n = (int64_t)(L.hp / 64) * (sh.d_model / 16) * 256 + (int64_t)(sh.d_model / 128) * (L.hp / 16) * 256;
-  hipLaunchKernelGGL(pack_gemm_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const bf16_t*)w_gate,
-                     (const bf16_t*)w_up, (const bf16_t*)w_down, (bf16_t*)(base + L.up_off), (bf16_t*)(base + L.dn_off),
-                     sh.d_model, sh.n_experts, sh.expert_dim, L.edp, L.hp);
+  const int hb = sh.gated ? 64 : 128;
+  const int64_t n = (int64_t)(L.hp / hb) * (sh.d_model / 16) * 256 + (int64_t)(sh.d_model / 128) * (L.hp / 16) * 256 + L.hp;
+  hipLaunchKernelGGL(pack_gemm_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const bf16_t*)w1,
+                     (const bf16_t*)w_up, (const bf16_t*)w2, (const bf16_t*)b1, (bf16_t*)(base + L.up_off),
+                     (bf16_t*)(base + L.dn_off), (bf16_t*)(base + L.b_off), sh.d_model, sh.n_experts, sh.expert_dim, L.edp,
+                     L.hp, sh.gated);
   return hipGetLastError();
 }
 
@@ -143,6 +158,7 @@ struct GemmArgs {
   const bf16_t* x;         // [N, D] rows of this pass
   const bf16_t* routing;   // [N, E]
   const bf16x8* w;         // packed weight stream of this product
+  const bf16_t* bias;      // [HP] first-layer bias (ungated)
   bf16x8* hfrag;           // [token tile N/32][kstep2 HP/16][lane] hidden activations as A fragments
   float* partial;          // [ksplit][N][D] float32 sums of the down product
   int N; int D; int E; int edp; int hp; int act;
@@ -155,7 +171,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // MODE 0: up product (weights = A operand, x = B operand through LDS); MODE 1: down product (H = A operand through
 // LDS, weights = B operand).
-template <int MODE, int ACT>
+template <int MODE, int ACT, bool GATED>
 __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16x8* lds0 = (bf16x8*)smem_raw;          // [8 token tiles][4 ksteps][64 lanes]
@@ -269,23 +285,37 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
   }
 
   if (MODE == 0) {
-    // weight tiles 0,1 = gate rows, 2,3 = up rows of the same 64 hidden units; lane = token c32 of token tile j
+    // gated: weight tiles 0,1 = gate rows, 2,3 = up rows of the same 64 hidden units; ungated: four tiles of 32 hidden
+    // units.  lane = token c32 of token tile j; accumulator row r = hidden unit 8*(r/4) + 4g + r%4 of the tile
+    constexpr int NH = GATED ? 2 : 4;          // hidden tiles per wave
+    constexpr int HW = GATED ? 64 : 128;       // hidden units per wave
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int tl = wn * 4 + j;
       const int64_t tok = (int64_t)tt * GM_BT + tl * 32 + c32;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int h0 = (nb * 2 + wm) * 64 + 32 * i;
+      for (int i = 0; i < NH; ++i) {
+        const int h0 = (nb * 2 + wm) * HW + 32 * i;
         const int e = h0 / A.edp;
         const bool live = tok < N && e < A.E;
         const float rw = live ? bf16_to_f32(A.routing[tok * A.E + e]) : 0.f;
         float hv[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float gv = (ACT >= 0) ? act_fn<ACT>(acc[i][j][r]) : apply_act(A.act, acc[i][j][r]);
-          const float v = gv * acc[2 + i][j][r] * rw;
-          hv[r] = (live && rw != 0.f) ? v : 0.f;
+        for (int q = 0; q < 4; ++q) {
+          float bq[4] = {0.f, 0.f, 0.f, 0.f};
+          if (!GATED) {
+            const uint2 bb = *(const uint2*)(A.bias + h0 + 8 * q + 4 * g);
+            bq[0] = __uint_as_float(bb.x << 16); bq[1] = __uint_as_float(bb.x & 0xffff0000u);
+            bq[2] = __uint_as_float(bb.y << 16); bq[3] = __uint_as_float(bb.y & 0xffff0000u);
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int r = 4 * q + u;
+            const float pre = GATED ? acc[i][j][r] : (acc[i][j][r] + bq[u]);
+            const float gv = (ACT >= 0) ? act_fn<ACT>(pre) : apply_act(A.act, pre);
+            const float v = (GATED ? gv * acc[2 + (i & 1)][j][r] : gv) * rw;
+            hv[r] = (live && rw != 0.f) ? v : 0.f;
+          }
         }
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
@@ -351,15 +381,15 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restric
   *(uint4*)(out + n * D + col) = o;
 }
 
-template <int ACT>
+template <int ACT, bool GATED>
 static hipError_t launch_gemm_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
                                   const void* last_bias, void* out, void* workspace, hipStream_t s) {
   const GemmLayout L = gemm_layout(sh);
   const GemmPlan P = gemm_plan(sh);
   const char* pk = (const char*)packed_section;
   const size_t lds = 2 * 8 * 4 * 64 * 16;
-  auto k_up = gated_gemm_kernel<0, ACT>;
-  auto k_dn = gated_gemm_kernel<1, -1>;
+  auto k_up = gated_gemm_kernel<0, ACT, GATED>;
+  auto k_dn = gated_gemm_kernel<1, -1, true>;
   hipError_t e = hipFuncSetAttribute((const void*)k_up, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   e = hipFuncSetAttribute((const void*)k_dn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -369,6 +399,7 @@ static hipError_t launch_gemm_act(const d2dmoe_shape& sh, const void* x, const v
     GemmArgs A;
     A.x = (const bf16_t*)x + t0 * sh.d_model;
     A.routing = (const bf16_t*)routing + t0 * sh.n_experts;
+    A.bias = (const bf16_t*)(pk + L.b_off);
     A.hfrag = (bf16x8*)workspace;
     A.partial = (float*)((char*)workspace + P.h_bytes);
     A.N = n; A.D = sh.d_model; A.E = sh.n_experts; A.edp = L.edp; A.hp = L.hp; A.act = sh.activation;
@@ -376,7 +407,7 @@ static hipError_t launch_gemm_act(const d2dmoe_shape& sh, const void* x, const v
     A.tpx = (A.n_ttiles + 7) / 8;
     A.ksplit = P.ksplit;
     A.w = (const bf16x8*)(pk + L.up_off);
-    hipLaunchKernelGGL(k_up, dim3((unsigned)(8 * A.tpx * (L.hp / 128))), dim3(256), lds, s, A);
+    hipLaunchKernelGGL(k_up, dim3((unsigned)(8 * A.tpx * (L.hp / (GATED ? 128 : 256)))), dim3(256), lds, s, A);
     A.w = (const bf16x8*)(pk + L.dn_off);
     hipLaunchKernelGGL(k_dn, dim3((unsigned)(8 * A.tpx * (sh.d_model / 256) * P.ksplit)), dim3(256), lds, s, A);
     const int64_t items = (int64_t)n * (sh.d_model / 8);
@@ -389,15 +420,22 @@ static hipError_t launch_gemm_act(const d2dmoe_shape& sh, const void* x, const v
   return hipSuccess;
 }
 
+template <bool GATED>
+static hipError_t launch_gemm_gated(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
+                                    const void* last_bias, void* out, void* workspace, hipStream_t s) {
+  switch (sh.activation) {
+    case D2DMOE_ACT_RELU: return launch_gemm_act<D2DMOE_ACT_RELU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_GELU: return launch_gemm_act<D2DMOE_ACT_GELU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_GELU_TANH: return launch_gemm_act<D2DMOE_ACT_GELU_TANH, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_SILU: return launch_gemm_act<D2DMOE_ACT_SILU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    default: return launch_gemm_act<-1, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+  }
+}
+
 hipError_t launch_mfma_gemm(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
                             const void* last_bias, void* out, void* workspace, hipStream_t s) {
-  switch (sh.activation) {
-    case D2DMOE_ACT_RELU: return launch_gemm_act<D2DMOE_ACT_RELU>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    case D2DMOE_ACT_GELU: return launch_gemm_act<D2DMOE_ACT_GELU>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    case D2DMOE_ACT_GELU_TANH: return launch_gemm_act<D2DMOE_ACT_GELU_TANH>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    case D2DMOE_ACT_SILU: return launch_gemm_act<D2DMOE_ACT_SILU>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    default: return launch_gemm_act<-1>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-  }
+  if (sh.gated) return launch_gemm_gated<true>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+  return launch_gemm_gated<false>(sh, x, routing, packed_section, last_bias, out, workspace, s);
 }
 
 }  // namespace d2dmoe

@@ -191,7 +191,7 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
     if (e != hipSuccess) return e;
   }
   if (L.has_gemm) {
-    hipError_t e = launch_gemm_pack(sh, w1, w2, w_up, base + L.gm_off, s);
+    hipError_t e = launch_gemm_pack(sh, w1, b1, w2, w_up, base + L.gm_off, s);
     if (e != hipSuccess) return e;
   }
   if (!L.has_dense) return hipGetLastError();

@@ -61,12 +61,12 @@ hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void*
 size_t mfma_decode_section_offset(const d2dmoe_shape& sh);
 bool linear_skinny_supported(int64_t N, int K, int dtype);
 hipError_t launch_linear_skinny(const void* A, const void* B, void* C, int N, int K, int Nout, int act, hipStream_t s);
-// ---- large-batch gated path: two tiled bf16 MFMA products (kernels_gemm.hip) ----
+// ---- two tiled bf16 MFMA products with the hidden activations in the workspace (kernels_gemm.hip) ----
 bool mfma_gemm_supported(const d2dmoe_shape& sh);
 size_t mfma_gemm_packed_bytes(const d2dmoe_shape& sh);
 size_t mfma_gemm_workspace_bytes(const d2dmoe_shape& sh);
 size_t mfma_gemm_section_offset(const d2dmoe_shape& sh);
-hipError_t launch_gemm_pack(const d2dmoe_shape& sh, const void* w_gate, const void* w_down, const void* w_up,
+hipError_t launch_gemm_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                             void* packed_section, hipStream_t s);
 hipError_t launch_mfma_gemm(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
                             const void* last_bias, void* out, void* workspace, hipStream_t s);
