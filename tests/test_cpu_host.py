@@ -86,6 +86,33 @@ def test_shape_struct_matches_header_and_argument_checks():
         abi.check(-6, 'x')
 
 
+def test_packed_and_workspace_sizes_follow_the_documented_layouts():
+    """Host-only size queries (no device is touched): packed sections and workspace of the shapes the benchmarks use."""
+    from d2dmoe_amd import hip_abi as abi, ops
+    lib = abi.load()
+    lib.d2dmoe_packed_bytes.restype = ctypes.c_size_t
+    # Gemma-2B FFN: small-batch section (gate|up + down, 3 matrices + padded bias) + tiled-products section (3 matrices +
+    # bias) + router section
+    mat = 256 * 64 * 2048 * 2
+    g = ops.make_shape(4096, 2048, 256, 64, 256, abi.BF16, 'gelu_tanh', gated=True)
+    want = (3 * mat + 256 * 64 * 2) + (3 * mat + 256 * 64 * 2) + (256 * 2048 + 256 * 256) * 2
+    got = lib.d2dmoe_packed_bytes(ctypes.byref(g))
+    assert want <= got <= want + 4 * 256 and got % 256 == 0
+    # workspace at 4096 tokens: router hidden + norms, then H fragments (4096 x 16384 bf16) + 2 float32 partial sums
+    ws = lib.d2dmoe_workspace_bytes(ctypes.byref(g))
+    want_ws = 4096 * 256 * 2 * 2 + 4096 * 16384 * 2 + 2 * 4096 * 2048 * 4
+    assert want_ws <= ws <= want_ws + 4 * 256
+    # 16 tokens: the small-batch path needs the hidden fragments and one flag per expert only
+    g16 = ops.make_shape(16, 2048, 256, 64, 256, abi.BF16, 'gelu_tanh', gated=True)
+    assert lib.d2dmoe_workspace_bytes(ctypes.byref(g16)) < 2 << 20
+    # float32 layers have no packed form
+    f = ops.make_shape(100, 768, 128, 24, 128, abi.F32)
+    assert lib.d2dmoe_packed_bytes(ctypes.byref(f)) == 0
+    # ViT-B shape: dense-sweep stream (4 waves x 12 chunks x 192 fragments of 1 KB) is part of the buffer
+    v = ops.make_shape(50432, 768, 128, 24, 128, abi.BF16)
+    assert lib.d2dmoe_packed_bytes(ctypes.byref(v)) >= 4 * 12 * 192 * 1024
+
+
 # ------------------------------------------------------------------ host-side module mirror -------------
 def _toy_layer(act=nn.ReLU, experts_class='hip_kernel'):
     from d2dmoe_amd import MoeficationMoE, MoeficationRouter
