@@ -641,7 +641,7 @@ hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* 
 // A lane ends up with one token and 4 consecutive experts per accumulator quad, stored as 8-byte pieces.
 // Optional outputs: the norms, and per-expert token counts (wave ballots + one integer atomic per expert).
 // ---------------------------------------------------------------------------------------------------
-template <int WT, int ET>
+template <int WT, int ET, int U>
 __global__ __launch_bounds__(256) void router_select_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16x8* __restrict__ w1f, const bf16x8* __restrict__ w2f,
     bf16_t* __restrict__ routing, bf16_t* __restrict__ norms_out, int32_t* __restrict__ counts, int64_t N, int D,
@@ -661,17 +661,29 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
   for (int a = 0; a < WT; ++a)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc1[a][r] = 0.f;
-  for (int ks0 = 0; ks0 < KS1; ks0 += 4) {
-    bf16x8 b[4];   // four K steps of x fetched together
+  // two register buffers of U K steps each (x rows and W1 fragments): one is multiplied while the other fills;
+  // KS1 is a multiple of 2*U (the launcher picks U that way)
+  bf16x8 xA[U], wA[U][WT], xB[U], wB[U][WT];
+  auto fill = [&](bf16x8 (&xb)[U], bf16x8 (&wr)[U][WT], int ks0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) b[i] = xrow[2 * (ks0 + i) + g];
+    for (int u = 0; u < U; ++u) {
+      xb[u] = xrow[2 * (ks0 + u) + g];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+      for (int rt = 0; rt < WT; ++rt) wr[u][rt] = w1f[(int64_t)((ks0 + u) * WT + rt) * 64 + lane];
+    }
+  };
+  auto multiply = [&](bf16x8 (&xb)[U], bf16x8 (&wr)[U][WT]) __attribute__((always_inline)) {
 #pragma unroll
-      for (int rt = 0; rt < WT; ++rt) {
-        const bf16x8 a = w1f[(int64_t)((ks0 + i) * WT + rt) * 64 + lane];
-        acc1[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[i], acc1[rt], 0, 0, 0);
-      }
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int rt = 0; rt < WT; ++rt) acc1[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wr[u][rt], xb[u], acc1[rt], 0, 0, 0);
+  };
+  fill(xA, wA, 0);
+  for (int ks0 = 0; ks0 < KS1; ks0 += 2 * U) {
+    fill(xB, wB, ks0 + U);
+    multiply(xA, wA);
+    fill(xA, wA, (ks0 + 2 * U < KS1) ? (ks0 + 2 * U) : ks0);   // the last trip re-reads its own steps: in bounds, unused
+    multiply(xB, wB);
   }
   // hidden activations as B fragments of the second product
   bf16x8 hb[2 * WT];
@@ -914,12 +926,17 @@ hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, cons
     return hipGetLastError();
   }
   const unsigned grid = (unsigned)cdiv64(sh.n_tokens, 128);
-  if (sh.router_width == 128)
-    hipLaunchKernelGGL((router_select_mfma_kernel<4, 4>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+  if (sh.router_width == 128) {
+    if ((sh.d_model / 16) % 8 == 0)
+      hipLaunchKernelGGL((router_select_mfma_kernel<4, 4, 4>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+                         (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+    else
+      hipLaunchKernelGGL((router_select_mfma_kernel<4, 4, 2>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+                         (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+  } else {
+    hipLaunchKernelGGL((router_select_mfma_kernel<8, 8, 2>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
                        (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
-  else
-    hipLaunchKernelGGL((router_select_mfma_kernel<8, 8>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
-                       (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+  }
   return hipGetLastError();
 }
 
