@@ -614,3 +614,51 @@ def test_gpt_with_hip_moe_layers(shape, dtype):
     frac = gating[names[-1]][0].float().mean().item()
     assert out.shape == (4, cfg.block_size, cfg.vocab_size) and 0.0 < frac < 1.0
     assert torch.isfinite(out.float()).all()
+
+
+# =================================================================== HIP graph capture ================
+@pytest.mark.parametrize('case', ['vit_dense', 'vit_sparse', 'gemma_decode', 'gemma_tiled'])
+def test_layer_replays_from_a_hip_graph(case):
+    """The whole layer captured into a HIP graph (no allocation, memset or host sync inside the C ABI calls) and
+    replayed on new inputs, with eager work and synchronisations between the replays: every replay equals eager."""
+    _say('graph', case)
+    if case.startswith('vit'):
+        N, D, E, Ed, W, act, gated, tau = 300, 768, 128, 24, 128, 'relu', False, (0.9 if case == 'vit_dense' else 0.1)
+    elif case == 'gemma_decode':
+        N, D, E, Ed, W, act, gated, tau = 16, 2048, 256, 64, 256, 'gelu_tanh', True, 0.9
+    else:
+        N, D, E, Ed, W, act, gated, tau = 300, 2048, 256, 64, 256, 'gelu_tanh', True, 0.9
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=11, dtype=torch.bfloat16, gated=gated, bias=not gated)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, W, 1, act, gated=gated)
+    if gated:
+        packed = _ops().pack_weights(sh, d['w_gate'], None, d['w_down'], d['w_up'], d['router_w1'], d['router_w2'])
+        args = (d['w_gate'], None, d['w_down'], d['w_up'], None)
+    else:
+        packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, d['router_w1'], d['router_w2'])
+        args = (d['w1'], d['b1'], d['w2'], None, d['last_bias'].view(-1))
+
+    def layer(inp):
+        return _ops().forward(inp, d['router_w1'], d['router_w2'], float(1.0 - tau), *args, act, False, None, False, True,
+                              'auto', packed)
+
+    static_x = x.to(DEV).clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            layer(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_out, g_routing, _, g_counts = layer(static_x)
+    for rep in range(3):
+        new_x = (torch.randn(N, D, generator=torch.Generator().manual_seed(100 + rep)) * (1.0 + rep)).bfloat16().to(DEV)
+        want_out, want_routing, _, want_counts = layer(new_x)       # eager work between the replays
+        torch.cuda.synchronize()
+        static_x.copy_(new_x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_routing, want_routing) and torch.equal(g_counts, want_counts), (case, rep)
+        assert torch.equal(g_out, want_out), (case, rep)
