@@ -121,6 +121,11 @@ class MoeficationMoE(MoELayer):
         self.k = None
         self.tau = None
         self.add_residual_connection = add_residual_connection
+        # Cost accounting (the reference sums (routing > 0) over the dense routing tensor on the host side of every
+        # batch, eval.py:176-177): with collect_counts set, the fused HIP call also returns the per-expert number of
+        # routed tokens from its own device-side counters; it stays on the device, nothing synchronises.
+        self.collect_counts = False
+        self.last_expert_counts: Optional[torch.Tensor] = None
 
     # ------------------------------------------------------------------------------ gating
     def gate(self, x):
@@ -177,11 +182,12 @@ class MoeficationMoE(MoELayer):
                 rw1, rw2 = router.layers[0].weight, router.layers[2].weight
             ract = router.activation if router.activation in ACT else 'relu'
             roact = router.output_activation if router.output_activation in ACT else 'abs'
-            out, routing, _, _ = ops.forward(
+            out, routing, _, counts = ops.forward(
                 x2, rw1, rw2, float(1.0 - self.tau), ex.w1, ex.b1, ex.w2, None, last_bias, ex.activation_str,
-                self.add_residual_connection, norms_in=norms_in, path=ex.kernel_path,
+                self.add_residual_connection, norms_in=norms_in, want_counts=self.collect_counts, path=ex.kernel_path,
                 packed=ex.packed_weights(rw1, rw2, ract, roact), router_activation=ract, router_output_activation=roact)
             routing_tensor = routing.view(*orig_size[:-1], self.num_experts)
+            self.last_expert_counts = counts
             return out.view(orig_size), {self.name: (routing_tensor,)}
         routing_tensor = self.gate(x)
         x2 = x.reshape(-1, x.size(-1))

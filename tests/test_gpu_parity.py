@@ -613,6 +613,12 @@ def test_gpt_with_hip_moe_layers(shape, dtype):
             torch.cuda.set_sync_debug_mode('default')
     frac = gating[names[-1]][0].float().mean().item()
     assert out.shape == (4, cfg.block_size, cfg.vocab_size) and 0.0 < frac < 1.0
+    # cost accounting: executed (token, expert) pairs per layer from the kernel's own counters
+    last = gpt2.get_module_by_name(moe, names[-1])
+    last.collect_counts = True
+    with torch.no_grad():
+        _, gating = moe(idx, return_gating_data=True)
+    assert torch.equal(last.last_expert_counts.long().cpu(), (gating[names[-1]][0] > 0).long().sum((0, 1)).cpu())
     assert torch.isfinite(out.float()).all()
 
 
