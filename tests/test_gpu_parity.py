@@ -668,3 +668,40 @@ def test_layer_replays_from_a_hip_graph(case):
         torch.cuda.synchronize()
         assert torch.equal(g_routing, want_routing) and torch.equal(g_counts, want_counts), (case, rep)
         assert torch.equal(g_out, want_out), (case, rep)
+
+
+# =================================================================== argument checks on real device pointers ==========
+def test_entry_points_reject_bad_workspace_alignment_and_paths():
+    """Status codes instead of launches: workspace too small or misaligned, tensor pointer off by 2 bytes, a path the
+    shape has no kernel for, packed buffer missing for an MFMA path."""
+    import ctypes
+    from d2dmoe_amd import hip_abi as abi
+    ops = _ops()
+    lib = abi.load()
+    N, D, E, Ed = 64, 768, 128, 24
+    x, routing, p = H.random_case(N, D, E, Ed, 128, seed=3, dtype=torch.bfloat16)
+    d = H.to_dev(p, DEV)
+    xg, rg = x.to(DEV), routing.to(DEV)
+    out = torch.empty_like(xg)
+    sh = ops.make_shape(N, D, E, Ed, 0, abi.BF16)
+    packed = ops.pack_weights(sh, d['w1'], d['b1'], d['w2'], None, None, None)
+    need = lib.d2dmoe_workspace_bytes(ctypes.byref(sh))
+    ws = torch.empty(need + 512, dtype=torch.uint8, device=DEV)
+    base = ws.data_ptr() + (-ws.data_ptr()) % 256
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call(xp=xg.data_ptr(), path='mfma_sparse', wsp=base, wsb=need, pk=packed.data_ptr(), shape=sh):
+        return lib.d2dmoe_experts(ctypes.byref(shape), xp, rg.data_ptr(), d['w1'].data_ptr(), d['b1'].data_ptr(),
+                                  d['w2'].data_ptr(), None, None, pk, out.data_ptr(), abi.PATH[path], wsp, wsb, stream)
+
+    assert call() == 0
+    assert call(wsb=1024) == -5                  # workspace too small for the expert-major plan
+    assert call(wsp=base + 16) == -5             # workspace not 256-byte aligned
+    assert call(xp=xg.data_ptr() + 2) == -7      # x not 16-byte aligned
+    assert call(pk=None, path='mfma_dense') == -1
+    assert call(path='mfma_decode') == -6        # more than 16 tokens
+    f32 = ops.make_shape(N, D, E, Ed, 0, abi.F32)
+    assert call(shape=f32, path='mfma_dense') == -6
+    torch.cuda.synchronize()
+    # the call that went through left a correct result behind
+    assert H.rel_err(out.cpu(), _experts_want(x, routing, {k: v for k, v in p.items() if k != 'last_bias'}, 'relu')) < H.TOL_BF16
