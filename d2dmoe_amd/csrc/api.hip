@@ -43,6 +43,8 @@ ForwardWorkspace plan_workspace(const d2dmoe_shape& sh) {
   if (sparse > scratch) scratch = sparse;
   const size_t decode = mfma_decode_workspace_bytes(sh);   // per-expert result rows of the small-batch path
   if (decode > scratch) scratch = decode;
+  const size_t dsplit = mfma_dense_workspace_bytes(sh);    // float32 sums of the chunk-split dense sweep (few tokens)
+  if (dsplit > scratch) scratch = dsplit;
   const size_t gemm = (sh.n_tokens > 16) ? mfma_gemm_workspace_bytes(sh) : 0;   // H fragments + partial sums of the gated path
   if (gemm > scratch) scratch = gemm;
   w.perm_off = off;   off += align_up(scratch);
@@ -193,7 +195,7 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
     case D2DMOE_PATH_MFMA_DENSE: {
       if (!mfma_dense_supported(sh)) return D2DMOE_E_UNSUPPORTED;
       if (!packed) return D2DMOE_E_NULL;
-      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, nullptr, s);
+      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, nullptr, workspace, workspace_bytes, s);
     }
     case D2DMOE_PATH_MFMA_SPARSE: {
       // expert-major when the routed pairs fit the provisioned capacity, else the dense sweep: decided on the device
@@ -204,7 +206,7 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
       const int* flag = nullptr;
       hipError_t e = launch_mfma_sparse(sh, x, routing, packed, last_bias, out, workspace, 8, &flag, s);
       if (e != hipSuccess) return (int)e;
-      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, s);
+      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, nullptr, 0, s);
     }
     case D2DMOE_PATH_MFMA_DECODE: {
       if (!mfma_decode_supported(sh) || sh.n_tokens > 16) return D2DMOE_E_UNSUPPORTED;

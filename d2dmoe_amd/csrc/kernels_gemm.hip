@@ -381,6 +381,14 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restric
   *(uint4*)(out + n * D + col) = o;
 }
 
+hipError_t launch_sum_partials(const float* partial, const void* last_bias, const void* x, void* out, int64_t N, int D,
+                               int n_splits, int add_residual, hipStream_t s) {
+  const int64_t items = N * (D / 8);
+  hipLaunchKernelGGL(gemm_finish_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, partial, (const bf16_t*)last_bias,
+                     (const bf16_t*)x, (bf16_t*)out, N, D, n_splits, add_residual);
+  return hipGetLastError();
+}
+
 template <int ACT, bool GATED>
 static hipError_t launch_gemm_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
                                   const void* last_bias, void* out, void* workspace, hipStream_t s) {

@@ -227,11 +227,16 @@ struct DenseArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* wp; const bf16_t* b1p; const uint8_t* eidx;
   const bf16_t* last_bias; bf16_t* out;
   const int* skip_flag;   // optional device flag: non-zero = the expert-major path handles this call
+  float* partial;         // [csplit][N][D] float32 sums of the chunk-split variant
+  int csplit; int chunks_per_split;
   int64_t N; int E; int expert_dim; int n_chunks; int hidden; int act_rt; int add_residual; int n_full; int n_tiles;
 };
 
-template <int D, int ACT, bool ED8, int TT>
-__device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw) {
+// SPLIT: the workgroup handles only chunks [c_begin, c_end) of its tile and leaves its float32 sums, without bias or
+// residual, in A.partial[split]; a finishing kernel adds the splits in ascending order.
+template <int D, int ACT, bool ED8, int TT, bool SPLIT = false>
+__device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw,
+                                           const int c_begin = 0, const int c_end = 1 << 30, const int split = 0) {
   constexpr int KS1 = D / 16;          // K steps of GEMM1
   constexpr int CT = D / 128;          // 32-wide column tiles per wave in GEMM2
   const int E = A.E, n_chunks = A.n_chunks;
@@ -262,8 +267,9 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   // first active chunk turns out to be another one the ring is reloaded below.
   const bf16x8* wbase = A.wp + (int64_t)w * n_chunks * PIECES * 64 + lane;   // this wave's stream
   bf16x8 ring[R];
+  const int first_guess = SPLIT ? c_begin : 0;
 #pragma unroll
-  for (int i = 0; i < R; ++i) ring[i] = wbase[i * 64];
+  for (int i = 0; i < R; ++i) ring[i] = wbase[((int64_t)first_guess * PIECES + i) * 64];
 
   // ---- stage x (as B fragments), routing, bias and expert-index tables; all loads of a kind are issued together
   {
@@ -323,7 +329,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   if (t == 0) {
     int n_act = 0;
     for (int ch = 0; ch < n_chunks; ++ch)
-      if (cact[ch]) clist[n_act++] = ch;
+      if (cact[ch] && (!SPLIT || (ch >= c_begin && ch < c_end))) clist[n_act++] = ch;
     *n_act_p = n_act;
   }
   __syncthreads();
@@ -340,7 +346,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   if (n_act > 0) {
     f32x16 acc1[2][TT];   // GEMM1 accumulators [row-tile][token tile]
     const bf16x8* cur = wbase + (int64_t)clist[0] * PIECES * 64;
-    if (clist[0] != 0) {
+    if (clist[0] != first_guess) {
 #pragma unroll
       for (int i = 0; i < R; ++i) ring[i] = cur[i * 64];
     }
@@ -518,6 +524,12 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
           const float4 v1 = *(const float4*)(ot + m * OS + c8 + 4);
           float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
           const int col = pass * HALF + c8;
+          if constexpr (SPLIT) {
+            float* prow = A.partial + ((int64_t)split * N + n) * D + col;
+            *(float4*)prow = v0;
+            *(float4*)(prow + 4) = v1;
+            continue;
+          }
           if (A.last_bias != nullptr) {
             const uint4 lb = *(const uint4*)(A.last_bias + col);
             const uint32_t lw[4] = {lb.x, lb.y, lb.z, lb.w};
@@ -562,6 +574,18 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_dense_walk_kernel(const D
   }
 }
 
+// Few tokens: the tiles alone would leave most CUs idle, so each tile's chunks are dealt to csplit workgroups.
+template <int D, int ACT, bool ED8>
+__global__ __launch_bounds__(256, 1) void experts_mfma_dense_split_kernel(const DenseArgs A) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  const int b = blockIdx.x / A.csplit, split = blockIdx.x % A.csplit;
+  const int c_begin = split * A.chunks_per_split, c_end = c_begin + A.chunks_per_split;
+  if (b < A.n_full)
+    dense_tile<D, ACT, ED8, 2, true>(A, (int64_t)b * 64, smem_raw, c_begin, c_end, split);
+  else
+    dense_tile<D, ACT, ED8, 1, true>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw, c_begin, c_end, split);
+}
+
 template <int D, int ACT, bool ED8>
 __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -583,32 +607,71 @@ int device_cu_count() {
   return n;
 }
 
+struct DenseTiling {
+  int64_t n_full, n_half;   // tiles of 64 and of 32 tokens
+  int csplit, per;          // workgroups per tile and chunks per workgroup (1, n_chunks when the tiles fill the machine)
+};
+
+// Tiles of 64 tokens fill whole rounds of one workgroup per CU; when the last round would be at most half full its
+// tokens go to tiles of 32 instead (twice the workgroups, half the time each).  When even those leave at least half of
+// the CUs without a tile, every tile's chunks are dealt to several workgroups.
+static DenseTiling dense_tiling(const d2dmoe_shape& sh) {
+  const int cus = device_cu_count();
+  const int n_chunks = (sh.n_experts * sh.expert_dim + MD_HC - 1) / MD_HC;
+  DenseTiling T;
+  const int64_t t64 = cdiv64(sh.n_tokens, 64);
+  const int64_t leftover = t64 % cus;
+  T.n_full = t64; T.n_half = 0;
+  if (leftover > 0 && leftover * 2 <= cus) {
+    T.n_full = t64 - leftover;
+    T.n_half = cdiv64(sh.n_tokens - T.n_full * 64, 32);
+  }
+  T.csplit = 1; T.per = n_chunks;
+  const int64_t tiles = T.n_full + T.n_half;
+  if (tiles > 0 && tiles * 2 <= cus && n_chunks >= 2) {
+    int cs = (int)(cus / tiles);
+    if (cs > n_chunks) cs = n_chunks;
+    T.per = (n_chunks + cs - 1) / cs;
+    T.csplit = (n_chunks + T.per - 1) / T.per;
+  }
+  return T;
+}
+
+size_t mfma_dense_workspace_bytes(const d2dmoe_shape& sh) {
+  if (!mfma_dense_supported(sh) || sh.n_tokens <= 0) return 0;
+  const DenseTiling T = dense_tiling(sh);
+  return T.csplit > 1 ? (size_t)T.csplit * sh.n_tokens * sh.d_model * 4 : 0;
+}
+
 template <int D, int ACT, bool ED8>
 static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
-                                   const void* last_bias, void* out, const int* skip_flag, hipStream_t s) {
+                                   const void* last_bias, void* out, const int* skip_flag, void* workspace,
+                                   size_t workspace_bytes, hipStream_t s) {
   const PackedLayout L = packed_layout(sh);
   const char* base = (const char*)packed;
   const size_t lds = dense_lds_bytes(sh);
   if (lds > 160 * 1024) return hipErrorInvalidValue;
-  auto kern = (skip_flag != nullptr) ? experts_mfma_dense_walk_kernel<D, ACT, ED8> : experts_mfma_dense_kernel<D, ACT, ED8>;
+  const int cus = device_cu_count();
+  const DenseTiling T = dense_tiling(sh);
+  const bool split = T.csplit > 1 && skip_flag == nullptr && workspace != nullptr &&
+                     workspace_bytes >= mfma_dense_workspace_bytes(sh);
+  auto kern = split ? experts_mfma_dense_split_kernel<D, ACT, ED8>
+                    : ((skip_flag != nullptr) ? experts_mfma_dense_walk_kernel<D, ACT, ED8> : experts_mfma_dense_kernel<D, ACT, ED8>);
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
-  // Tiles of 64 tokens fill whole rounds of one workgroup per CU; when the last round would be at most half full its
-  // tokens go to tiles of 32 instead (twice the workgroups, half the time each).
-  const int cus = device_cu_count();
-  const int64_t t64 = cdiv64(sh.n_tokens, 64);
-  const int64_t leftover = t64 % cus;
-  int64_t n_full = t64, n_half = 0;
-  if (leftover > 0 && leftover * 2 <= cus) {
-    n_full = t64 - leftover;
-    n_half = cdiv64(sh.n_tokens - n_full * 64, 32);
-  }
   DenseArgs A;
   A.x = (const bf16_t*)x; A.routing = (const bf16_t*)routing; A.wp = (const bf16x8*)(base + L.w_off);
   A.b1p = (const bf16_t*)(base + L.b1_off); A.eidx = (const uint8_t*)(base + L.eidx_off);
   A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.N = sh.n_tokens; A.E = sh.n_experts; A.expert_dim = sh.expert_dim;
   A.n_chunks = L.n_chunks; A.hidden = L.hidden; A.act_rt = sh.activation; A.add_residual = sh.add_residual;
-  A.n_full = (int)n_full; A.n_tiles = (int)(n_full + n_half); A.skip_flag = skip_flag;
+  A.n_full = (int)T.n_full; A.n_tiles = (int)(T.n_full + T.n_half); A.skip_flag = skip_flag;
+  A.partial = (float*)workspace; A.csplit = split ? T.csplit : 1; A.chunks_per_split = T.per;
+  if (split) {
+    hipLaunchKernelGGL(kern, dim3((unsigned)(A.n_tiles * T.csplit)), dim3(256), lds, s, A);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return launch_sum_partials(A.partial, last_bias, x, out, sh.n_tokens, sh.d_model, T.csplit, sh.add_residual, s);
+  }
   const int64_t grid = (skip_flag != nullptr && A.n_tiles > cus) ? cus : A.n_tiles;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, s, A);
   return hipGetLastError();
@@ -616,17 +679,23 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
 
 template <int D, int ACT>
 static hipError_t launch_dense_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
-                                   const void* last_bias, void* out, const int* skip_flag, hipStream_t s) {
-  if (sh.expert_dim % 8 == 0) return launch_dense_cfg<D, ACT, true>(sh, x, routing, packed, last_bias, out, skip_flag, s);
-  return launch_dense_cfg<D, ACT, false>(sh, x, routing, packed, last_bias, out, skip_flag, s);
+                                   const void* last_bias, void* out, const int* skip_flag, void* workspace,
+                                   size_t workspace_bytes, hipStream_t s) {
+  if (sh.expert_dim % 8 == 0)
+    return launch_dense_cfg<D, ACT, true>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+  return launch_dense_cfg<D, ACT, false>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
 }
 
 hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
-                             const void* last_bias, void* out, const int* skip_flag, hipStream_t s) {
+                             const void* last_bias, void* out, const int* skip_flag, void* workspace, size_t workspace_bytes,
+                             hipStream_t s) {
   switch (sh.activation) {
-    case D2DMOE_ACT_RELU: return launch_dense_act<768, D2DMOE_ACT_RELU>(sh, x, routing, packed, last_bias, out, skip_flag, s);
-    case D2DMOE_ACT_GELU: return launch_dense_act<768, D2DMOE_ACT_GELU>(sh, x, routing, packed, last_bias, out, skip_flag, s);
-    default: return launch_dense_act<768, -1>(sh, x, routing, packed, last_bias, out, skip_flag, s);
+    case D2DMOE_ACT_RELU:
+      return launch_dense_act<768, D2DMOE_ACT_RELU>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+    case D2DMOE_ACT_GELU:
+      return launch_dense_act<768, D2DMOE_ACT_GELU>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+    default:
+      return launch_dense_act<768, -1>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
   }
 }
 

@@ -41,8 +41,15 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
                             const void* router_w1, const void* router_w2, void* packed, hipStream_t s);
 hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
                                      void* norms_out, int32_t* counts, float thr_scale, hipStream_t s);
+// With few tokens the sweep deals each tile's chunks to several workgroups and needs mfma_dense_workspace_bytes() of
+// workspace for their float32 sums (without it, or with skip_flag, it runs one workgroup per tile).
+size_t mfma_dense_workspace_bytes(const d2dmoe_shape& sh);
 hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
-                             const void* last_bias, void* out, const int* skip_flag, hipStream_t s);
+                             const void* last_bias, void* out, const int* skip_flag, void* workspace, size_t workspace_bytes,
+                             hipStream_t s);
+// out = round(sum over splits (ascending) of partial[split] + last_bias (+ x)); partial is [n_splits][N][D] float32
+hipError_t launch_sum_partials(const float* partial, const void* last_bias, const void* x, void* out, int64_t N, int D,
+                               int n_splits, int add_residual, hipStream_t s);
 
 // ---- bf16 MFMA expert-major path (kernels_sparse.hip) ----
 bool mfma_sparse_supported(const d2dmoe_shape& sh);
