@@ -227,8 +227,8 @@ struct DenseArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* wp; const bf16_t* b1p; const uint8_t* eidx;
   const bf16_t* last_bias; bf16_t* out;
   const int* skip_flag;   // optional device flag: non-zero = the expert-major path handles this call
-  float* partial;         // [csplit][N][D] float32 sums of the chunk-split variant
-  int csplit; int chunks_per_split;
+  float* partial;         // [csplit][part_rows][D] float32 sums of the chunk-split tiles (tokens from part_base on)
+  int csplit; int chunks_per_split; int64_t part_base; int64_t part_rows;
   int64_t N; int E; int expert_dim; int n_chunks; int hidden; int act_rt; int add_residual; int n_full; int n_tiles;
 };
 
@@ -525,7 +525,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
           float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
           const int col = pass * HALF + c8;
           if constexpr (SPLIT) {
-            float* prow = A.partial + ((int64_t)split * N + n) * D + col;
+            float* prow = A.partial + ((int64_t)split * A.part_rows + (n - A.part_base)) * D + col;
             *(float4*)prow = v0;
             *(float4*)(prow + 4) = v1;
             continue;
@@ -574,27 +574,25 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_dense_walk_kernel(const D
   }
 }
 
-// Few tokens: the tiles alone would leave most CUs idle, so each tile's chunks are dealt to csplit workgroups.
-template <int D, int ACT, bool ED8>
-__global__ __launch_bounds__(256, 1) void experts_mfma_dense_split_kernel(const DenseArgs A) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  const int b = blockIdx.x / A.csplit, split = blockIdx.x % A.csplit;
-  const int c_begin = split * A.chunks_per_split, c_end = c_begin + A.chunks_per_split;
-  if (b < A.n_full)
-    dense_tile<D, ACT, ED8, 2, true>(A, (int64_t)b * 64, smem_raw, c_begin, c_end, split);
-  else
-    dense_tile<D, ACT, ED8, 1, true>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw, c_begin, c_end, split);
-}
-
+// Workgroups [0, n_full) take tiles of 64 tokens.  The tokens left over after the last full round of the machine go to
+// tiles of 32; if those would still leave most CUs idle, each of them is dealt to csplit workgroups by chunk ranges,
+// which leave float32 sums in A.partial for the finishing kernel.
 template <int D, int ACT, bool ED8>
 __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
   const int b = blockIdx.x;
-  if (b < A.n_full)
+  if (b < A.n_full) {
     dense_tile<D, ACT, ED8, 2>(A, (int64_t)b * 64, smem_raw);
-  else
+  } else if (A.csplit <= 1) {
     dense_tile<D, ACT, ED8, 1>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
+  } else {
+    const int idx = b - A.n_full;
+    const int tile = idx / A.csplit, split = idx % A.csplit;
+    const int c_begin = split * A.chunks_per_split;
+    dense_tile<D, ACT, ED8, 1, true>(A, (int64_t)A.n_full * 64 + (int64_t)tile * 32, smem_raw, c_begin,
+                                     c_begin + A.chunks_per_split, split);
+  }
 }
 
 int device_cu_count() {
@@ -609,38 +607,44 @@ int device_cu_count() {
 
 struct DenseTiling {
   int64_t n_full, n_half;   // tiles of 64 and of 32 tokens
-  int csplit, per;          // workgroups per tile and chunks per workgroup (1, n_chunks when the tiles fill the machine)
+  int csplit, per;          // workgroups per tile of 32 and chunks per workgroup (1, n_chunks: not split)
+  int64_t part_base, part_rows;   // tokens covered by split tiles
 };
 
-// Tiles of 64 tokens fill whole rounds of one workgroup per CU; when the last round would be at most half full its
-// tokens go to tiles of 32 instead (twice the workgroups, half the time each).  When even those leave at least half of
-// the CUs without a tile, every tile's chunks are dealt to several workgroups.
-static DenseTiling dense_tiling(const d2dmoe_shape& sh) {
+// Tiles of 64 tokens fill whole rounds of one workgroup per CU.  When the last round would be at most half full its
+// tokens go to tiles of 32 instead, and if those still leave CUs idle each of them is dealt to several workgroups by
+// chunk ranges -- so the tail of the launch (or, with few tokens, the whole launch) spreads over the machine.
+static DenseTiling dense_tiling(const d2dmoe_shape& sh, bool allow_split) {
   const int cus = device_cu_count();
   const int n_chunks = (sh.n_experts * sh.expert_dim + MD_HC - 1) / MD_HC;
   DenseTiling T;
   const int64_t t64 = cdiv64(sh.n_tokens, 64);
   const int64_t leftover = t64 % cus;
   T.n_full = t64; T.n_half = 0;
+  T.csplit = 1; T.per = n_chunks; T.part_base = 0; T.part_rows = 0;
   if (leftover > 0 && leftover * 2 <= cus) {
     T.n_full = t64 - leftover;
     T.n_half = cdiv64(sh.n_tokens - T.n_full * 64, 32);
-  }
-  T.csplit = 1; T.per = n_chunks;
-  const int64_t tiles = T.n_full + T.n_half;
-  if (tiles > 0 && tiles * 2 <= cus && n_chunks >= 2) {
-    int cs = (int)(cus / tiles);
-    if (cs > n_chunks) cs = n_chunks;
-    T.per = (n_chunks + cs - 1) / cs;
-    T.csplit = (n_chunks + T.per - 1) / T.per;
+    if (allow_split && n_chunks >= 2 && T.n_half * 2 <= cus) {
+      int cs = (int)(cus / T.n_half);
+      if (cs > n_chunks) cs = n_chunks;
+      T.per = (n_chunks + cs - 1) / cs;
+      T.csplit = (n_chunks + T.per - 1) / T.per;
+      if (T.csplit > 1) {
+        T.part_base = T.n_full * 64;
+        T.part_rows = sh.n_tokens - T.part_base;
+      } else {
+        T.per = n_chunks;
+      }
+    }
   }
   return T;
 }
 
 size_t mfma_dense_workspace_bytes(const d2dmoe_shape& sh) {
   if (!mfma_dense_supported(sh) || sh.n_tokens <= 0) return 0;
-  const DenseTiling T = dense_tiling(sh);
-  return T.csplit > 1 ? (size_t)T.csplit * sh.n_tokens * sh.d_model * 4 : 0;
+  const DenseTiling T = dense_tiling(sh, true);
+  return T.csplit > 1 ? (size_t)T.csplit * T.part_rows * sh.d_model * 4 : 0;
 }
 
 template <int D, int ACT, bool ED8>
@@ -652,11 +656,9 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   const size_t lds = dense_lds_bytes(sh);
   if (lds > 160 * 1024) return hipErrorInvalidValue;
   const int cus = device_cu_count();
-  const DenseTiling T = dense_tiling(sh);
-  const bool split = T.csplit > 1 && skip_flag == nullptr && workspace != nullptr &&
-                     workspace_bytes >= mfma_dense_workspace_bytes(sh);
-  auto kern = split ? experts_mfma_dense_split_kernel<D, ACT, ED8>
-                    : ((skip_flag != nullptr) ? experts_mfma_dense_walk_kernel<D, ACT, ED8> : experts_mfma_dense_kernel<D, ACT, ED8>);
+  const bool allow_split = skip_flag == nullptr && workspace != nullptr && workspace_bytes >= mfma_dense_workspace_bytes(sh);
+  const DenseTiling T = dense_tiling(sh, allow_split);
+  auto kern = (skip_flag != nullptr) ? experts_mfma_dense_walk_kernel<D, ACT, ED8> : experts_mfma_dense_kernel<D, ACT, ED8>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   DenseArgs A;
@@ -665,16 +667,15 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.N = sh.n_tokens; A.E = sh.n_experts; A.expert_dim = sh.expert_dim;
   A.n_chunks = L.n_chunks; A.hidden = L.hidden; A.act_rt = sh.activation; A.add_residual = sh.add_residual;
   A.n_full = (int)T.n_full; A.n_tiles = (int)(T.n_full + T.n_half); A.skip_flag = skip_flag;
-  A.partial = (float*)workspace; A.csplit = split ? T.csplit : 1; A.chunks_per_split = T.per;
-  if (split) {
-    hipLaunchKernelGGL(kern, dim3((unsigned)(A.n_tiles * T.csplit)), dim3(256), lds, s, A);
-    e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    return launch_sum_partials(A.partial, last_bias, x, out, sh.n_tokens, sh.d_model, T.csplit, sh.add_residual, s);
-  }
-  const int64_t grid = (skip_flag != nullptr && A.n_tiles > cus) ? cus : A.n_tiles;
+  A.partial = (float*)workspace; A.csplit = T.csplit; A.chunks_per_split = T.per;
+  A.part_base = T.part_base; A.part_rows = T.part_rows;
+  int64_t grid = T.n_full + T.n_half * T.csplit;
+  if (skip_flag != nullptr && A.n_tiles > cus) grid = cus;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, s, A);
-  return hipGetLastError();
+  e = hipGetLastError();
+  if (e != hipSuccess || T.csplit <= 1) return e;
+  return launch_sum_partials(A.partial, last_bias, (const bf16_t*)x + T.part_base * sh.d_model,
+                             (bf16_t*)out + T.part_base * sh.d_model, T.part_rows, sh.d_model, T.csplit, sh.add_residual, s);
 }
 
 template <int D, int ACT>
