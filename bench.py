@@ -47,7 +47,7 @@ WORKLOADS = {
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (profiles/), scaled by
 # the factors a plain copy kernel of known size gives for the same counters (2.0 and 1.0); None = not measured
 MEASURED_TRAFFIC = {
-    'vit_b_50k': 472.8e6,     # experts_mfma_dense_kernel
+    'vit_b_50k': 468.0e6,     # experts_mfma_dense_kernel
     'gemma_16': 207.1e6,      # decode_hidden_kernel + decode_out_kernel
     'gemma_1': 163.7e6,
     'gemma_4096': 2169.8e6,   # up product + down product + finish
