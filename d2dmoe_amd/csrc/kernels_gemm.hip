@@ -1,5 +1,6 @@
-// Experts on bf16 MFMA as two tiled products with the hidden activations kept in memory between them.  Serves gated
-// experts (Gemma shape) at more than 16 tokens, and ungated experts whose width the fused sweep is not built for:
+// Experts on MFMA as two tiled products with the hidden activations kept in memory between them.  Serves gated experts
+// (Gemma shape) at more than 16 tokens, ungated experts whose width the fused sweep is not built for, and every
+// float32 layer (bf16 storage: v_mfma_f32_32x32x16_bf16; float32 storage: v_mfma_f32_32x32x2_f32, float32 throughout):
 //
 //   up    gated:   H^T[hidden, token] = act(Wg^T . X^T) * (Wu^T . X^T) * routing[token, expert(hidden)]
 //                  (ExecuteAllExperts with intermediate gating, moe_layers.py:71-78, 91-96)
@@ -15,15 +16,20 @@
 // (per K split), which is the ascending-expert order of the reference's merge kernel (moe_impls.py:485-514).
 //
 // One kernel template serves both products.  Workgroup = 4 waves (2 x 2), tile = 256 tokens x 256 rows/columns of the
-// weight operand, wave tile 128 x 128 = 16 accumulator tiles of v_mfma_f32_32x32x16_bf16 (256 AGPRs).  The token
-// operand (x, or H) goes through LDS in fragment order, double-buffered, 64 K values per stage; the weight operand is
-// read straight from its packed fragment stream through a register ring refilled one stage ahead.  One LDS-only
-// barrier per stage (64 MFMAs per wave).
+// weight operand, wave tile 128 x 128 = 16 accumulator tiles of 32 x 32 (256 AGPRs).  The token operand (x, or H) goes
+// through LDS in fragment order, double-buffered, four fragments of K per stage; the weight operand is read straight
+// from its packed fragment stream through a register ring refilled one stage ahead.  One LDS-only barrier per stage.
 //
-// The up product is computed transposed so that each lane ends up with ONE token and 16 hidden units per tile; the 8
-// values of accumulator rows r = 8k .. 8k+7 are exactly one A fragment of the down product (32 tokens x 16 hidden
-// units, k order: slot (g, i) <-> hidden 16*kstep + 8*(i/4) + 4g + i%4, baked into the packed W2 fragments).  H is
-// therefore written as 1 KB fragments, fully coalesced, and staged into LDS by the down product with straight copies.
+// A fragment is 64 lanes x 16 bytes: lane (c = lane % 32, g = lane / 32) holds row/column c and, in bf16, the 8 K values
+// 8g .. 8g+7 of a 16-wide K step (one MFMA); in float32 the 4 K values 4g .. 4g+3 of an 8-wide K group, consumed by four
+// MFMAs of K = 2 that pair value i of the g = 0 lanes with value i of the g = 1 lanes (any pairing is a valid order of
+// the K sum as long as both operands use it).  Byte for byte the two element types share every layout below.
+//
+// The up product is computed transposed so that each lane ends up with ONE token and 16 hidden units per tile, which
+// already is the A-fragment arrangement of the down product: in bf16 accumulator rows r = 8k .. 8k+7 form one fragment
+// (k order: slot (g, i) <-> hidden 16*kstep + 8*(i/4) + 4g + i%4, baked into the packed W2 fragments); in float32 rows
+// r = 4q .. 4q+3 form the fragment of K group q in natural order.  H is therefore written as 1 KB fragments, fully
+// coalesced, and staged into LDS by the down product with straight copies.
 #include "mfma_common.hpp"
 
 namespace d2dmoe {
@@ -32,26 +38,39 @@ constexpr int GM_BT = 256;         // tokens per workgroup tile
 constexpr int GM_SLAB = 8192;      // tokens per pass: bounds the workspace (H fragments + float32 partial sums)
 constexpr int GM_MAX_SPLIT = 8;
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+// Per element type: K values per fragment, elements per 16-byte piece.
+template <typename T> struct GemmElem;
+template <> struct GemmElem<bf16_t> { static constexpr int KPF = 16, EPP = 8; };
+template <> struct GemmElem<float> { static constexpr int KPF = 8, EPP = 4; };
+
+static inline int gemm_kpf(const d2dmoe_shape& sh) { return sh.dtype == D2DMOE_F32 ? 8 : 16; }
+static inline size_t gemm_esize(const d2dmoe_shape& sh) { return sh.dtype == D2DMOE_F32 ? 4 : 2; }
+
 struct GemmLayout {
-  int edp;   // neurons per expert padded to a multiple of 32: every 32-row MFMA tile belongs to one expert
+  int edp;   // neurons per expert in the hidden index space: Ed itself when it is a multiple of 4 (every group of 4
+             // accumulator rows then belongs to one expert), else Ed padded to a multiple of 32
   int hp;    // padded hidden size: a multiple of 128 (gated) or 256 (ungated), the hidden units one workgroup covers
   size_t up_off, dn_off, b_off, total;
 };
 
 static GemmLayout gemm_layout(const d2dmoe_shape& sh) {
   GemmLayout L;
-  L.edp = (sh.expert_dim + 31) / 32 * 32;
+  const size_t es = gemm_esize(sh);
+  L.edp = (sh.expert_dim % 4 == 0) ? sh.expert_dim : (sh.expert_dim + 31) / 32 * 32;
   const int quantum = sh.gated ? 128 : 256;
   L.hp = (sh.n_experts * L.edp + quantum - 1) / quantum * quantum;
   L.up_off = 0;
-  L.dn_off = (size_t)L.hp * (sh.gated ? 2 : 1) * sh.d_model * 2;
-  L.b_off = L.dn_off + (size_t)L.hp * sh.d_model * 2;
-  L.total = (L.b_off + (size_t)L.hp * 2 + 255) / 256 * 256;
+  L.dn_off = (size_t)L.hp * (sh.gated ? 2 : 1) * sh.d_model * es;
+  L.b_off = L.dn_off + (size_t)L.hp * sh.d_model * es;
+  L.total = (L.b_off + (size_t)L.hp * es + 255) / 256 * 256;
   return L;
 }
 
 bool mfma_gemm_supported(const d2dmoe_shape& sh) {
-  return sh.dtype == D2DMOE_BF16 && sh.d_model % 256 == 0 && sh.d_model >= 256;
+  return (sh.dtype == D2DMOE_BF16 || sh.dtype == D2DMOE_F32) && sh.d_model % 256 == 0 && sh.d_model >= 256;
 }
 
 size_t mfma_gemm_packed_bytes(const d2dmoe_shape& sh) { return mfma_gemm_supported(sh) ? gemm_layout(sh).total : 0; }
@@ -68,13 +87,13 @@ static GemmPlan gemm_plan(const d2dmoe_shape& sh) {
   GemmPlan P;
   P.slab = (int)(sh.n_tokens < GM_SLAB ? sh.n_tokens : GM_SLAB);
   P.n_ttiles = (P.slab + GM_BT - 1) / GM_BT;
-  // the down product has n_ttiles * D/256 tiles; split K until the machine is covered (the K steps of every split
+  // the down product has n_ttiles * D/256 tiles; split K until the machine is covered (the fragments of every split
   // must still be whole stages of 4)
   const int tiles = P.n_ttiles * (sh.d_model / 256);
-  const int ks2 = L.hp / 16;
+  const int ks2 = L.hp / gemm_kpf(sh);
   P.ksplit = 1;
   while (P.ksplit < GM_MAX_SPLIT && tiles * P.ksplit < device_cu_count() && (ks2 / (P.ksplit * 2)) % 4 == 0) P.ksplit *= 2;
-  P.h_bytes = ((size_t)P.n_ttiles * GM_BT * L.hp * 2 + 255) / 256 * 256;
+  P.h_bytes = ((size_t)P.n_ttiles * GM_BT * L.hp * gemm_esize(sh) + 255) / 256 * 256;
   P.partial_bytes = ((size_t)P.ksplit * P.slab * sh.d_model * 4 + 255) / 256 * 256;
   return P;
 }
@@ -86,19 +105,23 @@ size_t mfma_gemm_workspace_bytes(const d2dmoe_shape& sh) {
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Packing (lane = 32 g + c).  KS = D/16, KS2 = HP/16; hidden index h = e*EdP + j, zero beyond Ed and beyond E.
-//   up stream   gated:   [hidden block HP/64][kstep KS][tile 4: gate 0,1, up 0,1][lane][8]   A fragment:
-//                        row h = 64*block + 32*(tile%2) + c,  d = 16*kstep + 8g + i            value w[e][d][j]
-//               ungated: [hidden block HP/128][kstep KS][tile 4][lane][8]:  row h = 128*block + 32*tile + c
-//   down stream [column block D/128][kstep2 KS2][tile 4][lane][8]                   B fragment:
-//               column = 128*block + 32*tile + c,  h = 16*kstep2 + 8*(i/4) + 4g + i%4   value w2[e][j][column]
-//   bias        [HP] bf16 (ungated; zeros when the experts have none)
+// Packing (lane = 32 g + c).  KPF = K values per fragment (16 bf16 / 8 float32), EPP = elements per lane (8 / 4),
+// KS = D/KPF, KS2 = HP/KPF; hidden index h = e*EdP + j, zero beyond Ed and beyond E.
+//   up stream   gated:   [hidden block HP/64][fragment KS][tile 4: gate 0,1, up 0,1][lane][EPP]   A fragment:
+//                        row h = 64*block + 32*(tile%2) + c,  d = KPF*fragment + EPP*g + i          value w[e][d][j]
+//               ungated: [hidden block HP/128][fragment KS][tile 4][lane][EPP]:  row h = 128*block + 32*tile + c
+//   down stream [column block D/128][fragment KS2][tile 4][lane][EPP]                   B fragment:
+//               column = 128*block + 32*tile + c;  bf16: h = 16*fragment + 8*(i/4) + 4g + i%4,
+//               float32: h = 8*fragment + 4g + i                                         value w2[e][j][column]
+//   bias        [HP] (ungated; zeros when the experts have none)
 // ---------------------------------------------------------------------------------------------------
-__global__ void pack_gemm_kernel(const bf16_t* __restrict__ wg, const bf16_t* __restrict__ wu, const bf16_t* __restrict__ wd,
-                                 const bf16_t* __restrict__ b1, bf16_t* __restrict__ dup, bf16_t* __restrict__ ddn,
-                                 bf16_t* __restrict__ db, int D, int E, int Ed, int edp, int hp, int gated) {
+template <typename T>
+__global__ void pack_gemm_kernel(const T* __restrict__ wg, const T* __restrict__ wu, const T* __restrict__ wd,
+                                 const T* __restrict__ b1, T* __restrict__ dup, T* __restrict__ ddn, T* __restrict__ db, int D,
+                                 int E, int Ed, int edp, int hp, int gated) {
+  constexpr int KPF = GemmElem<T>::KPF, EPP = GemmElem<T>::EPP;
   const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int KS = D / 16, KS2 = hp / 16;
+  const int KS = D / KPF, KS2 = hp / KPF;
   const int hb = gated ? 64 : 128;   // hidden units per block of the up stream
   const int64_t n_up = (int64_t)(hp / hb) * KS * 4 * 64;
   const int64_t n_dn = (int64_t)(D / 128) * KS2 * 4 * 64;
@@ -111,12 +134,12 @@ __global__ void pack_gemm_kernel(const bf16_t* __restrict__ wg, const bf16_t* __
     const int g = lane >> 5, c = lane & 31;
     const int h = gated ? (64 * blk + 32 * (tile & 1) + c) : (128 * blk + 32 * tile + c);
     const int e = h / edp, j = h % edp;
-    const bf16_t* src = (gated && tile >= 2) ? wu : wg;
+    const T* src = (gated && tile >= 2) ? wu : wg;
     const bool ok = e < E && j < Ed;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int d = 16 * ks + 8 * g + i;
-      dup[p * 8 + i] = ok ? src[((int64_t)e * D + d) * Ed + j] : (bf16_t)0;
+    for (int i = 0; i < EPP; ++i) {
+      const int d = KPF * ks + EPP * g + i;
+      dup[p * EPP + i] = ok ? src[((int64_t)e * D + d) * Ed + j] : (T)0;
     }
   } else if (p < n_up + n_dn) {
     const int64_t pp = p - n_up;
@@ -128,38 +151,46 @@ __global__ void pack_gemm_kernel(const bf16_t* __restrict__ wg, const bf16_t* __
     const int g = lane >> 5, c = lane & 31;
     const int col = 128 * blk + 32 * tile + c;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int h = 16 * ks2 + 8 * (i / 4) + 4 * g + (i % 4);
+    for (int i = 0; i < EPP; ++i) {
+      const int h = (EPP == 8) ? (16 * ks2 + 8 * (i / 4) + 4 * g + (i % 4)) : (8 * ks2 + 4 * g + i);
       const int e = h / edp, j = h % edp;
-      ddn[pp * 8 + i] = (e < E && j < Ed) ? wd[((int64_t)e * Ed + j) * D + col] : (bf16_t)0;
+      ddn[pp * EPP + i] = (e < E && j < Ed) ? wd[((int64_t)e * Ed + j) * D + col] : (T)0;
     }
   } else if (p < n_up + n_dn + hp) {
     const int h = (int)(p - n_up - n_dn);
     const int e = h / edp, j = h % edp;
-    db[h] = (b1 != nullptr && e < E && j < Ed) ? b1[(int64_t)e * Ed + j] : (bf16_t)0;
+    db[h] = (b1 != nullptr && e < E && j < Ed) ? b1[(int64_t)e * Ed + j] : (T)0;
   }
+}
+
+template <typename T>
+static hipError_t launch_gemm_pack_t(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
+                                     void* packed_section, hipStream_t s) {
+  constexpr int KPF = GemmElem<T>::KPF;
+  const GemmLayout L = gemm_layout(sh);
+  char* base = (char*)packed_section;
+  const int hb = sh.gated ? 64 : 128;
+  const int64_t n = (int64_t)(L.hp / hb) * (sh.d_model / KPF) * 256 + (int64_t)(sh.d_model / 128) * (L.hp / KPF) * 256 + L.hp;
+  hipLaunchKernelGGL(pack_gemm_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const T*)w1, (const T*)w_up,
+                     (const T*)w2, (const T*)b1, (T*)(base + L.up_off), (T*)(base + L.dn_off), (T*)(base + L.b_off), sh.d_model,
+                     sh.n_experts, sh.expert_dim, L.edp, L.hp, sh.gated);
+  return hipGetLastError();
 }
 
 hipError_t launch_gemm_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                             void* packed_section, hipStream_t s) {
-  const GemmLayout L = gemm_layout(sh);
-  char* base = (char*)packed_section;
-  const int hb = sh.gated ? 64 : 128;
-  const int64_t n = (int64_t)(L.hp / hb) * (sh.d_model / 16) * 256 + (int64_t)(sh.d_model / 128) * (L.hp / 16) * 256 + L.hp;
-  hipLaunchKernelGGL(pack_gemm_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const bf16_t*)w1,
-                     (const bf16_t*)w_up, (const bf16_t*)w2, (const bf16_t*)b1, (bf16_t*)(base + L.up_off),
-                     (bf16_t*)(base + L.dn_off), (bf16_t*)(base + L.b_off), sh.d_model, sh.n_experts, sh.expert_dim, L.edp,
-                     L.hp, sh.gated);
-  return hipGetLastError();
+  if (sh.dtype == D2DMOE_F32) return launch_gemm_pack_t<float>(sh, w1, b1, w2, w_up, packed_section, s);
+  return launch_gemm_pack_t<bf16_t>(sh, w1, b1, w2, w_up, packed_section, s);
 }
 
 // ---------------------------------------------------------------------------------------------------
+template <typename T>
 struct GemmArgs {
-  const bf16_t* x;         // [N, D] rows of this pass
-  const bf16_t* routing;   // [N, E]
-  const bf16x8* w;         // packed weight stream of this product
-  const bf16_t* bias;      // [HP] first-layer bias (ungated)
-  bf16x8* hfrag;           // [token tile N/32][kstep2 HP/16][lane] hidden activations as A fragments
+  const T* x;              // [N, D] rows of this pass
+  const T* routing;        // [N, E]
+  const u32x4* w;          // packed weight stream of this product (fragments of 16 bytes per lane)
+  const T* bias;           // [HP] first-layer bias (ungated)
+  u32x4* hfrag;            // [token tile N/32][fragment HP/KPF][lane] hidden activations as A fragments
   float* partial;          // [ksplit][N][D] float32 sums of the down product
   int N; int D; int E; int edp; int hp; int act;
   int n_ttiles;            // 256-token tiles
@@ -167,15 +198,29 @@ struct GemmArgs {
   int ksplit;
 };
 
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+// one fragment pair into a 32 x 32 accumulator tile
+template <typename T>
+__device__ __forceinline__ void frag_mfma(const u32x4& a, const u32x4& b, f32x16& c) {
+  if constexpr (sizeof(T) == 2) {
+    bf16x8 av, bv;
+    __builtin_memcpy(&av, &a, 16);
+    __builtin_memcpy(&bv, &b, 16);
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, c, 0, 0, 0);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[i]), __uint_as_float(b[i]), c, 0, 0, 0);
+  }
+}
 
 // MODE 0: up product (weights = A operand, x = B operand through LDS); MODE 1: down product (H = A operand through
 // LDS, weights = B operand).
-template <int MODE, int ACT, bool GATED>
-__global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
+template <typename T, int MODE, int ACT, bool GATED>
+__global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs<T> A) {
+  constexpr int KPF = GemmElem<T>::KPF, EPP = GemmElem<T>::EPP;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  bf16x8* lds0 = (bf16x8*)smem_raw;          // [8 token tiles][4 ksteps][64 lanes]
-  bf16x8* lds1 = lds0 + 8 * 4 * 64;
+  u32x4* lds0 = (u32x4*)smem_raw;            // [8 token tiles][4 fragments][64 lanes]
+  u32x4* lds1 = lds0 + 8 * 4 * 64;
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
   const int wm = w >> 1, wn = w & 1;         // half of the weight rows/columns, half of the tokens
   const int g = lane >> 5, c32 = lane & 31;
@@ -188,12 +233,12 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
   int split = 0;
   if (MODE == 1) { split = nb % A.ksplit; nb /= A.ksplit; }
   const int N = A.N, D = A.D;
-  const int KS2T = A.hp / 16;                                    // K steps of the whole down product
-  const int n_ks = (MODE == 0) ? (D / 16) : (KS2T / A.ksplit);   // K steps of this workgroup
+  const int KS2T = A.hp / KPF;                                    // fragments along K of the whole down product
+  const int n_ks = (MODE == 0) ? (D / KPF) : (KS2T / A.ksplit);   // ... of this workgroup
   const int ks_begin = (MODE == 0) ? 0 : split * n_ks;
-  const int S = n_ks / 4;                                        // stages
-  const int KST = (MODE == 0) ? (D / 16) : KS2T;
-  const bf16x8* wbase = A.w + ((int64_t)(nb * 2 + wm) * KST + ks_begin) * 256 + lane;
+  const int S = n_ks / 4;                                         // stages
+  const int KST = (MODE == 0) ? (D / KPF) : KS2T;
+  const u32x4* wbase = A.w + ((int64_t)(nb * 2 + wm) * KST + ks_begin) * 256 + lane;
 
   f32x16 acc[4][4];   // [weight tile][token tile]
 #pragma unroll
@@ -205,9 +250,9 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
 
   // ---- token operand: global -> registers -> LDS, 8 pieces of 16 bytes per thread and stage
   u32x4 xv[8];
-  const int xrow = t >> 3, xpc = t & 7;   // MODE 0: row within a 32-token tile, 16-byte piece of the 64-wide K slice
+  const int xrow = t >> 3, xpc = t & 7;   // MODE 0: row within a 32-token tile, 16-byte piece of the stage's K slice
   // MODE 0 stores 8 pieces of one row per 8 lanes; inside a fragment the row slot is XORed with the piece index (and
-  // bit 3 with the row's parity) so that those stores spread over all LDS banks.  A read of fragment (kstep, half)
+  // bit 3 with the row's parity) so that those stores spread over all LDS banks.  A read of fragment (index, half)
   // applies the same XOR, which only permutes its 32 consecutive slots.
   int xoff[4];
 #pragma unroll
@@ -219,50 +264,50 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
       if (MODE == 0) {
         int64_t tok = (int64_t)tt * GM_BT + i * 32 + xrow;
         tok = tok < N ? tok : (N - 1);   // rows beyond N repeat the last row; their H is forced to zero below
-        xv[i] = *(const u32x4*)(A.x + tok * D + s * 64 + xpc * 8);
+        xv[i] = *(const u32x4*)(A.x + tok * D + s * (4 * KPF) + xpc * EPP);
       } else {
-        xv[i] = *(const u32x4*)(A.hfrag + (((int64_t)tt * 8 + i) * KS2T + ks_begin + s * 4 + w) * 64 + lane);
+        xv[i] = A.hfrag[(((int64_t)tt * 8 + i) * KS2T + ks_begin + s * 4 + w) * 64 + lane];
       }
     }
   };
-  auto store_x = [&](bf16x8* buf) __attribute__((always_inline)) {
+  auto store_x = [&](u32x4* buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      if (MODE == 0) ((u32x4*)buf)[(i * 4 + (xpc >> 1)) * 64 + 32 * (xpc & 1) + (xrow ^ xpc ^ ((xrow & 1) << 3))] = xv[i];
-      else ((u32x4*)buf)[i * 256 + t] = xv[i];
+      if (MODE == 0) buf[(i * 4 + (xpc >> 1)) * 64 + 32 * (xpc & 1) + (xrow ^ xpc ^ ((xrow & 1) << 3))] = xv[i];
+      else buf[i * 256 + t] = xv[i];
     }
   };
   // ---- weight operand: a register ring of 16 fragments (one stage); a slot is refilled with the fragment one stage
   // ahead as soon as it has been handed to the MFMAs
-  bf16x8 ring[4][4];   // [kstep][tile]
+  u32x4 ring[4][4];   // [fragment][tile]
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
     for (int i = 0; i < 4; ++i) ring[ks][i] = wbase[(ks * 4 + i) * 64];
-  auto compute = [&](const bf16x8* buf, int s_next) __attribute__((always_inline)) {
-    const bf16x8* xl = buf + (wn * 4) * 4 * 64;
-    const bf16x8* wn_ = wbase + (int64_t)s_next * 16 * 64;
-    bf16x8 xb[4];
+  auto compute = [&](const u32x4* buf, int s_next) __attribute__((always_inline)) {
+    const u32x4* xl = buf + (wn * 4) * 4 * 64;
+    const u32x4* wn_ = wbase + (int64_t)s_next * 16 * 64;
+    u32x4 xb[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) xb[j] = xl[(j * 4 + 0) * 64 + xoff[0]];
     static_for<0, 4>([&](auto ks_c) __attribute__((always_inline)) {
       constexpr int ks = decltype(ks_c)::value;
       constexpr int kn = (ks + 1 < 4) ? ks + 1 : ks;
-      bf16x8 wv[4];
+      u32x4 wv[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         wv[i] = ring[ks][i];
         ring[ks][i] = wn_[(ks * 4 + i) * 64];
       }
-      bf16x8 nxb[4];
+      u32x4 nxb[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) nxb[j] = xl[(j * 4 + kn) * 64 + xoff[kn]];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          if (MODE == 0) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv[i], xb[j], acc[i][j], 0, 0, 0);
-          else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xb[j], wv[i], acc[i][j], 0, 0, 0);
+          if (MODE == 0) frag_mfma<T>(wv[i], xb[j], acc[i][j]);
+          else frag_mfma<T>(xb[j], wv[i], acc[i][j]);
         }
 #pragma unroll
       for (int j = 0; j < 4; ++j) xb[j] = nxb[j];
@@ -274,8 +319,8 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
   store_x(lds0);
   __syncthreads();
   for (int s = 0; s < S; ++s) {
-    bf16x8* cur = (s & 1) ? lds1 : lds0;
-    bf16x8* nxt = (s & 1) ? lds0 : lds1;
+    u32x4* cur = (s & 1) ? lds1 : lds0;
+    u32x4* nxt = (s & 1) ? lds0 : lds1;
     const bool more = s + 1 < S;
     if (more) load_x(s + 1);
     __builtin_amdgcn_sched_barrier(0);
@@ -296,17 +341,16 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
 #pragma unroll
       for (int i = 0; i < NH; ++i) {
         const int h0 = (nb * 2 + wm) * HW + 32 * i;
-        const int e = h0 / A.edp;
-        const bool live = tok < N && e < A.E;
-        const float rw = live ? bf16_to_f32(A.routing[tok * A.E + e]) : 0.f;
         float hv[16];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
+          const int e = (h0 + 8 * q + 4 * g) / A.edp;   // the expert of these four rows
+          const bool live = tok < N && e < A.E;
+          const float rw = live ? Elem<T>::load(A.routing + tok * A.E + e) : 0.f;
           float bq[4] = {0.f, 0.f, 0.f, 0.f};
           if (!GATED) {
-            const uint2 bb = *(const uint2*)(A.bias + h0 + 8 * q + 4 * g);
-            bq[0] = __uint_as_float(bb.x << 16); bq[1] = __uint_as_float(bb.x & 0xffff0000u);
-            bq[2] = __uint_as_float(bb.y << 16); bq[3] = __uint_as_float(bb.y & 0xffff0000u);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) bq[u] = Elem<T>::load(A.bias + h0 + 8 * q + 4 * g + u);
           }
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
@@ -317,13 +361,23 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
             hv[r] = (live && rw != 0.f) ? v : 0.f;
           }
         }
+        u32x4* hdst = A.hfrag + (((int64_t)tt * 8 + tl) * KS2T + h0 / KPF) * 64 + lane;
+        if constexpr (sizeof(T) == 2) {
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
-          u32x4 pk;
-          pk.x = pack2_bf16(hv[8 * k + 0], hv[8 * k + 1]); pk.y = pack2_bf16(hv[8 * k + 2], hv[8 * k + 3]);
-          pk.z = pack2_bf16(hv[8 * k + 4], hv[8 * k + 5]); pk.w = pack2_bf16(hv[8 * k + 6], hv[8 * k + 7]);
-          const int ks2 = h0 / 16 + k;
-          *(u32x4*)(A.hfrag + (((int64_t)tt * 8 + tl) * KS2T + ks2) * 64 + lane) = pk;
+          for (int k = 0; k < 2; ++k) {
+            u32x4 pk;
+            pk.x = pack2_bf16(hv[8 * k + 0], hv[8 * k + 1]); pk.y = pack2_bf16(hv[8 * k + 2], hv[8 * k + 3]);
+            pk.z = pack2_bf16(hv[8 * k + 4], hv[8 * k + 5]); pk.w = pack2_bf16(hv[8 * k + 6], hv[8 * k + 7]);
+            hdst[k * 64] = pk;
+          }
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            u32x4 pk;
+            pk.x = __float_as_uint(hv[4 * q + 0]); pk.y = __float_as_uint(hv[4 * q + 1]);
+            pk.z = __float_as_uint(hv[4 * q + 2]); pk.w = __float_as_uint(hv[4 * q + 3]);
+            hdst[q * 64] = pk;
+          }
         }
       }
     }
@@ -347,8 +401,9 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs A) {
 }
 
 // out[n, :] = round(sum over splits (ascending) + last_bias + x), 8 columns per thread
-__global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restrict__ partial, const bf16_t* __restrict__ last_bias,
-                                                          const bf16_t* __restrict__ x, bf16_t* __restrict__ out, int64_t N, int D,
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restrict__ partial, const T* __restrict__ last_bias,
+                                                          const T* __restrict__ x, T* __restrict__ out, int64_t N, int D,
                                                           int ksplit, int add_residual) {
   const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int per_row = D / 8;
@@ -364,86 +419,94 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restric
     v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w; v[4] += b.x; v[5] += b.y; v[6] += b.z; v[7] += b.w;
   }
   if (last_bias != nullptr) {
-    const uint4 lb = *(const uint4*)(last_bias + col);
-    const uint32_t lw[4] = {lb.x, lb.y, lb.z, lb.w};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] += __uint_as_float((i & 1) ? (lw[i >> 1] & 0xffff0000u) : (lw[i >> 1] << 16));
+    for (int i = 0; i < 8; ++i) v[i] += Elem<T>::load(last_bias + col + i);
   }
   if (add_residual) {
-    const uint4 xr = *(const uint4*)(x + n * D + col);
-    const uint32_t xw[4] = {xr.x, xr.y, xr.z, xr.w};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] += __uint_as_float((i & 1) ? (xw[i >> 1] & 0xffff0000u) : (xw[i >> 1] << 16));
+    for (int i = 0; i < 8; ++i) v[i] += Elem<T>::load(x + n * D + col + i);
   }
-  uint4 o;
-  o.x = pack2_bf16(v[0], v[1]); o.y = pack2_bf16(v[2], v[3]);
-  o.z = pack2_bf16(v[4], v[5]); o.w = pack2_bf16(v[6], v[7]);
-  *(uint4*)(out + n * D + col) = o;
+  if constexpr (sizeof(T) == 2) {
+    uint4 o;
+    o.x = pack2_bf16(v[0], v[1]); o.y = pack2_bf16(v[2], v[3]);
+    o.z = pack2_bf16(v[4], v[5]); o.w = pack2_bf16(v[6], v[7]);
+    *(uint4*)(out + n * D + col) = o;
+  } else {
+    *(float4*)(out + n * D + col) = float4{v[0], v[1], v[2], v[3]};
+    *(float4*)(out + n * D + col + 4) = float4{v[4], v[5], v[6], v[7]};
+  }
+}
+
+template <typename T>
+static hipError_t launch_sum_partials_t(const float* partial, const void* last_bias, const void* x, void* out, int64_t N, int D,
+                                        int n_splits, int add_residual, hipStream_t s) {
+  const int64_t items = N * (D / 8);
+  hipLaunchKernelGGL(gemm_finish_kernel<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, partial, (const T*)last_bias,
+                     (const T*)x, (T*)out, N, D, n_splits, add_residual);
+  return hipGetLastError();
 }
 
 hipError_t launch_sum_partials(const float* partial, const void* last_bias, const void* x, void* out, int64_t N, int D,
                                int n_splits, int add_residual, hipStream_t s) {
-  const int64_t items = N * (D / 8);
-  hipLaunchKernelGGL(gemm_finish_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, partial, (const bf16_t*)last_bias,
-                     (const bf16_t*)x, (bf16_t*)out, N, D, n_splits, add_residual);
-  return hipGetLastError();
+  return launch_sum_partials_t<bf16_t>(partial, last_bias, x, out, N, D, n_splits, add_residual, s);
 }
 
-template <int ACT, bool GATED>
+template <typename T, int ACT, bool GATED>
 static hipError_t launch_gemm_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
                                   const void* last_bias, void* out, void* workspace, hipStream_t s) {
   const GemmLayout L = gemm_layout(sh);
   const GemmPlan P = gemm_plan(sh);
   const char* pk = (const char*)packed_section;
   const size_t lds = 2 * 8 * 4 * 64 * 16;
-  auto k_up = gated_gemm_kernel<0, ACT, GATED>;
-  auto k_dn = gated_gemm_kernel<1, -1, true>;
+  auto k_up = gated_gemm_kernel<T, 0, ACT, GATED>;
+  auto k_dn = gated_gemm_kernel<T, 1, -1, true>;
   hipError_t e = hipFuncSetAttribute((const void*)k_up, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   e = hipFuncSetAttribute((const void*)k_dn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   for (int64_t t0 = 0; t0 < sh.n_tokens; t0 += P.slab) {
     const int n = (int)((sh.n_tokens - t0) < P.slab ? (sh.n_tokens - t0) : P.slab);
-    GemmArgs A;
-    A.x = (const bf16_t*)x + t0 * sh.d_model;
-    A.routing = (const bf16_t*)routing + t0 * sh.n_experts;
-    A.bias = (const bf16_t*)(pk + L.b_off);
-    A.hfrag = (bf16x8*)workspace;
+    GemmArgs<T> A;
+    A.x = (const T*)x + t0 * sh.d_model;
+    A.routing = (const T*)routing + t0 * sh.n_experts;
+    A.bias = (const T*)(pk + L.b_off);
+    A.hfrag = (u32x4*)workspace;
     A.partial = (float*)((char*)workspace + P.h_bytes);
     A.N = n; A.D = sh.d_model; A.E = sh.n_experts; A.edp = L.edp; A.hp = L.hp; A.act = sh.activation;
     A.n_ttiles = (n + GM_BT - 1) / GM_BT;
     A.tpx = (A.n_ttiles + 7) / 8;
     A.ksplit = P.ksplit;
-    A.w = (const bf16x8*)(pk + L.up_off);
+    A.w = (const u32x4*)(pk + L.up_off);
     hipLaunchKernelGGL(k_up, dim3((unsigned)(8 * A.tpx * (L.hp / (GATED ? 128 : 256)))), dim3(256), lds, s, A);
-    A.w = (const bf16x8*)(pk + L.dn_off);
+    A.w = (const u32x4*)(pk + L.dn_off);
     hipLaunchKernelGGL(k_dn, dim3((unsigned)(8 * A.tpx * (sh.d_model / 256) * P.ksplit)), dim3(256), lds, s, A);
-    const int64_t items = (int64_t)n * (sh.d_model / 8);
-    hipLaunchKernelGGL(gemm_finish_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, (const float*)A.partial,
-                       (const bf16_t*)last_bias, A.x, (bf16_t*)out + t0 * sh.d_model, (int64_t)n, sh.d_model, P.ksplit,
-                       sh.add_residual);
-    e = hipGetLastError();
+    e = launch_sum_partials_t<T>(A.partial, last_bias, A.x, (T*)out + t0 * sh.d_model, (int64_t)n, sh.d_model, P.ksplit,
+                                 sh.add_residual, s);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;
 }
 
-template <bool GATED>
+template <typename T, bool GATED>
 static hipError_t launch_gemm_gated(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
                                     const void* last_bias, void* out, void* workspace, hipStream_t s) {
   switch (sh.activation) {
-    case D2DMOE_ACT_RELU: return launch_gemm_act<D2DMOE_ACT_RELU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    case D2DMOE_ACT_GELU: return launch_gemm_act<D2DMOE_ACT_GELU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    case D2DMOE_ACT_GELU_TANH: return launch_gemm_act<D2DMOE_ACT_GELU_TANH, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    case D2DMOE_ACT_SILU: return launch_gemm_act<D2DMOE_ACT_SILU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    default: return launch_gemm_act<-1, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_RELU: return launch_gemm_act<T, D2DMOE_ACT_RELU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_GELU: return launch_gemm_act<T, D2DMOE_ACT_GELU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_GELU_TANH: return launch_gemm_act<T, D2DMOE_ACT_GELU_TANH, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_SILU: return launch_gemm_act<T, D2DMOE_ACT_SILU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    default: return launch_gemm_act<T, -1, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
   }
 }
 
 hipError_t launch_mfma_gemm(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
                             const void* last_bias, void* out, void* workspace, hipStream_t s) {
-  if (sh.gated) return launch_gemm_gated<true>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-  return launch_gemm_gated<false>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+  if (sh.dtype == D2DMOE_F32) {
+    if (sh.gated) return launch_gemm_gated<float, true>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    return launch_gemm_gated<float, false>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+  }
+  if (sh.gated) return launch_gemm_gated<bf16_t, true>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+  return launch_gemm_gated<bf16_t, false>(sh, x, routing, packed_section, last_bias, out, workspace, s);
 }
 
 }  // namespace d2dmoe

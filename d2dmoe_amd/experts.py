@@ -132,7 +132,7 @@ class HipKernelExperts(ExpertsLayer):
 
     # -- derived buffers --------------------------------------------------------------------
     def packed_weights(self, router_w1=None, router_w2=None, router_activation='relu', router_output_activation='abs'):
-        if not self.w1.is_cuda or self.w1.dtype != torch.bfloat16:
+        if not self.w1.is_cuda or self.w1.dtype not in (torch.bfloat16, torch.float32):
             return None
         sh = ops.make_shape(0, self.hidden_dim, self.num_experts, self.expert_dim,
                             router_w1.size(0) if router_w1 is not None else 0, ops._dtype_code(self.w1),

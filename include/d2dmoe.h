@@ -73,7 +73,7 @@ enum {
                                  sweep runs.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 */
   D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 MFMA for at most 16 tokens: one workgroup per expert streams that expert's packed
                                  weights once (gated or ungated experts); AUTO picks it when it applies */
-  D2DMOE_PATH_MFMA_GEMM = 5   /* bf16 MFMA, D a multiple of 256, gated or ungated experts: two tiled products over all
+  D2DMOE_PATH_MFMA_GEMM = 5   /* bf16 or f32 MFMA, D a multiple of 256, gated or ungated experts: two tiled products over all
                                  experts with the routing value as a factor of the hidden activations, which stay in
                                  the workspace between them; AUTO picks it for more than 16 tokens when the dense sweep
                                  does not cover the shape */

@@ -105,9 +105,12 @@ def test_packed_and_workspace_sizes_follow_the_documented_layouts():
     # 16 tokens: the small-batch path needs the hidden fragments and one flag per expert only
     g16 = ops.make_shape(16, 2048, 256, 64, 256, abi.BF16, 'gelu_tanh', gated=True)
     assert lib.d2dmoe_workspace_bytes(ctypes.byref(g16)) < 2 << 20
-    # float32 layers have no packed form
+    # float32 layers: the tiled-products section only (hidden size 128 x 24 = 3072 neurons, float32 fragments)
     f = ops.make_shape(100, 768, 128, 24, 128, abi.F32)
-    assert lib.d2dmoe_packed_bytes(ctypes.byref(f)) == 0
+    want_f = (2 * 3072 * 768 + 3072) * 4
+    assert want_f <= lib.d2dmoe_packed_bytes(ctypes.byref(f)) <= want_f + 256
+    odd = ops.make_shape(100, 700, 128, 24, 128, abi.F32)   # width not a multiple of 256: generic kernel only
+    assert lib.d2dmoe_packed_bytes(ctypes.byref(odd)) == 0
     # ViT-B shape: dense-sweep stream (4 waves x 12 chunks x 192 fragments of 1 KB) is part of the buffer
     v = ops.make_shape(50432, 768, 128, 24, 128, abi.BF16)
     assert lib.d2dmoe_packed_bytes(ctypes.byref(v)) >= 4 * 12 * 192 * 1024
