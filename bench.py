@@ -35,6 +35,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_F32_TFLOPS = 157.3     # MI355X float32 matrix
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 
 WORKLOADS = {
@@ -43,6 +44,8 @@ WORKLOADS = {
     'vit_b_1576': (8, 197, 768, 128, 24, 128, 'relu'),
     # skewed routing: router bypassed, norms = |randn| * w_e with w_e = rank_e^-1.2 (a few experts draw most tokens)
     'vit_b_skew': (256, 197, 768, 128, 24, 128, 'relu'),
+    # the CPU baseline's own case (8 x 197 tokens, float32) on the GPU: float32 storage and float32 matrix arithmetic
+    'vit_b_1576_f32': (8, 197, 768, 128, 24, 128, 'relu'),
 }
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (profiles/), scaled by
 # the factors a plain copy kernel of known size gives for the same counters (2.0 and 1.0); None = not measured
@@ -175,10 +178,10 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, pa
     torch.cuda.synchronize()
     ms_layer = (time.perf_counter() - t0) * 1e3 / steps
     # dominant kernel alone (same routing), HIP events on the launch stream
+    # the experts call the layer makes: under AUTO d2dmoe_forward takes the expert-major path for high thresholds (bf16)
+    experts_path = path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 and x.dtype == torch.bfloat16 else 'auto')
     ms_experts = time_events(lambda: ops.experts(x, routing, p['w1'], p['b1'], p['w2'], None, p['last_bias'], act, False,
-                                                 path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 else 'auto'),
-                                                 packed), steps, warmup)
-    experts_path = path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 else 'auto')
+                                                 experts_path, packed), steps, warmup)
     quant = None
     if quantile_iters:
         quant = time_quantiles(lambda: ops.experts(x, routing, p['w1'], p['b1'], p['w2'], None, p['last_bias'], act, False,
@@ -384,7 +387,9 @@ def main():
         return
     B, T, D, E, Ed, W, act = WORKLOADS[args.workload]
     N = B * T
-    dtype = torch.bfloat16
+    f32 = args.workload.endswith('_f32')
+    dtype = torch.float32 if f32 else torch.bfloat16
+    peak = PEAK_F32_TFLOPS if f32 else PEAK_BF16_TFLOPS
     p = make_params(D, E, Ed, W, seed=0, dtype=dtype, device=dev)
     x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
     shape = ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x), act)
@@ -414,7 +419,7 @@ def main():
         'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
         'value': main_r['tokens_per_s'], 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': main_r['ms_layer'], 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
-        'dtype': 'bf16', 'data': 'synthetic',
+        'dtype': 'f32' if f32 else 'bf16', 'data': 'synthetic',
         'config': {'workload': f'{args.workload}: {B}x{T}={N} tokens, D={D}, {E} experts x {Ed}, {act}, router {D}->{W}->{E}, '
                                f'module tau={args.tau} (keep norm >= {1 - args.tau:.2f}*max), whole layer',
                    'mean_active_experts': main_r['mean_active'], 'p99_active_experts': main_r['p99_active'],
@@ -422,7 +427,7 @@ def main():
         'ms_per_step_eager_launches': main_r['ms_layer_eager'],
         'active_tflops': main_r['active_tflops_layer'], 'hbm_gbps': main_r['hbm_gbps_layer'],
         'roofline': {'bound': 'mfma', 'kernel': 'experts', 'achieved': main_r['active_tflops_kernel'],
-                     'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s', 'frac': main_r['active_tflops_kernel'] / PEAK_BF16_TFLOPS,
+                     'peak': peak, 'unit': 'TFLOP/s', 'frac': main_r['active_tflops_kernel'] / peak,
                      'traffic': MEASURED_TRAFFIC.get(args.workload), 'kernel_ms': main_r['ms_experts'],
                      'kernel_quantiles': main_r['experts_quantiles'], 'router_select_ms': main_r['ms_router'],
                      'frac_of_library_gemm': main_r['active_tflops_kernel'] / ceil['library_gemm_bf16_8192_tflops']},
