@@ -322,7 +322,7 @@ def run_gpt2(args, dev):
     print(json.dumps(line))
 
 
-def cpu_baseline(D, E, Ed, W, act, tau, budget_s=15.0):
+def cpu_baseline(D, E, Ed, W, act, tau, budget_s=12.0):
     """The oracle's restatement of the reference CPU path (router -> dynk_max gate -> per-expert loop), float32,
     8 x 197 tokens of the same layer shape, repeated until about budget_s seconds have been spent."""
     from oracle import d2dmoe_oracle as O
@@ -335,7 +335,7 @@ def cpu_baseline(D, E, Ed, W, act, tau, budget_s=15.0):
         O.moe_layer_forward(x, p, tau, act, 'naive')
         times = []
         t_start = time.perf_counter()
-        while (time.perf_counter() - t_start < budget_s and len(times) < 50) or len(times) < 3:
+        while (time.perf_counter() - t_start < budget_s and len(times) < 400) or len(times) < 3:
             t0 = time.perf_counter()
             O.moe_layer_forward(x, p, tau, act, 'naive')
             times.append(time.perf_counter() - t0)
