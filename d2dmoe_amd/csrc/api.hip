@@ -41,7 +41,7 @@ ForwardWorkspace plan_workspace(const d2dmoe_shape& sh) {
   size_t scratch = perm_workspace_bytes(sh.n_tokens, sh.n_experts);
   const size_t sparse = mfma_sparse_workspace_bytes(sh);   // plan + result rows of the expert-major path
   if (sparse > scratch) scratch = sparse;
-  const size_t decode = mfma_decode_workspace_bytes(sh);   // per-expert result rows of the small-batch path
+  const size_t decode = mfma_decode_workspace_bytes(sh);   // hidden fragments + expert flags of the small-batch path
   if (decode > scratch) scratch = decode;
   const size_t dsplit = mfma_dense_workspace_bytes(sh);    // float32 sums of the chunk-split dense sweep (few tokens)
   if (dsplit > scratch) scratch = dsplit;

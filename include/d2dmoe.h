@@ -161,15 +161,20 @@ int d2dmoe_build_permutation(const void* routing, int64_t n_tokens, int32_t n_ex
  * For 0/1 routing this equals the reference's naive and Triton modes; for weighted routing it equals its
  * 'masked' mode (forward_all, moe_layers.py:193-198).
  * packed: optional buffer written by d2dmoe_pack_weights for the same weights (required by the MFMA paths;
- * D2DMOE_PATH_AUTO without it uses the generic kernel). */
+ * D2DMOE_PATH_AUTO without it uses the generic kernel).
+ * workspace: d2dmoe_workspace_bytes() of the same shape, 256-byte aligned.  Required by the expert-major, small-batch
+ * and tiled-products paths; the dense sweep uses it when given (with few tokens it deals every tile's work to several
+ * workgroups through it) and runs without it otherwise. */
 int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing,
                    const void* w1, const void* b1, const void* w2, const void* w_up,
                    const void* last_bias, const void* packed, void* out, int32_t path,
                    void* workspace, size_t workspace_bytes, void* stream);
 
-/* Bytes of the derived weight buffer for the MFMA kernels (0 when `shape` has no MFMA kernel).  The buffer has an
- * experts section (when the fused experts kernel covers the shape) and a router section (when shape.router_width
- * > 0 and the fused router+selection kernel covers the router: bf16, ReLU/abs, width = experts = 128 or 256). */
+/* Bytes of the derived weight buffer for the MFMA kernels (0 when `shape` has no MFMA kernel).  The buffer has one
+ * section per kernel family that covers the shape (dense sweep and expert-major: bf16, D = 768, ungated; small batch:
+ * bf16, D a multiple of 256; tiled products: bf16 or f32, D a multiple of 256) and a router section (when
+ * shape.router_width > 0 and the fused router+selection kernel covers the router: bf16, ReLU/abs, width = experts =
+ * 128 or 256). */
 size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape);
 
 /* Re-tiles expert and router weights into MFMA fragment order.  A derived, cacheable buffer: call once per
