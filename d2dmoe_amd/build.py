@@ -10,6 +10,7 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, 'csrc')
@@ -25,10 +26,7 @@ def hipcc_path() -> str:
     raise RuntimeError('hipcc not found')
 
 
-def build(verbose: bool = False) -> str:
-    cmd = [hipcc_path(), f'--offload-arch={ARCH}', '-O3', '-std=c++17', '-fPIC', '-shared',
-           '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
-           *[os.path.join(CSRC, s) for s in SOURCES], '-o', OUTPUT + '.tmp']
+def _run(cmd, verbose):
     if verbose:
         print(' '.join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -38,6 +36,22 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError(f'hipcc failed ({res.returncode}):\n{err}')
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build(verbose: bool = False) -> str:
+    """One object per source, compiled side by side (a handful of processes), then one link."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = hipcc_path()
+    flags = [f'--offload-arch={ARCH}', '-O3', '-std=c++17', '-fPIC', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops']
+    objdir = tempfile.mkdtemp(prefix='d2dmoe_build_')
+    try:
+        objs = [os.path.join(objdir, s.replace('.hip', '.o')) for s in SOURCES]
+        jobs = [[hipcc, *flags, '-c', os.path.join(CSRC, s), '-o', o] for s, o in zip(SOURCES, objs)]
+        with ThreadPoolExecutor(max_workers=min(len(jobs), max(1, min(os.cpu_count() or 1, 8)))) as pool:
+            list(pool.map(lambda c: _run(c, verbose), jobs))
+        _run([hipcc, f'--offload-arch={ARCH}', '-shared', '-fPIC', *objs, '-o', OUTPUT + '.tmp'], verbose)
+    finally:
+        shutil.rmtree(objdir, ignore_errors=True)
     os.replace(OUTPUT + '.tmp', OUTPUT)
     return OUTPUT
 
