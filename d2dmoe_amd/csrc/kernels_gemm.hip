@@ -38,7 +38,6 @@ constexpr int GM_BT = 256;         // tokens per workgroup tile
 constexpr int GM_SLAB = 8192;      // tokens per pass: bounds the workspace (H fragments + float32 partial sums)
 constexpr int GM_MAX_SPLIT = 8;
 
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 // Per element type: K values per fragment, elements per 16-byte piece.

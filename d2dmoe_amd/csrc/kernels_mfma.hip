@@ -22,7 +22,7 @@ static size_t dense_lds_bytes(const d2dmoe_shape& sh) {
   return (size_t)(2 * KS1 * 64 + 2 * MD_KS2 * 64) * 16            // x fragments, h fragments
          + (size_t)MD_BM * (sh.n_experts + 8) * 2                  // routing tile, rows padded by 8 elements
          + (size_t)n_chunks * MD_HC * 3                            // b1 (bf16) and expert index (uint8) per neuron
-         + (size_t)(2 * n_chunks + 1) * sizeof(int);               // chunk-activity flags, active-chunk list
+         + (size_t)((sh.n_experts + 7) / 8 * 8 + 4) * sizeof(uint32_t);   // chunk bits per expert, active-chunk mask
 }
 
 // The fused experts kernel is instantiated for D = 768 (ViT-B, GPT-2 small, BERT-base), ungated experts, bf16.
@@ -31,6 +31,7 @@ bool mfma_dense_supported(const d2dmoe_shape& sh) {
   if (sh.d_model != 768) return false;
   if (sh.n_experts > 256) return false;          // expert indices are staged as uint8
   if (sh.expert_dim > MD_HC) return false;       // an expert spans at most two chunks
+  if ((sh.n_experts * sh.expert_dim + MD_HC - 1) / MD_HC > MD_MAX_CHUNKS) return false;   // staging registers, chunk mask
   return dense_lds_bytes(sh) <= 160 * 1024;      // x tile + h tile + routing tile + bias/expert-index tables
 }
 
@@ -247,10 +248,9 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   const int HP = n_chunks * MD_HC;
   bf16_t* rs = (bf16_t*)(hs + 2 * MD_KS2 * 64);                // [64][E+8] routing tile
   bf16_t* b1s = rs + MD_BM * RS;                               // [HP] first-layer bias
-  int* cact = (int*)(b1s + HP);                                // [n_chunks] chunk-activity flags
-  int* clist = cact + n_chunks;                                // [n_chunks] active chunks, then their number
-  int* n_act_p = clist + n_chunks;
-  uint8_t* eis = (uint8_t*)(n_act_p + 1);                      // [HP] expert index of each neuron
+  uint8_t* eis = (uint8_t*)(b1s + HP);                         // [HP] expert index of each neuron
+  uint32_t* ebits = (uint32_t*)(eis + HP);                     // [E rounded up to 8] chunks each expert's neurons lie in
+  uint32_t* cmask_lds = ebits + ((E + 7) & ~7);                // chunks some token of the tile needs (bit per chunk)
 
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -263,77 +263,135 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   constexpr int BM = 32 * TT;
   static_assert(NW1 % R == 0 && NW2 % R == 0, "every phase must start at ring slot 0");
 
-  // The weight stream of chunk 0 is requested before anything else (almost every tile starts there); if the tile's
-  // first active chunk turns out to be another one the ring is reloaded below.
+  // ---- staging.  Every global load of the tile's inputs is issued up front, in the order the data is needed:
+  // routing pieces and the two tables (short, and the active-chunk mask hangs on them), the x tile, then the weight
+  // stream of the first chunk (almost every tile starts at chunk 0; if its first active chunk turns out to be another
+  // one the ring is reloaded below).  Loads complete in order, so each stage below waits only for what precedes it.
+  //
+  // A wave stages RW consecutive rows of the tile.  Lane (r = lane & 7, c = lane >> 3) takes row r of a block of 8
+  // rows and the 16-byte pieces c, c + 8, c + 16 ... of it: 8 lanes read 128 contiguous bytes of a row, 8 lanes write
+  // 128 contiguous bytes of LDS (the rows of a fragment), and all further addresses are compile-time offsets from a
+  // handful of lane values -- this part of the kernel is bound by instruction issue, not by memory.
+  // Rows past the end of the batch are read from the last row instead (rows never mix, and their results are not
+  // stored).
   const bf16x8* wbase = A.wp + (int64_t)w * n_chunks * PIECES * 64 + lane;   // this wave's stream
   bf16x8 ring[R];
   const int first_guess = SPLIT ? c_begin : 0;
-#pragma unroll
-  for (int i = 0; i < R; ++i) ring[i] = wbase[((int64_t)first_guess * PIECES + i) * 64];
-
-  // ---- stage x (as B fragments), routing, bias and expert-index tables; all loads of a kind are issued together
+  const int r8 = lane & 7, c8l = lane >> 3;
+  const int last_row = (int)((N - 1 - tok0) < (int64_t)(BM - 1) ? (N - 1 - tok0) : (int64_t)(BM - 1));
   {
-    for (int i = t; i < n_chunks; i += 256) cact[i] = 0;
-    constexpr int PIECES_PER_ROW = D / 8;
-    constexpr int XP = BM * PIECES_PER_ROW / 256;   // 16-byte pieces of x per thread
-    static_assert(BM * PIECES_PER_ROW % 256 == 0, "x tile must divide over the workgroup");
-    const uint4 zero4 = {0u, 0u, 0u, 0u};
-    uint4 xv[XP];
-#pragma unroll
-    for (int k = 0; k < XP; ++k) {
-      const int p = t + k * 256;
-      const int m = p / PIECES_PER_ROW, kk = p - m * PIECES_PER_ROW;
-      const int64_t n = tok0 + m;
-      xv[k] = *(const uint4*)(A.x + (n < N ? n : N - 1) * D + kk * 8);   // clamped address, value zeroed below
-      if (n >= N) xv[k] = zero4;
-    }
-    for (int i = t; i < HP / 8; i += 256) ((uint4*)b1s)[i] = ((const uint4*)A.b1p)[i];
-    for (int i = t; i < HP / 16; i += 256) ((uint4*)eis)[i] = ((const uint4*)A.eidx)[i];
-    __syncthreads();   // cact zeroed before the flags below are raised
-    auto raise_flags = [&](int e) __attribute__((always_inline)) {   // expert e is routed to: mark its chunks active
+    constexpr int RW = BM / 4;                      // rows per wave
+    constexpr int RB = RW / 8;                      // blocks of 8 rows per wave
+    constexpr int XK = D / 64;                      // 16-byte pieces of a row per lane (12)
+    constexpr int RK = 4;                           // routing pieces of a row per lane (E <= 256)
+    constexpr int TB1 = MD_MAX_CHUNKS / 8, TEI = MD_MAX_CHUNKS / 16;   // table pieces per thread
+    const bool wide = (E & 7) == 0;                 // routing rows are whole 16-byte pieces
+    const int EP = E >> 3;
+    if (t == 0) *cmask_lds = 0u;
+    for (int e = t; e < E; e += 256) {
       const int h0 = e * A.expert_dim;
-      cact[h0 >> 8] = 1;                                      // benign race: every writer stores 1
-      cact[(h0 + A.expert_dim - 1) >> 8] = 1;
-    };
-    if ((E & 7) == 0) {
-      const int EP = E / 8;   // 16-byte pieces per routing row
-      for (int p = t; p < BM * EP; p += 256) {
-        const int m = p / EP, e0 = (p - m * EP) * 8;
-        const int64_t n = tok0 + m;
-        uint4 rv = *(const uint4*)(A.routing + (n < N ? n : N - 1) * E + e0);
-        if (n >= N) rv = zero4;
-        *(uint4*)(rs + m * RS + e0) = rv;
-        const uint32_t wd[4] = {rv.x, rv.y, rv.z, rv.w};
+      ebits[e] = (1u << (h0 >> 8)) | (1u << ((h0 + A.expert_dim - 1) >> 8));
+    }
+    int mrow[RB];                                   // tile row of each row block, clamped to the last real row
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          if (((wd[i >> 1] >> (16 * (i & 1))) & 0x7fffu) != 0) raise_flags(e0 + i);
+    for (int rb = 0; rb < RB; ++rb) {
+      const int m = w * RW + rb * 8 + r8;
+      mrow[rb] = m < last_row ? m : last_row;
+    }
+    u32x4 rv[RB][RK];
+    if (wide) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const u32x4* rrow = (const u32x4*)(A.routing + (tok0 + mrow[rb]) * E);
+#pragma unroll
+        for (int kb = 0; kb < RK; ++kb)
+          if (kb * 8 < EP) rv[rb][kb] = rrow[c8l + kb * 8 < EP ? c8l + kb * 8 : 0];   // lanes past the row: piece 0
       }
-    } else {
+    }
+    u32x4 tb[TB1], te[TEI];
+#pragma unroll
+    for (int k = 0; k < TB1; ++k) {
+      const int i = t + k * 256;
+      tb[k] = ((const u32x4*)A.b1p)[i < HP / 8 ? i : 0];
+    }
+#pragma unroll
+    for (int k = 0; k < TEI; ++k) {
+      const int i = t + k * 256;
+      te[k] = ((const u32x4*)A.eidx)[i < HP / 16 ? i : 0];
+    }
+    u32x4 xv[RB][XK];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const u32x4* xrow = (const u32x4*)(A.x + (tok0 + mrow[rb]) * D) + c8l;
+#pragma unroll
+      for (int kb = 0; kb < XK; ++kb) xv[rb][kb] = xrow[kb * 8];
+    }
+    lds_barrier();   // chunk bits per expert written, mask cleared
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t need = 0u;                             // chunks the rows staged by this thread need
+    if (wide) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const int m = w * RW + rb * 8 + r8;
+#pragma unroll
+        for (int kb = 0; kb < RK; ++kb) {
+          if (kb * 8 < EP && c8l + kb * 8 < EP) {
+            const int piece = c8l + kb * 8;
+            const u32x4 r4 = rv[rb][kb];
+            *(u32x4*)(rs + m * RS + piece * 8) = r4;
+            const u32x4 eb0 = *(const u32x4*)(ebits + piece * 8);
+            const u32x4 eb1 = *(const u32x4*)(ebits + piece * 8 + 4);
+            const uint32_t wd[4] = {r4.x, r4.y, r4.z, r4.w};
+            const uint32_t eb[8] = {eb0.x, eb0.y, eb0.z, eb0.w, eb1.x, eb1.y, eb1.z, eb1.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              need |= (wd[i >> 1] & ((i & 1) ? 0x7fff0000u : 0x7fffu)) != 0 ? eb[i] : 0u;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < TB1; ++k) {
+      const int i = t + k * 256;
+      if (i < HP / 8) ((u32x4*)b1s)[i] = tb[k];
+    }
+#pragma unroll
+    for (int k = 0; k < TEI; ++k) {
+      const int i = t + k * 256;
+      if (i < HP / 16) ((u32x4*)eis)[i] = te[k];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < R; ++i) ring[i] = wbase[((int64_t)first_guess * PIECES + i) * 64];
+    __builtin_amdgcn_sched_barrier(0);
+    if (!wide) {
       for (int i = t; i < BM * E; i += 256) {
         const int m = i / E, e = i - m * E;
-        const int64_t n = tok0 + m;
-        const bf16_t rv = (n < N) ? A.routing[n * E + e] : (bf16_t)0;
-        rs[m * RS + e] = rv;
-        if ((rv & 0x7fff) != 0) raise_flags(e);
+        const bf16_t r1 = A.routing[(tok0 + (m < last_row ? m : last_row)) * E + e];
+        rs[m * RS + e] = r1;
+        if ((r1 & 0x7fff) != 0) need |= ebits[e];
       }
     }
+    if (need != 0u)
+      __hip_atomic_fetch_or((__attribute__((address_space(3))) uint32_t*)cmask_lds, need, __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_WORKGROUP);
+    // x fragments: piece kk of row m goes to fragment kk / 2 (K step), slot (m & 31) + 32 * (kk & 1)
 #pragma unroll
-    for (int k = 0; k < XP; ++k) {
-      const int p = t + k * 256;
-      const int m = p / PIECES_PER_ROW, kk = p - m * PIECES_PER_ROW;
-      const int ks = kk >> 1, gg = kk & 1;
-      ((uint4*)xs)[((m >> 5) * KS1 + ks) * 64 + (m & 31) + 32 * gg] = xv[k];
+    for (int rb = 0; rb < RB; ++rb) {
+      const int m = w * RW + rb * 8 + r8;
+      u32x4* xdst = (u32x4*)xs + ((m >> 5) * KS1 + (c8l >> 1)) * 64 + (m & 31) + 32 * (c8l & 1);
+#pragma unroll
+      for (int kb = 0; kb < XK; ++kb) xdst[kb * 4 * 64] = xv[rb][kb];
     }
   }
-  __syncthreads();
-  if (t == 0) {
-    int n_act = 0;
-    for (int ch = 0; ch < n_chunks; ++ch)
-      if (cact[ch] && (!SPLIT || (ch >= c_begin && ch < c_end))) clist[n_act++] = ch;
-    *n_act_p = n_act;
+  lds_barrier();
+  // Active chunks as a bit mask, the same in every wave: the chunk loop walks its set bits.
+  uint32_t cmask = __builtin_amdgcn_readfirstlane(*cmask_lds);
+  if constexpr (SPLIT) {
+    const uint32_t below_end = (c_end >= 32) ? ~0u : ((1u << c_end) - 1u);
+    cmask &= below_end & ~((1u << c_begin) - 1u);
   }
-  __syncthreads();
-  const int n_act = *n_act_p;
+  const int n_act = __popc(cmask);
 
   f32x16 acc2[TT][CT];
 #pragma unroll
@@ -345,15 +403,17 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
 
   if (n_act > 0) {
     f32x16 acc1[2][TT];   // GEMM1 accumulators [row-tile][token tile]
-    const bf16x8* cur = wbase + (int64_t)clist[0] * PIECES * 64;
-    if (clist[0] != first_guess) {
+    const int first_chunk = __builtin_ctz(cmask);
+    const bf16x8* cur = wbase + (int64_t)first_chunk * PIECES * 64;
+    if (first_chunk != first_guess) {
 #pragma unroll
       for (int i = 0; i < R; ++i) ring[i] = cur[i * 64];
     }
 
     for (int ci = 0; ci < n_act; ++ci) {
-      const int chunk = clist[ci];
-      const bf16x8* nxt = (ci + 1 < n_act) ? (wbase + (int64_t)clist[ci + 1] * PIECES * 64) : cur;
+      const int chunk = __builtin_ctz(cmask);
+      cmask &= cmask - 1;
+      const bf16x8* nxt = (cmask != 0) ? (wbase + (int64_t)__builtin_ctz(cmask) * PIECES * 64) : cur;
       const int hb0 = chunk * MD_HC + w * 64 + 4 * g;   // first neuron of this lane's accumulator rows, row-tile 0
 
       // epilogue state, filled and consumed in slices between MFMAs
@@ -490,62 +550,73 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     }
   }
 
-  // ---- final epilogue: OUT tile -> LDS as float pairs are not needed; the accumulators are rounded to bf16 AFTER
-  // + last_bias (+ x) in float32, so they go through LDS as float in two passes of D/2 columns: write [tokens][D/2]
-  // float, then every thread reads 8 consecutive columns, adds bias / residual, rounds once, stores 16 bytes.
+  // ---- final epilogue: the accumulators are rounded to bf16 once, AFTER + last_bias (+ x) in float32, and leave as
+  // whole rows.  One pass per 32-token tile: every wave writes its D/4 columns of the pass's rows to LDS as float
+  // [32][D + 4] (bias added on the way: a lane's accumulators share CT columns), then wave w takes rows 8w .. 8w + 7
+  // with the lane mapping of the staging above -- lane (r, c) reads 8 consecutive columns c, c + 8, ... of row r, adds
+  // the residual, rounds, stores 16 bytes; 8 lanes cover 128 contiguous bytes of an output row.  The residual rows
+  // are requested before the pass's LDS traffic; the read loop has no branches and no address arithmetic.
   {
-    constexpr int HALF = D / 2;
-    constexpr int OS = HALF + 4;                    // row stride in floats (+16 bytes: the two lane halves use
-    float* ot = (float*)smem_raw;                   // different banks); BM * OS * 4 <= x + h regions
-    static_assert((size_t)64 * OS * 4 <= (size_t)(2 * KS1 * 64 + 2 * MD_KS2 * 64) * 16, "out staging fits");
-    constexpr int OP = BM * (HALF / 8) / 256;       // 8-column pieces per thread and pass
-    static_assert(BM * (HALF / 8) % 256 == 0, "out tile must divide over the workgroup");
+    constexpr int OS = D + 4;                       // row stride in floats (+16 bytes: rows shift by 4 banks, so the
+    float* ot = (float*)smem_raw;                   // 8 rows a wave reads at once cover all 32); fits in x + h regions
+    static_assert((size_t)32 * OS * 4 <= (size_t)(2 * KS1 * 64 + 2 * MD_KS2 * 64) * 16, "out staging fits");
+    constexpr int OP = D / 64;                      // 8-column pieces per thread and pass
+    const bool with_bias = !SPLIT && A.last_bias != nullptr;
+    const bool with_res = !SPLIT && A.add_residual != 0;
+    float lb[CT];
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-      __syncthreads();                              // previous readers of this LDS region are done
-      if ((w >> 1) == pass) {                       // waves 0,1 own columns [0, D/2), waves 2,3 own [D/2, D)
+    for (int ct = 0; ct < CT; ++ct)
+      lb[ct] = with_bias ? bf16_to_f32(A.last_bias[w * (D / 4) + ct * 32 + c32]) : 0.f;
+    const int row = w * 8 + r8;                     // row of the pass this thread finishes
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-          const int colh = (w & 1) * (D / 4) + ct * 32 + c32;
+    for (int tt = 0; tt < TT; ++tt) {
+      const int64_t n = tok0 + tt * 32 + row;
+      const bool live = n < N;
+      u32x4 xr[OP];
+      if (with_res) {
+        const u32x4* xrow = (const u32x4*)(A.x + (live ? n : N - 1) * D) + c8l;
 #pragma unroll
-          for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) ot[(tt * 32 + 8 * (r / 4) + 4 * g + (r % 4)) * OS + colh] = acc2[tt][ct][r];
-        }
+        for (int k = 0; k < OP; ++k) xr[k] = xrow[k * 8];
       }
-      __syncthreads();
+      lds_barrier();                                // previous readers of this LDS region are done
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        const int col = w * (D / 4) + ct * 32 + c32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          ot[(8 * (r / 4) + 4 * g + (r % 4)) * OS + col] = with_bias ? acc2[tt][ct][r] + lb[ct] : acc2[tt][ct][r];
+      }
+      lds_barrier();
+      const float* orow = ot + row * OS + c8l * 8;
+      u32x4 o[OP];
+      float4 pv0[OP], pv1[OP];
 #pragma unroll
       for (int k = 0; k < OP; ++k) {
-        const int p = t + k * 256;
-        const int m = p / (HALF / 8), c8 = (p - m * (HALF / 8)) * 8;
-        const int64_t n = tok0 + m;
-        if (n < N) {
-          const float4 v0 = *(const float4*)(ot + m * OS + c8);
-          const float4 v1 = *(const float4*)(ot + m * OS + c8 + 4);
-          float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-          const int col = pass * HALF + c8;
-          if constexpr (SPLIT) {
-            float* prow = A.partial + ((int64_t)split * A.part_rows + (n - A.part_base)) * D + col;
-            *(float4*)prow = v0;
-            *(float4*)(prow + 4) = v1;
-            continue;
-          }
-          if (A.last_bias != nullptr) {
-            const uint4 lb = *(const uint4*)(A.last_bias + col);
-            const uint32_t lw[4] = {lb.x, lb.y, lb.z, lb.w};
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] += __uint_as_float((i & 1) ? (lw[i >> 1] & 0xffff0000u) : (lw[i >> 1] << 16));
-          }
-          if (A.add_residual) {
-            const uint4 xr = *(const uint4*)(A.x + n * D + col);
-            const uint32_t xw[4] = {xr.x, xr.y, xr.z, xr.w};
+        pv0[k] = *(const float4*)(orow + k * 64);
+        pv1[k] = *(const float4*)(orow + k * 64 + 4);
+        if constexpr (!SPLIT) {
+          float v[8] = {pv0[k].x, pv0[k].y, pv0[k].z, pv0[k].w, pv1[k].x, pv1[k].y, pv1[k].z, pv1[k].w};
+          if (with_res) {
+            const uint32_t xw[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[i] += __uint_as_float((i & 1) ? (xw[i >> 1] & 0xffff0000u) : (xw[i >> 1] << 16));
           }
-          uint4 o;
-          o.x = pack2_bf16(v[0], v[1]); o.y = pack2_bf16(v[2], v[3]);
-          o.z = pack2_bf16(v[4], v[5]); o.w = pack2_bf16(v[6], v[7]);
-          *(uint4*)(A.out + n * D + col) = o;
+          o[k].x = pack2_bf16(v[0], v[1]); o[k].y = pack2_bf16(v[2], v[3]);
+          o[k].z = pack2_bf16(v[4], v[5]); o[k].w = pack2_bf16(v[6], v[7]);
+        }
+      }
+      if (live) {
+        if constexpr (SPLIT) {
+          float* prow = A.partial + ((int64_t)split * A.part_rows + (n - A.part_base)) * D + c8l * 8;
+#pragma unroll
+          for (int k = 0; k < OP; ++k) {
+            *(float4*)(prow + k * 64) = pv0[k];
+            *(float4*)(prow + k * 64 + 4) = pv1[k];
+          }
+        } else {
+          u32x4* grow = (u32x4*)(A.out + n * D) + c8l;
+#pragma unroll
+          for (int k = 0; k < OP; ++k) grow[k * 8] = o[k];
         }
       }
     }

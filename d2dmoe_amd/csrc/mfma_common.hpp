@@ -13,11 +13,13 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // 16 raw bytes that stay in registers
 
 constexpr int MD_BM = 64;       // tokens per workgroup of the dense sweep
 constexpr int MD_HC = 256;      // hidden neurons per chunk (4 waves x 64)
 constexpr int MD_WAVES = 4;
 constexpr int MD_KS2 = MD_HC / 16;  // K=16 steps of the second GEMM per chunk
+constexpr int MD_MAX_CHUNKS = 32;   // chunks per layer the dense sweep stages tables for (hidden <= 8192)
 constexpr int MD_RING = 32;     // weight fragments kept in flight per wave (16 bytes per lane each)
 constexpr int SP_MAX_MEAN_K = 8;    // the expert-major path is provisioned for at most N * 8 routed pairs
 

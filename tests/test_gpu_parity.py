@@ -200,7 +200,7 @@ def _packed_for(p, act='relu', with_router=False):
 
 @pytest.mark.parametrize('N,E,Ed,density', [(197, 128, 24, 0.8), (197, 128, 24, 0.02), (1576, 128, 24, 0.79), (64, 128, 24, 1.0),
                                             (65, 128, 24, 0.5), (1, 128, 24, 0.5), (300, 24, 128, 0.5), (130, 100, 30, 0.5),
-                                            (100, 7, 5, 0.5)])
+                                            (100, 7, 5, 0.5), (70, 16, 192, 0.5), (96, 160, 16, 0.3)])
 def test_experts_mfma_dense_matches_oracle(N, E, Ed, density):
     _say('experts mfma', N, E, Ed, density)
     x, routing, p = H.random_case(N, 768, E, Ed, 8, seed=N + E, dtype=torch.bfloat16, density=density)
