@@ -114,7 +114,8 @@ __global__ __launch_bounds__(256) void select_kernel(const T* __restrict__ norms
     for (int k = 0; k < SEL_MAX_VPT; ++k) {
       if (k < vpt) {
         const int e = lane + k * kWave;
-        v[k] = (e < E) ? Elem<T>::load(norms + n * E + e) : -INFINITY;
+        const float nv = Elem<T>::load(norms + n * E + (e < E ? e : E - 1));   // unconditional (clamped) load
+        v[k] = (e < E) ? nv : -INFINITY;
         m = nanmax(m, v[k]);
       }
     }
@@ -183,14 +184,21 @@ __global__ __launch_bounds__(256) void perm_count_kernel(const T* __restrict__ r
   int cnt[PERM_MAX_VPT];
 #pragma unroll
   for (int k = 0; k < PERM_MAX_VPT; ++k) cnt[k] = 0;
-  for (int r = 0; r < rows; ++r) {
-    const T* row = routing + (t0 + r) * E;
+  // a lane group's whole segment is requested at once, every load unconditional (clamped address): one round trip
+  // to memory per group of 64 experts
 #pragma unroll
-    for (int k = 0; k < PERM_MAX_VPT; ++k) {
-      if (k < vpt) {
-        const int e = lane + k * kWave;
-        if (e < E) cnt[k] += (Elem<T>::load(row + e) > 0.f) ? 1 : 0;
+  for (int k = 0; k < PERM_MAX_VPT; ++k) {
+    if (k < vpt) {
+      const int e = lane + k * kWave;
+      const int ec = (e < E) ? e : (E - 1);
+      float v[PERM_SEG];
+#pragma unroll
+      for (int i = 0; i < PERM_SEG; ++i) {
+        const int r = (i < rows) ? i : (rows - 1);
+        v[i] = Elem<T>::load(routing + (t0 + r) * E + ec);
       }
+#pragma unroll
+      for (int i = 0; i < PERM_SEG; ++i) cnt[k] += (i < rows && e < E && v[i] > 0.f) ? 1 : 0;
     }
   }
 #pragma unroll
@@ -298,15 +306,34 @@ __global__ __launch_bounds__(256) void perm_scatter_kernel(const T* __restrict__
       }
     }
   }
-  for (int r = 0; r < rows; ++r) {
-    const int64_t tok = t0 + r;
-    const T* row = routing + tok * E;
+  // the segment's routing entries of this lane's experts as bit masks (bit i = token i routes to the expert); a lane
+  // group's rows are requested together, unconditionally (clamped addresses)
+  static_assert(PERM_SEG <= 64, "one 64-bit mask per lane group");
+  unsigned long long onbits[PERM_MAX_VPT];
+#pragma unroll
+  for (int k = 0; k < PERM_MAX_VPT; ++k) {
+    onbits[k] = 0ull;
+    if (k < vpt) {
+      const int e = lane + k * kWave;
+      const int ec = (e < E) ? e : (E - 1);
+      float v[PERM_SEG];
+#pragma unroll
+      for (int i = 0; i < PERM_SEG; ++i) {
+        const int r = (i < rows) ? i : (rows - 1);
+        v[i] = Elem<T>::load(routing + (t0 + r) * E + ec);
+      }
+#pragma unroll
+      for (int i = 0; i < PERM_SEG; ++i) onbits[k] |= (unsigned long long)(v[i] > 0.f ? 1 : 0) << i;
+    }
+  }
+  for (int i = 0; i < rows; ++i) {
+    const int64_t tok = t0 + i;
 #pragma unroll
     for (int k = 0; k < PERM_MAX_VPT; ++k) {
       if (k < vpt) {
         const int e = lane + k * kWave;
         if (e < E) {
-          const bool on = Elem<T>::load(row + e) > 0.f;
+          const bool on = ((onbits[k] >> i) & 1ull) != 0ull;
           // position inside column e of the full (routed first, then the rest) ordering
           const int64_t pos = on ? (int64_t)run[k] : (int64_t)total[k] + (tok - run[k]);
           if (on) token_idx[(int64_t)base[k] + run[k]] = (int32_t)tok;

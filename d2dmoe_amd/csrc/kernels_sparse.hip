@@ -16,11 +16,12 @@
 namespace d2dmoe {
 
 constexpr int SP_BT = 32;        // pairs per tile
-constexpr int SP_SEG = 16;       // tokens per plan segment (one wave); small, so a pass is one round trip to memory
+constexpr int SP_SEG = 32;       // tokens per plan segment (one wave): the tile of the fused router kernel, which can
+                                 // leave the per-segment counts itself
 
 struct SparseWorkspace {
   int64_t n_seg, cap;
-  size_t seg_counts, seg_offsets, totals, seg_pairs, seg_pairbase, offsets, tile_off, flag, tok_off, token_idx, pair_dst, y,
+  size_t seg_counts, seg_offsets, totals, seg_pairs, offsets, tile_off, flag, tok_off, token_idx, pair_dst, y,
       total;
 };
 
@@ -36,7 +37,6 @@ static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) 
   W.seg_offsets = take((size_t)W.n_seg * E * 4);
   W.totals = take((size_t)E * 4);
   W.seg_pairs = take((size_t)W.n_seg * 4);
-  W.seg_pairbase = take((size_t)W.n_seg * 4);
   W.offsets = take((size_t)(E + 1) * 4);
   W.tile_off = take((size_t)(E + 1) * 4);
   W.flag = take(16);
@@ -109,7 +109,7 @@ hipError_t launch_sparse_pack(const d2dmoe_shape& sh, const PackedLayout& L, con
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Plan, pass 1: per segment of 64 tokens (one wave, lanes = experts) the number of routed tokens per expert and the
+// Plan, pass 1: per segment of SP_SEG tokens (one wave, lanes = experts) the number of routed tokens per expert and the
 // segment's number of pairs.
 // ---------------------------------------------------------------------------------------------------
 template <int VPT>
@@ -132,11 +132,11 @@ __global__ __launch_bounds__(256) void plan_count_kernel(const bf16_t* __restric
 #pragma unroll
       for (int i = 0; i < SP_SEG; ++i) {
         const int r = (i < rows) ? i : (rows - 1);
-        v[i] = (e < E) ? routing[(t0 + r) * E + e] : (bf16_t)0;
+        v[i] = routing[(t0 + r) * E + (e < E ? e : E - 1)];   // unconditional (clamped): the loads go out together
       }
 #pragma unroll
       for (int i = 0; i < SP_SEG; ++i)
-        if (i < rows) cnt[k] += ((v[i] & 0x7fff) != 0) ? 1 : 0;   // non-zero routing weight
+        if (i < rows && e < E) cnt[k] += ((v[i] & 0x7fff) != 0) ? 1 : 0;   // non-zero routing weight
     }
   }
   int tot = 0;
@@ -151,125 +151,127 @@ __global__ __launch_bounds__(256) void plan_count_kernel(const bf16_t* __restric
   if (lane == 0) seg_pairs[seg] = tot;
 }
 
-// Plan, pass 3 (after the per-expert scan over segments): expert offsets, tile offsets, segment pair bases, the
-// path flag and tok_off[N].  One workgroup of 1024 threads.
-__global__ __launch_bounds__(1024) void plan_finish_kernel(const int32_t* __restrict__ totals, const int32_t* __restrict__ seg_pairs,
-                                                           int32_t* __restrict__ seg_pairbase, int32_t* __restrict__ offsets,
-                                                           int32_t* __restrict__ tile_off, int32_t* __restrict__ flag,
-                                                           int32_t* __restrict__ tok_off, int E, int64_t n_seg, int64_t N,
-                                                           int64_t cap) {
-  __shared__ int32_t a[1024];
-  __shared__ int32_t b[1024];
-  const int t = threadIdx.x;
-  const int c = (t < E) ? totals[t] : 0;
-  a[t] = c;
-  b[t] = (c + SP_BT - 1) / SP_BT;
-  __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {   // inclusive scans of counts and of tile counts
-    const int va = (t >= off) ? a[t - off] : 0;
-    const int vb = (t >= off) ? b[t - off] : 0;
-    __syncthreads();
-    a[t] += va;
-    b[t] += vb;
-    __syncthreads();
+// Plan, pass 3 (after the per-expert scan over segments): scatter.  A wave walks its segment's tokens in order;
+// lanes = experts, so a lane's running counter is the token's rank inside the expert's list (expert-major position)
+// and a prefix count over the lanes is the expert's rank inside the token's list (token-major position).
+// What a wave needs of the global picture it derives itself from the small arrays of the earlier passes: the experts'
+// offsets (a scan over E totals), its segment's first token-major slot (a sum over the segments before it) and the
+// path flag (all pairs <= capacity).  The first wave also publishes offsets, tile offsets, the flag and tok_off[N]
+// for the kernels that follow, so no single-workgroup pass sits between the scan and this one.
+// ---------------------------------------------------------------------------------------------------
+__device__ inline int wave_incl_scan_i32(int v, int lane) {
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int t = __shfl_up(v, off, 64);
+    if (lane >= off) v += t;
   }
-  if (t < E) {
-    offsets[t + 1] = a[t];
-    tile_off[t + 1] = b[t];
-  }
-  if (t == 0) {
-    offsets[0] = 0;
-    tile_off[0] = 0;
-  }
-  const int64_t P = a[E - 1];
-  if (t == 0) {
-    flag[0] = (P <= cap) ? 1 : 0;
-    tok_off[N] = (int32_t)P;
-  }
-  __syncthreads();
-  // exclusive scan of the segments' pair counts: each thread owns a contiguous run of segments
-  const int64_t per = (n_seg + 1023) / 1024;
-  const int64_t s0 = (int64_t)t * per, s1 = (s0 + per < n_seg) ? (s0 + per) : n_seg;
-  int sum = 0;
-  for (int64_t s = s0; s < s1; ++s) sum += seg_pairs[s];
-  a[t] = sum;
-  __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {
-    const int v = (t >= off) ? a[t - off] : 0;
-    __syncthreads();
-    a[t] += v;
-    __syncthreads();
-  }
-  int run = a[t] - sum;
-  for (int64_t s = s0; s < s1; ++s) {
-    seg_pairbase[s] = run;
-    run += seg_pairs[s];
-  }
+  return v;
 }
 
-// Plan, pass 4: scatter.  A wave walks its 64 tokens in order; lanes = experts, so a lane's running counter is the
-// token's rank inside the expert's list (expert-major position) and a prefix count over the lanes is the expert's
-// rank inside the token's list (token-major position).
 template <int VPT>
 __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restrict__ routing, const int32_t* __restrict__ seg_offsets,
-                                                           const int32_t* __restrict__ seg_pairbase, const int32_t* __restrict__ offsets,
-                                                           const int32_t* __restrict__ flag, int32_t* __restrict__ tok_off,
+                                                           const int32_t* __restrict__ totals, const int32_t* __restrict__ seg_pairs,
+                                                           int32_t* __restrict__ offsets, int32_t* __restrict__ tile_off,
+                                                           int32_t* __restrict__ flag, int32_t* __restrict__ tok_off,
                                                            int32_t* __restrict__ token_idx, int32_t* __restrict__ pair_dst,
-                                                           int64_t N, int E, int64_t n_seg) {
-  if (flag[0] == 0) return;
+                                                           int64_t N, int E, int64_t n_seg, int64_t cap) {
   const int lane = threadIdx.x & 63;
   const int64_t seg = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / 64;
   if (seg >= n_seg) return;
   const int vpt = (E + 63) / 64;
   const int64_t t0 = seg * SP_SEG;
   const int rows = (int)((N - t0) < SP_SEG ? (N - t0) : SP_SEG);
-  int pos[VPT];   // next expert-major position of expert e
+  // Every load of the prologue is issued before anything is computed from it, none of them under a branch (lane
+  // groups past the last expert read clamped addresses and are masked), so the wave pays about one round trip.
+  int tot[VPT], segoff[VPT];
+  unsigned onbits[VPT];    // bit i = token i of the segment routes to expert e
+  static_assert(SP_SEG <= 32, "one 32-bit mask per lane group");
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
-    pos[k] = 0;
-    if (k < vpt) {
-      const int e = lane + k * 64;
-      if (e < E) pos[k] = offsets[e] + seg_offsets[seg * E + e];
+    const int e = lane + k * 64;
+    const int ec = (e < E) ? e : (E - 1);
+    tot[k] = totals[ec];
+    segoff[k] = seg_offsets[seg * E + ec];
+    bf16_t v[SP_SEG];
+#pragma unroll
+    for (int i = 0; i < SP_SEG; ++i) {
+      const int r = (i < rows) ? i : (rows - 1);
+      v[i] = routing[(t0 + r) * E + ec];
     }
+    onbits[k] = 0u;
+#pragma unroll
+    for (int i = 0; i < SP_SEG; ++i) onbits[k] |= ((i < rows && e < E && (v[i] & 0x7fff) != 0) ? 1u : 0u) << i;
   }
-  int tokbase = seg_pairbase[seg];
-  const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-  for (int r0 = 0; r0 < rows; r0 += 4) {
-    bf16_t v[4][VPT];   // four rows fetched together, then walked in order
+  // pairs of all earlier segments = this segment's first token-major slot; eight loads per trip
+  int before_segs = 0;
+  for (int64_t s0 = 0; s0 < seg; s0 += 512) {
+    int part[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = (r0 + i < rows) ? (r0 + i) : (rows - 1);
-      const bf16_t* row = routing + (t0 + r) * E;
-#pragma unroll
-      for (int k = 0; k < VPT; ++k)
-        if (k < vpt) {
-          const int e = lane + k * 64;
-          v[i][k] = (e < E) ? row[e] : (bf16_t)0;
-        }
+    for (int u = 0; u < 8; ++u) {
+      const int64_t sgi = s0 + u * 64 + lane;
+      part[u] = seg_pairs[sgi < seg ? sgi : 0];
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (r0 + i < rows) {   // uniform
-        const int64_t tok = t0 + r0 + i;
-        int before = 0;   // routed experts of this token with a smaller index, over the previous lane groups
+    for (int u = 0; u < 8; ++u) before_segs += (s0 + u * 64 + lane < seg) ? part[u] : 0;
+  }
+  before_segs = wave_sum_i32(before_segs);
+  // exclusive scans over the experts (e = lane + 64 k) of the pair counts and of the tile counts
+  int eoff[VPT], toff[VPT];
+  int run = 0, trun = 0;
 #pragma unroll
-        for (int k = 0; k < VPT; ++k) {
-          if (k < vpt) {
-            const bool on = (v[i][k] & 0x7fff) != 0;
-            const unsigned long long bal = __ballot(on);
-            if (on) {
-              const int rank_in_token = before + __popcll(bal & lt_mask);
-              token_idx[pos[k]] = (int32_t)tok;
-              pair_dst[pos[k]] = tokbase + rank_in_token;
-              pos[k] += 1;
-            }
-            before += __popcll(bal);
-          }
-        }
-        if (lane == 0) tok_off[tok] = tokbase;
-        tokbase += before;
+  for (int k = 0; k < VPT; ++k) {
+    const int e = lane + k * 64;
+    const int c = (e < E) ? tot[k] : 0;
+    const int tc = (c + SP_BT - 1) / SP_BT;
+    const int ci = wave_incl_scan_i32(c, lane), ti = wave_incl_scan_i32(tc, lane);
+    eoff[k] = run + ci - c;
+    toff[k] = trun + ti - tc;
+    run += __shfl(ci, 63, 64);
+    trun += __shfl(ti, 63, 64);
+  }
+  const int64_t P = run;
+  const bool sparse_ok = P <= cap;
+  if (seg == 0) {
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int e = lane + k * 64;
+      if (e < E) {
+        offsets[e] = eoff[k];
+        tile_off[e] = toff[k];
       }
     }
+    if (lane == 0) {
+      offsets[E] = run;
+      tile_off[E] = trun;
+      flag[0] = sparse_ok ? 1 : 0;
+      tok_off[N] = (int32_t)P;
+    }
+  }
+  if (!sparse_ok) return;
+  int pos[VPT];            // next expert-major position of expert e
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) pos[k] = eoff[k] + segoff[k];
+  int tokbase = before_segs;
+  const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int i = 0; i < rows; ++i) {
+    const int64_t tok = t0 + i;
+    int before = 0;   // routed experts of this token with a smaller index, over the previous lane groups
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      if (k < vpt) {
+        const bool on = ((onbits[k] >> i) & 1u) != 0u;
+        const unsigned long long bal = __ballot(on);
+        if (on) {
+          const int rank_in_token = before + __popcll(bal & lt_mask);
+          token_idx[pos[k]] = (int32_t)tok;
+          pair_dst[pos[k]] = tokbase + rank_in_token;
+          pos[k] += 1;
+        }
+        before += __popcll(bal);
+      }
+    }
+    if (lane == 0) tok_off[tok] = tokbase;
+    tokbase += before;
   }
 }
 
@@ -470,7 +472,6 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   int32_t* seg_offsets = (int32_t*)(ws + W.seg_offsets);
   int32_t* totals = (int32_t*)(ws + W.totals);
   int32_t* seg_pairs = (int32_t*)(ws + W.seg_pairs);
-  int32_t* seg_pairbase = (int32_t*)(ws + W.seg_pairbase);
   int32_t* offsets = (int32_t*)(ws + W.offsets);
   int32_t* tile_off = (int32_t*)(ws + W.tile_off);
   int32_t* flag = (int32_t*)(ws + W.flag);
@@ -487,11 +488,10 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   else if (vpt <= 8) D2DMOE_PLAN_DISPATCH(8); else D2DMOE_PLAN_DISPATCH(16);
 #undef D2DMOE_PLAN_DISPATCH
   launch_perm_scan(seg_counts, seg_offsets, totals, E, W.n_seg, s);
-  hipLaunchKernelGGL(plan_finish_kernel, dim3(1), dim3(1024), 0, s, totals, seg_pairs, seg_pairbase, offsets, tile_off, flag,
-                     tok_off, E, W.n_seg, N, N * (int64_t)max_mean_k);
 #define D2DMOE_PLAN_DISPATCH(V)                                                                                          \
   hipLaunchKernelGGL(plan_scatter_kernel<V>, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_offsets,    \
-                     seg_pairbase, offsets, flag, tok_off, token_idx, pair_dst, N, E, W.n_seg)
+                     totals, seg_pairs, offsets, tile_off, flag, tok_off, token_idx, pair_dst, N, E, W.n_seg,           \
+                     N * (int64_t)max_mean_k)
   if (vpt <= 1) D2DMOE_PLAN_DISPATCH(1); else if (vpt <= 2) D2DMOE_PLAN_DISPATCH(2); else if (vpt <= 4) D2DMOE_PLAN_DISPATCH(4);
   else if (vpt <= 8) D2DMOE_PLAN_DISPATCH(8); else D2DMOE_PLAN_DISPATCH(16);
 #undef D2DMOE_PLAN_DISPATCH
