@@ -306,6 +306,20 @@ def run_gpt2(args, dev):
                              args.steps, args.warmup)
     active = r0.float().sum().item() * 4.0 * 768 * 24
     N = B * T
+    # the literal rule (keep norm >= tau * max) on the same model: module tau = 1 - tau
+    for layer in layers:
+        layer.tau = 1.0 - args.tau
+    lit_k = {}
+    hooks = [layer.register_forward_hook(lambda m, inp, out, n=n: lit_k.__setitem__(n, out[1][n][0].float().sum(-1).mean().item()))
+             for n, layer in zip(names, layers)]
+    moe(idx)
+    for h in hooks:
+        h.remove()
+    torch.cuda.synchronize()
+    ms_lit_model = time_events(lambda: moe(idx), args.steps, args.warmup)
+    ms_lit_layers = sum(time_events(lambda: layer(captured[n][0]), args.steps, args.warmup) for n, layer in zip(names, layers))
+    for layer in layers:
+        layer.tau = args.tau
     line = {
         'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
         'value': N / ms_moe_model * 1e3, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
@@ -315,6 +329,9 @@ def run_gpt2(args, dev):
                                f'(gelu, biases), router 768->128->128, module tau={args.tau}; one step = one model forward'},
         'moe_layers_ms': ms_moe_layers, 'moe_share_of_model': ms_moe_layers / ms_moe_model,
         'dense_model_ms': ms_dense_model, 'dense_ffn_layer_ms': ms_dense_ffn, 'per_layer': per_layer,
+        'literal_rule': {'rule': f'keep norm >= {args.tau}*max', 'model_ms': ms_lit_model, 'tokens_per_s': N / ms_lit_model * 1e3,
+                         'moe_layers_ms': ms_lit_layers,
+                         'mean_active_experts': sum(lit_k.values()) / max(len(lit_k), 1)},
         'roofline': {'bound': 'mfma', 'kernel': 'experts (first MoE layer, its real input and routing)',
                      'achieved': active / ms_experts / 1e9, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': active / ms_experts / 1e9 / PEAK_BF16_TFLOPS, 'traffic': None, 'kernel_ms': ms_experts},
