@@ -289,6 +289,7 @@ struct SparseArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* w1s; const bf16x8* w2s; const bf16_t* b1s;
   const int32_t* offsets; const int32_t* tile_off; const int32_t* token_idx; const int32_t* pair_dst; const int32_t* flag;
   bf16_t* y; int E; int act_rt;
+  const int32_t* tok_off; const bf16_t* last_bias; bf16_t* out; int add_residual;   // tokens with ONE routed expert
 };
 
 template <int D, int NT, int ACT>
@@ -299,9 +300,11 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
   static_assert(KS1 % 4 == 0, "the model dimension must split over four waves");
   __shared__ int32_t s_tile_off[1025];
   __shared__ float part[4][NT * 16][64];
+  __shared__ __attribute__((aligned(16))) bf16_t s_last_bias[D];
   if (A.flag[0] == 0) return;
   const int E = A.E;
   for (int i = threadIdx.x; i <= E; i += 256) s_tile_off[i] = A.tile_off[i];
+  for (int i = threadIdx.x; i < D; i += 256) s_last_bias[i] = (A.last_bias != nullptr) ? A.last_bias[i] : (bf16_t)0;
   __syncthreads();
   const int n_tiles = s_tile_off[E];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -321,6 +324,9 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
     const int pj = base + j0 + (valid ? c32 : rows - 1);
     const int tok = A.token_idx[pj];
     const int dst = A.pair_dst[pj];
+    // A token with a single routed expert has nothing to be summed with: its row leaves this kernel as the finished
+    // output row (float32 accumulator + last_bias (+ x), one rounding) and the combine kernel skips the token.
+    const bool single = valid && (A.tok_off[tok + 1] - A.tok_off[tok] == 1);
     const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)tok * D) + 2 * w * KQ + g;
     const float rw = bf16_to_f32(A.routing[(int64_t)tok * E + e]);
 
@@ -392,8 +398,34 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
 #pragma unroll
       for (int ks2 = 0; ks2 < 2 * NT; ++ks2)
         acc2[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w2r[ct * 2 * NT + ks2], hb[ks2], acc2[ct], 0, 0, 0);
+    const bool any_single = __ballot(single) != 0ull;   // uniform
+    const int col0 = w * (D / 4) + 4 * g;
+    bf16_t* yrow = single ? (A.out + (int64_t)tok * D + col0) : (A.y + (int64_t)dst * D + col0);
+    if (any_single) {
+      // the bias (and residual) pieces are fetched by every lane, unconditionally, and added under a mask
+      const uint32_t keep = single ? 0xffffffffu : 0u;
+      const bf16_t* xres = A.x + (int64_t)tok * D + col0;
+#pragma unroll
+      for (int ct = 0; ct < CTW; ++ct)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint2 lb = *(const uint2*)(s_last_bias + col0 + ct * 32 + 8 * q);
+          lb.x &= keep; lb.y &= keep;
+          acc2[ct][q * 4 + 0] += __uint_as_float(lb.x << 16);
+          acc2[ct][q * 4 + 1] += __uint_as_float(lb.x & 0xffff0000u);
+          acc2[ct][q * 4 + 2] += __uint_as_float(lb.y << 16);
+          acc2[ct][q * 4 + 3] += __uint_as_float(lb.y & 0xffff0000u);
+          if (A.add_residual) {   // uniform
+            uint2 xv = *(const uint2*)(xres + ct * 32 + 8 * q);
+            xv.x &= keep; xv.y &= keep;
+            acc2[ct][q * 4 + 0] += __uint_as_float(xv.x << 16);
+            acc2[ct][q * 4 + 1] += __uint_as_float(xv.x & 0xffff0000u);
+            acc2[ct][q * 4 + 2] += __uint_as_float(xv.y << 16);
+            acc2[ct][q * 4 + 3] += __uint_as_float(xv.y & 0xffff0000u);
+          }
+        }
+    }
     if (valid) {
-      bf16_t* yrow = A.y + (int64_t)dst * D + w * (D / 4) + 4 * g;
 #pragma unroll
       for (int ct = 0; ct < CTW; ++ct)
 #pragma unroll
@@ -422,6 +454,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   const int q0 = tok_off[n], q1 = tok_off[n + 1];
+  if (q1 - q0 == 1) return;   // finished by the experts kernel
   for (int q = q0; q < q1; ++q) {
     const uint4 v = *(const uint4*)(y + (int64_t)q * D + col);
     const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
@@ -500,6 +533,7 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   A.w2s = (const bf16x8*)(pk + L.s2_off); A.b1s = (const bf16_t*)(pk + L.sb_off); A.offsets = offsets;
   A.tile_off = tile_off; A.token_idx = token_idx; A.pair_dst = pair_dst; A.flag = flag; A.y = y; A.E = E;
   A.act_rt = sh.activation;
+  A.tok_off = tok_off; A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.add_residual = sh.add_residual;
   const unsigned grid = (unsigned)(8 * device_cu_count());
   if (L.nt == 1) launch_sparse_experts<1>(A, sh.activation, grid, s);
   else if (L.nt == 2) launch_sparse_experts<2>(A, sh.activation, grid, s);

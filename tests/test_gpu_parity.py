@@ -280,6 +280,13 @@ def test_experts_mfma_sparse_activations_weights_edges(act):
     one[:, 77] = 1
     got = _experts_got(x, one, p, act, path='mfma_sparse', packed=packed)
     assert H.rel_err(got, _experts_want(x, one, p, act)) < H.TOL_BF16
+    # tokens with ONE routed expert are finished inside the experts kernel: weighted, with the residual, without last_bias
+    lone = torch.zeros_like(routing)
+    lone[torch.arange(500), torch.arange(500) % 128] = 0.75
+    lone[::7, 5] = 1.0   # some tokens get a second expert and go through the combine kernel
+    q = {k: v for k, v in p.items() if k != 'last_bias'}
+    got = _experts_got(x, lone, q, act, residual=True, path='mfma_sparse', packed=_packed_for(q, act))
+    assert H.rel_err(got, _experts_want(x, lone, q, act, True)) < H.TOL_BF16
 
 
 def test_experts_mfma_sparse_full_size_and_auto_switch():
