@@ -214,7 +214,7 @@ __global__ __launch_bounds__(256) void perm_count_kernel(const T* __restrict__ r
 // segments); a workgroup has 16 waves, lanes = experts.  A workgroup first adds up everything before its block (its
 // waves share that range), then wave w scans its own slice of the block; partial sums meet in LDS.  Integer sums, so
 // the result does not depend on the split.
-constexpr int PERM_SCAN_BLOCKS = 16;
+constexpr int PERM_SCAN_BLOCKS = 32;
 
 __global__ __launch_bounds__(1024) void perm_scan_kernel(const int32_t* __restrict__ seg_counts,
                                                          int32_t* __restrict__ seg_offsets, int32_t* __restrict__ totals,
