@@ -167,6 +167,26 @@ class MoeficationMoE(MoELayer):
         return self.router is not None and (self.router.test_override_outputs_p is not None
                                             or self.router.hip_compatible())
 
+    def _router_operands(self):
+        """(router_w1, router_w2, hidden activation, output activation) as the fused HIP call takes them; the weights are
+        None when the router's outputs are overridden (test hook) and the norms are passed in instead."""
+        router = self.router
+        if router.test_override_outputs_p is not None:
+            rw1 = rw2 = None
+        else:
+            rw1, rw2 = router.layers[0].weight, router.layers[2].weight
+        ract = router.activation if router.activation in ACT else 'relu'
+        roact = router.output_activation if router.output_activation in ACT else 'abs'
+        return rw1, rw2, ract, roact
+
+    def packed_weights(self):
+        """The derived, MFMA-ordered weight buffer the fused forward of this layer uses (built on first use, rebuilt when
+        a parameter changes); None where no MFMA kernel applies.  Calling it ahead of time moves the packing out of the
+        first forward."""
+        if not isinstance(self.experts, HipKernelExperts) or self.router is None or not self.router.hip_compatible():
+            return None
+        return self.experts.packed_weights(*self._router_operands())
+
     def forward(self, x):
         orig_size = x.size()
         if self._fused_ok(x):
@@ -174,14 +194,10 @@ class MoeficationMoE(MoELayer):
             x2 = x.reshape(-1, x.size(-1)).contiguous()
             router = self.router
             last_bias = self.last_bias.view(-1) if self.bias else None
+            norms_in = None
             if router.test_override_outputs_p is not None:
                 norms_in = router(x).reshape(-1, self.num_experts).contiguous()
-                rw1 = rw2 = None
-            else:
-                norms_in = None
-                rw1, rw2 = router.layers[0].weight, router.layers[2].weight
-            ract = router.activation if router.activation in ACT else 'relu'
-            roact = router.output_activation if router.output_activation in ACT else 'abs'
+            rw1, rw2, ract, roact = self._router_operands()
             out, routing, _, counts = ops.forward(
                 x2, rw1, rw2, float(1.0 - self.tau), ex.w1, ex.b1, ex.w2, None, last_bias, ex.activation_str,
                 self.add_residual_connection, norms_in=norms_in, want_counts=self.collect_counts, path=ex.kernel_path,

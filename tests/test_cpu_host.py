@@ -285,3 +285,82 @@ def test_gpt_dynk_max_on_cpu_matches_oracle_layer():
     assert torch.equal(captured['routing'], want_routing.view_as(captured['routing']))
     assert H.rel_err(captured['out'], want_out.view_as(captured['out'])) < 1e-5
     assert 0 < captured['routing'].mean().item() < 1
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Checkpoint import (reference: train.py:295-320 writes final.pth; utils.py:580-672 rebuilds and load_state_dict()s)
+# ---------------------------------------------------------------------------------------------------------------------
+def _tiny_moe_gpt(seed):
+    from d2dmoe_amd import add_routers, gpt2
+    torch.manual_seed(seed)
+    cfg = gpt2.GPTConfig(block_size=16, vocab_size=64, n_layer=2, n_head=2, n_embd=32)
+    dense = gpt2.GPT(cfg).eval()
+    moe, names = gpt2.replace_with_moes(dense, num_experts=8, experts_class='hip_kernel')
+    gpt2.split_original_parameters(dense, moe, names)
+    add_routers(moe, dict(width=16, depth=2, bias=False, activation='relu', output_activation='abs'))
+    return moe, names
+
+
+def test_reference_checkpoint_layout_loads_unchanged(tmp_path):
+    import d2dmoe_amd as P
+    src, names = _tiny_moe_gpt(0)
+    state = src.state_dict()
+    # the parameter names and shapes a reference model_state carries for a MoE layer
+    n0 = names[0]
+    assert tuple(state[f'{n0}.experts.w1'].shape) == (8, 32, 16)
+    assert tuple(state[f'{n0}.experts.b1'].shape) == (8, 16)
+    assert tuple(state[f'{n0}.experts.w2'].shape) == (8, 16, 32)
+    assert tuple(state[f'{n0}.last_bias'].shape) == (1, 32)
+    assert tuple(state[f'{n0}.router.layers.0.weight'].shape) == (16, 32)
+    assert tuple(state[f'{n0}.router.layers.2.weight'].shape) == (8, 16)
+    # final.pth as the reference's driver writes it, minus the arbitrary `args` object; keys wrapped as accelerate
+    # / DataParallel / torch.compile leave them
+    path = tmp_path / 'final.pth'
+    wrapped = {'module._orig_mod.' + k: v for k, v in state.items()}
+    torch.save({'model_state': wrapped, 'final_score': 0.5, 'model_flops': 123}, path)
+    got = P.read_model_state(path)
+    assert set(got) == set(state)
+    dst, _ = _tiny_moe_gpt(1)
+    assert not torch.equal(dst.state_dict()[f'{n0}.experts.w1'], state[f'{n0}.experts.w1'])
+    missing, unexpected = P.load_model_state(dst, got)
+    assert missing == [] and unexpected == []
+    for k, v in state.items():
+        assert torch.equal(dst.state_dict()[k], v), k
+    idx = torch.randint(0, 64, (2, 16), generator=torch.Generator().manual_seed(3))
+    from d2dmoe_amd import gpt2
+    for m in (src, dst):
+        for n in names:
+            layer = gpt2.get_module_by_name(m, n)
+            layer.forward_mode, layer.tau = 'dynk_max', 0.9
+            layer.experts.forward_mode = 'naive'
+    with torch.no_grad():
+        assert torch.equal(src(idx)[0], dst(idx)[0])
+    # a bare state dict is accepted as well
+    torch.save(state, tmp_path / 'bare.pth')
+    assert set(P.read_model_state(tmp_path / 'bare.pth')) == set(state)
+
+
+def test_checkpoint_import_refuses_what_it_should(tmp_path):
+    import argparse
+    import d2dmoe_amd as P
+    src, names = _tiny_moe_gpt(0)
+    # an arbitrary Python object in the file: the safe loader refuses it and the error says what to do
+    torch.save({'args': argparse.Namespace(lr=0.1), 'model_state': src.state_dict()}, tmp_path / 'with_args.pth')
+    with pytest.raises(ValueError, match='weights_only'):
+        P.read_model_state(tmp_path / 'with_args.pth')
+    torch.save({'model_state': [1, 2, 3]}, tmp_path / 'junk.pth')
+    with pytest.raises(ValueError, match='state dict'):
+        P.read_model_state(tmp_path / 'junk.pth')
+    # converted with another number of experts: named shape error instead of a wall of mismatches
+    from d2dmoe_amd import gpt2
+    torch.manual_seed(0)
+    cfg = gpt2.GPTConfig(block_size=16, vocab_size=64, n_layer=2, n_head=2, n_embd=32)
+    other, _ = gpt2.replace_with_moes(gpt2.GPT(cfg).eval(), num_experts=4, experts_class='hip_kernel')
+    state = {k: v for k, v in src.state_dict().items() if 'router' not in k}
+    with pytest.raises(ValueError, match='number of experts'):
+        P.load_model_state(other, state)
+    # prefixes are only stripped when every key carries them
+    mixed = {'module.a': torch.zeros(1), 'b': torch.zeros(1)}
+    assert set(P.strip_wrapper_prefixes(mixed)) == {'module.a', 'b'}
+    # without a GPU there is nothing to pack
+    assert P.prepack(src) == 0

@@ -612,9 +612,21 @@ def test_gpt_with_hip_moe_layers(shape, dtype):
     for n in names:
         layer = gpt2.get_module_by_name(moe, n)
         layer.forward_mode, layer.tau = 'dynk_max', 0.5
+    # packing ahead of time: the buffers the first forward would build, and the forward then reuses them
+    from d2dmoe_amd import prepack
+    nbytes = prepack(moe)
+    layers = [gpt2.get_module_by_name(moe, n) for n in names]
+    if dtype == torch.bfloat16 and shape != 'tiny':
+        assert nbytes > 0
+    ahead = [layer.packed_weights() for layer in layers]
+    assert nbytes == sum(pk.numel() * pk.element_size() for pk in ahead if pk is not None)
     with torch.no_grad():
         moe(idx)
         torch.cuda.synchronize()
+    for layer, pk in zip(layers, ahead):
+        now = layer.packed_weights()
+        assert (now is None and pk is None) or now.data_ptr() == pk.data_ptr()
+    with torch.no_grad():
         torch.cuda.set_sync_debug_mode('error')
         try:
             out, gating = moe(idx, return_gating_data=True)
