@@ -339,6 +339,41 @@ def run_gpt2(args, dev):
     print(json.dumps(line))
 
 
+def run_norms(args, ops, dev):
+    """Router-training targets: the L2 norm of every expert's output for every token (ViT-B layer, 256 x 197 tokens),
+    by the HIP kernel and, beside it, by the reference's route on the same GPU (masked-mode stubs + vector_norm over
+    the [E,N,D] outputs).  One step = one pass over the batch."""
+    from d2dmoe_amd import HipKernelExperts
+    torch.manual_seed(0)
+    B, T, D, E, Ed = 256, 197, 768, 128, 24
+    N = B * T
+    ex = HipKernelExperts(D, E, 2, Ed, 'without_last', torch.nn.ReLU).to(dev).bfloat16()
+    ex.b1.normal_(0.0, 0.1)
+    x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).bfloat16().to(dev)
+
+    def stubs():
+        h = ex.intermediate_activation_extraction_stub(x.unsqueeze(0), ex.w1, ex.b1, ex.act)
+        return torch.linalg.vector_norm(ex.output_activation_extraction_stub(h, ex.w2), ord=2, dim=-1)
+
+    ms = time_events(lambda: ex.output_norms(x), args.steps, args.warmup)
+    ms_stubs = time_events(stubs, 3, 1)
+    executed = N * E * 2.0 * D * 32          # first product with experts padded to 32 neurons
+    useful = N * E * 2.0 * D * Ed
+    line = {
+        'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
+        'value': N / ms * 1e3, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': ms, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16',
+        'data': 'synthetic',
+        'config': {'workload': f'vit_b_50k_norms: per-expert output norms (router-training targets), {B}x{T}={N} tokens, '
+                               f'D={D}, {E} experts x {Ed}, relu; one step = norms [E,N] of one batch'},
+        'reference_route_ms': ms_stubs,
+        'roofline': {'bound': 'mfma', 'kernel': 'expert_norms_kernel', 'achieved': useful / ms / 1e9, 'peak': PEAK_BF16_TFLOPS,
+                     'unit': 'TFLOP/s', 'frac': useful / ms / 1e9 / PEAK_BF16_TFLOPS, 'traffic': None, 'kernel_ms': ms,
+                     'executed_tflops': executed / ms / 1e9},
+    }
+    print(json.dumps(line))
+
+
 def cpu_baseline(D, E, Ed, W, act, tau, budget_s=12.0):
     """The oracle's restatement of the reference CPU path (router -> dynk_max gate -> per-expert loop), float32,
     8 x 197 tokens of the same layer shape, repeated until about budget_s seconds have been spent."""
@@ -368,7 +403,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS) + sorted(GATED_WORKLOADS) + ['gpt2_small'])
+    ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS) + sorted(GATED_WORKLOADS) + ['gpt2_small', 'vit_b_50k_norms'])
     ap.add_argument('--tau', type=float, default=0.9, help='module tau (keep expert when norm >= (1 - tau) * max)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-sweep', action='store_true', help='skip the threshold sweep (5 values x 2 readings)')
@@ -401,6 +436,10 @@ def main():
     if args.workload == 'gpt2_small':
         with torch.no_grad():
             run_gpt2(args, dev)
+        return
+    if args.workload == 'vit_b_50k_norms':
+        with torch.no_grad():
+            run_norms(args, ops, dev)
         return
     B, T, D, E, Ed, W, act = WORKLOADS[args.workload]
     N = B * T

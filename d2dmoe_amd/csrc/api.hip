@@ -283,4 +283,29 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
                         plan.total - plan.perm_off, stream);
 }
 
+size_t d2dmoe_norms_packed_bytes(const d2dmoe_shape* shape) {
+  if (check_shape(shape) != D2DMOE_OK) return 0;
+  return mfma_norms_packed_bytes(*shape);
+}
+
+int d2dmoe_pack_norms(const d2dmoe_shape* shape, const void* w1, const void* b1, const void* w2, void* packed,
+                      size_t packed_bytes, void* stream) {
+  int st = check_shape(shape);
+  if (st != D2DMOE_OK) return st;
+  if (!w1 || !w2 || !packed) return D2DMOE_E_NULL;
+  if (!mfma_norms_supported(*shape)) return D2DMOE_E_UNSUPPORTED;
+  if (packed_bytes < mfma_norms_packed_bytes(*shape) || !aligned16(packed)) return D2DMOE_E_WORKSPACE;
+  return (int)launch_norms_pack(*shape, w1, b1, w2, packed, (hipStream_t)stream);
+}
+
+int d2dmoe_expert_output_norms(const d2dmoe_shape* shape, const void* x, const void* packed, void* norms, void* stream) {
+  int st = check_shape(shape);
+  if (st != D2DMOE_OK) return st;
+  if (shape->n_tokens == 0) return D2DMOE_OK;
+  if (!x || !packed || !norms) return D2DMOE_E_NULL;
+  if (!mfma_norms_supported(*shape)) return D2DMOE_E_UNSUPPORTED;
+  if (!aligned16(x) || !aligned16(packed)) return D2DMOE_E_ALIGN;
+  return (int)launch_mfma_norms(*shape, x, packed, norms, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -79,4 +79,10 @@ hipError_t launch_mfma_gemm(const d2dmoe_shape& sh, const void* x, const void* r
                             const void* last_bias, void* out, void* workspace, hipStream_t s);
 void launch_perm_scan(const int32_t* seg_counts, int32_t* seg_offsets, int32_t* totals, int E, int64_t n_seg, hipStream_t s);
 
+// ---- per-expert output norms, the router-training targets (kernels_norms.hip) ----
+bool mfma_norms_supported(const d2dmoe_shape& sh);
+size_t mfma_norms_packed_bytes(const d2dmoe_shape& sh);
+hipError_t launch_norms_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, void* packed, hipStream_t s);
+hipError_t launch_mfma_norms(const d2dmoe_shape& sh, const void* x, const void* packed, void* norms, hipStream_t s);
+
 }  // namespace d2dmoe

@@ -121,6 +121,7 @@ class HipKernelExperts(ExpertsLayer):
         self.intermediate_activation_extraction_stub = _IntermediateStub()
         self.output_activation_extraction_stub = _OutputStub()
         self._packed = _PackedCache()
+        self._norms_packed = None   # (key, buffer) of the derived buffer output_norms() uses
 
     @property
     def forward_mode(self):
@@ -139,6 +140,26 @@ class HipKernelExperts(ExpertsLayer):
                             self.activation_str, router_activation=router_activation,
                             router_output_activation=router_output_activation)
         return self._packed.get(sh, (self.w1, self.b1, self.w2, None, router_w1, router_w2))
+
+    def output_norms(self, x):
+        """L2 norm of every expert's output for every token, [E,N]: the router-training targets the reference reads off
+        a forward hook on `output_activation_extraction_stub` in 'masked' mode (train_routers.py:49-86,
+        utils.py:353-369).  On a ROCm device in bf16 with D = 768 and experts of at most 32 neurons one HIP kernel computes
+        them without forming the [E,N,D] outputs; anything else takes the reference's own route through the stubs."""
+        assert x.dim() == 2, f'{x.size()=}'
+        if x.is_cuda and not (torch.is_grad_enabled() and (x.requires_grad or self.w1.requires_grad)):
+            sh = ops.make_shape(0, self.hidden_dim, self.num_experts, self.expert_dim, 0, ops._dtype_code(x),
+                                self.activation_str) if x.dtype in (torch.bfloat16, torch.float32) else None
+            if sh is not None and x.dtype == self.w1.dtype:
+                key = tuple((t.data_ptr(), t._version, t.dtype, t.device) for t in (self.w1, self.b1, self.w2))
+                if self._norms_packed is None or self._norms_packed[0] != key:
+                    self._norms_packed = (key, ops.pack_norms(sh, self.w1, self.b1, self.w2))
+                if self._norms_packed[1] is not None:
+                    return ops.expert_output_norms(x.contiguous(), self.w1, self.b1, self.w2, self.activation_str,
+                                                   self._norms_packed[1])
+        h = self.intermediate_activation_extraction_stub(x.unsqueeze(0), self.w1, self.b1, self.act)
+        y = self.output_activation_extraction_stub(h, self.w2)
+        return torch.linalg.vector_norm(y, ord=2, dim=-1)
 
     # -- forward ----------------------------------------------------------------------------
     def forward(self, x, routing_tensor):

@@ -23,6 +23,7 @@ EXPORTS = (
     'd2dmoe_version', 'd2dmoe_status_string', 'd2dmoe_workspace_bytes', 'd2dmoe_router', 'd2dmoe_select',
     'd2dmoe_router_select',
     'd2dmoe_build_permutation', 'd2dmoe_experts', 'd2dmoe_packed_bytes', 'd2dmoe_pack_weights', 'd2dmoe_forward',
+    'd2dmoe_norms_packed_bytes', 'd2dmoe_pack_norms', 'd2dmoe_expert_output_norms',
 )
 
 
@@ -75,6 +76,12 @@ def load() -> ctypes.CDLL:
     lib.d2dmoe_pack_weights.argtypes = [SH, P, P, P, P, P, P, P, SZ, P]
     lib.d2dmoe_forward.restype = ctypes.c_int
     lib.d2dmoe_forward.argtypes = [SH, P, P, P, c_float, P, P, P, P, P, P, P, P, P, P, P, I32, P, SZ, P]
+    lib.d2dmoe_norms_packed_bytes.restype = SZ
+    lib.d2dmoe_norms_packed_bytes.argtypes = [SH]
+    lib.d2dmoe_pack_norms.restype = ctypes.c_int
+    lib.d2dmoe_pack_norms.argtypes = [SH, P, P, P, P, SZ, P]
+    lib.d2dmoe_expert_output_norms.restype = ctypes.c_int
+    lib.d2dmoe_expert_output_norms.argtypes = [SH, P, P, P, P]
     _lib = lib
     return lib
 

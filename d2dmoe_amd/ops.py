@@ -160,6 +160,38 @@ def pack_weights(shape: abi.Shape, w1, b1, w2, w_up=None, router_w1=None, router
     return packed
 
 
+def pack_norms(shape: abi.Shape, w1, b1, w2) -> Optional[torch.Tensor]:
+    """Derived buffer of d2dmoe_expert_output_norms (first-layer fragments, bias, per-expert Gram matrices), or None
+    when the kernel does not cover the shape."""
+    dev = _require_gpu(w1, b1, w2)
+    lib = abi.load()
+    nbytes = lib.d2dmoe_norms_packed_bytes(ctypes.byref(shape))
+    if nbytes == 0:
+        return None
+    packed = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    abi.check(lib.d2dmoe_pack_norms(ctypes.byref(shape), _ptr(w1), _ptr(b1), _ptr(w2), _ptr(packed), nbytes, _stream()),
+              'd2dmoe_pack_norms')
+    return packed
+
+
+def expert_output_norms(x: torch.Tensor, w1: torch.Tensor, b1: Optional[torch.Tensor], w2: torch.Tensor,
+                        activation: str = 'relu', packed: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """norms [E,N] = | act(x w1[e] + b1[e]) w2[e] |_2 through d2dmoe_expert_output_norms (bf16, D = 768, Ed <= 32)."""
+    dev = _require_gpu(x, w1, b1, w2, packed)
+    lib = abi.load()
+    n, d = x.shape
+    e, _, ed = w1.shape
+    sh = make_shape(n, d, e, ed, 0, _dtype_code(x), activation)
+    if packed is None:
+        packed = pack_norms(sh, w1, b1, w2)
+    if packed is None:
+        raise abi.D2DMoEError('d2dmoe_expert_output_norms does not cover this shape (bf16, D = 768, experts of <= 32 neurons)')
+    out = torch.empty(e, n, dtype=x.dtype, device=dev)
+    abi.check(lib.d2dmoe_expert_output_norms(ctypes.byref(sh), _ptr(x), _ptr(packed), _ptr(out), _stream()),
+              'd2dmoe_expert_output_norms')
+    return out
+
+
 def experts(x: torch.Tensor, routing: torch.Tensor, w1: torch.Tensor, b1: Optional[torch.Tensor], w2: torch.Tensor,
             w_up: Optional[torch.Tensor] = None, last_bias: Optional[torch.Tensor] = None, activation: str = 'relu',
             add_residual: bool = False, path: str = 'auto', packed: Optional[torch.Tensor] = None) -> torch.Tensor:

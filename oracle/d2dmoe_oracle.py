@@ -24,6 +24,9 @@ mathematical; they live in tests/test_oracle_pins.py):
                         pinned: composition equals experts_forward_all on 0/1 routing
   gated variants        pinned: same three formulations with act(gate) * up
   moe_layer_forward     pinned: composition of the above + bias/residual closed form
+  expert_output_norms   pinned: per-(token, expert) brute force in numpy float64; the Gram identity
+                        |h W2|^2 = h (W2 W2^T) h^T; zero second layer -> zeros; one expert, identity
+                        activation -> |x A| for the product matrix A through a library GEMM
   activations           pinned: torch.nn.functional counterparts / closed forms in float64
 
 No function is "parity unpinned".
@@ -255,6 +258,23 @@ def experts_forward_all(x: torch.Tensor, routing: torch.Tensor, w1: torch.Tensor
     h = ACTIVATIONS[activation](h)
     y = torch.einsum('eni,eio->eno', h, w2)
     return torch.einsum('end,ne->nd', y, routing)
+
+
+def expert_output_norms(x: torch.Tensor, w1: torch.Tensor, b1: Optional[torch.Tensor], w2: torch.Tensor,
+                        activation: str = 'relu') -> torch.Tensor:
+    """L2 norm of every expert's output for every token: the regression targets of router training.
+
+    The reference runs the layer in 'masked' mode, captures the output of
+    `output_activation_extraction_stub` ([E,N,D], moe_layers.py:125-133, 193-198) with a forward hook and takes
+    `torch.linalg.vector_norm(output, ord=2, dim=-1)` (utils.py:353-369, train_routers.py:49-86).
+    x [N,D], w1 [E,D,Ed], b1 [E,Ed] or None, w2 [E,Ed,D] -> [E,N].
+    """
+    h = torch.einsum('eni,eio->eno', x.unsqueeze(0).expand(w1.size(0), -1, -1), w1)
+    if b1 is not None:
+        h = h + b1.unsqueeze(-2)
+    h = ACTIVATIONS[activation](h)
+    y = torch.einsum('eni,eio->eno', h, w2)
+    return torch.linalg.vector_norm(y, ord=2, dim=-1)
 
 
 def experts_forward_naive(x: torch.Tensor, routing: torch.Tensor, w1: torch.Tensor,

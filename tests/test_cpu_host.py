@@ -364,3 +364,20 @@ def test_checkpoint_import_refuses_what_it_should(tmp_path):
     assert set(P.strip_wrapper_prefixes(mixed)) == {'module.a', 'b'}
     # without a GPU there is nothing to pack
     assert P.prepack(src) == 0
+
+
+def test_output_norms_on_cpu_follow_the_reference_route():
+    """Without a GPU the router-training targets come from the two stub submodules, as in the reference."""
+    from d2dmoe_amd import HipKernelExperts
+    torch.manual_seed(0)
+    ex = HipKernelExperts(48, 6, 2, 8, 'without_last', torch.nn.GELU)
+    with torch.no_grad():
+        ex.b1.normal_(0.0, 0.1)
+    x = torch.randn(11, 48)
+    seen = {}
+    h = ex.output_activation_extraction_stub.register_forward_hook(lambda m, i, o: seen.__setitem__('y', o))
+    got = ex.output_norms(x)
+    h.remove()
+    assert got.shape == (6, 11) and tuple(seen['y'].shape) == (6, 11, 48)
+    want = O.expert_output_norms(x.double(), ex.w1.double(), ex.b1.double(), ex.w2.double(), 'gelu')
+    assert torch.allclose(got.double(), want, rtol=1e-4, atol=1e-6)

@@ -726,3 +726,57 @@ def test_entry_points_reject_bad_workspace_alignment_and_paths():
     torch.cuda.synchronize()
     # the call that went through left a correct result behind
     assert H.rel_err(out.cpu(), _experts_want(x, routing, {k: v for k, v in p.items() if k != 'last_bias'}, 'relu')) < H.TOL_BF16
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Router-training targets: per-expert output norms (reference: train_routers.py:49-86, utils.py:353-369)
+# ---------------------------------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize('N,E,Ed,act', [(197, 128, 24, 'relu'), (65, 100, 30, 'gelu'), (1, 7, 5, 'relu'),
+                                        (300, 16, 32, 'tanh'), (130, 9, 24, 'leaky_relu')])
+def test_expert_output_norms_match_oracle(N, E, Ed, act):
+    _say('expert output norms', N, E, Ed, act)
+    x, _, p = H.random_case(N, 768, E, Ed, 8, seed=N + E + 5, dtype=torch.bfloat16)
+    d = H.to_dev(p, DEV)
+    got = _ops().expert_output_norms(x.to(DEV), d['w1'], d['b1'], d['w2'], act)
+    assert got.shape == (E, N) and got.dtype == torch.bfloat16
+    q = O.upcast(p)
+    want = O.expert_output_norms(x.double(), q['w1'], q['b1'], q['w2'], act)
+    assert H.rel_err(got.cpu(), want) < H.TOL_BF16
+    # element-wise as well: a norm is a sum of squares, there is no cancellation to hide behind
+    rel = ((got.cpu().double() - want).abs() / want.clamp_min(1e-3)).max().item()
+    assert rel < 2e-2, rel
+    # without the first-layer bias
+    got = _ops().expert_output_norms(x.to(DEV), d['w1'], None, d['w2'], act)
+    want = O.expert_output_norms(x.double(), q['w1'], None, q['w2'], act)
+    assert H.rel_err(got.cpu(), want) < H.TOL_BF16
+
+
+@pytest.mark.gpu
+def test_expert_output_norms_module_method_and_full_size():
+    from d2dmoe_amd import HipKernelExperts
+    torch.manual_seed(0)
+    ex = HipKernelExperts(768, 128, 2, 24, 'without_last', torch.nn.ReLU).to(DEV).bfloat16()
+    with torch.no_grad():
+        ex.b1.normal_(0.0, 0.1)
+    N = 50432
+    x = torch.randn(N, 768, generator=torch.Generator().manual_seed(3)).bfloat16().to(DEV)
+    with torch.no_grad():
+        got = ex.output_norms(x)                       # HIP kernel
+        assert got.shape == (128, N)
+        rows = torch.cat([torch.arange(0, 96), torch.arange(N - 70, N)]).to(DEV)
+        ref = torch.linalg.vector_norm(ex.output_activation_extraction_stub(
+            ex.intermediate_activation_extraction_stub(x[rows].unsqueeze(0), ex.w1, ex.b1, ex.act), ex.w2), ord=2, dim=-1)
+        assert H.rel_err(got[:, rows].float().cpu(), ref.float().cpu()) < H.TOL_BF16
+        want = O.expert_output_norms(x[rows].double().cpu(), ex.w1.double().cpu(), ex.b1.double().cpu(), ex.w2.double().cpu(), 'relu')
+        assert H.rel_err(got[:, rows].cpu(), want) < H.TOL_BF16
+        assert torch.equal(got, ex.output_norms(x))    # deterministic
+        # the packed buffer follows parameter updates
+        ex.w2.mul_(2.0)
+        assert H.rel_err(ex.output_norms(x)[:, rows].cpu(), 2.0 * want) < H.TOL_BF16
+        # float32 parameters: the reference's own route through the stubs
+        ex32 = HipKernelExperts(768, 16, 2, 24, 'without_last', torch.nn.ReLU).to(DEV)
+        x32 = x[:40].float()
+        got32 = ex32.output_norms(x32)
+        want32 = O.expert_output_norms(x32.double().cpu(), ex32.w1.double().cpu(), ex32.b1.double().cpu(), ex32.w2.double().cpu(), 'relu')
+        assert H.rel_err(got32.cpu(), want32) < H.TOL_F32

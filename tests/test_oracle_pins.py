@@ -334,3 +334,31 @@ def test_layer_forward_composition_and_epilogue():
 def test_threshold_fraction_round_trip():
     # the bench takes the threshold fraction f ("0.9 x max") and sets module tau = 1 - f
     assert 1.0 - 0.1 == 0.9
+
+
+def test_expert_output_norms_brute_force_gram_identity_and_special_cases():
+    g = torch.Generator().manual_seed(17)
+    N, D, E, Ed = 9, 12, 5, 7
+    x = torch.randn(N, D, generator=g, dtype=torch.float64)
+    w1 = torch.randn(E, D, Ed, generator=g, dtype=torch.float64)
+    b1 = torch.randn(E, Ed, generator=g, dtype=torch.float64)
+    w2 = torch.randn(E, Ed, D, generator=g, dtype=torch.float64)
+    got = O.expert_output_norms(x, w1, b1, w2, 'relu')
+    assert got.shape == (E, N)
+    xn, w1n, b1n, w2n = x.numpy(), w1.numpy(), b1.numpy(), w2.numpy()
+    for e in range(E):
+        for n in range(N):
+            h = np.maximum(xn[n] @ w1n[e] + b1n[e], 0.0)
+            y = h @ w2n[e]
+            assert abs(got[e, n].item() - math.sqrt(float((y * y).sum()))) < 1e-10
+            # the quadratic form over the expert's Gram matrix gives the same number
+            gram = w2n[e] @ w2n[e].T
+            assert abs(got[e, n].item() ** 2 - float(h @ gram @ h)) < 1e-8
+    # a zero second layer gives zero norms; norms are non-negative and scale with the second layer
+    assert torch.equal(O.expert_output_norms(x, w1, b1, torch.zeros_like(w2), 'relu'), torch.zeros(E, N, dtype=torch.float64))
+    assert (got >= 0).all()
+    assert torch.allclose(O.expert_output_norms(x, w1, b1, -3.0 * w2, 'relu'), 3.0 * got, rtol=1e-12)
+    # one expert, identity activation, no bias: |x (W1 W2)| through a library GEMM
+    a = w1[0] @ w2[0]
+    want = torch.linalg.vector_norm(x @ a, dim=-1)
+    assert torch.allclose(O.expert_output_norms(x, w1[:1], None, w2[:1], 'identity')[0], want, rtol=1e-12)
