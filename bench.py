@@ -339,6 +339,57 @@ def run_gpt2(args, dev):
     print(json.dumps(line))
 
 
+def run_vit(args, dev):
+    """Whole-model workload: ViT-B/16 (12 blocks, D = 768, 12 heads, 197 tokens per image) with every FFN replaced by a
+    MoE layer of 128 experts x 24 neurons (GELU, biases) and a 768 -> 128 -> 128 router; 256 images = 50432 tokens per
+    layer; bf16; random weights.  Attention, LayerNorm, patch embedding and head are stock PyTorch."""
+    from d2dmoe_amd import add_routers, gpt2, vit
+    torch.manual_seed(0)
+    dense = vit.VisionTransformer().eval().to(dev).to(torch.bfloat16)
+    moe, names = gpt2.replace_with_moes(dense, num_experts=128, experts_class='hip_kernel')
+    gpt2.split_original_parameters(dense, moe, names)
+    add_routers(moe, dict(width=128, depth=2, bias=False, activation='relu', output_activation='abs'))
+    moe = moe.to(dev).to(torch.bfloat16)
+    layers = [gpt2.get_module_by_name(moe, n) for n in names]
+    B = 256
+    x = torch.randn(B, 3, 224, 224, generator=torch.Generator().manual_seed(1)).to(dev).to(torch.bfloat16)
+    N = B * 197
+
+    def measure(tau):
+        ks = {}
+        for layer in layers:
+            layer.forward_mode, layer.tau = 'dynk_max', tau
+            layer.experts.forward_mode = 'hip'
+        hooks = [layer.register_forward_hook(lambda m, inp, out, n=n: ks.__setitem__(n, out[1][n][0].float().sum(-1).mean().item()))
+                 for n, layer in zip(names, layers)]
+        moe(x)
+        for h in hooks:
+            h.remove()
+        torch.cuda.synchronize()
+        return time_events(lambda: moe(x), args.steps, args.warmup), sum(ks.values()) / len(ks)
+
+    ms_moe, k_moe = measure(args.tau)
+    ms_lit, k_lit = measure(1.0 - args.tau)
+    ms_dense = time_events(lambda: dense(x), args.steps, args.warmup)
+    xin = torch.randn(B, 197, 768, generator=torch.Generator().manual_seed(2)).to(dev).to(torch.bfloat16)
+    ms_dense_ffn = time_events(lambda: dense.encoder.layers[0].mlp(xin), args.steps, args.warmup)
+    line = {
+        'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
+        'value': N / ms_moe * 1e3, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': ms_moe, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16',
+        'data': 'synthetic',
+        'config': {'workload': f'vit_b_model: whole ViT-B/16 forward, 12 blocks, {B} images x 197 tokens = {N} tokens per layer, '
+                               f'MoE FFN 128 experts x 24 (gelu, biases), router 768->128->128, module tau={args.tau}; '
+                               f'one step = one model forward', 'mean_active_experts': k_moe},
+        'images_per_s': B / ms_moe * 1e3, 'dense_model_ms': ms_dense, 'dense_ffn_layer_ms': ms_dense_ffn,
+        'literal_rule': {'rule': f'keep norm >= {args.tau}*max', 'model_ms': ms_lit, 'images_per_s': B / ms_lit * 1e3,
+                         'mean_active_experts': k_lit},
+        'roofline': {'bound': 'mfma', 'kernel': 'see workload vit_b_50k (the same layer shape and token count)', 'achieved': None,
+                     'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s', 'frac': None, 'traffic': None},
+    }
+    print(json.dumps(line))
+
+
 def run_norms(args, ops, dev):
     """Router-training targets: the L2 norm of every expert's output for every token (ViT-B layer, 256 x 197 tokens),
     by the HIP kernel and, beside it, by the reference's route on the same GPU (masked-mode stubs + vector_norm over
@@ -403,7 +454,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS) + sorted(GATED_WORKLOADS) + ['gpt2_small', 'vit_b_50k_norms'])
+    ap.add_argument('--workload', default='vit_b_50k', choices=sorted(WORKLOADS) + sorted(GATED_WORKLOADS) + ['gpt2_small', 'vit_b_50k_norms', 'vit_b_model'])
     ap.add_argument('--tau', type=float, default=0.9, help='module tau (keep expert when norm >= (1 - tau) * max)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-sweep', action='store_true', help='skip the threshold sweep (5 values x 2 readings)')
@@ -436,6 +487,10 @@ def main():
     if args.workload == 'gpt2_small':
         with torch.no_grad():
             run_gpt2(args, dev)
+        return
+    if args.workload == 'vit_b_model':
+        with torch.no_grad():
+            run_vit(args, dev)
         return
     if args.workload == 'vit_b_50k_norms':
         with torch.no_grad():

@@ -180,8 +180,21 @@ def moe_gpt_main_forward(self, x: torch.Tensor, return_gating_data: bool = False
 
 
 # ------------------------------------------------------------------------------------------- model surgery
+def ffn_parts(ffn: nn.Module):
+    """(first Linear, activation module, second Linear, dropout probability) of a dense FFN block: this file's `MLP`
+    (c_fc, act, c_proj, dropout) or an index-addressed Linear/act/Dropout/Linear/Dropout sequence (torchvision's
+    MLPBlock, `vit.MLPBlock`)."""
+    if isinstance(ffn, MLP):
+        return ffn.c_fc, ffn.act, ffn.c_proj, ffn.dropout.p
+    if isinstance(ffn, nn.Sequential) and len(ffn) == 5 and isinstance(ffn[0], nn.Linear) and isinstance(ffn[3], nn.Linear):
+        return ffn[0], ffn[1], ffn[3], ffn[4].p if isinstance(ffn[4], nn.Dropout) else 0.0
+    raise ValueError(f'Unsupported ffn type: {type(ffn)}')
+
+
 def ffn_filter_condition(_model: nn.Module, m: nn.Module) -> bool:
-    return isinstance(m, MLP)
+    if isinstance(m, MLP):
+        return True
+    return isinstance(m, nn.Sequential) and len(m) == 5 and isinstance(m[0], nn.Linear) and isinstance(m[3], nn.Linear)
 
 
 def find_module_names(model: nn.Module, condition=None) -> List[str]:
@@ -212,9 +225,7 @@ def set_module_by_name(model: nn.Module, name: str, module: Optional[nn.Module])
 
 def replace_layer_with_moe(model: nn.Module, name: str, num_experts=None, expert_size=None, experts_class='hip_kernel'):
     original = get_module_by_name(model, name)
-    if not isinstance(original, MLP):
-        raise ValueError(f'Unsupported ffn type: {type(original)}')
-    w1 = original.c_fc
+    w1, act, _, dropout_p = ffn_parts(original)
     hidden_dim, d_ff = w1.in_features, w1.out_features
     if num_experts is not None:
         assert d_ff % num_experts == 0, 'd_ff has to be divisible by the number of experts'
@@ -222,36 +233,40 @@ def replace_layer_with_moe(model: nn.Module, name: str, num_experts=None, expert
     else:
         assert d_ff % expert_size == 0, 'd_ff has to be divisible by the expert size'
         num_experts = d_ff // expert_size
-    moe_layer = MoeficationMoE(name, hidden_dim, num_experts, w1.bias is not None, expert_size, type(original.act),
-                               experts_class)
+    moe_layer = MoeficationMoE(name, hidden_dim, num_experts, w1.bias is not None, expert_size, type(act), experts_class)
     moe_layer = moe_layer.to(device=w1.weight.device, dtype=w1.weight.dtype)
     set_module_by_name(model, name, moe_layer)
-    set_module_by_name(model, f'{name}.dropout', nn.Dropout(original.dropout.p))
+    set_module_by_name(model, f'{name}.dropout', nn.Dropout(dropout_p))
 
 
-def replace_with_moes(original_model: GPT, num_experts: int = None, expert_size: int = None,
+def replace_with_moes(original_model: nn.Module, num_experts: int = None, expert_size: int = None,
                       experts_class: str = 'hip_kernel', module_filter_condition=None):
-    """Deep copy of `original_model` with every selected FFN replaced by a MoE layer and the forwards patched to
-    return gating data; returns (model, names of the replaced modules)."""
+    """Deep copy of `original_model` (this package's GPT or VisionTransformer) with every selected FFN replaced by a MoE
+    layer and the forwards patched to return gating data; returns (model, names of the replaced modules)."""
+    from . import vit
     assert (num_experts is None) != (expert_size is None), 'pass exactly one of num_experts and expert_size'
-    if not isinstance(original_model, GPT):
+    if not isinstance(original_model, (GPT, vit.VisionTransformer)):
         raise ValueError(f'Unsupported model type: {type(original_model)}')
     original_model.eval()
     model = deepcopy(original_model)
     names = find_module_names(original_model, module_filter_condition)
     for name in names:
         replace_layer_with_moe(model, name, num_experts, expert_size, experts_class)
-    for block in model.transformer.h:
-        block.forward = partial(moe_gpt_block_forward, block)
-    model.forward = partial(moe_gpt_main_forward, model)
+    if isinstance(model, GPT):
+        for block in model.transformer.h:
+            block.forward = partial(moe_gpt_block_forward, block)
+        model.forward = partial(moe_gpt_main_forward, model)
+    else:
+        vit.patch_forwards(model)
     return model, names
 
 
-def param_split(ffn: MLP, moe_layer: MoeficationMoE, labels: Optional[Sequence[int]] = None):
+def param_split(ffn: nn.Module, moe_layer: MoeficationMoE, labels: Optional[Sequence[int]] = None):
     """Moves the dense FFN's neurons into the experts: neuron n goes to expert labels[n], in order of appearance."""
     ex = moe_layer.experts
     E, Ed = moe_layer.num_experts, moe_layer.expert_dim
-    d_ff = ffn.c_fc.out_features
+    fc1, _, fc2, _ = ffn_parts(ffn)
+    d_ff = fc1.out_features
     if labels is None:
         labels = torch.arange(d_ff) // Ed
     labels = torch.as_tensor(labels, dtype=torch.long)
@@ -262,16 +277,16 @@ def param_split(ffn: MLP, moe_layer: MoeficationMoE, labels: Optional[Sequence[i
     slot = torch.empty_like(order)
     slot[order] = torch.arange(d_ff) % Ed
     with torch.no_grad():
-        w_fc = ffn.c_fc.weight.detach()                 # [d_ff, D]
-        w_proj = ffn.c_proj.weight.detach()             # [D, d_ff]
+        w_fc = fc1.weight.detach()                      # [d_ff, D]
+        w_proj = fc2.weight.detach()                    # [D, d_ff]
         ex.w1[labels, :, slot] = w_fc.to(ex.w1.dtype).to(ex.w1.device)
         ex.w2[labels, slot, :] = w_proj.t().to(ex.w2.dtype).to(ex.w2.device)
         if moe_layer.bias:
-            ex.b1[labels, slot] = ffn.c_fc.bias.detach().to(ex.b1.dtype).to(ex.b1.device)
-            moe_layer.last_bias.copy_(ffn.c_proj.bias.detach().view(1, -1))
+            ex.b1[labels, slot] = fc1.bias.detach().to(ex.b1.dtype).to(ex.b1.device)
+            moe_layer.last_bias.copy_(fc2.bias.detach().view(1, -1))
 
 
-def split_original_parameters(original_model: GPT, moe_model: GPT, replaced_module_names: List[str],
+def split_original_parameters(original_model: nn.Module, moe_model: nn.Module, replaced_module_names: List[str],
                               labels: Optional[Dict[str, Sequence[int]]] = None):
     assert len(replaced_module_names) > 0
     original_model.eval()

@@ -381,3 +381,45 @@ def test_output_norms_on_cpu_follow_the_reference_route():
     assert got.shape == (6, 11) and tuple(seen['y'].shape) == (6, 11, 48)
     want = O.expert_output_norms(x.double(), ex.w1.double(), ex.b1.double(), ex.w2.double(), 'gelu')
     assert torch.allclose(got.double(), want, rtol=1e-4, atol=1e-6)
+
+
+def test_vit_surgery_keeps_the_function_and_the_parameter_names():
+    """ViT with torchvision's module tree: FFNs (mlp.0 / mlp.3) -> MoE layers, same logits with every expert running,
+    gating data of every block from the patched forwards (reference: moe_models.py:55-78, 103-127)."""
+    from d2dmoe_amd import add_routers, gpt2, vit
+    torch.manual_seed(0)
+    m = vit.VisionTransformer(image_size=32, patch_size=8, num_layers=2, num_heads=2, hidden_dim=32, mlp_dim=64,
+                              num_classes=10).eval()
+    with torch.no_grad():
+        for n, prm in m.named_parameters():
+            if n.endswith('bias'):
+                prm.normal_(0.0, 0.05)
+        m.class_token.normal_(0.0, 0.02)
+    keys = set(m.state_dict())
+    for k in ('conv_proj.weight', 'class_token', 'encoder.pos_embedding', 'encoder.layers.encoder_layer_1.ln_2.bias',
+              'encoder.layers.encoder_layer_0.self_attention.in_proj_weight',
+              'encoder.layers.encoder_layer_0.mlp.0.weight', 'encoder.layers.encoder_layer_0.mlp.3.bias',
+              'encoder.ln.weight', 'heads.head.weight'):
+        assert k in keys, k
+    moe, names = gpt2.replace_with_moes(m, num_experts=8, experts_class='hip_kernel')
+    assert names == ['encoder.layers.encoder_layer_0.mlp', 'encoder.layers.encoder_layer_1.mlp']
+    labels = {n: torch.randperm(64, generator=torch.Generator().manual_seed(i)) % 8 for i, n in enumerate(names)}
+    gpt2.split_original_parameters(m, moe, names, labels)
+    x = torch.randn(3, 3, 32, 32, generator=torch.Generator().manual_seed(5))
+    for n in names:
+        layer = gpt2.get_module_by_name(moe, n)
+        layer.forward_mode = 'all'
+        layer.experts.forward_mode = 'naive'
+    with torch.no_grad():
+        want = m(x)
+        got, gating = moe(x, return_gating_data=True)
+    assert H.rel_err(got, want) < 1e-5 and set(gating) == set(names)
+    assert tuple(gating[names[0]][0].shape) == (3, 17, 8)
+    add_routers(moe, dict(width=16, depth=2, bias=False, activation='relu', output_activation='abs'))
+    for n in names:
+        layer = gpt2.get_module_by_name(moe, n)
+        layer.forward_mode, layer.tau = 'dynk_max', 0.5
+    with torch.no_grad():
+        out, gating = moe(x, return_gating_data=True)
+    frac = gating[names[1]][0].float().mean().item()
+    assert out.shape == (3, 10) and 0.0 < frac < 1.0

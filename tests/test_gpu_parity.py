@@ -780,3 +780,39 @@ def test_expert_output_norms_module_method_and_full_size():
         got32 = ex32.output_norms(x32)
         want32 = O.expert_output_norms(x32.double().cpu(), ex32.w1.double().cpu(), ex32.b1.double().cpu(), ex32.w2.double().cpu(), 'relu')
         assert H.rel_err(got32.cpu(), want32) < H.TOL_F32
+
+
+@pytest.mark.gpu
+def test_vit_with_hip_moe_layers():
+    """ViT-B width on the GPU in bf16: 2 encoder blocks, 197 tokens per image; with every expert running the MoE model
+    (HIP experts) reproduces the dense model's logits; under dynk_max the fused layers return their gating data."""
+    from d2dmoe_amd import add_routers, gpt2, vit
+    torch.manual_seed(0)
+    m = vit.VisionTransformer(image_size=224, patch_size=16, num_layers=2, num_heads=12, hidden_dim=768, mlp_dim=3072,
+                              num_classes=100).eval()
+    with torch.no_grad():
+        for n, prm in m.named_parameters():
+            if n.endswith('bias'):
+                prm.normal_(0.0, 0.05)
+    m = m.to(DEV).bfloat16()
+    moe, names = gpt2.replace_with_moes(m, num_experts=128, experts_class='hip_kernel')
+    gpt2.split_original_parameters(m, moe, names)
+    for n in names:
+        layer = gpt2.get_module_by_name(moe, n)
+        layer.forward_mode = 'all'
+        layer.experts.forward_mode = 'hip'
+    x = torch.randn(4, 3, 224, 224, generator=torch.Generator().manual_seed(1)).to(DEV).bfloat16()
+    with torch.no_grad():
+        want = m(x)
+        got, gating = moe(x, return_gating_data=True)
+    assert H.rel_err(got.float().cpu(), want.float().cpu()) < H.TOL_BF16
+    assert set(gating) == set(names) and tuple(gating[names[0]][0].shape) == (4, 197, 128)
+    add_routers(moe, dict(width=128, depth=2, bias=False, activation='relu', output_activation='abs'))
+    moe = moe.to(DEV).bfloat16()
+    for n in names:
+        layer = gpt2.get_module_by_name(moe, n)
+        layer.forward_mode, layer.tau = 'dynk_max', 0.5
+    with torch.no_grad():
+        out, gating = moe(x, return_gating_data=True)
+    frac = gating[names[-1]][0].float().mean().item()
+    assert out.shape == (4, 100) and 0.0 < frac < 1.0 and torch.isfinite(out.float()).all()
