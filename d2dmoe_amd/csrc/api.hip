@@ -96,8 +96,14 @@ int d2dmoe_router(const void* x, const void* router_w1, const void* router_w2, v
     e = launch_linear_skinny(x, router_w1, workspace, (int)n_tokens, d_model, router_width, activation, s);
     if (e == hipSuccess) e = launch_linear_skinny(workspace, router_w2, norms, (int)n_tokens, router_width, n_experts, output_activation, s);
   } else if (dtype == D2DMOE_F32) {
-    e = launch_linear_act<float>(x, router_w1, workspace, n_tokens, d_model, router_width, activation, s);
-    if (e == hipSuccess) e = launch_linear_act<float>(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s);
+    // float32 on the matrix cores where the widths allow 16-byte operand loads and whole 32-column tiles
+    const bool m1 = linear_mfma_f32_supported(n_tokens, d_model, router_width) && aligned16(x) && aligned16(router_w1);
+    const bool m2 = linear_mfma_f32_supported(n_tokens, router_width, n_experts) && aligned16(router_w2);
+    e = m1 ? launch_linear_mfma_f32(x, router_w1, workspace, n_tokens, d_model, router_width, activation, s)
+           : launch_linear_act<float>(x, router_w1, workspace, n_tokens, d_model, router_width, activation, s);
+    if (e == hipSuccess)
+      e = m2 ? launch_linear_mfma_f32(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s)
+             : launch_linear_act<float>(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s);
   } else {
     e = launch_linear_act<bf16_t>(x, router_w1, workspace, n_tokens, d_model, router_width, activation, s);
     if (e == hipSuccess) e = launch_linear_act<bf16_t>(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s);

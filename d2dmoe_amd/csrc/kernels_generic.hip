@@ -74,6 +74,68 @@ hipError_t launch_linear_act(const void* A, const void* B, void* C, int64_t M, i
 template hipError_t launch_linear_act<float>(const void*, const void*, void*, int64_t, int, int, int, hipStream_t);
 template hipError_t launch_linear_act<bf16_t>(const void*, const void*, void*, int64_t, int, int, int, hipStream_t);
 
+// The same layer in float32 on the matrix cores (v_mfma_f32_32x32x2_f32: float32 operands, products and sums), for
+// K a multiple of 32 and Nout a multiple of 32.  Workgroup = 32 rows x 128 columns, one 32 x 32 tile per wave, no LDS:
+// lane (c, h) holds 4 consecutive K values of row c of each operand per step of 8 (h = which half of the 8), read
+// straight from global memory; the four waves share their A rows through the L1.  Two register buffers of 32 K values
+// each alternate, so the loads of one are in flight while the other is multiplied.
+typedef float f32x16_g __attribute__((ext_vector_type(16)));
+typedef float f32x4_g __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void linear_act_mfma_f32_kernel(const float* __restrict__ A, const float* __restrict__ B,
+                                                                  float* __restrict__ C, int64_t M, int K, int Nout, int act) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int c32 = lane & 31, kh = lane >> 5;
+  const int64_t row0 = (int64_t)blockIdx.x * 32;
+  const int col0 = (blockIdx.y * 4 + w) * 32;
+  if (col0 >= Nout) return;   // whole waves leave; the kernel has no barrier
+  int64_t ar = row0 + c32;
+  ar = ar < M ? ar : (M - 1);   // rows beyond M repeat the last row and are not stored
+  const f32x4_g* ap = (const f32x4_g*)(A + ar * K) + kh;
+  const f32x4_g* bp = (const f32x4_g*)(B + (int64_t)(col0 + c32) * K) + kh;
+  f32x16_g acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  f32x4_g a0[4], b0[4], a1[4], b1[4];
+  auto fill = [&](f32x4_g (&a)[4], f32x4_g (&b)[4], int k0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      a[u] = ap[(k0 >> 2) + 2 * u];
+      b[u] = bp[(k0 >> 2) + 2 * u];
+    }
+  };
+  auto multiply = [&](const f32x4_g (&a)[4], const f32x4_g (&b)[4]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][q], b[u][q], acc, 0, 0, 0);
+  };
+  const int k_last = K - 32;
+  fill(a0, b0, 0);
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    fill(a1, b1, (k0 + 32 < K) ? (k0 + 32) : k_last);   // past the end: an in-bounds re-read that is not multiplied
+    multiply(a0, b0);
+    if (k0 + 32 < K) {
+      fill(a0, b0, (k0 + 64 < K) ? (k0 + 64) : k_last);
+      multiply(a1, b1);
+    }
+  }
+  // lane = column c32; accumulator r = row 8*(r/4) + 4*kh + r%4
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int64_t row = row0 + 8 * (r / 4) + 4 * kh + (r % 4);
+    if (row < M) C[row * Nout + col0 + c32] = apply_act(act, acc[r]);
+  }
+}
+
+bool linear_mfma_f32_supported(int64_t M, int K, int Nout) { return M > 0 && K >= 32 && K % 32 == 0 && Nout % 32 == 0; }
+
+hipError_t launch_linear_mfma_f32(const void* A, const void* B, void* C, int64_t M, int K, int Nout, int act, hipStream_t s) {
+  dim3 grid((unsigned)cdiv64(M, 32), (unsigned)((Nout + 127) / 128));
+  hipLaunchKernelGGL(linear_act_mfma_f32_kernel, grid, dim3(256), 0, s, (const float*)A, (const float*)B, (float*)C, M, K, Nout, act);
+  return hipGetLastError();
+}
+
 // =====================================================================================================
 // small fill kernel (used instead of a memset node so the path stays graph-capture friendly)
 // =====================================================================================================

@@ -12,6 +12,8 @@ namespace d2dmoe {
 // ---- generic kernels (kernels_generic.hip) ----
 template <typename T>
 hipError_t launch_linear_act(const void* A, const void* B, void* C, int64_t M, int K, int Nout, int act, hipStream_t s);
+bool linear_mfma_f32_supported(int64_t M, int K, int Nout);
+hipError_t launch_linear_mfma_f32(const void* A, const void* B, void* C, int64_t M, int K, int Nout, int act, hipStream_t s);
 
 hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s);
 

@@ -31,7 +31,9 @@ def _say(*a):
 # =================================================================== router ===========================
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('N,D,W,E', [(1, 64, 128, 4), (10, 64, 128, 4), (197, 768, 128, 128), (1576, 768, 128, 128),
-                                     (16, 2048, 256, 256), (70, 100, 37, 19)])
+                                     (16, 2048, 256, 256), (70, 100, 37, 19),
+                                     # widths that are multiples of 32: the float32 layers run on the matrix cores
+                                     (33, 96, 160, 32), (50, 32, 32, 64), (100, 64, 96, 288)])
 def test_router_matches_oracle(dtype, N, D, W, E):
     _say('router', dtype, N, D, W, E)
     x, _, p = H.random_case(N, D, E, 8, W, seed=N + D, dtype=dtype)
