@@ -299,42 +299,75 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
   constexpr int CTW = D / 128;   // column tiles per wave
   static_assert(KS1 % 4 == 0, "the model dimension must split over four waves");
   __shared__ int32_t s_tile_off[1025];
+  __shared__ int32_t s_offsets[1025];
   __shared__ float part[4][NT * 16][64];
   __shared__ __attribute__((aligned(16))) bf16_t s_last_bias[D];
   if (A.flag[0] == 0) return;
   const int E = A.E;
-  for (int i = threadIdx.x; i <= E; i += 256) s_tile_off[i] = A.tile_off[i];
+  for (int i = threadIdx.x; i <= E; i += 256) {
+    s_tile_off[i] = A.tile_off[i];
+    s_offsets[i] = A.offsets[i];
+  }
   for (int i = threadIdx.x; i < D; i += 256) s_last_bias[i] = (A.last_bias != nullptr) ? A.last_bias[i] : (bf16_t)0;
   __syncthreads();
   const int n_tiles = s_tile_off[E];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int g = lane >> 5, c32 = lane & 31;
-  for (int T = blockIdx.x; T < n_tiles; T += gridDim.x) {
+  // Workgroups are dealt to the 8 XCDs round-robin.  Each XCD takes one contiguous eighth of the tiles (tiles are in
+  // expert order), so an expert's weights pass through one L2, or two, instead of all eight.
+  const int xcd = blockIdx.x & 7, wg = blockIdx.x >> 3, nwg = gridDim.x >> 3;   // the grid is a multiple of 8
+  const int t_lo = (int)((int64_t)n_tiles * xcd / 8), t_hi = (int)((int64_t)n_tiles * (xcd + 1) / 8);
+  // What a tile needs before its first x load hangs on two dependent global reads (pair -> token -> that token's pair
+  // range and routing value).  They are made one tile ahead, in stages placed between the phases of the current tile,
+  // so that each has returned long before its result is used.
+  struct TileInfo {
+    int e, rows, tok, dst, t0, t1;
+    bf16_t rbits;
+  };
+  auto tile_begin = [&](int T, TileInfo& ti) __attribute__((always_inline)) {   // LDS lookups, then the pair's token and row
     int lo = 0, hi = E;   // largest e with tile_off[e] <= T (experts without tiles share their successor's offset)
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
       if (s_tile_off[mid] <= T) lo = mid; else hi = mid;
     }
-    const int e = lo;
-    const int base = A.offsets[e];
-    const int cnt = A.offsets[e + 1] - base;
-    const int j0 = (T - s_tile_off[e]) * SP_BT;
-    const int rows = (cnt - j0 < SP_BT) ? (cnt - j0) : SP_BT;
+    ti.e = lo;
+    const int base = s_offsets[lo];
+    const int cnt = s_offsets[lo + 1] - base;
+    const int j0 = (T - s_tile_off[lo]) * SP_BT;
+    ti.rows = (cnt - j0 < SP_BT) ? (cnt - j0) : SP_BT;
+    const int pj = base + j0 + (c32 < ti.rows ? c32 : ti.rows - 1);
+    ti.tok = A.token_idx[pj];
+    ti.dst = A.pair_dst[pj];
+  };
+  auto tile_token = [&](TileInfo& ti) __attribute__((always_inline)) {          // the token's pair range and routing value
+    ti.t0 = A.tok_off[ti.tok];
+    ti.t1 = A.tok_off[ti.tok + 1];
+    ti.rbits = A.routing[(int64_t)ti.tok * E + ti.e];
+  };
+  int T = t_lo + wg;
+  TileInfo cur = {0, 1, 0, 0, 0, 0, 0}, nxt = {0, 1, 0, 0, 0, 0, 0};
+  if (T < t_hi) {
+    tile_begin(T, cur);
+    tile_token(cur);
+  }
+  for (; T < t_hi; T += nwg) {
+    const bool has_next = T + nwg < t_hi;   // uniform
+    const int e = cur.e, rows = cur.rows, tok = cur.tok, dst = cur.dst;
     const bool valid = c32 < rows;
-    const int pj = base + j0 + (valid ? c32 : rows - 1);
-    const int tok = A.token_idx[pj];
-    const int dst = A.pair_dst[pj];
     // A token with a single routed expert has nothing to be summed with: its row leaves this kernel as the finished
     // output row (float32 accumulator + last_bias (+ x), one rounding) and the combine kernel skips the token.
-    const bool single = valid && (A.tok_off[tok + 1] - A.tok_off[tok] == 1);
+    const bool single = valid && (cur.t1 - cur.t0 == 1);
+    const float rw = bf16_to_f32(cur.rbits);
     const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)tok * D) + 2 * w * KQ + g;
-    const float rw = bf16_to_f32(A.routing[(int64_t)tok * E + e]);
 
     // GEMM1, this wave's quarter of K: all loads are issued before the first MFMA
     const bf16x8* w1f = A.w1s + ((int64_t)e * KS1 + w * KQ) * NT * 64 + lane;
     bf16x8 xb[KQ];
 #pragma unroll
     for (int ks = 0; ks < KQ; ++ks) xb[ks] = xrow[2 * ks];
+    __builtin_amdgcn_sched_barrier(0);
+    if (has_next) tile_begin(T + nwg, nxt);
+    __builtin_amdgcn_sched_barrier(0);
     f32x16 acc1[NT];
 #pragma unroll
     for (int a = 0; a < NT; ++a)
@@ -350,6 +383,9 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
     bf16x8 w2r[CTW * 2 * NT];
 #pragma unroll
     for (int i = 0; i < CTW * 2 * NT; ++i) w2r[i] = w2f[i * 64];
+    __builtin_amdgcn_sched_barrier(0);
+    if (has_next) tile_token(nxt);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -400,7 +436,6 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
         acc2[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w2r[ct * 2 * NT + ks2], hb[ks2], acc2[ct], 0, 0, 0);
     const bool any_single = __ballot(single) != 0ull;   // uniform
     const int col0 = w * (D / 4) + 4 * g;
-    bf16_t* yrow = single ? (A.out + (int64_t)tok * D + col0) : (A.y + (int64_t)dst * D + col0);
     if (any_single) {
       // the bias (and residual) pieces are fetched by every lane, unconditionally, and added under a mask
       const uint32_t keep = single ? 0xffffffffu : 0u;
@@ -425,17 +460,47 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
           }
         }
     }
-    if (valid) {
+    // The rows leave through this wave's slice of the partial-sum buffer (idle until the next tile, and touched by no
+    // other wave outside the two barriers above), two column tiles at a time: a lane holds 4 columns of one row, the
+    // transposed read gives 8 lanes 128 contiguous bytes of a row.  16-byte pieces are XORed with the row so that both
+    // directions spread over the banks.
+    {
+      static_assert(CTW % 2 == 0, "column tiles are written in pairs");
+      unsigned char* stage = (unsigned char*)&part[w][0][0];   // 32 rows x 128 bytes
+      const int ridx = single ? tok : dst;
+      const int rl = lane >> 3, pc = lane & 7;
+      bf16_t* rptr[4];   // where row rl + 8 i goes: a finished row of out, or a row of y for the combine kernel
+      bool rlive[4];
 #pragma unroll
-      for (int ct = 0; ct < CTW; ++ct)
+      for (int i = 0; i < 4; ++i) {
+        const int R = rl + 8 * i;
+        const int idx = __shfl(ridx, R, kWave);
+        const int sg = __shfl((int)single, R, kWave);
+        rptr[i] = (sg ? A.out : A.y) + (int64_t)idx * D + w * (D / 4) + pc * 8;
+        rlive[i] = R < rows;
+      }
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          uint2 o;
-          o.x = pack2_bf16(acc2[ct][q * 4 + 0], acc2[ct][q * 4 + 1]);
-          o.y = pack2_bf16(acc2[ct][q * 4 + 2], acc2[ct][q * 4 + 3]);
-          *(uint2*)(yrow + ct * 32 + 8 * q) = o;
-        }
+      for (int ps = 0; ps < CTW / 2; ++ps) {
+#pragma unroll
+        for (int cta = 0; cta < 2; ++cta)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            uint2 o;
+            o.x = pack2_bf16(acc2[2 * ps + cta][q * 4 + 0], acc2[2 * ps + cta][q * 4 + 1]);
+            o.y = pack2_bf16(acc2[2 * ps + cta][q * 4 + 2], acc2[2 * ps + cta][q * 4 + 3]);
+            *(uint2*)(stage + c32 * 128 + (((cta * 4 + q) ^ (c32 & 7)) * 16) + 8 * g) = o;
+          }
+        __builtin_amdgcn_wave_barrier();
+        u32x4 rowv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rowv[i] = *(const u32x4*)(stage + (rl + 8 * i) * 128 + ((pc ^ rl) * 16));
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (rlive[i]) *(u32x4*)(rptr[i] + ps * 64) = rowv[i];
+      }
     }
+    cur = nxt;
   }
 }
 
