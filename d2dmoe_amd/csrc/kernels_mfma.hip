@@ -788,6 +788,7 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
     bf16_t* __restrict__ routing, bf16_t* __restrict__ norms_out, int32_t* __restrict__ counts, int64_t N, int D,
     float thr_scale) {
   constexpr int E = ET * 32;
+  __shared__ __attribute__((aligned(16))) unsigned char stage_all[4 * 32 * E * 2];   // per wave: 32 rows of routing
   const int lane = threadIdx.x & 63;
   const int g = lane >> 5, c32 = lane & 31;
   const int64_t tok0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 32;
@@ -865,38 +866,64 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
     }
   m = nanmax(m, __shfl_xor(m, 32, kWave));
   const float thr = __uint_as_float(pack2_bf16(m * thr_scale, 0.f) << 16);
+  // A lane holds 4 consecutive experts of one token per accumulator quad.  The rows go through a wave-private LDS tile
+  // (16-byte pieces XORed with the row, so both directions spread over the banks) and leave as whole rows: CH lanes
+  // write the E * 2 contiguous bytes of a token's routing (or norms) row.
+  constexpr int CH = E / 8;            // 16-byte pieces per row
+  constexpr int RPI = 64 / CH;         // rows per store instruction
+  u32x4* stage = (u32x4*)stage_all + (threadIdx.x >> 6) * (32 * CH);
+  const int srow = lane / CH, spc = lane % CH;
+  auto flush = [&](bf16_t* dst) __attribute__((always_inline)) {
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; ++i) {
+      const int row = srow + RPI * i;
+      const u32x4 v = stage[row * CH + (spc ^ (row & (CH - 1)))];
+      if (tok0 + row < N) *(u32x4*)(dst + (tok0 + row) * E + spc * 8) = v;
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  uint2* srow_w = (uint2*)(stage + c32 * CH);   // this lane's row; piece p at index (p ^ (c32 & (CH-1))) * 2 + g
+  bool on[ET][16];
 #pragma unroll
   for (int et = 0; et < ET; ++et) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int e0 = et * 32 + 8 * q + 4 * g;
-      bool on[4];
 #pragma unroll
-      for (int s = 0; s < 4; ++s) on[s] = acc2[et][q * 4 + s] >= thr;
-      if (valid) {
-        uint2 rv;
-        rv.x = (on[0] ? 0x3F80u : 0u) | (on[1] ? 0x3F800000u : 0u);   // bf16 1.0 = 0x3F80
-        rv.y = (on[2] ? 0x3F80u : 0u) | (on[3] ? 0x3F800000u : 0u);
-        *(uint2*)(routing + token * E + e0) = rv;
-        if (norms_out != nullptr) {
-          uint2 nv;
-          nv.x = (__float_as_uint(acc2[et][q * 4 + 0]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 1]) & 0xffff0000u);
-          nv.y = (__float_as_uint(acc2[et][q * 4 + 2]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 3]) & 0xffff0000u);
-          *(uint2*)(norms_out + token * E + e0) = nv;
-        }
+      for (int s = 0; s < 4; ++s) on[et][q * 4 + s] = acc2[et][q * 4 + s] >= thr;
+      uint2 rv;
+      rv.x = (on[et][q * 4 + 0] ? 0x3F80u : 0u) | (on[et][q * 4 + 1] ? 0x3F800000u : 0u);   // bf16 1.0 = 0x3F80
+      rv.y = (on[et][q * 4 + 2] ? 0x3F80u : 0u) | (on[et][q * 4 + 3] ? 0x3F800000u : 0u);
+      srow_w[(((et * 4 + q) ^ (c32 & (CH - 1))) << 1) + g] = rv;
+    }
+  }
+  flush(routing);
+  if (norms_out != nullptr) {
+#pragma unroll
+    for (int et = 0; et < ET; ++et)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        uint2 nv;
+        nv.x = (__float_as_uint(acc2[et][q * 4 + 0]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 1]) & 0xffff0000u);
+        nv.y = (__float_as_uint(acc2[et][q * 4 + 2]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 3]) & 0xffff0000u);
+        srow_w[(((et * 4 + q) ^ (c32 & (CH - 1))) << 1) + g] = nv;
       }
-      if (counts != nullptr) {
+    flush(norms_out);
+  }
+  if (counts != nullptr) {
+#pragma unroll
+    for (int et = 0; et < ET; ++et)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-          const unsigned long long bal = __ballot(on[s] && valid);
+          const unsigned long long bal = __ballot(on[et][q * 4 + s] && valid);
           if (lane == 0) {
             const int lo = __popcll(bal & 0xffffffffull), hi = __popcll(bal >> 32);
             if (lo) atomicAdd(counts + et * 32 + 8 * q + s, lo);
             if (hi) atomicAdd(counts + et * 32 + 8 * q + 4 + s, hi);
           }
         }
-      }
-    }
   }
 }
 
