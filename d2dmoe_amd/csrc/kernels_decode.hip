@@ -133,8 +133,8 @@ hipError_t launch_decode_pack(const d2dmoe_shape& sh, const void* w1, const void
 //
 // decode_out_kernel: workgroup = 8 output columns, 8 waves.
 //   the routed experts are listed in ascending order and cut into 8 consecutive runs, one per wave; a wave chains
-//   OUT^T += W2[e]^T . H[e]^T over its run in one float32 accumulator (rows 8..15 of the 16-row MFMA tile are zero
-//   and dropped); the 8 partial tiles are added in wave order, then last_bias and the residual, one
+//   OUT^T += W2[e]^T . H[e]^T over its run in one float32 accumulator (rows 8..15 of the 16-row MFMA tile repeat
+//   rows 0..7 and are dropped); the 8 partial tiles are added in wave order, then last_bias and the residual, one
 //   rounding.  The summation order depends on the routing only.
 // ---------------------------------------------------------------------------------------------------
 struct DecodeArgs {
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
   const int EW = (E + DO_WAVES - 1) / DO_WAVES;
   const int e_lo = w * EW, e_hi = (e_lo + EW < E) ? (e_lo + EW) : E;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  // A fragment rows 0..7 only (lanes c16 < 8); result rows 8..15 are dropped
+  // A fragment rows 0..7 only (lanes c16 >= 8 repeat them); result rows 8..15 are dropped
   const bf16x8* wdf = A.wd + (int64_t)cb * E * KS2 * 32 + gq * 8 + (c16 & 7);
   const bf16x8* hf = A.hfrag + lane;
   bf16x8 aA[UB][KS2], bA[UB][KS2], aB[UB][KS2], bB[UB][KS2];
@@ -260,10 +260,6 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
       int e = e0;
       int es[UB];
 #pragma unroll
-      for (int j = 0; j < UB; ++j)
-#pragma unroll
-        for (int k2 = 0; k2 < KS2; ++k2) a[j][k2] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
       for (int j = 0; j < UB; ++j) {
         if (mask != 0ull) {
           e = e0 + (int)__builtin_ctzll(mask);
@@ -274,13 +270,12 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
         for (int k2 = 0; k2 < KS2; ++k2) b[j][k2] = hf[((int64_t)e * KS2 + k2) * 64];
         es[j] = e;
       }
-      // rows 8..15 of the A tile are not needed: those lanes request nothing and multiply zeros
-      if (c16 < 8) {
+      // rows 8..15 of the A tile are not needed: their lanes read the same 16 bytes as rows 0..7 (no extra traffic, and
+      // no load under a lane-dependent branch), and the result rows they produce are dropped
 #pragma unroll
-        for (int j = 0; j < UB; ++j)
+      for (int j = 0; j < UB; ++j)
 #pragma unroll
-          for (int k2 = 0; k2 < KS2; ++k2) a[j][k2] = wdf[((int64_t)es[j] * KS2 + k2) * 32];
-      }
+        for (int k2 = 0; k2 < KS2; ++k2) a[j][k2] = wdf[((int64_t)es[j] * KS2 + k2) * 32];
     };
     auto multiply = [&](bf16x8 (&a)[UB][KS2], bf16x8 (&b)[UB][KS2], int cnt) __attribute__((always_inline)) {
 #pragma unroll
