@@ -340,12 +340,25 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs<T> A)
 #pragma unroll
       for (int i = 0; i < NH; ++i) {
         const int h0 = (nb * 2 + wm) * HW + 32 * i;
+        // experts of a multiple of 32 neurons: the whole 32-row tile belongs to one expert, one routing value serves it
+        const bool one_expert = (A.edp & 31) == 0;   // uniform
+        float rw_tile = 0.f;
+        bool live_tile = false;
+        if (one_expert) {
+          const int e = h0 / A.edp;
+          live_tile = tok < N && e < A.E;
+          rw_tile = live_tile ? Elem<T>::load(A.routing + tok * A.E + e) : 0.f;
+        }
         float hv[16];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int e = (h0 + 8 * q + 4 * g) / A.edp;   // the expert of these four rows
-          const bool live = tok < N && e < A.E;
-          const float rw = live ? Elem<T>::load(A.routing + tok * A.E + e) : 0.f;
+          float rw = rw_tile;
+          bool live = live_tile;
+          if (!one_expert) {
+            const int e = (h0 + 8 * q + 4 * g) / A.edp;   // the expert of these four rows
+            live = tok < N && e < A.E;
+            rw = live ? Elem<T>::load(A.routing + tok * A.E + e) : 0.f;
+          }
           float bq[4] = {0.f, 0.f, 0.f, 0.f};
           if (!GATED) {
 #pragma unroll
