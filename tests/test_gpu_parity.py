@@ -312,6 +312,37 @@ def test_experts_mfma_sparse_full_size_and_auto_switch():
     assert torch.equal(r_auto, r_dense) and H.rel_err(out_auto, out_dense) < 1e-2
     want = O.layer_from_routing(x[rows].double(), O.upcast(p), r_auto.cpu()[rows].double(), 'relu', 'all')
     assert H.rel_err(out_auto.cpu()[rows], want) < H.TOL_BF16
+def test_full_size_token_permutation_equivariance():
+    """50432 tokens: a token's output does not depend on where in the batch it sits.  Expert-major path: bit-exact under
+    a random permutation of the tokens (every token's sum runs over its experts in ascending order, whatever its
+    neighbours).  Token-tile-major sweep: bit-exact for tokens that sit in full 64-token tiles before and after (the
+    tail tiles add their chunk ranges' float32 sums in a second step, which may move the last bf16 bit), and within
+    one bf16 ulp everywhere."""
+    N = 50432
+    g = torch.Generator().manual_seed(77)
+    perm = torch.randperm(N, generator=g)
+    x, routing, p = H.random_case(N, 768, 128, 24, 8, seed=78, dtype=torch.bfloat16, density=0.0165)
+    packed = _packed_for(p)
+    d = H.to_dev(p, DEV)
+    lb = d['last_bias'].view(-1)
+    xg, rg, pg = x.to(DEV), routing.to(DEV), perm.to(DEV)
+    xp, rp = xg[pg].contiguous(), rg[pg].contiguous()
+    a = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, 'relu', True, 'mfma_sparse', packed)
+    b = _ops().experts(xp, rp, d['w1'], d['b1'], d['w2'], None, lb, 'relu', True, 'mfma_sparse', packed)
+    assert torch.equal(a[pg], b)
+    x2, routing2, _ = H.random_case(N, 768, 128, 24, 8, seed=79, dtype=torch.bfloat16, density=0.79)
+    xg, rg = x2.to(DEV), routing2.to(DEV)
+    xp, rp = xg[pg].contiguous(), rg[pg].contiguous()
+    a = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, 'relu', True, 'mfma_dense', packed)
+    b = _ops().experts(xp, rp, d['w1'], d['b1'], d['w2'], None, lb, 'relu', True, 'mfma_dense', packed)
+    full = (N // (64 * 256)) * 64 * 256          # tokens in whole rounds of 64-token tiles on 256 CUs at most
+    pos_after = torch.empty(N, dtype=torch.long, device=DEV)
+    pos_after[pg] = torch.arange(N, device=DEV)   # token n sits at row pos_after[n] of the permuted batch
+    both_full = (torch.arange(N, device=DEV) < full) & (pos_after < full)
+    assert both_full.float().mean() > 0.8
+    assert torch.equal(a[both_full], b[pos_after[both_full]])
+    diff = (a.float() - b[pos_after].float()).abs()
+    assert (diff <= a.float().abs() * 2 ** -7 + 1e-6).all()
 
 
 def test_packed_weights_cache_tracks_parameter_updates():
