@@ -423,3 +423,13 @@ def test_vit_surgery_keeps_the_function_and_the_parameter_names():
         out, gating = moe(x, return_gating_data=True)
     frac = gating[names[1]][0].float().mean().item()
     assert out.shape == (3, 10) and 0.0 < frac < 1.0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The path is measured on one GPU; asking bench.py for more ends with a message that says so, before any GPU call."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--gpus', '2'], capture_output=True, text=True, timeout=120)
+    assert res.returncode != 0
+    assert 'single-GPU' in (res.stderr + res.stdout)
