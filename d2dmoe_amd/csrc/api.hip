@@ -205,13 +205,17 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
     }
     case D2DMOE_PATH_MFMA_SPARSE: {
       // expert-major when the routed pairs fit the provisioned capacity, else the dense sweep: decided on the device
-      if (!mfma_sparse_supported(sh) || !mfma_dense_supported(sh)) return D2DMOE_E_UNSUPPORTED;
+      if (!mfma_sparse_supported(sh)) return D2DMOE_E_UNSUPPORTED;
+      if (sh.gated ? !mfma_gemm_supported(sh) : !mfma_dense_supported(sh)) return D2DMOE_E_UNSUPPORTED;
       if (!packed) return D2DMOE_E_NULL;
       const size_t need = mfma_sparse_workspace_bytes(sh);
       if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
       const int* flag = nullptr;
       hipError_t e = launch_mfma_sparse(sh, x, routing, packed, last_bias, out, workspace, 8, &flag, s);
       if (e != hipSuccess) return (int)e;
+      if (sh.gated)   // gated layers fall back to the tiled products, which work behind the plan in the same workspace
+        return (int)launch_mfma_gemm(sh, x, routing, (const char*)packed + mfma_gemm_section_offset(sh), last_bias, out,
+                                     (char*)workspace + mfma_sparse_fallback_offset(sh), s, flag);
       return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, nullptr, 0, s);
     }
     case D2DMOE_PATH_MFMA_DECODE: {
@@ -283,7 +287,7 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   // A high threshold fraction keeps few experts per token: take the expert-major path (it falls back to the dense
   // sweep on the device if the routing turns out dense after all).
   if (path == D2DMOE_PATH_AUTO && sh.n_tokens > 16 && packed != nullptr && thr_scale >= 0.75f && mfma_sparse_supported(sh) &&
-      mfma_dense_supported(sh))
+      (sh.gated ? mfma_gemm_supported(sh) : mfma_dense_supported(sh)))
     path = D2DMOE_PATH_MFMA_SPARSE;
   return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,
                         plan.total - plan.perm_off, stream);

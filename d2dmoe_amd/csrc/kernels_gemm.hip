@@ -195,6 +195,7 @@ struct GemmArgs {
   int n_ttiles;            // 256-token tiles
   int tpx;                 // token tiles per XCD: ceil(n_ttiles / 8)
   int ksplit;
+  const int* skip_flag;    // optional device flag: non-zero = another path has handled this call
 };
 
 // one fragment pair into a 32 x 32 accumulator tile
@@ -218,6 +219,7 @@ template <typename T, int MODE, int ACT, bool GATED>
 __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs<T> A) {
   constexpr int KPF = GemmElem<T>::KPF, EPP = GemmElem<T>::EPP;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
   u32x4* lds0 = (u32x4*)smem_raw;            // [8 token tiles][4 fragments][64 lanes]
   u32x4* lds1 = lds0 + 8 * 4 * 64;
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
@@ -416,7 +418,8 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs<T> A)
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restrict__ partial, const T* __restrict__ last_bias,
                                                           const T* __restrict__ x, T* __restrict__ out, int64_t N, int D,
-                                                          int ksplit, int add_residual) {
+                                                          int ksplit, int add_residual, const int* __restrict__ skip_flag) {
+  if (skip_flag != nullptr && *skip_flag != 0) return;   // uniform over the whole grid
   const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int per_row = D / 8;
   if (p >= N * per_row) return;
@@ -451,10 +454,10 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restric
 
 template <typename T>
 static hipError_t launch_sum_partials_t(const float* partial, const void* last_bias, const void* x, void* out, int64_t N, int D,
-                                        int n_splits, int add_residual, hipStream_t s) {
+                                        int n_splits, int add_residual, hipStream_t s, const int* skip_flag = nullptr) {
   const int64_t items = N * (D / 8);
   hipLaunchKernelGGL(gemm_finish_kernel<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, partial, (const T*)last_bias,
-                     (const T*)x, (T*)out, N, D, n_splits, add_residual);
+                     (const T*)x, (T*)out, N, D, n_splits, add_residual, skip_flag);
   return hipGetLastError();
 }
 
@@ -465,7 +468,7 @@ hipError_t launch_sum_partials(const float* partial, const void* last_bias, cons
 
 template <typename T, int ACT, bool GATED>
 static hipError_t launch_gemm_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
-                                  const void* last_bias, void* out, void* workspace, hipStream_t s) {
+                                  const void* last_bias, void* out, void* workspace, hipStream_t s, const int* skip_flag) {
   const GemmLayout L = gemm_layout(sh);
   const GemmPlan P = gemm_plan(sh);
   const char* pk = (const char*)packed_section;
@@ -488,12 +491,13 @@ static hipError_t launch_gemm_act(const d2dmoe_shape& sh, const void* x, const v
     A.n_ttiles = (n + GM_BT - 1) / GM_BT;
     A.tpx = (A.n_ttiles + 7) / 8;
     A.ksplit = P.ksplit;
+    A.skip_flag = skip_flag;
     A.w = (const u32x4*)(pk + L.up_off);
     hipLaunchKernelGGL(k_up, dim3((unsigned)(8 * A.tpx * (L.hp / (GATED ? 128 : 256)))), dim3(256), lds, s, A);
     A.w = (const u32x4*)(pk + L.dn_off);
     hipLaunchKernelGGL(k_dn, dim3((unsigned)(8 * A.tpx * (sh.d_model / 256) * P.ksplit)), dim3(256), lds, s, A);
     e = launch_sum_partials_t<T>(A.partial, last_bias, A.x, (T*)out + t0 * sh.d_model, (int64_t)n, sh.d_model, P.ksplit,
-                                 sh.add_residual, s);
+                                 sh.add_residual, s, skip_flag);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;
@@ -501,24 +505,24 @@ static hipError_t launch_gemm_act(const d2dmoe_shape& sh, const void* x, const v
 
 template <typename T, bool GATED>
 static hipError_t launch_gemm_gated(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
-                                    const void* last_bias, void* out, void* workspace, hipStream_t s) {
+                                    const void* last_bias, void* out, void* workspace, hipStream_t s, const int* skip_flag) {
   switch (sh.activation) {
-    case D2DMOE_ACT_RELU: return launch_gemm_act<T, D2DMOE_ACT_RELU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    case D2DMOE_ACT_GELU: return launch_gemm_act<T, D2DMOE_ACT_GELU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    case D2DMOE_ACT_GELU_TANH: return launch_gemm_act<T, D2DMOE_ACT_GELU_TANH, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    case D2DMOE_ACT_SILU: return launch_gemm_act<T, D2DMOE_ACT_SILU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    default: return launch_gemm_act<T, -1, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    case D2DMOE_ACT_RELU: return launch_gemm_act<T, D2DMOE_ACT_RELU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
+    case D2DMOE_ACT_GELU: return launch_gemm_act<T, D2DMOE_ACT_GELU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
+    case D2DMOE_ACT_GELU_TANH: return launch_gemm_act<T, D2DMOE_ACT_GELU_TANH, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
+    case D2DMOE_ACT_SILU: return launch_gemm_act<T, D2DMOE_ACT_SILU, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
+    default: return launch_gemm_act<T, -1, GATED>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
   }
 }
 
 hipError_t launch_mfma_gemm(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
-                            const void* last_bias, void* out, void* workspace, hipStream_t s) {
+                            const void* last_bias, void* out, void* workspace, hipStream_t s, const int* skip_flag) {
   if (sh.dtype == D2DMOE_F32) {
-    if (sh.gated) return launch_gemm_gated<float, true>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-    return launch_gemm_gated<float, false>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+    if (sh.gated) return launch_gemm_gated<float, true>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
+    return launch_gemm_gated<float, false>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
   }
-  if (sh.gated) return launch_gemm_gated<bf16_t, true>(sh, x, routing, packed_section, last_bias, out, workspace, s);
-  return launch_gemm_gated<bf16_t, false>(sh, x, routing, packed_section, last_bias, out, workspace, s);
+  if (sh.gated) return launch_gemm_gated<bf16_t, true>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
+  return launch_gemm_gated<bf16_t, false>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
 }
 
 }  // namespace d2dmoe

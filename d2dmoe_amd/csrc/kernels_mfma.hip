@@ -45,8 +45,10 @@ bool mfma_router_supported(const d2dmoe_shape& sh) {
 }
 
 // The expert-major kernel covers the same layers as the dense sweep with experts of at most 128 neurons.
+// Gated experts have their own expert-major kernel, instantiated for D = 2048 and experts of at most 64 neurons (Gemma).
 bool mfma_sparse_supported(const d2dmoe_shape& sh) {
-  if (sh.dtype != D2DMOE_BF16 || sh.gated) return false;
+  if (sh.dtype != D2DMOE_BF16) return false;
+  if (sh.gated) return sh.d_model == 2048 && sh.expert_dim <= 64 && sh.n_experts <= 1024;
   if (sh.d_model != 768) return false;
   return sh.expert_dim <= 128 && sh.n_experts <= 1024;
 }
@@ -66,8 +68,10 @@ PackedLayout packed_layout(const d2dmoe_shape& sh) {
   L.has_sparse = mfma_sparse_supported(sh);
   const int nt = (sh.expert_dim + 31) / 32;
   L.nt = (nt <= 1) ? 1 : (nt == 2 ? 2 : 4);   // kernels are instantiated for 1, 2 and 4 row tiles
+  if (sh.gated) L.nt = 2;                      // the gated kernel always works on two tiles per projection
   const size_t frag_bytes = (size_t)sh.n_experts * L.nt * 32 * sh.d_model * 2;
   L.s1_off = off;   if (L.has_sparse) off += frag_bytes;
+  L.su_off = off;   if (L.has_sparse && sh.gated) off += frag_bytes;
   L.s2_off = off;   if (L.has_sparse) off += frag_bytes;
   L.sb_off = off;   if (L.has_sparse) off += (size_t)sh.n_experts * L.nt * 32 * 2;
   off = (off + 255) / 256 * 256;
@@ -184,7 +188,7 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
                        sh.router_width, sh.n_experts);
   }
   if (L.has_sparse) {
-    hipError_t e = launch_sparse_pack(sh, L, w1, b1, w2, packed, s);
+    hipError_t e = launch_sparse_pack(sh, L, w1, b1, w2, w_up, packed, s);
     if (e != hipSuccess) return e;
   }
   if (L.has_decode) {

@@ -43,10 +43,17 @@ static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) 
   W.tok_off = take((size_t)(N + 1) * 4);
   W.token_idx = take((size_t)W.cap * 4);
   W.pair_dst = take((size_t)W.cap * 4);
-  W.y = take((size_t)W.cap * sh.d_model * 2);
+  size_t ybytes = (size_t)W.cap * sh.d_model * 2;
+  if (sh.gated) {   // the fall-back of a gated layer (tiled products) works in the same region
+    const size_t g = mfma_gemm_workspace_bytes(sh);
+    if (g > ybytes) ybytes = g;
+  }
+  W.y = take(ybytes);
   W.total = off;
   return W;
 }
+
+size_t mfma_sparse_fallback_offset(const d2dmoe_shape& sh) { return sparse_workspace(sh, SP_MAX_MEAN_K).y; }
 
 size_t mfma_sparse_workspace_bytes(const d2dmoe_shape& sh) {
   if (!mfma_sparse_supported(sh)) return 0;
@@ -69,6 +76,7 @@ __global__ void pack_sparse_kernel(const bf16_t* __restrict__ w1, const bf16_t* 
   const int lane = (int)(p % 64);
   const int g = lane / 32, c = lane % 32;
   if (p < n) {
+    if (w1 == nullptr) return;
     const int e = (int)(p / per_expert);
     int64_t q = (p % per_expert) / 64;
     const int t = (int)(q % nt);
@@ -80,6 +88,7 @@ __global__ void pack_sparse_kernel(const bf16_t* __restrict__ w1, const bf16_t* 
       d1[p * 8 + i] = (j < Ed) ? w1[((int64_t)e * D + d) * Ed + j] : (bf16_t)0;
     }
   } else if (p < 2 * n) {
+    if (w2 == nullptr) return;
     const int64_t pp = p - n;
     const int e = (int)(pp / per_expert);
     int64_t q = (pp % per_expert) / 64;
@@ -92,6 +101,7 @@ __global__ void pack_sparse_kernel(const bf16_t* __restrict__ w1, const bf16_t* 
       d2[pp * 8 + i] = (j < Ed) ? w2[((int64_t)e * Ed + j) * D + col] : (bf16_t)0;
     }
   } else if (p < 2 * n + (int64_t)E * nt * 32) {
+    if (db == nullptr) return;
     const int64_t pp = p - 2 * n;
     const int e = (int)(pp / (nt * 32)), j = (int)(pp % (nt * 32));
     db[pp] = (j < Ed && b1 != nullptr) ? b1[(int64_t)e * Ed + j] : (bf16_t)0;
@@ -99,9 +109,15 @@ __global__ void pack_sparse_kernel(const bf16_t* __restrict__ w1, const bf16_t* 
 }
 
 hipError_t launch_sparse_pack(const d2dmoe_shape& sh, const PackedLayout& L, const void* w1, const void* b1, const void* w2,
-                              void* packed, hipStream_t s) {
+                              const void* w_up, void* packed, hipStream_t s) {
   char* base = (char*)packed;
   const int64_t n = 2 * (int64_t)sh.n_experts * L.nt * 32 * sh.d_model / 8 + (int64_t)sh.n_experts * L.nt * 32;
+  if (sh.gated) {
+    // gated experts: the up projection is a second stream in the W1 arrangement; there is no bias
+    hipLaunchKernelGGL(pack_sparse_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const bf16_t*)w_up,
+                       (const bf16_t*)nullptr, (const bf16_t*)nullptr, (bf16_t*)(base + L.su_off), (bf16_t*)nullptr,
+                       (bf16_t*)nullptr, sh.d_model, sh.n_experts, sh.expert_dim, L.nt);
+  }
   hipLaunchKernelGGL(pack_sparse_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const bf16_t*)w1,
                      (const bf16_t*)b1, (const bf16_t*)w2, (bf16_t*)(base + L.s1_off), (bf16_t*)(base + L.s2_off),
                      (bf16_t*)(base + L.sb_off), sh.d_model, sh.n_experts, sh.expert_dim, L.nt);
@@ -287,6 +303,7 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restr
 // ---------------------------------------------------------------------------------------------------
 struct SparseArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* w1s; const bf16x8* w2s; const bf16_t* b1s;
+  const bf16x8* wus;   // gated experts: fragments of the up projection, arranged like w1s
   const int32_t* offsets; const int32_t* tile_off; const int32_t* token_idx; const int32_t* pair_dst; const int32_t* flag;
   bf16_t* y; int E; int act_rt;
   const int32_t* tok_off; const bf16_t* last_bias; bf16_t* out; int add_residual;   // tokens with ONE routed expert
@@ -508,7 +525,7 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
 __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__ y, const int32_t* __restrict__ tok_off,
                                                       const int32_t* __restrict__ flag, const bf16_t* __restrict__ x,
                                                       const bf16_t* __restrict__ last_bias, bf16_t* __restrict__ out, int64_t N,
-                                                      int D, int add_residual) {
+                                                      int D, int add_residual, int singles_done) {
   if (flag[0] == 0) return;
   const int ppr = D / 8;
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -519,7 +536,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   const int q0 = tok_off[n], q1 = tok_off[n + 1];
-  if (q1 - q0 == 1) return;   // finished by the experts kernel
+  if (singles_done && q1 - q0 == 1) return;   // finished by the experts kernel
   for (int q = q0; q < q1; ++q) {
     const uint4 v = *(const uint4*)(y + (int64_t)q * D + col);
     const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
@@ -542,6 +559,184 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__
   o.x = pack2_bf16(acc[0], acc[1]); o.y = pack2_bf16(acc[2], acc[3]);
   o.z = pack2_bf16(acc[4], acc[5]); o.w = pack2_bf16(acc[6], acc[7]);
   *(uint4*)(out + n * D + col) = o;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Gated experts, expert-major (Gemma shape: D = 2048, experts of at most 64 neurons, no biases):
+//   y[pair, :] = routing . (act(x Wg[e]) * (x Wu[e])) Wd[e]      for the 32 pairs of a tile of expert e
+// The layer is bound by the weight stream (786 KB per expert against 128 KB of x rows per tile), so the work is dealt to
+// keep four independent streams going.  First products: wave w owns ONE 32-neuron tile over all of K -- waves 0,1 the
+// gate tiles, waves 2,3 the up tiles -- with x rows read from their gathered positions (the four waves share them
+// through the L1) and two register buffers of 8 K steps; nothing is summed across waves.  The up waves hand their tile
+// to the gate waves through LDS, which apply the activation, the product and the routing weight and leave H as B
+// fragments in LDS.  Second product: wave w owns 512 output columns, 4 column tiles at a time, fragments of the next
+// four in flight while the current are multiplied; rows leave through a wave-private LDS tile as whole 256-byte
+// segments.  Every pair's row goes to y, tokens with one expert included; the combine kernel sums them.
+// ---------------------------------------------------------------------------------------------------
+template <int D, int ACT>
+__global__ __launch_bounds__(256, 2) void experts_gated_sparse_kernel(const SparseArgs A) {
+  constexpr int KS1 = D / 16;
+  constexpr int NT = 2;          // 32-neuron tiles per projection (expert size <= 64)
+  constexpr int CTW = D / 128;   // column tiles per wave
+  constexpr int U = 8;           // K steps per register buffer
+  static_assert(KS1 % (2 * U) == 0 && CTW % 8 == 0, "buffers alternate in pairs");
+  __shared__ int32_t s_tile_off[1025];
+  __shared__ int32_t s_offsets[1025];
+  __shared__ float upx[2][16][64];
+  __shared__ __attribute__((aligned(16))) bf16x8 hs[2 * NT][64];
+  __shared__ __attribute__((aligned(16))) u32x4 stage_all[4][32 * 16];
+  if (A.flag[0] == 0) return;
+  const int E = A.E;
+  for (int i = threadIdx.x; i <= E; i += 256) {
+    s_tile_off[i] = A.tile_off[i];
+    s_offsets[i] = A.offsets[i];
+  }
+  __syncthreads();
+  const int n_tiles = s_tile_off[E];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int g = lane >> 5, c32 = lane & 31;
+  const int xcd = blockIdx.x & 7, wg = blockIdx.x >> 3, nwg = gridDim.x >> 3;   // the grid is a multiple of 8
+  const int t_lo = (int)((int64_t)n_tiles * xcd / 8), t_hi = (int)((int64_t)n_tiles * (xcd + 1) / 8);
+  for (int T = t_lo + wg; T < t_hi; T += nwg) {
+    int lo = 0, hi = E;   // largest e with tile_off[e] <= T
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (s_tile_off[mid] <= T) lo = mid; else hi = mid;
+    }
+    const int e = lo;
+    const int base = s_offsets[e];
+    const int cnt = s_offsets[e + 1] - base;
+    const int j0 = (T - s_tile_off[e]) * SP_BT;
+    const int rows = (cnt - j0 < SP_BT) ? (cnt - j0) : SP_BT;
+    const int pj = base + j0 + (c32 < rows ? c32 : rows - 1);
+    const int tok = A.token_idx[pj];
+    const int dst = A.pair_dst[pj];
+    const float rw = bf16_to_f32(A.routing[(int64_t)tok * E + e]);
+
+    // ---- first products: this wave's tile over all of K
+    const bf16x8* wf = ((w >> 1) ? A.wus : A.w1s) + ((int64_t)e * KS1 * NT + (w & 1)) * 64 + lane;   // + NT * 64 per K step
+    const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)tok * D) + g;                               // + 2 per K step
+    f32x16 acc1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc1[r] = 0.f;
+    bf16x8 xA[U], wA[U], xB[U], wB[U];
+    auto fill = [&](bf16x8 (&xb)[U], bf16x8 (&wb)[U], int ks0) __attribute__((always_inline)) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        xb[u] = xrow[2 * (ks0 + u)];
+        wb[u] = wf[(int64_t)(ks0 + u) * NT * 64];
+      }
+    };
+    auto multiply = [&](bf16x8 (&xb)[U], bf16x8 (&wb)[U]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[u], xb[u], acc1, 0, 0, 0);
+    };
+    fill(xA, wA, 0);
+    for (int ks0 = 0; ks0 < KS1; ks0 += 2 * U) {
+      fill(xB, wB, ks0 + U);
+      multiply(xA, wA);
+      fill(xA, wA, (ks0 + 2 * U < KS1) ? (ks0 + 2 * U) : ks0);   // the last trip re-reads its own steps: in bounds, unused
+      multiply(xB, wB);
+    }
+    // the first column tiles of the second product are requested before the exchange
+    const bf16x8* w2f = A.w2s + ((int64_t)e * (D / 32) + w * CTW) * (2 * NT) * 64 + lane;   // [col tile][K step 2 NT][lane]
+    bf16x8 fA[4][2 * NT], fB[4][2 * NT];
+    auto fill2 = [&](bf16x8 (&f)[4][2 * NT], int ct0) __attribute__((always_inline)) {
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int k = 0; k < 2 * NT; ++k) f[ct][k] = w2f[((ct0 + ct) * (2 * NT) + k) * 64];
+    };
+    fill2(fA, 0);
+    if (w >= 2) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) upx[w - 2][r][lane] = acc1[r];
+    }
+    __syncthreads();
+    if (w < 2) {
+      float hv[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float gv = (ACT >= 0) ? act_fn<ACT>(acc1[r]) : apply_act(A.act_rt, acc1[r]);
+        hv[r] = gv * upx[w][r][lane] * rw;
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        uint4 pk;
+        pk.x = pack2_bf16(hv[half * 8 + 0], hv[half * 8 + 1]);
+        pk.y = pack2_bf16(hv[half * 8 + 2], hv[half * 8 + 3]);
+        pk.z = pack2_bf16(hv[half * 8 + 4], hv[half * 8 + 5]);
+        pk.w = pack2_bf16(hv[half * 8 + 6], hv[half * 8 + 7]);
+        ((uint4*)hs)[(w * 2 + half) * 64 + lane] = pk;
+      }
+    }
+    __syncthreads();
+    bf16x8 hb[2 * NT];
+#pragma unroll
+    for (int k = 0; k < 2 * NT; ++k) hb[k] = hs[k][lane];
+
+    // ---- second product (transposed): OUT^T[512 columns of this wave, 32 pairs], 4 column tiles per pass
+    u32x4* stage = stage_all[w];                    // 32 rows x 256 bytes
+    const int rl = lane >> 4, pc = lane & 15;
+    bf16_t* rptr[8];
+    bool rlive[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int R = rl + 4 * i;
+      const int rd = __shfl(dst, R, kWave);
+      rptr[i] = A.y + (int64_t)rd * D + w * (D / 4) + pc * 8;
+      rlive[i] = R < rows;
+    }
+    auto pass = [&](bf16x8 (&f)[4][2 * NT], int ct0) __attribute__((always_inline)) {
+      f32x16 acc2[4];
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc2[ct][r] = 0.f;
+#pragma unroll
+        for (int k = 0; k < 2 * NT; ++k) acc2[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[ct][k], hb[k], acc2[ct], 0, 0, 0);
+      }
+      // lane = pair c32, accumulator r = column 8*(r/4) + 4g + r%4 of the tile -> 16-byte piece ct*4 + r/4, half g
+      uint2* srow = (uint2*)(stage + c32 * 16);
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint2 o;
+          o.x = pack2_bf16(acc2[ct][q * 4 + 0], acc2[ct][q * 4 + 1]);
+          o.y = pack2_bf16(acc2[ct][q * 4 + 2], acc2[ct][q * 4 + 3]);
+          srow[(((ct * 4 + q) ^ (c32 & 15)) << 1) + g] = o;
+        }
+      __builtin_amdgcn_wave_barrier();
+      u32x4 rowv[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int R = rl + 4 * i;
+        rowv[i] = stage[R * 16 + (pc ^ (R & 15))];
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (rlive[i]) *(u32x4*)(rptr[i] + ct0 * 32) = rowv[i];
+    };
+    for (int ct0 = 0; ct0 < CTW; ct0 += 8) {
+      fill2(fB, ct0 + 4);
+      pass(fA, ct0);
+      fill2(fA, (ct0 + 8 < CTW) ? (ct0 + 8) : ct0);   // the last trip re-reads its own tiles: in bounds, unused
+      pass(fB, ct0 + 4);
+    }
+  }
+}
+
+static void launch_gated_sparse_experts(const SparseArgs& A, int act, unsigned grid, hipStream_t s) {
+  switch (act) {
+    case D2DMOE_ACT_GELU_TANH:
+      hipLaunchKernelGGL((experts_gated_sparse_kernel<2048, D2DMOE_ACT_GELU_TANH>), dim3(grid), dim3(256), 0, s, A); break;
+    case D2DMOE_ACT_RELU:
+      hipLaunchKernelGGL((experts_gated_sparse_kernel<2048, D2DMOE_ACT_RELU>), dim3(grid), dim3(256), 0, s, A); break;
+    default:
+      hipLaunchKernelGGL((experts_gated_sparse_kernel<2048, -1>), dim3(grid), dim3(256), 0, s, A); break;
+  }
 }
 
 template <int NT>
@@ -599,13 +794,15 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   A.tile_off = tile_off; A.token_idx = token_idx; A.pair_dst = pair_dst; A.flag = flag; A.y = y; A.E = E;
   A.act_rt = sh.activation;
   A.tok_off = tok_off; A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.add_residual = sh.add_residual;
+  A.wus = (const bf16x8*)(pk + L.su_off);
   const unsigned grid = (unsigned)(8 * device_cu_count());
-  if (L.nt == 1) launch_sparse_experts<1>(A, sh.activation, grid, s);
+  if (sh.gated) launch_gated_sparse_experts(A, sh.activation, grid, s);
+  else if (L.nt == 1) launch_sparse_experts<1>(A, sh.activation, grid, s);
   else if (L.nt == 2) launch_sparse_experts<2>(A, sh.activation, grid, s);
   else launch_sparse_experts<4>(A, sh.activation, grid, s);
   const int64_t n_threads = N * (sh.d_model / 8);
   hipLaunchKernelGGL(combine_kernel, dim3((unsigned)cdiv64(n_threads, 256)), dim3(256), 0, s, y, tok_off, flag, (const bf16_t*)x,
-                     (const bf16_t*)last_bias, (bf16_t*)out, N, sh.d_model, sh.add_residual);
+                     (const bf16_t*)last_bias, (bf16_t*)out, N, sh.d_model, sh.add_residual, sh.gated ? 0 : 1);
   *flag_out = flag;
   return hipGetLastError();
 }

@@ -56,6 +56,9 @@ hipError_t launch_sum_partials(const float* partial, const void* last_bias, cons
 // ---- bf16 MFMA expert-major path (kernels_sparse.hip) ----
 bool mfma_sparse_supported(const d2dmoe_shape& sh);
 size_t mfma_sparse_workspace_bytes(const d2dmoe_shape& sh);
+// Offset inside the expert-major workspace at which a gated layer's fall-back (the tiled products) may work: behind the
+// plan, in the region the per-pair rows would have used.
+size_t mfma_sparse_fallback_offset(const d2dmoe_shape& sh);
 // Plans the call on the device (permutation, tiles, path flag), runs the expert-major kernels when the number of routed
 // pairs is at most n_tokens * max_mean_k, and leaves *flag == 0 otherwise so that the dense sweep (launched by the
 // caller with skip_flag = the returned pointer) does the work instead.
@@ -78,7 +81,7 @@ size_t mfma_gemm_section_offset(const d2dmoe_shape& sh);
 hipError_t launch_gemm_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                             void* packed_section, hipStream_t s);
 hipError_t launch_mfma_gemm(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
-                            const void* last_bias, void* out, void* workspace, hipStream_t s);
+                            const void* last_bias, void* out, void* workspace, hipStream_t s, const int* skip_flag = nullptr);
 void launch_perm_scan(const int32_t* seg_counts, int32_t* seg_offsets, int32_t* totals, int E, int64_t n_seg, hipStream_t s);
 
 // ---- per-expert output norms, the router-training targets (kernels_norms.hip) ----

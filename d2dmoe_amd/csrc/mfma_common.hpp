@@ -33,6 +33,7 @@ struct PackedLayout {
   size_t w_off, b1_off, eidx_off;        // dense sweep: weight stream, bias (bf16), expert index per neuron (uint8)
   size_t r1_off, r2_off;                 // router fragments
   size_t s1_off, s2_off, sb_off;         // expert-major: W1 fragments, W2^T fragments, bias (bf16, padded to nt*32)
+  size_t su_off;                         // expert-major, gated experts: fragments of the up projection
   size_t dc_off;                         // small-batch (decode) section
   size_t gm_off;                         // large-batch gated section (tiled products)
   size_t total;
@@ -44,7 +45,7 @@ size_t mfma_decode_packed_bytes(const d2dmoe_shape& sh);
 hipError_t launch_decode_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                               void* packed_section, hipStream_t s);
 hipError_t launch_sparse_pack(const d2dmoe_shape& sh, const PackedLayout& L, const void* w1, const void* b1, const void* w2,
-                              void* packed, hipStream_t s);
+                              const void* w_up, void* packed, hipStream_t s);
 
 // two float32 -> packed bf16 pair, round-to-nearest-even (one v_cvt_pk_bf16_f32 on gfx950)
 __device__ inline uint32_t pack2_bf16(float lo, float hi) {

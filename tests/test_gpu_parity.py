@@ -476,6 +476,57 @@ def test_tiled_products_path_matches_oracle(N, D, E, Ed, W, act, gated, dtype):
     assert torch.equal(got, _experts_got(x, weights, p, act, residual=True, path='mfma_gemm', packed=packed))
 
 
+@pytest.mark.parametrize('N,E,Ed,density,act', [(300, 16, 64, 0.15, 'gelu_tanh'), (4096, 256, 64, 0.009, 'gelu_tanh'),
+                                                (77, 8, 40, 0.3, 'relu'), (1, 4, 64, 0.5, 'silu'), (33, 40, 64, 0.05, 'gelu_tanh'),
+                                                (200, 16, 64, 0.7, 'gelu_tanh')])
+def test_gated_expert_major_path_matches_oracle(N, E, Ed, density, act):
+    """Gated experts at D = 2048 with few experts per token: plan -> per-expert gated kernel -> ordered combine.  The
+    last case routes more pairs than the path is provisioned for; the device-side flag then hands the call to the tiled
+    products, which work in the same workspace."""
+    _say('gated expert-major', N, E, Ed, density, act)
+    D = 2048
+    x, routing, p = H.random_case(N, D, E, Ed, 64, seed=N + E, dtype=torch.bfloat16, gated=True, bias=False, density=density)
+    routing[0] = 0
+    routing[0, E - 1] = 1            # a token with a single expert
+    if N > 2:
+        routing[2] = 0               # a token with none: zeros (gated experts carry no biases)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, 64, 1, act, gated=True)
+    packed = _ops().pack_weights(sh, d['w_gate'], None, d['w_down'], d['w_up'], d['router_w1'], d['router_w2'])
+    assert packed is not None
+    rows = torch.arange(N) if N <= 400 else torch.cat([torch.arange(64), torch.arange(N - 64, N)])
+    got = _experts_got(x, routing, p, act, path='mfma_sparse', packed=packed)
+    assert H.rel_err(got[rows], _experts_want(x[rows], routing[rows], p, act)) < H.TOL_BF16
+    if N > 2:
+        assert torch.equal(got[2].float(), torch.zeros(D))
+    assert torch.equal(got, _experts_got(x, routing, p, act, path='mfma_sparse', packed=packed))   # deterministic
+    # against the tiled products on every row
+    assert H.rel_err(got, _experts_got(x, routing, p, act, path='mfma_gemm', packed=packed)) < 1e-2
+    # weighted routing + residual
+    g = torch.Generator().manual_seed(5)
+    weights = (routing.float() * (torch.rand(N, E, generator=g) + 0.5)).to(torch.bfloat16)
+    got = _experts_got(x, weights, p, act, residual=True, path='mfma_sparse', packed=packed)
+    assert H.rel_err(got[rows], _experts_want(x[rows], weights[rows], p, act, True)) < H.TOL_BF16
+
+
+def test_gated_layer_takes_the_expert_major_path_for_a_high_threshold():
+    """Whole gated layer at the Gemma shape, 4096 tokens, keep norm >= 0.9 * max: AUTO plans on the device and runs the
+    expert-major kernels; the result equals the tiled products' on the same routing within the bf16 tolerance."""
+    N, D, E, Ed, W = 4096, 2048, 256, 64, 256
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=7, dtype=torch.bfloat16, gated=True, bias=False)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, W, 1, 'gelu_tanh', gated=True)
+    packed = _ops().pack_weights(sh, d['w_gate'], None, d['w_down'], d['w_up'], d['router_w1'], d['router_w2'])
+    out_a, r_a, _, _ = _forward(x, p, 0.1, 'gelu_tanh', path='auto', packed=packed)
+    out_g, r_g, _, _ = _forward(x, p, 0.1, 'gelu_tanh', path='mfma_gemm', packed=packed)
+    assert torch.equal(r_a, r_g)
+    assert 1.0 <= r_a.float().sum(1).mean().item() < 8.0
+    assert H.rel_err(out_a, out_g) < 1e-2
+    rows = torch.cat([torch.arange(48), torch.arange(N - 48, N)])
+    want = O.layer_from_routing(x[rows].double(), O.upcast(p), r_a.cpu()[rows].double(), 'gelu_tanh', 'all')
+    assert H.rel_err(out_a.cpu()[rows], want) < H.TOL_BF16
+
+
 # =================================================================== whole layer ======================
 def _forward(x, p, tau, act='relu', norms_in=None, path='auto', packed=None, residual=False):
     d = H.to_dev(p, DEV)
