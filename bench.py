@@ -258,6 +258,24 @@ def run_gated(args, ops, dev):
                             'frac': active / ms_experts / 1e9 / PEAK_BF16_TFLOPS,
                             'traffic': MEASURED_TRAFFIC.get(args.workload), 'kernel_ms': ms_experts,
                             'executed_tflops': executed / ms_experts / 1e9}
+        # the literal reading of the same number (keep norm >= tau * max): a few experts per token, the layer is bound by
+        # the weight stream again and takes the expert-major path
+        lit_scale = float(args.tau)
+
+        def layer_lit():
+            return ops.forward(x, rw1, rw2, lit_scale, wg, None, wd, wu, None, act, False, None, False, False, 'auto', packed)
+
+        _, r_lit, _, _ = layer_lit()
+        torch.cuda.synchronize()
+        ms_lit = time_events(layer_lit, args.steps, args.warmup)
+        union_lit = int((r_lit.float().sum(0) > 0).sum().item())
+        pairs_lit = int(r_lit.float().sum().item())
+        bytes_lit = (W * D + E * W) * s + union_lit * 3 * D * Ed * s + 2 * N * D * s + N * E * s
+        line['literal_rule'] = {'rule': f'keep norm >= {args.tau}*max', 'ms_per_step': ms_lit, 'tokens_per_s': N / ms_lit * 1e3,
+                                'mean_active_experts': pairs_lit / N, 'experts_routed_to': union_lit,
+                                'roofline': {'bound': 'hbm', 'achieved': bytes_lit / ms_lit / 1e6, 'peak': PEAK_HBM_GBPS,
+                                             'unit': 'GB/s', 'frac': bytes_lit / ms_lit / 1e6 / PEAK_HBM_GBPS,
+                                             'algorithmic_bytes': bytes_lit}}
     print(json.dumps(line))
 
 
