@@ -91,20 +91,23 @@ def test_packed_and_workspace_sizes_follow_the_documented_layouts():
     from d2dmoe_amd import hip_abi as abi, ops
     lib = abi.load()
     lib.d2dmoe_packed_bytes.restype = ctypes.c_size_t
-    # Gemma-2B FFN: small-batch section (gate|up + down, 3 matrices + padded bias) + tiled-products section (3 matrices +
-    # bias) + router section
+    # Gemma-2B FFN: expert-major section (gate, up, down fragments + padded bias) + small-batch section (gate|up + down,
+    # 3 matrices + padded bias) + tiled-products section (3 matrices + bias) + router section
     mat = 256 * 64 * 2048 * 2
     g = ops.make_shape(4096, 2048, 256, 64, 256, abi.BF16, 'gelu_tanh', gated=True)
-    want = (3 * mat + 256 * 64 * 2) + (3 * mat + 256 * 64 * 2) + (256 * 2048 + 256 * 256) * 2
+    want = 3 * (3 * mat + 256 * 64 * 2) + (256 * 2048 + 256 * 256) * 2
     got = lib.d2dmoe_packed_bytes(ctypes.byref(g))
-    assert want <= got <= want + 4 * 256 and got % 256 == 0
-    # workspace at 4096 tokens: router hidden + norms, then H fragments (4096 x 16384 bf16) + 2 float32 partial sums
+    assert want <= got <= want + 6 * 256 and got % 256 == 0
+    # workspace at 4096 tokens: router hidden + norms, then the expert-major plan (under 1 MB of counts, offsets and
+    # lists) in front of the region its fall-back, the tiled products, works in: H fragments (4096 x 16384 bf16) +
+    # 2 float32 partial sums (the per-pair rows, 8 x 4096 x 2048 bf16, are smaller)
     ws = lib.d2dmoe_workspace_bytes(ctypes.byref(g))
     want_ws = 4096 * 256 * 2 * 2 + 4096 * 16384 * 2 + 2 * 4096 * 2048 * 4
-    assert want_ws <= ws <= want_ws + 4 * 256
-    # 16 tokens: the small-batch path needs the hidden fragments and one flag per expert only
+    assert want_ws <= ws <= want_ws + (1 << 20)
+    # 16 tokens: the small-batch path needs the hidden fragments and one flag per expert only; the size query also covers
+    # the expert-major path on request, whose fall-back works on one 256-token tile of H fragments (8 MB)
     g16 = ops.make_shape(16, 2048, 256, 64, 256, abi.BF16, 'gelu_tanh', gated=True)
-    assert lib.d2dmoe_workspace_bytes(ctypes.byref(g16)) < 2 << 20
+    assert lib.d2dmoe_workspace_bytes(ctypes.byref(g16)) < 10 << 20
     # float32 layers: the tiled-products section only (hidden size 128 x 24 = 3072 neurons, float32 fragments)
     f = ops.make_shape(100, 768, 128, 24, 128, abi.F32)
     want_f = (2 * 3072 * 768 + 3072) * 4
