@@ -211,7 +211,7 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
       const size_t need = mfma_sparse_workspace_bytes(sh);
       if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
       const int* flag = nullptr;
-      hipError_t e = launch_mfma_sparse(sh, x, routing, packed, last_bias, out, workspace, 8, &flag, s);
+      hipError_t e = launch_mfma_sparse(sh, x, routing, packed, last_bias, out, workspace, mfma_sparse_capacity_k(sh), &flag, s);
       if (e != hipSuccess) return (int)e;
       if (sh.gated)   // gated layers fall back to the tiled products, which work behind the plan in the same workspace
         return (int)launch_mfma_gemm(sh, x, routing, (const char*)packed + mfma_gemm_section_offset(sh), last_bias, out,
@@ -286,7 +286,9 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   if (st != D2DMOE_OK) return st;
   // A high threshold fraction keeps few experts per token: take the expert-major path (it falls back to the dense
   // sweep on the device if the routing turns out dense after all).
-  if (path == D2DMOE_PATH_AUTO && sh.n_tokens > 16 && packed != nullptr && thr_scale >= 0.75f && mfma_sparse_supported(sh) &&
+  // (gated experts: from a lower fraction on -- their dense alternative costs ten times the expert-major path at few
+  // experts per token and the device-side switch is cheap next to it)
+  if (path == D2DMOE_PATH_AUTO && sh.n_tokens > 16 && packed != nullptr && thr_scale >= (sh.gated ? 0.5f : 0.75f) && mfma_sparse_supported(sh) &&
       (sh.gated ? mfma_gemm_supported(sh) : mfma_dense_supported(sh)))
     path = D2DMOE_PATH_MFMA_SPARSE;
   return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,

@@ -25,6 +25,14 @@ struct SparseWorkspace {
       total;
 };
 
+// Routed pairs per token the path is provisioned for.  Ungated experts (36 KB each at the ViT-B shape): 8 -- the dense
+// sweep is as fast from about 7 on.  Gated experts at the Gemma shape (786 KB each): the tiled products cost 0.8 ms per
+// 4096 tokens whatever the routing and the expert-major kernels stay below that up to about 40 pairs per token, so the
+// capacity is 32 -- up to 16 384 tokens, where the per-pair rows (4 KB each) take 2 GB; beyond that 8.
+int mfma_sparse_capacity_k(const d2dmoe_shape& sh) {
+  return (sh.gated && sh.n_tokens <= 16384) ? SP_MAX_MEAN_K_GATED : SP_MAX_MEAN_K;
+}
+
 static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) {
   SparseWorkspace W;
   const int64_t N = sh.n_tokens;
@@ -53,11 +61,11 @@ static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) 
   return W;
 }
 
-size_t mfma_sparse_fallback_offset(const d2dmoe_shape& sh) { return sparse_workspace(sh, SP_MAX_MEAN_K).y; }
+size_t mfma_sparse_fallback_offset(const d2dmoe_shape& sh) { return sparse_workspace(sh, mfma_sparse_capacity_k(sh)).y; }
 
 size_t mfma_sparse_workspace_bytes(const d2dmoe_shape& sh) {
   if (!mfma_sparse_supported(sh)) return 0;
-  return sparse_workspace(sh, SP_MAX_MEAN_K).total;
+  return sparse_workspace(sh, mfma_sparse_capacity_k(sh)).total;
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -754,8 +762,9 @@ static void launch_sparse_experts(const SparseArgs& A, int act, unsigned grid, h
 hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                               const void* last_bias, void* out, void* workspace, int max_mean_k, const int** flag_out,
                               hipStream_t s) {
-  if (max_mean_k > SP_MAX_MEAN_K) max_mean_k = SP_MAX_MEAN_K;
-  const SparseWorkspace W = sparse_workspace(sh, SP_MAX_MEAN_K);   // sized for the maximum; the flag uses max_mean_k
+  const int cap_k = mfma_sparse_capacity_k(sh);
+  if (max_mean_k > cap_k) max_mean_k = cap_k;
+  const SparseWorkspace W = sparse_workspace(sh, cap_k);   // sized for the maximum; the flag uses max_mean_k
   const PackedLayout L = packed_layout(sh);
   char* ws = (char*)workspace;
   const char* pk = (const char*)packed;

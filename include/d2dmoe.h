@@ -70,9 +70,9 @@ enum {
   D2DMOE_PATH_MFMA_DENSE = 2, /* bf16 MFMA, token-tile-major, masked dense sweep over all experts */
   D2DMOE_PATH_MFMA_SPARSE = 3, /* bf16 MFMA, expert-major over the permutation, then ordered combine; taken when at most
                                  8 experts per token are routed on average (checked on the device), else the dense
-                                 sweep runs (for gated experts: the tiled products).  Ungated experts at D = 768, gated
-                                 experts at D = 2048 with at most 64 neurons.  d2dmoe_forward picks it under AUTO when
-                                 thr_scale >= 0.75 */
+                                 sweep runs.  Ungated experts at D = 768.  Gated experts at D = 2048 with at most 64
+                                 neurons: up to 32 experts per token (8 beyond 16 384 tokens), else the tiled products
+                                 run.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 (gated: >= 0.5) */
   D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 MFMA for at most 16 tokens: one workgroup per expert streams that expert's packed
                                  weights once (gated or ungated experts); AUTO picks it when it applies */
   D2DMOE_PATH_MFMA_GEMM = 5   /* bf16 or f32 MFMA, D a multiple of 256, gated or ungated experts: two tiled products over all

@@ -98,12 +98,14 @@ def test_packed_and_workspace_sizes_follow_the_documented_layouts():
     want = 3 * (3 * mat + 256 * 64 * 2) + (256 * 2048 + 256 * 256) * 2
     got = lib.d2dmoe_packed_bytes(ctypes.byref(g))
     assert want <= got <= want + 6 * 256 and got % 256 == 0
-    # workspace at 4096 tokens: router hidden + norms, then the expert-major plan (under 1 MB of counts, offsets and
-    # lists) in front of the region its fall-back, the tiled products, works in: H fragments (4096 x 16384 bf16) +
-    # 2 float32 partial sums (the per-pair rows, 8 x 4096 x 2048 bf16, are smaller)
+    # workspace at 4096 tokens: router hidden + norms, then the expert-major plan (under 2 MB of counts, offsets and
+    # lists) and its per-pair result rows, provisioned for 32 routed experts per token (32 x 4096 rows of 2048 bf16); the
+    # fall-back, the tiled products, works in the same region (H fragments 4096 x 16384 bf16 + 2 float32 partial sums:
+    # smaller)
     ws = lib.d2dmoe_workspace_bytes(ctypes.byref(g))
-    want_ws = 4096 * 256 * 2 * 2 + 4096 * 16384 * 2 + 2 * 4096 * 2048 * 4
-    assert want_ws <= ws <= want_ws + (1 << 20)
+    want_ws = 4096 * 256 * 2 * 2 + 32 * 4096 * 2048 * 2
+    assert want_ws <= ws <= want_ws + (2 << 20)
+    assert 32 * 4096 * 2048 * 2 >= 4096 * 16384 * 2 + 2 * 4096 * 2048 * 4
     # 16 tokens: the small-batch path needs the hidden fragments and one flag per expert only; the size query also covers
     # the expert-major path on request, whose fall-back works on one 256-token tile of H fragments (8 MB)
     g16 = ops.make_shape(16, 2048, 256, 64, 256, abi.BF16, 'gelu_tanh', gated=True)
