@@ -478,11 +478,13 @@ def test_tiled_products_path_matches_oracle(N, D, E, Ed, W, act, gated, dtype):
 
 @pytest.mark.parametrize('N,E,Ed,density,act', [(300, 16, 64, 0.15, 'gelu_tanh'), (4096, 256, 64, 0.009, 'gelu_tanh'),
                                                 (77, 8, 40, 0.3, 'relu'), (1, 4, 64, 0.5, 'silu'), (33, 40, 64, 0.05, 'gelu_tanh'),
-                                                (200, 64, 64, 0.7, 'gelu_tanh'), (200, 16, 64, 0.7, 'gelu_tanh')])
+                                                (200, 64, 64, 0.7, 'gelu_tanh'), (200, 16, 64, 0.7, 'gelu_tanh'),
+                                                (16400, 16, 64, 0.2, 'gelu_tanh')])
 def test_gated_expert_major_path_matches_oracle(N, E, Ed, density, act):
     """Gated experts at D = 2048 with few experts per token: plan -> per-expert gated kernel -> ordered combine.  The
     last but one case routes 45 pairs per token, more than the 32 the path is provisioned for; the device-side flag then
-    hands the call to the tiled products, which work in the same workspace.  The last (11 per token) stays expert-major."""
+    hands the call to the tiled products, which work in the same workspace.  The next (11 per token) stays expert-major;
+    the last has more than 16 384 tokens, where the capacity is 8 per token and the fall-back runs in three passes."""
     _say('gated expert-major', N, E, Ed, density, act)
     D = 2048
     x, routing, p = H.random_case(N, D, E, Ed, 64, seed=N + E, dtype=torch.bfloat16, gated=True, bias=False, density=density)
