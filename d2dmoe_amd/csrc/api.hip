@@ -185,7 +185,9 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
   if (!aligned16(x) || !aligned16(out) || !aligned16(routing)) return D2DMOE_E_ALIGN;
   hipStream_t s = (hipStream_t)stream;
   if (path == D2DMOE_PATH_AUTO) {
-    if (packed != nullptr && sh.n_tokens <= 16 && mfma_decode_supported(sh)) path = D2DMOE_PATH_MFMA_DECODE;
+    // the small-batch kernels take 16 tokens per pass; gated experts (bound by the weight stream up to a few hundred
+    // tokens) are worth up to three passes
+    if (packed != nullptr && sh.n_tokens <= (sh.gated ? 48 : 16) && mfma_decode_supported(sh)) path = D2DMOE_PATH_MFMA_DECODE;
     else if (packed != nullptr && mfma_dense_supported(sh)) path = D2DMOE_PATH_MFMA_DENSE;
     else if (packed != nullptr && mfma_gemm_supported(sh)) path = D2DMOE_PATH_MFMA_GEMM;
     else path = D2DMOE_PATH_GENERIC;
@@ -219,12 +221,21 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
       return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, nullptr, 0, s);
     }
     case D2DMOE_PATH_MFMA_DECODE: {
-      if (!mfma_decode_supported(sh) || sh.n_tokens > 16) return D2DMOE_E_UNSUPPORTED;
+      if (!mfma_decode_supported(sh) || sh.n_tokens > 48) return D2DMOE_E_UNSUPPORTED;
       if (!packed) return D2DMOE_E_NULL;
       const size_t need = mfma_decode_workspace_bytes(sh);
       if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
-      return (int)launch_mfma_decode(sh, x, routing, (const char*)packed + mfma_decode_section_offset(sh), last_bias, out,
-                                     workspace, s);
+      // passes of 16 tokens, one after the other on the stream, sharing the workspace
+      const size_t es = elem_size(sh.dtype);
+      for (int64_t t0 = 0; t0 < sh.n_tokens; t0 += 16) {
+        d2dmoe_shape part = sh;
+        part.n_tokens = (sh.n_tokens - t0 < 16) ? (sh.n_tokens - t0) : 16;
+        const hipError_t e = launch_mfma_decode(part, (const char*)x + t0 * sh.d_model * es, (const char*)routing + t0 * sh.n_experts * es,
+                                                (const char*)packed + mfma_decode_section_offset(sh), last_bias,
+                                                (char*)out + t0 * sh.d_model * es, workspace, s);
+        if (e != hipSuccess) return (int)e;
+      }
+      return D2DMOE_OK;
     }
     case D2DMOE_PATH_MFMA_GEMM: {
       if (!mfma_gemm_supported(sh)) return D2DMOE_E_UNSUPPORTED;
@@ -287,8 +298,11 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   // A high threshold fraction keeps few experts per token: take the expert-major path (it falls back to the dense
   // sweep on the device if the routing turns out dense after all).
   // (gated experts: from a lower fraction on -- their dense alternative costs ten times the expert-major path at few
-  // experts per token and the device-side switch is cheap next to it)
-  if (path == D2DMOE_PATH_AUTO && sh.n_tokens > 16 && packed != nullptr && thr_scale >= (sh.gated ? 0.5f : 0.75f) && mfma_sparse_supported(sh) &&
+  // experts per token and the device-side switch is cheap next to it;
+  // and with at most 128 tokens whatever the fraction -- the layer is bound by the weight stream there, which the tiled
+  // products pay for with whole 256-token tiles)
+  if (path == D2DMOE_PATH_AUTO && sh.n_tokens > (sh.gated && mfma_decode_supported(sh) ? 48 : 16) && packed != nullptr &&
+      (thr_scale >= (sh.gated ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128)) && mfma_sparse_supported(sh) &&
       (sh.gated ? mfma_gemm_supported(sh) : mfma_dense_supported(sh)))
     path = D2DMOE_PATH_MFMA_SPARSE;
   return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,

@@ -39,6 +39,9 @@ static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) 
   const int E = sh.n_experts;
   W.n_seg = cdiv64(N, SP_SEG);
   W.cap = N * max_mean_k;
+  // Gated experts, few tokens: whatever the routing, an expert's 786 KB of weights are streamed once or twice, so the
+  // path also pays with every expert routed to by every token -- room for at least 128 pairs per expert.
+  if (sh.gated && N > 16 && W.cap < (int64_t)E * SP_GATED_MIN_PAIRS_PER_EXPERT) W.cap = (int64_t)E * SP_GATED_MIN_PAIRS_PER_EXPERT;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += (bytes + 255) / 256 * 256; return o; };
   W.seg_counts = take((size_t)W.n_seg * E * 4);
@@ -793,7 +796,7 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
 #define D2DMOE_PLAN_DISPATCH(V)                                                                                          \
   hipLaunchKernelGGL(plan_scatter_kernel<V>, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_offsets,    \
                      totals, seg_pairs, offsets, tile_off, flag, tok_off, token_idx, pair_dst, N, E, W.n_seg,           \
-                     N * (int64_t)max_mean_k)
+                     (max_mean_k == cap_k) ? W.cap : N * (int64_t)max_mean_k)
   if (vpt <= 1) D2DMOE_PLAN_DISPATCH(1); else if (vpt <= 2) D2DMOE_PLAN_DISPATCH(2); else if (vpt <= 4) D2DMOE_PLAN_DISPATCH(4);
   else if (vpt <= 8) D2DMOE_PLAN_DISPATCH(8); else D2DMOE_PLAN_DISPATCH(16);
 #undef D2DMOE_PLAN_DISPATCH

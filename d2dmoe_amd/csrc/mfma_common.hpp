@@ -23,6 +23,7 @@ constexpr int MD_MAX_CHUNKS = 32;   // chunks per layer the dense sweep stages t
 constexpr int MD_RING = 32;     // weight fragments kept in flight per wave (16 bytes per lane each)
 constexpr int SP_MAX_MEAN_K = 8;    // the expert-major path is provisioned for at most N * 8 routed pairs
 constexpr int SP_MAX_MEAN_K_GATED = 32;   // ... N * 32 for gated experts (up to 16 384 tokens)
+constexpr int SP_GATED_MIN_PAIRS_PER_EXPERT = 128;   // ... and never fewer than E * 128 for gated experts
 
 // Sections of the buffer d2dmoe_pack_weights writes.  A section is present when its kernel covers the shape.
 struct PackedLayout {

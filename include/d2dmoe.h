@@ -73,8 +73,9 @@ enum {
                                  sweep runs.  Ungated experts at D = 768.  Gated experts at D = 2048 with at most 64
                                  neurons: up to 32 experts per token (8 beyond 16 384 tokens), else the tiled products
                                  run.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 (gated: >= 0.5) */
-  D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 MFMA for at most 16 tokens: one workgroup per expert streams that expert's packed
-                                 weights once (gated or ungated experts); AUTO picks it when it applies */
+  D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 MFMA for a handful of tokens: per pass of 16 tokens one workgroup per expert streams
+                                 that expert's packed weights once (gated or ungated experts); at most 48 tokens (three
+                                 passes).  AUTO picks it up to 16 tokens, for gated experts up to 48 */
   D2DMOE_PATH_MFMA_GEMM = 5   /* bf16 or f32 MFMA, D a multiple of 256, gated or ungated experts: two tiled products over all
                                  experts with the routing value as a factor of the hidden activations, which stay in
                                  the workspace between them; AUTO picks it for more than 16 tokens when the dense sweep
