@@ -188,6 +188,8 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
     // the small-batch kernels take 16 tokens per pass; gated experts (bound by the weight stream up to a few hundred
     // tokens) are worth up to three passes
     if (packed != nullptr && sh.n_tokens <= (sh.gated ? 48 : 16) && mfma_decode_supported(sh)) path = D2DMOE_PATH_MFMA_DECODE;
+    else if (packed != nullptr && sh.gated && sh.n_tokens <= 128 && mfma_sparse_supported(sh) && mfma_gemm_supported(sh))
+      path = D2DMOE_PATH_MFMA_SPARSE;   // still bound by the weight stream: expert-major whatever the routing
     else if (packed != nullptr && mfma_dense_supported(sh)) path = D2DMOE_PATH_MFMA_DENSE;
     else if (packed != nullptr && mfma_gemm_supported(sh)) path = D2DMOE_PATH_MFMA_GEMM;
     else path = D2DMOE_PATH_GENERIC;
