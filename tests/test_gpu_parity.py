@@ -531,6 +531,25 @@ def test_gated_layer_takes_the_expert_major_path_for_a_high_threshold():
     assert H.rel_err(out_a.cpu()[rows], want) < H.TOL_BF16
 
 
+@pytest.mark.parametrize('N', [17, 40, 48, 49, 100, 128, 129])
+@pytest.mark.parametrize('tau', [0.1, 0.9])
+def test_gated_layer_between_small_batch_and_tiled_products(N, tau):
+    """Whole gated layer at token counts where AUTO changes hands: small-batch kernels in passes of 16 (up to 48 tokens),
+    expert-major kernels (up to 128 tokens whatever the routing, beyond that for a high threshold fraction), tiled products
+    otherwise.  Outputs against the float64 oracle on the kernel's own routing; the routing against the oracle gate on
+    the kernel's own norms."""
+    D, E, Ed, W = 2048, 32, 64, 256
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=N, dtype=torch.bfloat16, gated=True, bias=False)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, W, 1, 'gelu_tanh', gated=True)
+    packed = _ops().pack_weights(sh, d['w_gate'], None, d['w_down'], d['w_up'], d['router_w1'], d['router_w2'])
+    out, r, norms, counts = _forward(x, p, tau, 'gelu_tanh', path='auto', packed=packed)
+    assert torch.equal(r.cpu(), O.gate_dynk_max(norms.cpu(), tau))
+    assert torch.equal(counts.cpu().long(), r.cpu().float().sum(0).long())
+    want = O.layer_from_routing(x.double(), O.upcast(p), r.cpu().double(), 'gelu_tanh', 'all')
+    assert H.rel_err(out.cpu(), want) < H.TOL_BF16
+
+
 # =================================================================== whole layer ======================
 def _forward(x, p, tau, act='relu', norms_in=None, path='auto', packed=None, residual=False):
     d = H.to_dev(p, DEV)
