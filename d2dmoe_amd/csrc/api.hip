@@ -217,6 +217,8 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
       const int* flag = nullptr;
       hipError_t e = launch_mfma_sparse(sh, x, routing, packed, last_bias, out, workspace, mfma_sparse_capacity_k(sh), &flag, s);
       if (e != hipSuccess) return (int)e;
+      // with every expert routed to by every token the pairs still fit: the fall-back can never be needed
+      if (sh.n_tokens * (int64_t)sh.n_experts <= mfma_sparse_capacity_pairs(sh)) return D2DMOE_OK;
       if (sh.gated)   // gated layers fall back to the tiled products, which work behind the plan in the same workspace
         return (int)launch_mfma_gemm(sh, x, routing, (const char*)packed + mfma_gemm_section_offset(sh), last_bias, out,
                                      (char*)workspace + mfma_sparse_fallback_offset(sh), s, flag);

@@ -64,6 +64,8 @@ static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) 
   return W;
 }
 
+int64_t mfma_sparse_capacity_pairs(const d2dmoe_shape& sh) { return sparse_workspace(sh, mfma_sparse_capacity_k(sh)).cap; }
+
 size_t mfma_sparse_fallback_offset(const d2dmoe_shape& sh) { return sparse_workspace(sh, mfma_sparse_capacity_k(sh)).y; }
 
 size_t mfma_sparse_workspace_bytes(const d2dmoe_shape& sh) {
@@ -548,7 +550,21 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   const int q0 = tok_off[n], q1 = tok_off[n + 1];
   if (singles_done && q1 - q0 == 1) return;   // finished by the experts kernel
-  for (int q = q0; q < q1; ++q) {
+  // rows are added in ascending order; eight of them are requested at a time (a token of a small batch may have a
+  // couple of hundred, and one load per trip would make the sum a chain of memory round trips)
+  int q = q0;
+  for (; q + 8 <= q1; q += 8) {
+    uint4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = *(const uint4*)(y + (int64_t)(q + u) * D + col);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const uint32_t wd[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+    }
+  }
+  for (; q < q1; ++q) {
     const uint4 v = *(const uint4*)(y + (int64_t)q * D + col);
     const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll

@@ -57,6 +57,7 @@ hipError_t launch_sum_partials(const float* partial, const void* last_bias, cons
 bool mfma_sparse_supported(const d2dmoe_shape& sh);
 size_t mfma_sparse_workspace_bytes(const d2dmoe_shape& sh);
 int mfma_sparse_capacity_k(const d2dmoe_shape& sh);   // routed pairs per token the path is provisioned for
+int64_t mfma_sparse_capacity_pairs(const d2dmoe_shape& sh);   // ... and in all, for this number of tokens
 // Offset inside the expert-major workspace at which a gated layer's fall-back (the tiled products) may work: behind the
 // plan, in the region the per-pair rows would have used.
 size_t mfma_sparse_fallback_offset(const d2dmoe_shape& sh);
