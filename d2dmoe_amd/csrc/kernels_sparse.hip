@@ -204,12 +204,18 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restr
                                                            int32_t* __restrict__ flag, int32_t* __restrict__ tok_off,
                                                            int32_t* __restrict__ token_idx, int32_t* __restrict__ pair_dst,
                                                            int64_t N, int E, int64_t n_seg, int64_t cap) {
-  const int lane = threadIdx.x & 63;
-  const int64_t seg = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / 64;
+  // One workgroup per segment; its four waves each scatter a quarter of the segment's tokens (the per-token loop is
+  // the serial part of this kernel), after the same prologue: where a wave's first token starts follows from the bits
+  // of the tokens before it.
+  const int lane = threadIdx.x & 63, wq = threadIdx.x >> 6;
+  const int64_t seg = blockIdx.x;
   if (seg >= n_seg) return;
   const int vpt = (E + 63) / 64;
   const int64_t t0 = seg * SP_SEG;
   const int rows = (int)((N - t0) < SP_SEG ? (N - t0) : SP_SEG);
+  constexpr int RPW = SP_SEG / 4;                 // tokens per wave
+  const int row_lo = wq * RPW;
+  const int row_hi = (row_lo + RPW < rows) ? (row_lo + RPW) : rows;
   // Every load of the prologue is issued before anything is computed from it, none of them under a branch (lane
   // groups past the last expert read clamped addresses and are masked), so the wave pays about one round trip.
   int tot[VPT], segoff[VPT];
@@ -260,7 +266,7 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restr
   }
   const int64_t P = run;
   const bool sparse_ok = P <= cap;
-  if (seg == 0) {
+  if (seg == 0 && wq == 0) {
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       const int e = lane + k * 64;
@@ -278,11 +284,17 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restr
   }
   if (!sparse_ok) return;
   int pos[VPT];            // next expert-major position of expert e
+  const unsigned below = (row_lo == 0) ? 0u : ((1u << row_lo) - 1u);   // the segment's tokens before this wave's
+  int earlier = 0;         // their pairs
 #pragma unroll
-  for (int k = 0; k < VPT; ++k) pos[k] = eoff[k] + segoff[k];
-  int tokbase = before_segs;
+  for (int k = 0; k < VPT; ++k) {
+    const int c = __popc(onbits[k] & below);
+    pos[k] = eoff[k] + segoff[k] + c;
+    earlier += c;
+  }
+  int tokbase = before_segs + wave_sum_i32(earlier);
   const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-  for (int i = 0; i < rows; ++i) {
+  for (int i = row_lo; i < row_hi; ++i) {
     const int64_t tok = t0 + i;
     int before = 0;   // routed experts of this token with a smaller index, over the previous lane groups
 #pragma unroll
@@ -810,7 +822,7 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
 #undef D2DMOE_PLAN_DISPATCH
   launch_perm_scan(seg_counts, seg_offsets, totals, E, W.n_seg, s);
 #define D2DMOE_PLAN_DISPATCH(V)                                                                                          \
-  hipLaunchKernelGGL(plan_scatter_kernel<V>, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_offsets,    \
+  hipLaunchKernelGGL(plan_scatter_kernel<V>, dim3((unsigned)W.n_seg), dim3(256), 0, s, (const bf16_t*)routing, seg_offsets, \
                      totals, seg_pairs, offsets, tile_off, flag, tok_off, token_idx, pair_dst, N, E, W.n_seg,           \
                      (max_mean_k == cap_k) ? W.cap : N * (int64_t)max_mean_k)
   if (vpt <= 1) D2DMOE_PLAN_DISPATCH(1); else if (vpt <= 2) D2DMOE_PLAN_DISPATCH(2); else if (vpt <= 4) D2DMOE_PLAN_DISPATCH(4);
