@@ -203,19 +203,20 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restr
                                                            int32_t* __restrict__ offsets, int32_t* __restrict__ tile_off,
                                                            int32_t* __restrict__ flag, int32_t* __restrict__ tok_off,
                                                            int32_t* __restrict__ token_idx, int32_t* __restrict__ pair_dst,
-                                                           int64_t N, int E, int64_t n_seg, int64_t cap) {
-  // One workgroup per segment; its four waves each scatter a quarter of the segment's tokens (the per-token loop is
-  // the serial part of this kernel), after the same prologue: where a wave's first token starts follows from the bits
-  // of the tokens before it.
+                                                           int64_t N, int E, int64_t n_seg, int64_t cap, int split) {
+  // split == 0: a wave per segment, four segments per workgroup.  split != 0 (few segments): a workgroup per segment,
+  // whose four waves each scatter a quarter of the segment's tokens (the per-token loop is the serial part of this
+  // kernel) after the same prologue: where a wave's first token starts follows from the bits of the tokens before it.
   const int lane = threadIdx.x & 63, wq = threadIdx.x >> 6;
-  const int64_t seg = blockIdx.x;
+  const int64_t seg = split ? (int64_t)blockIdx.x : ((int64_t)blockIdx.x * 4 + wq);
   if (seg >= n_seg) return;
   const int vpt = (E + 63) / 64;
   const int64_t t0 = seg * SP_SEG;
   const int rows = (int)((N - t0) < SP_SEG ? (N - t0) : SP_SEG);
-  constexpr int RPW = SP_SEG / 4;                 // tokens per wave
-  const int row_lo = wq * RPW;
-  const int row_hi = (row_lo + RPW < rows) ? (row_lo + RPW) : rows;
+  constexpr int RPW = SP_SEG / 4;                 // tokens per wave when the segment is split
+  const int row_lo = split ? wq * RPW : 0;
+  const int row_hi = split ? ((row_lo + RPW < rows) ? (row_lo + RPW) : rows) : rows;
+  const bool first_wave = (seg == 0) && (split ? wq == 0 : true);
   // Every load of the prologue is issued before anything is computed from it, none of them under a branch (lane
   // groups past the last expert read clamped addresses and are masked), so the wave pays about one round trip.
   int tot[VPT], segoff[VPT];
@@ -266,7 +267,7 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restr
   }
   const int64_t P = run;
   const bool sparse_ok = P <= cap;
-  if (seg == 0 && wq == 0) {
+  if (first_wave) {
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       const int e = lane + k * 64;
@@ -813,6 +814,10 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   int32_t* pair_dst = (int32_t*)(ws + W.pair_dst);
   bf16_t* y = (bf16_t*)(ws + W.y);
   const unsigned seg_blocks = (unsigned)cdiv64(W.n_seg, 4);
+  // up to 16 384 tokens the scatter gives each segment a workgroup (four waves on its tokens); beyond, the extra
+  // workgroups' repeated prologues cost more than the shorter token loops save (measured: -5 us at 4096 tokens, +3.6 us
+  // at 50 432)
+  const bool split_seg = W.n_seg <= 512;
   const int vpt = (E + 63) / 64;
 #define D2DMOE_PLAN_DISPATCH(V)                                                                                          \
   hipLaunchKernelGGL(plan_count_kernel<V>, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_counts, seg_pairs, N, \
@@ -822,9 +827,10 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
 #undef D2DMOE_PLAN_DISPATCH
   launch_perm_scan(seg_counts, seg_offsets, totals, E, W.n_seg, s);
 #define D2DMOE_PLAN_DISPATCH(V)                                                                                          \
-  hipLaunchKernelGGL(plan_scatter_kernel<V>, dim3((unsigned)W.n_seg), dim3(256), 0, s, (const bf16_t*)routing, seg_offsets, \
+  hipLaunchKernelGGL(plan_scatter_kernel<V>, dim3(split_seg ? (unsigned)W.n_seg : seg_blocks), dim3(256), 0, s,          \
+                     (const bf16_t*)routing, seg_offsets,                                                                \
                      totals, seg_pairs, offsets, tile_off, flag, tok_off, token_idx, pair_dst, N, E, W.n_seg,           \
-                     (max_mean_k == cap_k) ? W.cap : N * (int64_t)max_mean_k)
+                     (max_mean_k == cap_k) ? W.cap : N * (int64_t)max_mean_k, split_seg ? 1 : 0)
   if (vpt <= 1) D2DMOE_PLAN_DISPATCH(1); else if (vpt <= 2) D2DMOE_PLAN_DISPATCH(2); else if (vpt <= 4) D2DMOE_PLAN_DISPATCH(4);
   else if (vpt <= 8) D2DMOE_PLAN_DISPATCH(8); else D2DMOE_PLAN_DISPATCH(16);
 #undef D2DMOE_PLAN_DISPATCH
