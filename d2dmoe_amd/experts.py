@@ -85,7 +85,49 @@ class _PackedCache:
         return cached[1]
 
 
-class HipKernelExperts(ExpertsLayer):
+def _grad_wanted(*tensors) -> bool:
+    """True when autograd is on and one of the tensors asks for a gradient: the HIP kernels have no backward, so such a
+    call has to be refused (the reference's kernel wrappers raise in backward, moe_impls.py:60-64)."""
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+class _HipContainer(ExpertsLayer):
+    """What every experts container of this package shares: the route to the HIP kernels.
+
+    A container names its weights in the kernels' layout through ``hip_operands()`` ->
+    ``(w1 [E,D,Ed], b1 [E,Ed] | None, w2 [E,Ed,D], w_up [E,D,Ed] | None, activation name)``; the derived MFMA-ordered
+    buffer is cached on those tensors and rebuilt when one of them changes."""
+
+    HIP_MODES = ('hip', 'triton', 'triton_atomic')
+
+    def _init_hip(self):
+        self.kernel_path = 'auto'
+        self._packed = _PackedCache()
+
+    def hip_operands(self):
+        raise NotImplementedError
+
+    def packed_weights(self, router_w1=None, router_w2=None, router_activation='relu', router_output_activation='abs'):
+        w1, b1, w2, w_up, act = self.hip_operands()
+        if not w1.is_cuda or w1.dtype not in (torch.bfloat16, torch.float32):
+            return None
+        sh = ops.make_shape(0, w1.size(1), w1.size(0), w1.size(2), router_w1.size(0) if router_w1 is not None else 0,
+                            ops._dtype_code(w1), act, gated=w_up is not None, router_activation=router_activation,
+                            router_output_activation=router_output_activation)
+        return self._packed.get(sh, (w1, b1, w2, w_up, router_w1, router_w2))
+
+    def forward_hip(self, x, routing_tensor, last_bias=None, add_residual=False):
+        if not x.is_cuda:
+            raise D2DMoEError("forward_mode 'hip' needs a ROCm device; use a PyTorch mode on the CPU")
+        w1, b1, w2, w_up, act = self.hip_operands()
+        if _grad_wanted(x, routing_tensor, w1, b1, w2, w_up, last_bias):
+            # inference-only, like the reference's kernel wrappers (moe_impls.py:60-64)
+            raise NotImplementedError("the HIP experts path has no backward; wrap the call in torch.no_grad()")
+        return ops.experts(x.contiguous(), routing_tensor.contiguous(), w1, b1, w2, w_up, last_bias, act, add_residual,
+                           self.kernel_path, self.packed_weights())
+
+
+class HipKernelExperts(_HipContainer):
     """Two-layer experts with the first-layer bias only, run by the gfx950 HIP kernels.
 
     Drop-in for the reference's CustomKernelExperts (moe_layers.py:136-264): same constructor, same parameters
@@ -96,8 +138,6 @@ class HipKernelExperts(ExpertsLayer):
       'hip'     the HIP kernels; 'triton' and 'triton_atomic' are accepted as aliases so reference scripts that
                 select the Triton kernels get this path
     """
-
-    HIP_MODES = ('hip', 'triton', 'triton_atomic')
 
     def __init__(self, dim, num_experts, depth=2, expert_dim=None, bias=True, activation=nn.GELU,
                  intermediate_gating=False):
@@ -117,10 +157,9 @@ class HipKernelExperts(ExpertsLayer):
         self.w2 = init_(nn.Parameter(torch.empty(num_experts, self.expert_dim, dim)))
         self.act = activation()
         self._forward_mode = 'masked'
-        self.kernel_path = 'auto'
+        self._init_hip()
         self.intermediate_activation_extraction_stub = _IntermediateStub()
         self.output_activation_extraction_stub = _OutputStub()
-        self._packed = _PackedCache()
         self._norms_packed = None   # (key, buffer) of the derived buffer output_norms() uses
 
     @property
@@ -132,14 +171,16 @@ class HipKernelExperts(ExpertsLayer):
         self._forward_mode = value
 
     # -- derived buffers --------------------------------------------------------------------
-    def packed_weights(self, router_w1=None, router_w2=None, router_activation='relu', router_output_activation='abs'):
-        if not self.w1.is_cuda or self.w1.dtype not in (torch.bfloat16, torch.float32):
-            return None
-        sh = ops.make_shape(0, self.hidden_dim, self.num_experts, self.expert_dim,
-                            router_w1.size(0) if router_w1 is not None else 0, ops._dtype_code(self.w1),
-                            self.activation_str, router_activation=router_activation,
-                            router_output_activation=router_output_activation)
-        return self._packed.get(sh, (self.w1, self.b1, self.w2, None, router_w1, router_w2))
+    def hip_operands(self):
+        return self.w1, self.b1, self.w2, None, self.activation_str
+
+    def load_operands(self, w1, b1, w2, w_up=None):
+        assert w_up is None
+        with torch.no_grad():
+            self.w1.copy_(w1)
+            self.w2.copy_(w2)
+            if b1 is not None:
+                self.b1.copy_(b1)
 
     def output_norms(self, x):
         """L2 norm of every expert's output for every token, [E,N]: the router-training targets the reference reads off
@@ -185,15 +226,6 @@ class HipKernelExperts(ExpertsLayer):
             out[mask] += self.act(x[mask] @ self.w1[e] + self.b1[e]) @ self.w2[e]
         return out
 
-    def forward_hip(self, x, routing_tensor, last_bias=None, add_residual=False):
-        if not x.is_cuda:
-            raise D2DMoEError("forward_mode 'hip' needs a ROCm device; use 'naive' or 'masked' on CPU")
-        if torch.is_grad_enabled() and (x.requires_grad or self.w1.requires_grad):
-            # inference-only, like the reference's kernel wrappers (moe_impls.py:60-64)
-            raise NotImplementedError("the HIP experts path has no backward; wrap the call in torch.no_grad()")
-        return ops.experts(x.contiguous(), routing_tensor.contiguous(), self.w1, self.b1, self.w2, None, last_bias,
-                           self.activation_str, add_residual, self.kernel_path, self.packed_weights())
-
     # the reference exposes these two as static methods of the container (moe_layers.py:213-224, 241-249)
     @staticmethod
     def extract_indices(routing_tensor):
@@ -229,7 +261,7 @@ class _ExecuteAllLayer(nn.Module):
         return self.act(x)
 
 
-class HipExecuteAllExperts(ExpertsLayer):
+class HipExecuteAllExperts(_HipContainer):
     """Depth-2 experts, optionally with LLaMA/Gemma-style intermediate gating, parameters named as the reference's
     ExecuteAllExperts (moe_layers.py:50-101): ``layers.0.w`` first/gate projection, ``layers.1.w`` down projection,
     ``layers.2.w`` up projection (gated only).  ``forward_mode`` 'masked' is the reference's dense einsum; 'hip'
@@ -257,11 +289,30 @@ class HipExecuteAllExperts(ExpertsLayer):
             self.layers.append(_ExecuteAllLayer(dim, self.expert_dim, num_experts, first_bias, activation))
             self.layers.append(_ExecuteAllLayer(self.expert_dim, dim, num_experts, last_bias, nn.Identity))
         self.forward_mode = 'masked'
-        self.kernel_path = 'auto'
+        self._init_hip()
+
+    def hip_operands(self):
+        if self.layers[1].bias or (self.intermediate_gating and self.layers[0].bias):
+            raise NotImplementedError('the HIP path covers first-layer bias (ungated) or no bias (gated)')
+        b1 = self.layers[0].b.squeeze(1) if self.layers[0].bias else None   # a view: shares storage and version counter
+        w_up = self.layers[2].w if self.intermediate_gating else None
+        return self.layers[0].w, b1, self.layers[1].w, w_up, activation_name(self.layers[0].act)
+
+    def load_operands(self, w1, b1, w2, w_up=None):
+        """Fills the parameters from kernel-layout tensors (what the reference's param_clustering_split writes entry by
+        entry, moefication.py:253-271)."""
+        assert (w_up is not None) == self.intermediate_gating
+        with torch.no_grad():
+            self.layers[0].w.copy_(w1)
+            self.layers[1].w.copy_(w2)
+            if b1 is not None:
+                self.layers[0].b.copy_(b1.unsqueeze(1))
+            if w_up is not None:
+                self.layers[2].w.copy_(w_up)
 
     def forward(self, x, routing_tensor):
         assert x.dim() == 2, f'{x.size()=}'
-        if self.forward_mode == 'hip':
+        if self.forward_mode in self.HIP_MODES:
             return self.forward_hip(x, routing_tensor)
         x = x.unsqueeze(0)
         if self.intermediate_gating:
@@ -271,16 +322,178 @@ class HipExecuteAllExperts(ExpertsLayer):
                 x = layer(x)
         return torch.einsum('end,ne->nd', x, routing_tensor)
 
-    def forward_hip(self, x, routing_tensor, last_bias=None, add_residual=False):
-        if not x.is_cuda:
-            raise D2DMoEError("forward_mode 'hip' needs a ROCm device")
-        if self.layers[1].bias or (self.intermediate_gating and self.layers[0].bias):
-            raise NotImplementedError('the HIP path covers first-layer bias (ungated) or no bias (gated)')
-        b1 = self.layers[0].b.squeeze(1).contiguous() if self.layers[0].bias else None
-        w_up = self.layers[2].w if self.intermediate_gating else None
-        act = activation_name(self.layers[0].act)
-        return ops.experts(x.contiguous(), routing_tensor.contiguous(), self.layers[0].w, b1, self.layers[1].w, w_up,
-                           last_bias, act, add_residual, self.kernel_path, None)
+
+class _GLUExpert(nn.Module):
+    """One gated expert as a module (reference: moe_layers.py:104-113; same submodule names)."""
+
+    def __init__(self, d_model, d_intermediate, activation, bias, last_bias):
+        super().__init__()
+        self.gate = nn.Linear(d_model, d_intermediate, bias=bias)
+        self.up_scale = nn.Linear(d_model, d_intermediate, bias=bias)
+        self.activation = activation()
+        self.down_scale = nn.Linear(d_intermediate, d_model, bias=last_bias)
+
+    def forward(self, x):
+        return self.down_scale(self.activation(self.gate(x)) * self.up_scale(x))
+
+
+def _loop_over_experts(x, routing_tensor, num_experts, expert_fn):
+    """The reference's per-expert loop of its module containers (moe_layers.py:311-326, 385-399): every expert runs on the
+    rows routed to it and its output is scaled by the routing value.  (The reference first asserts that x holds no NaN,
+    which costs a host synchronisation per call; that check is left out.)"""
+    outputs = torch.zeros_like(x)
+    for i in range(num_experts):
+        col = routing_tensor[:, i]
+        mask = col != 0.0
+        outputs[mask] += expert_fn(x[mask], i) * col[mask].unsqueeze(1)
+    return outputs
+
+
+class _StackedOperands:
+    """Kernel-layout copies ([E,D,Ed] / [E,Ed] / [E,Ed,D]) of weights a container keeps per expert, rebuilt when one of the
+    source parameters changes (storage pointer or in-place version counter)."""
+
+    def __init__(self):
+        self.key = None
+        self.value = None
+
+    def get(self, sources, build):
+        key = tuple((t.data_ptr(), t._version, t.dtype, t.device) for t in sources)
+        if key != self.key:
+            with torch.no_grad():
+                self.value = build()
+            self.key = key
+        return self.value
+
+
+class HipModuleBatchedExperts(_HipContainer):
+    """Experts kept as one small module each, with the reference's ModuleBatchedExperts names (moe_layers.py:267-326):
+    ``e.<i>.0`` / ``e.<i>.2`` Linear layers (``e.<i>.gate`` / ``up_scale`` / ``down_scale`` for gated experts), so its
+    state_dicts load unchanged.  ``forward_mode`` 'naive' (the default) is the reference's per-expert loop; 'hip' runs the
+    HIP kernels on stacked copies of the weights (inference only)."""
+
+    def __init__(self, dim, num_experts, depth=2, expert_dim=None, bias=True, activation=nn.GELU,
+                 intermediate_gating=False):
+        super().__init__()
+        assert depth == 2, 'only two-layer experts'
+        self.num_experts = num_experts
+        self.depth = depth
+        self.expert_dim = dim * 2 if expert_dim is None else expert_dim
+        self.bias_mode = bias
+        self.intermediate_gating = intermediate_gating
+        first_bias = True if bias == 'without_last' else bias
+        last_bias = False if bias == 'without_last' else bias
+        self.e = nn.ModuleList()
+        for _ in range(num_experts):
+            if intermediate_gating:
+                self.e.append(_GLUExpert(dim, self.expert_dim, activation, bool(bias), bool(last_bias)))
+            else:
+                self.e.append(nn.Sequential(nn.Linear(dim, self.expert_dim, bias=first_bias), activation(),
+                                            nn.Linear(self.expert_dim, dim, bias=last_bias)))
+        self.forward_mode = 'naive'
+        self._init_hip()
+        self._stacked = _StackedOperands()
+
+    def hip_operands(self):
+        if self.intermediate_gating:
+            first = [m.gate for m in self.e]
+            up = [m.up_scale for m in self.e]
+            last = [m.down_scale for m in self.e]
+            act = activation_name(self.e[0].activation)
+            if first[0].bias is not None:
+                raise NotImplementedError('the HIP path covers gated experts without biases')
+        else:
+            first = [m[0] for m in self.e]
+            up = None
+            last = [m[2] for m in self.e]
+            act = activation_name(self.e[0][1])
+        if last[0].bias is not None:
+            raise NotImplementedError('the HIP path has no per-expert output bias')
+        sources = [l.weight for l in first] + [l.weight for l in last]
+        sources += [l.bias for l in first if l.bias is not None] + ([l.weight for l in up] if up else [])
+
+        def build():
+            w1 = torch.stack([l.weight.t() for l in first]).contiguous()
+            b1 = torch.stack([l.bias for l in first]).contiguous() if first[0].bias is not None else None
+            w2 = torch.stack([l.weight.t() for l in last]).contiguous()
+            w_up = torch.stack([l.weight.t() for l in up]).contiguous() if up else None
+            return w1, b1, w2, w_up
+
+        return (*self._stacked.get(sources, build), act)
+
+    def load_operands(self, w1, b1, w2, w_up=None):
+        assert (w_up is not None) == self.intermediate_gating
+        with torch.no_grad():
+            for i, m in enumerate(self.e):
+                first, last = (m.gate, m.down_scale) if self.intermediate_gating else (m[0], m[2])
+                first.weight.copy_(w1[i].t())
+                last.weight.copy_(w2[i].t())
+                if b1 is not None:
+                    first.bias.copy_(b1[i])
+                if w_up is not None:
+                    m.up_scale.weight.copy_(w_up[i].t())
+
+    def forward(self, x, routing_tensor):
+        assert x.dim() == 2, f'{x.size()=}'
+        if self.forward_mode in self.HIP_MODES:
+            return self.forward_hip(x, routing_tensor)
+        return _loop_over_experts(x, routing_tensor, self.num_experts, lambda rows, i: self.e[i](rows))
+
+
+class HipBatchedExperts(_HipContainer):
+    """Experts kept as stacked tensors in parameter lists, with the reference's BatchedExperts names
+    (moe_layers.py:329-399): ``weights.0 [E,D,Ed]``, ``weights.1 [E,Ed,D]``, ``biases.<i> [E,1,*]``.  As there, the list
+    of biases under bias='without_last' also holds an (unused) entry for the last layer.  ``forward_mode`` 'naive' (the
+    default) is the reference's per-expert loop; 'hip' runs the HIP kernels (inference only)."""
+
+    def __init__(self, dim, num_experts, depth=2, expert_dim=None, bias=True, activation=nn.GELU,
+                 intermediate_gating=False):
+        super().__init__()
+        assert depth == 2, 'only two-layer experts'
+        if intermediate_gating:
+            raise NotImplementedError()
+        self.num_experts = num_experts
+        self.depth = depth
+        self.expert_dim = dim * 2 if expert_dim is None else expert_dim
+        self.bias_mode = bias
+        has_bias = True if bias == 'without_last' else bias
+        self.weights = nn.ParameterList([init_(nn.Parameter(torch.empty(num_experts, dim, self.expert_dim))),
+                                         init_(nn.Parameter(torch.empty(num_experts, self.expert_dim, dim)))])
+        if has_bias:
+            self.biases = nn.ParameterList([nn.Parameter(torch.zeros(num_experts, 1, self.expert_dim)),
+                                            nn.Parameter(torch.zeros(num_experts, 1, dim))])
+        self.act = activation()
+        self.forward_mode = 'naive'
+        self._init_hip()
+
+    def expert_forward(self, x, expert_index):
+        if self.bias_mode is True:
+            x = self.act(x @ self.weights[0][expert_index] + self.biases[0][expert_index])
+            return x @ self.weights[1][expert_index] + self.biases[1][expert_index]
+        if self.bias_mode == 'without_last':
+            x = self.act(x @ self.weights[0][expert_index] + self.biases[0][expert_index])
+            return x @ self.weights[1][expert_index]
+        return self.act(x @ self.weights[0][expert_index]) @ self.weights[1][expert_index]
+
+    def hip_operands(self):
+        if self.bias_mode is True:
+            raise NotImplementedError('the HIP path has no per-expert output bias')
+        b1 = self.biases[0].squeeze(1) if self.bias_mode == 'without_last' else None
+        return self.weights[0], b1, self.weights[1], None, activation_name(self.act)
+
+    def load_operands(self, w1, b1, w2, w_up=None):
+        assert w_up is None
+        with torch.no_grad():
+            self.weights[0].copy_(w1)
+            self.weights[1].copy_(w2)
+            if b1 is not None:
+                self.biases[0].copy_(b1.unsqueeze(1))
+
+    def forward(self, x, routing_tensor):
+        assert x.dim() == 2, f'{x.size()=}'
+        if self.forward_mode in self.HIP_MODES:
+            return self.forward_hip(x, routing_tensor)
+        return _loop_over_experts(x, routing_tensor, self.num_experts, self.expert_forward)
 
 
 MOE_IMPL_MAP = {
@@ -288,4 +501,6 @@ MOE_IMPL_MAP = {
     'custom_kernel': HipKernelExperts,     # the reference's name for its Triton-backed container
     'hip_execute_all': HipExecuteAllExperts,
     'execute_all': HipExecuteAllExperts,   # the reference's dense container (the one its Gemma runs use)
+    'module': HipModuleBatchedExperts,     # one module per expert (the reference's default experts_class)
+    'batched': HipBatchedExperts,          # stacked tensors in parameter lists
 }

@@ -180,19 +180,28 @@ def moe_gpt_main_forward(self, x: torch.Tensor, return_gating_data: bool = False
 
 
 # ------------------------------------------------------------------------------------------- model surgery
+def is_gated_ffn(ffn: nn.Module) -> bool:
+    """A LLaMA/Gemma-style gated FFN: Linear submodules gate_proj, up_proj, down_proj and an activation act_fn (the
+    layout of transformers' GemmaMLP, which the reference converts with intermediate gating, moefication.py:115-129)."""
+    return all(isinstance(getattr(ffn, n, None), nn.Linear) for n in ('gate_proj', 'up_proj', 'down_proj')) and \
+        isinstance(getattr(ffn, 'act_fn', None), nn.Module)
+
+
 def ffn_parts(ffn: nn.Module):
     """(first Linear, activation module, second Linear, dropout probability) of a dense FFN block: this file's `MLP`
-    (c_fc, act, c_proj, dropout) or an index-addressed Linear/act/Dropout/Linear/Dropout sequence (torchvision's
-    MLPBlock, `vit.MLPBlock`)."""
+    (c_fc, act, c_proj, dropout), an index-addressed Linear/act/Dropout/Linear/Dropout sequence (torchvision's
+    MLPBlock, `vit.MLPBlock`), or a gated FFN, whose first Linear is the gate projection (`ffn.up_proj` is its third)."""
     if isinstance(ffn, MLP):
         return ffn.c_fc, ffn.act, ffn.c_proj, ffn.dropout.p
     if isinstance(ffn, nn.Sequential) and len(ffn) == 5 and isinstance(ffn[0], nn.Linear) and isinstance(ffn[3], nn.Linear):
         return ffn[0], ffn[1], ffn[3], ffn[4].p if isinstance(ffn[4], nn.Dropout) else 0.0
+    if is_gated_ffn(ffn):
+        return ffn.gate_proj, ffn.act_fn, ffn.down_proj, 0.0
     raise ValueError(f'Unsupported ffn type: {type(ffn)}')
 
 
 def ffn_filter_condition(_model: nn.Module, m: nn.Module) -> bool:
-    if isinstance(m, MLP):
+    if isinstance(m, MLP) or is_gated_ffn(m):
         return True
     return isinstance(m, nn.Sequential) and len(m) == 5 and isinstance(m[0], nn.Linear) and isinstance(m[3], nn.Linear)
 
@@ -233,10 +242,13 @@ def replace_layer_with_moe(model: nn.Module, name: str, num_experts=None, expert
     else:
         assert d_ff % expert_size == 0, 'd_ff has to be divisible by the expert size'
         num_experts = d_ff // expert_size
-    moe_layer = MoeficationMoE(name, hidden_dim, num_experts, w1.bias is not None, expert_size, type(act), experts_class)
+    gated = is_gated_ffn(original)
+    moe_layer = MoeficationMoE(name, hidden_dim, num_experts, w1.bias is not None, expert_size, type(act), experts_class,
+                               add_intermediate_gating=gated)
     moe_layer = moe_layer.to(device=w1.weight.device, dtype=w1.weight.dtype)
     set_module_by_name(model, name, moe_layer)
-    set_module_by_name(model, f'{name}.dropout', nn.Dropout(dropout_p))
+    if not gated:
+        set_module_by_name(model, f'{name}.dropout', nn.Dropout(dropout_p))
 
 
 def replace_with_moes(original_model: nn.Module, num_experts: int = None, expert_size: int = None,
@@ -262,11 +274,16 @@ def replace_with_moes(original_model: nn.Module, num_experts: int = None, expert
 
 
 def param_split(ffn: nn.Module, moe_layer: MoeficationMoE, labels: Optional[Sequence[int]] = None):
-    """Moves the dense FFN's neurons into the experts: neuron n goes to expert labels[n], in order of appearance."""
+    """Moves the dense FFN's neurons into the experts: neuron n goes to expert labels[n], in order of appearance (what the
+    reference's param_clustering_split does with its clustering labels, moefication.py:205-285).  Works for every
+    experts container of this package; for a gated FFN the gate projection is the first layer and the up projection is
+    split alongside it."""
     ex = moe_layer.experts
     E, Ed = moe_layer.num_experts, moe_layer.expert_dim
     fc1, _, fc2, _ = ffn_parts(ffn)
+    up = ffn.up_proj if is_gated_ffn(ffn) else None
     d_ff = fc1.out_features
+    D = fc1.in_features
     if labels is None:
         labels = torch.arange(d_ff) // Ed
     labels = torch.as_tensor(labels, dtype=torch.long)
@@ -276,13 +293,22 @@ def param_split(ffn: nn.Module, moe_layer: MoeficationMoE, labels: Optional[Sequ
     order = torch.argsort(labels, stable=True)          # neurons grouped by expert, original order kept
     slot = torch.empty_like(order)
     slot[order] = torch.arange(d_ff) % Ed
+    ref = next(ex.parameters())
     with torch.no_grad():
-        w_fc = fc1.weight.detach()                      # [d_ff, D]
-        w_proj = fc2.weight.detach()                    # [D, d_ff]
-        ex.w1[labels, :, slot] = w_fc.to(ex.w1.dtype).to(ex.w1.device)
-        ex.w2[labels, slot, :] = w_proj.t().to(ex.w2.dtype).to(ex.w2.device)
+        w1 = torch.empty(E, D, Ed, dtype=ref.dtype)
+        w2 = torch.empty(E, Ed, D, dtype=ref.dtype)
+        w1[labels, :, slot] = fc1.weight.detach().cpu().to(ref.dtype)               # fc1.weight [d_ff, D]
+        w2[labels, slot, :] = fc2.weight.detach().cpu().t().to(ref.dtype)           # fc2.weight [D, d_ff]
+        b1 = w_up = None
         if moe_layer.bias:
-            ex.b1[labels, slot] = fc1.bias.detach().to(ex.b1.dtype).to(ex.b1.device)
+            b1 = torch.empty(E, Ed, dtype=ref.dtype)
+            b1[labels, slot] = fc1.bias.detach().cpu().to(ref.dtype)
+        if up is not None:
+            w_up = torch.empty(E, D, Ed, dtype=ref.dtype)
+            w_up[labels, :, slot] = up.weight.detach().cpu().to(ref.dtype)
+        dev = ref.device
+        ex.load_operands(w1.to(dev), None if b1 is None else b1.to(dev), w2.to(dev), None if w_up is None else w_up.to(dev))
+        if moe_layer.bias:
             moe_layer.last_bias.copy_(fc2.bias.detach().view(1, -1))
 
 

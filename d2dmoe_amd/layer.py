@@ -18,7 +18,7 @@ import torch
 from torch import nn
 
 from . import ops
-from .experts import MOE_IMPL_MAP, HipExecuteAllExperts, HipKernelExperts, activation_name
+from .experts import MOE_IMPL_MAP, _HipContainer, _grad_wanted
 from .hip_abi import ACT
 
 
@@ -39,6 +39,20 @@ ACTIVATION_NAME_MAP = {
     'abs': _Abs,
     'identity': nn.Identity,
 }
+
+
+class _CallCache:
+    """Holder of a layer's prepared library call.  It is derived state: copies and pickles of the layer start empty."""
+    __slots__ = ('entry',)
+
+    def __init__(self):
+        self.entry = None
+
+    def __deepcopy__(self, memo):
+        return _CallCache()
+
+    def __reduce__(self):
+        return (_CallCache, ())
 
 
 class MoELayer(nn.Module):
@@ -125,6 +139,7 @@ class MoeficationMoE(MoELayer):
         # batch, eval.py:176-177): with collect_counts set, the fused HIP call also returns the per-expert number of
         # routed tokens from its own device-side counters; it stays on the device, nothing synchronises.
         self.collect_counts = False
+        self._prepared = _CallCache()   # (key, ops.PreparedForward) of the fused call
         self.last_expert_counts: Optional[torch.Tensor] = None
 
     # ------------------------------------------------------------------------------ gating
@@ -158,14 +173,21 @@ class MoeficationMoE(MoELayer):
 
     # ------------------------------------------------------------------------------ forward
     def _fused_ok(self, x) -> bool:
+        """True when the whole layer can run as one d2dmoe_forward call.  Raises, as the experts containers do, when that
+        call would be taken under autograd with a tensor that asks for a gradient: the kernels have no backward
+        (the reference's wrappers raise there too, moe_impls.py:60-64), and an output silently cut off from the graph
+        would leave the parameters without gradients."""
         if self.forward_mode != 'dynk_max' or not x.is_cuda or x.dtype not in (torch.float32, torch.bfloat16):
             return False
-        if torch.is_grad_enabled() and x.requires_grad:
+        ex = self.experts
+        if not isinstance(ex, _HipContainer) or ex.forward_mode not in ex.HIP_MODES:
             return False
-        if not isinstance(self.experts, HipKernelExperts) or self.experts.forward_mode not in HipKernelExperts.HIP_MODES:
+        if self.router is None or not (self.router.test_override_outputs_p is not None or self.router.hip_compatible()):
             return False
-        return self.router is not None and (self.router.test_override_outputs_p is not None
-                                            or self.router.hip_compatible())
+        if torch.is_grad_enabled() and _grad_wanted(x, *self.parameters()):
+            raise NotImplementedError("the HIP layer path has no backward; wrap the call in torch.no_grad(), or switch the "
+                                      "experts to a PyTorch forward_mode for training")
+        return True
 
     def _router_operands(self):
         """(router_w1, router_w2, hidden activation, output activation) as the fused HIP call takes them; the weights are
@@ -183,25 +205,39 @@ class MoeficationMoE(MoELayer):
         """The derived, MFMA-ordered weight buffer the fused forward of this layer uses (built on first use, rebuilt when
         a parameter changes); None where no MFMA kernel applies.  Calling it ahead of time moves the packing out of the
         first forward."""
-        if not isinstance(self.experts, HipKernelExperts) or self.router is None or not self.router.hip_compatible():
+        if not isinstance(self.experts, _HipContainer) or self.router is None or not self.router.hip_compatible():
             return None
         return self.experts.packed_weights(*self._router_operands())
+
+    def _prepared_forward(self, x):
+        """The layer's ops.PreparedForward, rebuilt when a parameter was replaced or updated in place, the dtype or device
+        changed, or a setting it bakes in did (residual, bias, router override)."""
+        ex = self.experts
+        rw1, rw2, ract, roact = self._router_operands()
+        w1, b1, w2, w_up, act = ex.hip_operands()
+        last_bias = self.last_bias if self.bias else None
+        sources = (rw1, rw2, w1, b1, w2, w_up, last_bias)
+        key = tuple((t.data_ptr(), t._version) if t is not None else None for t in sources) + \
+            (x.dtype, x.device, act, ract, roact, self.add_residual_connection)
+        cached = self._prepared.entry
+        if cached is None or cached[0] != key:
+            prepared = ops.PreparedForward(self.hidden_dim, x.dtype, rw1, rw2, w1, b1, w2, w_up,
+                                           last_bias.view(-1) if last_bias is not None else None, act,
+                                           self.add_residual_connection, ex.packed_weights(rw1, rw2, ract, roact), ract, roact)
+            cached = self._prepared.entry = (key, prepared)
+        return cached[1]
 
     def forward(self, x):
         orig_size = x.size()
         if self._fused_ok(x):
-            ex = self.experts
-            x2 = x.reshape(-1, x.size(-1)).contiguous()
+            x2 = x.reshape(-1, orig_size[-1]).contiguous()
             router = self.router
-            last_bias = self.last_bias.view(-1) if self.bias else None
             norms_in = None
             if router.test_override_outputs_p is not None:
                 norms_in = router(x).reshape(-1, self.num_experts).contiguous()
-            rw1, rw2, ract, roact = self._router_operands()
-            out, routing, _, counts = ops.forward(
-                x2, rw1, rw2, float(1.0 - self.tau), ex.w1, ex.b1, ex.w2, None, last_bias, ex.activation_str,
-                self.add_residual_connection, norms_in=norms_in, want_counts=self.collect_counts, path=ex.kernel_path,
-                packed=ex.packed_weights(rw1, rw2, ract, roact), router_activation=ract, router_output_activation=roact)
+            out, routing, _, counts = self._prepared_forward(x)(x2, float(1.0 - self.tau), norms_in,
+                                                                want_counts=self.collect_counts,
+                                                                path=self.experts.kernel_path)
             routing_tensor = routing.view(*orig_size[:-1], self.num_experts)
             self.last_expert_counts = counts
             return out.view(orig_size), {self.name: (routing_tensor,)}

@@ -23,6 +23,27 @@ def _dtype_code(t: torch.Tensor) -> int:
         raise abi.D2DMoEError(f'unsupported dtype {t.dtype}: the HIP path handles float32 and bfloat16') from None
 
 
+def _require_same_dtype(what: str, ref: torch.Tensor, **tensors: Optional[torch.Tensor]) -> None:
+    """The kernels read every operand with the element type of `ref` (d2dmoe_shape.dtype): an operand of another dtype
+    would be reinterpreted byte by byte, so it is refused here, before any pointer reaches the library."""
+    for name, t in tensors.items():
+        if t is not None and t.dtype != ref.dtype:
+            raise abi.D2DMoEError(f'{what}: {name} is {t.dtype} but the activations are {ref.dtype}; the HIP path needs one '
+                                  'element type for activations, routing and weights')
+
+
+def _check_packed(lib, shape: 'abi.Shape', packed: Optional[torch.Tensor]) -> None:
+    """A packed buffer carries no header: its size is the one thing that can be checked, and a buffer packed for another
+    shape, dtype or without the router section has another size."""
+    if packed is None:
+        return
+    need = lib.d2dmoe_packed_bytes(ctypes.byref(shape))
+    have = packed.numel() * packed.element_size()
+    if need == 0 or have < need:
+        raise abi.D2DMoEError(f'packed buffer holds {have} bytes but this shape/dtype needs {need}: it was packed for other '
+                              'weights (pack again with the shape of this call)')
+
+
 def _require_gpu(*tensors: Optional[torch.Tensor]) -> torch.device:
     dev = None
     for t in tensors:
@@ -47,9 +68,9 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
-def _workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+def _workspace(dev: torch.device, nbytes: int, stream: Optional[int] = None) -> torch.Tensor:
     """Per-(device, stream) scratch buffer, grown on demand and reused between calls on that stream."""
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _stream())
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _stream() if stream is None else stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
@@ -70,6 +91,7 @@ def make_shape(n_tokens: int, d_model: int, n_experts: int, expert_dim: int, rou
 def router(x: torch.Tensor, router_w1: torch.Tensor, router_w2: torch.Tensor, activation: str = 'relu',
            output_activation: str = 'abs') -> torch.Tensor:
     """norms [N,E] = out_act(act(x W1^T) W2^T) through d2dmoe_router."""
+    _require_same_dtype('router', x, router_w1=router_w1, router_w2=router_w2)
     dev = _require_gpu(x, router_w1, router_w2)
     lib = abi.load()
     n, d = x.shape
@@ -103,6 +125,7 @@ def router_select(x: torch.Tensor, router_w1: torch.Tensor, router_w2: torch.Ten
                   output_activation: str = 'abs'):
     """Router MLP + dynamic-k selection through d2dmoe_router_select (one fused MFMA kernel when `packed` carries a
     router section for this shape).  Returns (routing [N,E], norms or None, counts or None)."""
+    _require_same_dtype('router_select', x, router_w1=router_w1, router_w2=router_w2)
     dev = _require_gpu(x, router_w1, router_w2, packed)
     lib = abi.load()
     n, d = x.shape
@@ -149,6 +172,9 @@ def packed_bytes(shape: abi.Shape) -> int:
 
 def pack_weights(shape: abi.Shape, w1, b1, w2, w_up=None, router_w1=None, router_w2=None) -> Optional[torch.Tensor]:
     """Derived MFMA-fragment-ordered weight buffer, or None when the shape has no MFMA kernel."""
+    _require_same_dtype('pack_weights', w1, b1=b1, w2=w2, w_up=w_up, router_w1=router_w1, router_w2=router_w2)
+    if _dtype_code(w1) != shape.dtype:
+        raise abi.D2DMoEError(f'pack_weights: the weights are {w1.dtype} but the shape names dtype code {shape.dtype}')
     dev = _require_gpu(w1, b1, w2, w_up, router_w1, router_w2)
     lib = abi.load()
     nbytes = lib.d2dmoe_packed_bytes(ctypes.byref(shape))
@@ -163,6 +189,7 @@ def pack_weights(shape: abi.Shape, w1, b1, w2, w_up=None, router_w1=None, router
 def pack_norms(shape: abi.Shape, w1, b1, w2) -> Optional[torch.Tensor]:
     """Derived buffer of d2dmoe_expert_output_norms (first-layer fragments, bias, per-expert Gram matrices), or None
     when the kernel does not cover the shape."""
+    _require_same_dtype('pack_norms', w1, b1=b1, w2=w2)
     dev = _require_gpu(w1, b1, w2)
     lib = abi.load()
     nbytes = lib.d2dmoe_norms_packed_bytes(ctypes.byref(shape))
@@ -177,6 +204,7 @@ def pack_norms(shape: abi.Shape, w1, b1, w2) -> Optional[torch.Tensor]:
 def expert_output_norms(x: torch.Tensor, w1: torch.Tensor, b1: Optional[torch.Tensor], w2: torch.Tensor,
                         activation: str = 'relu', packed: Optional[torch.Tensor] = None) -> torch.Tensor:
     """norms [E,N] = | act(x w1[e] + b1[e]) w2[e] |_2 through d2dmoe_expert_output_norms (bf16, D = 768, Ed <= 32)."""
+    _require_same_dtype('expert_output_norms', x, w1=w1, b1=b1, w2=w2)
     dev = _require_gpu(x, w1, b1, w2, packed)
     lib = abi.load()
     n, d = x.shape
@@ -196,12 +224,14 @@ def experts(x: torch.Tensor, routing: torch.Tensor, w1: torch.Tensor, b1: Option
             w_up: Optional[torch.Tensor] = None, last_bias: Optional[torch.Tensor] = None, activation: str = 'relu',
             add_residual: bool = False, path: str = 'auto', packed: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out [N,D] = sum_e routing[n,e] * expert_e(x[n]) (+ last_bias) (+ x) through d2dmoe_experts."""
+    _require_same_dtype('experts', x, routing=routing, w1=w1, b1=b1, w2=w2, w_up=w_up, last_bias=last_bias)
     dev = _require_gpu(x, routing, w1, b1, w2, w_up, last_bias, packed)
     lib = abi.load()
     n, d = x.shape
     e, _, ed = w1.shape
-    assert routing.shape == (n, e) and w2.shape == (e, ed, d) and routing.dtype == x.dtype
+    assert routing.shape == (n, e) and w2.shape == (e, ed, d)
     sh = make_shape(n, d, e, ed, 0, _dtype_code(x), activation, gated=w_up is not None, add_residual=add_residual)
+    _check_packed(lib, sh, packed)
     out = torch.empty_like(x)
     need = max(lib.d2dmoe_workspace_bytes(ctypes.byref(sh)), 16)
     ws = _workspace(dev, need)
@@ -211,28 +241,102 @@ def experts(x: torch.Tensor, routing: torch.Tensor, w1: torch.Tensor, b1: Option
     return out
 
 
+class PreparedForward:
+    """d2dmoe_forward for one layer with everything that does not change from call to call resolved once: operand checks
+    (device, contiguity, one element type, packed-buffer size), the weights' device pointers, the d2dmoe_shape and
+    workspace size per token count.  A call then allocates the outputs, looks the stream and workspace up and makes the one
+    library call.  The object keeps references to the tensors it was built from; build a new one when a weight tensor is
+    replaced (in-place updates keep the pointers valid, but a packed buffer has to be rebuilt from them first)."""
+
+    def __init__(self, d_model: int, dtype: torch.dtype, router_w1, router_w2, w1, b1, w2, w_up=None, last_bias=None,
+                 activation: str = 'relu', add_residual: bool = False, packed=None, router_activation: str = 'relu',
+                 router_output_activation: str = 'abs'):
+        self.tensors = (router_w1, router_w2, w1, b1, w2, w_up, last_bias, packed)
+        for name, t in zip(('router_w1', 'router_w2', 'w1', 'b1', 'w2', 'w_up', 'last_bias'), self.tensors):
+            if t is not None and t.dtype != dtype:
+                raise abi.D2DMoEError(f'forward: {name} is {t.dtype} but the activations are {dtype}; the HIP path needs '
+                                      'one element type for activations, routing and weights')
+        self.dtype = dtype
+        self.code = _DTYPES.get(dtype)
+        if self.code is None:
+            raise abi.D2DMoEError(f'unsupported dtype {dtype}: the HIP path handles float32 and bfloat16')
+        self.dev = _require_gpu(*self.tensors)
+        self.lib = abi.load()
+        self.d = d_model
+        self.e, _, self.ed = w1.shape
+        assert w1.size(1) == d_model and w2.shape == (self.e, self.ed, d_model)
+        self.w = router_w1.size(0) if router_w1 is not None else 0
+        self.kw = dict(activation=activation, gated=w_up is not None, add_residual=add_residual,
+                       router_activation=router_activation, router_output_activation=router_output_activation)
+        self.ptrs = tuple(_ptr(t) for t in self.tensors)
+        self.shapes = {}
+        # the router section is the last one of a packed buffer: a buffer packed without it serves calls that bring their
+        # own predicted norms (norms_in), and only those
+        _check_packed(self.lib, make_shape(0, self.d, self.e, self.ed, 0, self.code, **self.kw), packed)
+        self.router_packed_ok = True
+        if packed is not None and self.w > 0:
+            need = self.lib.d2dmoe_packed_bytes(self.shape_for(0)[1])
+            self.router_packed_ok = packed.numel() * packed.element_size() >= need
+
+    def shape_for(self, n: int):
+        got = self.shapes.get(n)
+        if got is None:
+            sh = make_shape(n, self.d, self.e, self.ed, self.w, self.code, **self.kw)
+            got = (sh, ctypes.byref(sh), max(self.lib.d2dmoe_workspace_bytes(ctypes.byref(sh)), 256))
+            if len(self.shapes) > 64:
+                self.shapes.clear()
+            self.shapes[n] = got
+        return got
+
+    def __call__(self, x: torch.Tensor, thr_scale: float, norms_in=None, want_norms=False, want_counts=False,
+                 path: str = 'auto', static_workspace: bool = False, out=None, routing=None, norms=None, counts=None):
+        if x.dtype != self.dtype or (norms_in is not None and norms_in.dtype != self.dtype):
+            raise abi.D2DMoEError(f'forward: the activations are {x.dtype} but the layer was prepared for {self.dtype}')
+        if _require_gpu(x, norms_in, out, routing, norms, counts) != self.dev:
+            raise abi.D2DMoEError('all tensors must live on the same device')
+        if norms_in is None and not self.router_packed_ok:
+            raise abi.D2DMoEError('packed buffer has no router section for this layer, but the call runs the router: it was '
+                                  'packed for other weights (pack again with the router weights)')
+        n, d = x.shape
+        assert d == self.d
+        e = self.e
+        _, shref, need = self.shape_for(n)
+        dev = self.dev
+        out = torch.empty_like(x) if out is None else out
+        routing = torch.empty(n, e, dtype=x.dtype, device=dev) if routing is None else routing
+        assert out.shape == x.shape and out.dtype == x.dtype and routing.shape == (n, e) and routing.dtype == x.dtype
+        if norms is None and want_norms and norms_in is None:
+            norms = torch.empty(n, e, dtype=x.dtype, device=dev)
+        if counts is None and want_counts:
+            counts = torch.empty(e, dtype=torch.int32, device=dev)
+        rw1, rw2, w1, b1, w2, w_up, lb, pk = self.ptrs
+        stream = _stream()
+        if static_workspace:
+            abi.check(self.lib.d2dmoe_forward_static(shref, x.data_ptr(), rw1, rw2, ctypes.c_float(thr_scale), w1, b1, w2,
+                                                     w_up, lb, pk, _ptr(norms_in), _ptr(norms), routing.data_ptr(),
+                                                     _ptr(counts), out.data_ptr(), abi.PATH[path], stream),
+                      'd2dmoe_forward_static')
+        else:
+            ws = _workspace(dev, need, stream)
+            abi.check(self.lib.d2dmoe_forward(shref, x.data_ptr(), rw1, rw2, ctypes.c_float(thr_scale), w1, b1, w2, w_up, lb,
+                                              pk, _ptr(norms_in), _ptr(norms), routing.data_ptr(), _ptr(counts),
+                                              out.data_ptr(), abi.PATH[path], ws.data_ptr(), ws.numel(), stream),
+                      'd2dmoe_forward')
+        return out, routing, (norms_in if norms_in is not None else norms), counts
+
+
 def forward(x: torch.Tensor, router_w1: Optional[torch.Tensor], router_w2: Optional[torch.Tensor], thr_scale: float,
             w1: torch.Tensor, b1: Optional[torch.Tensor], w2: torch.Tensor, w_up: Optional[torch.Tensor] = None,
             last_bias: Optional[torch.Tensor] = None, activation: str = 'relu', add_residual: bool = False,
             norms_in: Optional[torch.Tensor] = None, want_norms: bool = False, want_counts: bool = False,
             path: str = 'auto', packed: Optional[torch.Tensor] = None, router_activation: str = 'relu',
-            router_output_activation: str = 'abs'):
-    """Whole layer through d2dmoe_forward.  x [N,D] -> (out [N,D], routing [N,E], norms or None, counts or None)."""
-    dev = _require_gpu(x, router_w1, router_w2, w1, b1, w2, w_up, last_bias, norms_in, packed)
-    lib = abi.load()
-    n, d = x.shape
-    e, _, ed = w1.shape
-    w = router_w1.size(0) if router_w1 is not None else 0
-    sh = make_shape(n, d, e, ed, w, _dtype_code(x), activation, gated=w_up is not None, add_residual=add_residual,
-                    router_activation=router_activation, router_output_activation=router_output_activation)
-    out = torch.empty_like(x)
-    routing = torch.empty(n, e, dtype=x.dtype, device=dev)
-    norms = torch.empty(n, e, dtype=x.dtype, device=dev) if (want_norms and norms_in is None) else None
-    counts = torch.empty(e, dtype=torch.int32, device=dev) if want_counts else None
-    need = max(lib.d2dmoe_workspace_bytes(ctypes.byref(sh)), 256)
-    ws = _workspace(dev, need)
-    abi.check(lib.d2dmoe_forward(ctypes.byref(sh), _ptr(x), _ptr(router_w1), _ptr(router_w2), ctypes.c_float(thr_scale),
-                                 _ptr(w1), _ptr(b1), _ptr(w2), _ptr(w_up), _ptr(last_bias), _ptr(packed),
-                                 _ptr(norms_in), _ptr(norms), _ptr(routing), _ptr(counts), _ptr(out), abi.PATH[path],
-                                 _ptr(ws), ws.numel(), _stream()), 'd2dmoe_forward')
-    return out, routing, (norms_in if norms_in is not None else norms), counts
+            router_output_activation: str = 'abs', static_workspace: bool = False, out: Optional[torch.Tensor] = None,
+            routing: Optional[torch.Tensor] = None, norms: Optional[torch.Tensor] = None,
+            counts: Optional[torch.Tensor] = None):
+    """Whole layer through d2dmoe_forward.  x [N,D] -> (out [N,D], routing [N,E], norms or None, counts or None).
+
+    static_workspace=True goes through d2dmoe_forward_static instead: the workspace is the array inside the library, and
+    when the caller also hands over `out` / `routing` (/ `norms` / `counts`) nothing at all is allocated by the call."""
+    prepared = PreparedForward(x.size(1), x.dtype, router_w1, router_w2, w1, b1, w2, w_up, last_bias, activation,
+                               add_residual, packed, router_activation, router_output_activation)
+    return prepared(x, thr_scale, norms_in, want_norms, want_counts, path, static_workspace, out, routing, norms, counts)

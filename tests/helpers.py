@@ -15,6 +15,14 @@ TOL_F32 = 1e-5
 TOL_BF16 = 2e-2
 
 
+class GELUTanh(torch.nn.GELU):
+    """An activation class of its own for the tanh form of GELU, as transformers has for Gemma (the layer and the surgery
+    rebuild an activation from its type alone, moefication.py:116)."""
+
+    def __init__(self):
+        super().__init__(approximate='tanh')
+
+
 def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
     got = got.detach().double().cpu()
     want = want.detach().double().cpu()

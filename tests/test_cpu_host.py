@@ -438,3 +438,116 @@ def test_bench_refuses_more_than_one_gpu():
     res = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--gpus', '2'], capture_output=True, text=True, timeout=120)
     assert res.returncode != 0
     assert 'single-GPU' in (res.stderr + res.stdout)
+
+
+# ------------------------------------------------------------------ every experts container of the registry ----
+def test_registry_holds_the_reference_keys():
+    from d2dmoe_amd import MOE_IMPL_MAP
+    assert {'execute_all', 'module', 'batched', 'custom_kernel'} <= set(MOE_IMPL_MAP)   # moe_layers.py:402-407
+
+
+def _container_params(ex):
+    """(w1, b1, w2, w_up) in the kernels' layout, read through the container's own accessor."""
+    w1, b1, w2, w_up, _ = ex.hip_operands()
+    return {'w1': w1.detach(), 'b1': None if b1 is None else b1.detach(), 'w2': w2.detach(),
+            'w_up': None if w_up is None else w_up.detach()}
+
+
+@pytest.mark.parametrize('experts_class,gated', [('custom_kernel', False), ('execute_all', False), ('execute_all', True),
+                                                 ('module', False), ('module', True), ('batched', False)])
+def test_container_pytorch_modes_match_oracle(experts_class, gated):
+    from d2dmoe_amd import MoeficationMoE
+    torch.manual_seed(3)
+    bias = not gated
+    moe = MoeficationMoE('m', 48, 5, bias, 12, nn.GELU, experts_class=experts_class, add_intermediate_gating=gated).eval()
+    ex = moe.experts
+    if bias and experts_class == 'batched':
+        with torch.no_grad():
+            ex.biases[0].uniform_(-0.2, 0.2)     # the reference initialises them to zero; make them count
+    x = torch.randn(11, 48)
+    routing = (torch.rand(11, 5) < 0.5).float() * torch.rand(11, 5)      # weighted routing, some zeros
+    p = _container_params(ex)
+    if gated:
+        want = O.experts_gated_forward_all(x.double(), routing.double(), p['w1'].double(), p['w_up'].double(),
+                                           p['w2'].double(), 'gelu')
+    else:
+        want = O.experts_forward_all(x.double(), routing.double(), p['w1'].double(), p['b1'].double(), p['w2'].double(),
+                                     'gelu')
+    with torch.no_grad():
+        got = ex(x, routing)
+    assert H.rel_err(got, want) < 1e-5
+    # state_dict names follow the reference's containers
+    keys = set(ex.state_dict())
+    if experts_class == 'module':
+        assert ('e.0.gate.weight' in keys and 'e.4.down_scale.weight' in keys) if gated else \
+            ({'e.0.0.weight', 'e.0.0.bias', 'e.4.2.weight'} <= keys and 'e.0.2.bias' not in keys)
+    if experts_class == 'batched':
+        assert keys == {'weights.0', 'weights.1', 'biases.0', 'biases.1'}
+    if experts_class == 'execute_all':
+        assert 'layers.0.w' in keys and ('layers.2.w' in keys) == gated
+
+
+class _GatedMLP(nn.Module):
+    """The submodule layout of transformers' GemmaMLP."""
+
+    def __init__(self, d, dff):
+        super().__init__()
+        self.gate_proj = nn.Linear(d, dff, bias=False)
+        self.up_proj = nn.Linear(d, dff, bias=False)
+        self.down_proj = nn.Linear(dff, d, bias=False)
+        self.act_fn = H.GELUTanh()
+
+    def forward(self, x):
+        return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+
+
+@pytest.mark.parametrize('experts_class,gated', [('custom_kernel', False), ('execute_all', False), ('execute_all', True),
+                                                 ('module', False), ('module', True), ('batched', False)])
+def test_param_split_fills_every_container(experts_class, gated):
+    """With every expert running, the converted layer reproduces the dense FFN, for contiguous and shuffled labels."""
+    from d2dmoe_amd import MoeficationMoE, gpt2
+    torch.manual_seed(4)
+    D, dff, E = 32, 48, 6
+    if gated:
+        ffn = _GatedMLP(D, dff).eval()
+    else:
+        ffn = nn.Sequential(nn.Linear(D, dff), nn.GELU(), nn.Dropout(0.0), nn.Linear(dff, D), nn.Dropout(0.0)).eval()
+    assert gpt2.ffn_filter_condition(None, ffn)
+    x = torch.randn(3, 4, D)
+    with torch.no_grad():
+        want = ffn(x)
+    for labels in (None, torch.randperm(dff) % E):
+        holder = nn.ModuleDict({'ffn': ffn})
+        holder = __import__('copy').deepcopy(holder)
+        gpt2.replace_layer_with_moe(holder, 'ffn', num_experts=E, experts_class=experts_class)
+        moe = holder['ffn']
+        assert isinstance(moe, MoeficationMoE) and moe.forward_mode == 'all'
+        gpt2.param_split(ffn, moe, labels)
+        with torch.no_grad():
+            got, gating = moe(x)
+        assert torch.allclose(got, want, rtol=1e-4, atol=1e-5), (experts_class, gated)
+        assert gating['ffn'][0].shape == (3, 4, E)
+
+
+def test_operand_dtype_mismatch_is_refused_before_any_device_call():
+    from d2dmoe_amd import D2DMoEError, ops
+    x = torch.randn(4, 64).bfloat16()
+    routing = torch.ones(4, 4).bfloat16()
+    w1, b1, w2 = torch.randn(4, 64, 32), torch.randn(4, 32), torch.randn(4, 32, 64)    # float32 weights
+    with pytest.raises(D2DMoEError, match='w1 is torch.float32'):
+        ops.experts(x, routing, w1, b1, w2)
+    with pytest.raises(D2DMoEError, match='routing is torch.float32'):
+        ops.experts(x, routing.float(), w1.bfloat16(), b1.bfloat16(), w2.bfloat16())
+    with pytest.raises(D2DMoEError, match='router_w1'):
+        ops.forward(x, torch.randn(128, 64), torch.randn(4, 128).bfloat16(), 0.1, w1.bfloat16(), b1.bfloat16(), w2.bfloat16())
+
+
+def test_grad_predicate_of_the_hip_paths():
+    from d2dmoe_amd.experts import _grad_wanted
+    w = nn.Parameter(torch.zeros(2))
+    x = torch.zeros(2)
+    assert _grad_wanted(x, w) and not _grad_wanted(x, None)
+    with torch.no_grad():
+        assert not _grad_wanted(x, w)
+    w.requires_grad_(False)
+    assert not _grad_wanted(x, w)
