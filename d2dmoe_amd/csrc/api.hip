@@ -2,12 +2,44 @@
 // Nothing here allocates, synchronises or reads device memory on the host.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "common.hpp"
 #include "launch.hpp"
 
 using namespace d2dmoe;
 
+// Workspace of d2dmoe_forward_static: one array per GPU, part of the loaded code object, held until the process ends.
+// Host code never uses this name as an address -- it is a host-side stand-in; the device address is looked up once per
+// device with hipGetSymbolAddress and kept in static_scratch_ptr[].
+static __device__ __align__(256) unsigned char scratch[D2DMOE_STATIC_WORKSPACE_BYTES];
+
+// Keeps the array in the device code object whatever the optimiser thinks of a variable no other kernel names.
+__global__ void static_scratch_anchor_kernel(int v) { scratch[0] = (unsigned char)v; }
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+void* static_scratch_ptr[kMaxDevices] = {};
+std::mutex static_scratch_mutex;
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return D2DMOE_E_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(static_scratch_mutex);
+  if (static_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr || (((uintptr_t)p) & 255u)) return D2DMOE_E_WORKSPACE;
+    static_scratch_ptr[dev] = p;
+  }
+  *out = static_scratch_ptr[dev];
+  return D2DMOE_OK;
+}
 
 inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 inline size_t elem_size(int dtype) { return dtype == D2DMOE_F32 ? 4 : 2; }
@@ -68,6 +100,7 @@ const char* d2dmoe_status_string(int status) {
     case D2DMOE_E_WORKSPACE: return "workspace missing, misaligned or too small";
     case D2DMOE_E_UNSUPPORTED: return "no kernel for this request in this build";
     case D2DMOE_E_ALIGN: return "tensor pointer not aligned to 16 bytes";
+    case D2DMOE_E_STATIC_LIMIT: return "shape needs more workspace than the static array of d2dmoe_forward_static holds";
     default: break;
   }
   if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -311,6 +344,22 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
     path = D2DMOE_PATH_MFMA_SPARSE;
   return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,
                         plan.total - plan.perm_off, stream);
+}
+
+int d2dmoe_forward_static(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
+                          float thr_scale, const void* w1, const void* b1, const void* w2, const void* w_up,
+                          const void* last_bias, const void* packed, const void* norms_in, void* norms_out, void* routing,
+                          int32_t* counts, void* out, int32_t path, void* stream) {
+  int st = check_shape(shape);
+  if (st != D2DMOE_OK) return st;
+  if (plan_workspace(*shape).total > (size_t)D2DMOE_STATIC_WORKSPACE_BYTES) return D2DMOE_E_STATIC_LIMIT;
+  void* ws = nullptr;
+  st = static_scratch(&ws);
+  if (st != D2DMOE_OK) return st;
+  // Every kernel behind d2dmoe_forward initialises what it reads of its workspace (counters, flags, partial sums) on the
+  // stream before use, so the contents the previous call left in the array are never seen.
+  return d2dmoe_forward(shape, x, router_w1, router_w2, thr_scale, w1, b1, w2, w_up, last_bias, packed, norms_in, norms_out,
+                        routing, counts, out, path, ws, (size_t)D2DMOE_STATIC_WORKSPACE_BYTES, stream);
 }
 
 size_t d2dmoe_norms_packed_bytes(const d2dmoe_shape* shape) {

@@ -15,6 +15,8 @@ LIB_PATH = os.environ.get('D2DMOE_LIB') or os.path.join(os.path.dirname(os.path.
 
 # enums of include/d2dmoe.h
 F32, BF16 = 0, 1
+E_STATIC_LIMIT = -8
+STATIC_WORKSPACE_BYTES = 256 << 20
 ACT = {'relu': 0, 'gelu': 1, 'tanh': 2, 'leaky_relu': 3, 'gelu_tanh': 4, 'silu': 5, 'identity': 6, 'abs': 7}
 PATH = {'auto': 0, 'generic': 1, 'mfma_dense': 2, 'mfma_sparse': 3, 'mfma_decode': 4, 'mfma_gemm': 5}
 
@@ -23,7 +25,7 @@ EXPORTS = (
     'd2dmoe_version', 'd2dmoe_status_string', 'd2dmoe_workspace_bytes', 'd2dmoe_router', 'd2dmoe_select',
     'd2dmoe_router_select',
     'd2dmoe_build_permutation', 'd2dmoe_experts', 'd2dmoe_packed_bytes', 'd2dmoe_pack_weights', 'd2dmoe_forward',
-    'd2dmoe_norms_packed_bytes', 'd2dmoe_pack_norms', 'd2dmoe_expert_output_norms',
+    'd2dmoe_norms_packed_bytes', 'd2dmoe_pack_norms', 'd2dmoe_expert_output_norms', 'd2dmoe_forward_static',
 )
 
 
@@ -76,6 +78,8 @@ def load() -> ctypes.CDLL:
     lib.d2dmoe_pack_weights.argtypes = [SH, P, P, P, P, P, P, P, SZ, P]
     lib.d2dmoe_forward.restype = ctypes.c_int
     lib.d2dmoe_forward.argtypes = [SH, P, P, P, c_float, P, P, P, P, P, P, P, P, P, P, P, I32, P, SZ, P]
+    lib.d2dmoe_forward_static.restype = ctypes.c_int
+    lib.d2dmoe_forward_static.argtypes = [SH, P, P, P, c_float, P, P, P, P, P, P, P, P, P, P, P, I32, P]
     lib.d2dmoe_norms_packed_bytes.restype = SZ
     lib.d2dmoe_norms_packed_bytes.argtypes = [SH]
     lib.d2dmoe_pack_norms.restype = ctypes.c_int

@@ -45,7 +45,8 @@ enum {
   D2DMOE_E_ACTIVATION = -4,  /* unknown activation */
   D2DMOE_E_WORKSPACE = -5,   /* workspace missing, misaligned or smaller than d2dmoe_workspace_bytes() */
   D2DMOE_E_UNSUPPORTED = -6, /* valid request that this build has no kernel for */
-  D2DMOE_E_ALIGN = -7        /* a tensor pointer is not aligned to 16 bytes */
+  D2DMOE_E_ALIGN = -7,       /* a tensor pointer is not aligned to 16 bytes */
+  D2DMOE_E_STATIC_LIMIT = -8 /* d2dmoe_forward_static: the shape needs more than D2DMOE_STATIC_WORKSPACE_BYTES of workspace */
 };
 
 /* element types */
@@ -202,6 +203,26 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x,
                    const void* packed, const void* norms_in,
                    void* norms_out, void* routing, int32_t* counts, void* out, int32_t path,
                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* d2dmoe_forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the same layer, the same kernels and bit-identical results, with the workspace taken
+ * from an array that is part of the library's device code instead of a caller-owned buffer.  No counterpart in the
+ * reference.  The entry point calls no hipMalloc / hipFree and no allocating library routine; the caller still passes
+ * every input and output.
+ *   - Limit: shapes whose d2dmoe_workspace_bytes() exceeds D2DMOE_STATIC_WORKSPACE_BYTES (256 MiB) are rejected with
+ *     D2DMOE_E_STATIC_LIMIT before anything is launched (the ViT-B / GPT-2 layer fits up to 20 808 tokens, the
+ *     Gemma-shape layer up to 2 027).  Each GPU the library runs on holds one such array until the process ends.
+ *   - Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race.  The
+ *     array keeps the previous call's contents; the kernels initialise what they read of it on the stream, as they do
+ *     with a caller-owned workspace.
+ *   - The first call on each device looks the array's device address up (hipGetSymbolAddress); make that call outside
+ *     stream capture. */
+#define D2DMOE_STATIC_WORKSPACE_BYTES (256u << 20)
+int d2dmoe_forward_static(const d2dmoe_shape* shape, const void* x,
+                          const void* router_w1, const void* router_w2, float thr_scale,
+                          const void* w1, const void* b1, const void* w2, const void* w_up, const void* last_bias,
+                          const void* packed, const void* norms_in,
+                          void* norms_out, void* routing, int32_t* counts, void* out, int32_t path, void* stream);
 
 /* L2 norm of every expert's output for every token, norms[e,n] = | act(x[n,:] . w1[e] + b1[e]) . w2[e] |_2 (bf16 [E,N]):
  * the regression targets of router training.  Replaces running the layer in 'masked' mode with a forward hook on
