@@ -79,6 +79,8 @@ ForwardWorkspace plan_workspace(const d2dmoe_shape& sh) {
   if (dsplit > scratch) scratch = dsplit;
   const size_t gemm = (sh.n_tokens > 16) ? mfma_gemm_workspace_bytes(sh) : 0;   // H fragments + partial sums of the gated path
   if (gemm > scratch) scratch = gemm;
+  const size_t mid = (sh.n_tokens > 16) ? mfma_mid_workspace_bytes(sh) : 0;     // plan + hidden rows of the compacted path
+  if (mid > scratch) scratch = mid;
   w.perm_off = off;   off += align_up(scratch);
   w.total = off;
   return w;
@@ -255,6 +257,19 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
       if (sh.gated)   // gated layers fall back to the tiled products, which work behind the plan in the same workspace
         return (int)launch_mfma_gemm(sh, x, routing, (const char*)packed + mfma_gemm_section_offset(sh), last_bias, out,
                                      (char*)workspace + mfma_sparse_fallback_offset(sh), s, flag);
+      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, nullptr, 0, s);
+    }
+    case D2DMOE_PATH_MFMA_MID: {
+      // compacted two-kernel path when the routed pairs fit the provisioned capacity, else the dense sweep: decided on
+      // the device
+      if (!mfma_mid_supported(sh) || !mfma_dense_supported(sh)) return D2DMOE_E_UNSUPPORTED;
+      if (!packed) return D2DMOE_E_NULL;
+      const size_t need = mfma_mid_workspace_bytes(sh);
+      if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
+      const int* flag = nullptr;
+      hipError_t e = launch_mfma_mid(sh, x, routing, packed, last_bias, out, workspace, &flag, s);
+      if (e != hipSuccess) return (int)e;
+      if (sh.n_tokens * (int64_t)sh.n_experts <= mfma_mid_capacity_pairs(sh)) return D2DMOE_OK;   // always fits
       return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, nullptr, 0, s);
     }
     case D2DMOE_PATH_MFMA_DECODE: {

@@ -79,6 +79,10 @@ PackedLayout packed_layout(const d2dmoe_shape& sh) {
   L.dc_off = off;   if (L.has_decode) off += mfma_decode_packed_bytes(sh);
   L.has_gemm = mfma_gemm_supported(sh);
   L.gm_off = off;   if (L.has_gemm) off += mfma_gemm_packed_bytes(sh);
+  L.has_mid = mfma_mid_supported(sh);     // experts padded to 32 neurons, both layers
+  const size_t mid_bytes = (size_t)sh.n_experts * MID_HROW * sh.d_model * 2;
+  L.m1_off = off;   if (L.has_mid) off += mid_bytes;
+  L.m2_off = off;   if (L.has_mid) off += mid_bytes;
   // the router section comes last, so the expert sections sit at the same offsets whether or not the shape handed
   // to a later call names the router
   L.has_router = mfma_router_supported(sh);
@@ -197,6 +201,10 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
   }
   if (L.has_gemm) {
     hipError_t e = launch_gemm_pack(sh, w1, b1, w2, w_up, base + L.gm_off, s);
+    if (e != hipSuccess) return e;
+  }
+  if (L.has_mid) {
+    hipError_t e = launch_mid_pack(sh, L, w1, w2, packed, s);
     if (e != hipSuccess) return e;
   }
   if (!L.has_dense) return hipGetLastError();

@@ -67,6 +67,14 @@ size_t mfma_sparse_fallback_offset(const d2dmoe_shape& sh);
 hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                               const void* last_bias, void* out, void* workspace, int max_mean_k, const int** flag_out,
                               hipStream_t s);
+// ---- compacted two-kernel bf16 MFMA path for middling routing density (kernels_mid.hip) ----
+bool mfma_mid_supported(const d2dmoe_shape& sh);
+size_t mfma_mid_workspace_bytes(const d2dmoe_shape& sh);
+int64_t mfma_mid_capacity_pairs(const d2dmoe_shape& sh);
+// Plans on the device and runs the two kernels when the routed pairs fit the capacity; otherwise *flag stays 0 and the
+// caller's dense sweep (skip_flag = the returned pointer) does the work.
+hipError_t launch_mfma_mid(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
+                           const void* last_bias, void* out, void* workspace, const int** flag_out, hipStream_t s);
 // ---- small-batch (<= 16 tokens) bf16 MFMA path (kernels_decode.hip) ----
 bool mfma_decode_supported(const d2dmoe_shape& sh);
 size_t mfma_decode_workspace_bytes(const d2dmoe_shape& sh);

@@ -24,6 +24,9 @@ constexpr int MD_RING = 32;     // weight fragments kept in flight per wave (16 
 constexpr int SP_MAX_MEAN_K = 8;    // the expert-major path is provisioned for at most N * 8 routed pairs
 constexpr int SP_MAX_MEAN_K_GATED = 32;   // ... N * 32 for gated experts (up to 16 384 tokens)
 constexpr int SP_GATED_MIN_PAIRS_PER_EXPERT = 128;   // ... and never fewer than E * 128 for gated experts
+constexpr int SP_SEG = 32;          // tokens per plan segment (one wave): the tile of the fused router kernel
+constexpr int MID_MAX_MEAN_K = 48;  // the compacted two-kernel path is provisioned for at most N * 48 routed pairs
+constexpr int MID_HROW = 32;        // hidden values kept per routed pair (experts of at most 32 neurons), bf16
 
 // Sections of the buffer d2dmoe_pack_weights writes.  A section is present when its kernel covers the shape.
 struct PackedLayout {
@@ -38,8 +41,9 @@ struct PackedLayout {
   size_t su_off;                         // expert-major, gated experts: fragments of the up projection
   size_t dc_off;                         // small-batch (decode) section
   size_t gm_off;                         // large-batch gated section (tiled products)
+  size_t m1_off, m2_off;                 // compacted two-kernel path: W1 and W2^T fragments of the 16x16x32 MFMA
   size_t total;
-  bool has_dense, has_router, has_sparse, has_decode, has_gemm;
+  bool has_dense, has_router, has_sparse, has_decode, has_gemm, has_mid;
 };
 PackedLayout packed_layout(const d2dmoe_shape& sh);
 int device_cu_count();
@@ -48,6 +52,13 @@ hipError_t launch_decode_pack(const d2dmoe_shape& sh, const void* w1, const void
                               void* packed_section, hipStream_t s);
 hipError_t launch_sparse_pack(const d2dmoe_shape& sh, const PackedLayout& L, const void* w1, const void* b1, const void* w2,
                               const void* w_up, void* packed, hipStream_t s);
+
+// Per-segment routed-token counts and their per-expert prefix over segments (plan passes 1 and 2 of the expert-major
+// paths): seg_counts[seg][e], seg_pairs[seg], then seg_offsets[seg][e] and totals[e].
+void launch_plan_count_scan(const void* routing, int64_t N, int E, int32_t* seg_counts, int32_t* seg_pairs,
+                            int32_t* seg_offsets, int32_t* totals, hipStream_t s);
+hipError_t launch_mid_pack(const d2dmoe_shape& sh, const PackedLayout& L, const void* w1, const void* w2, void* packed,
+                           hipStream_t s);
 
 // two float32 -> packed bf16 pair, round-to-nearest-even (one v_cvt_pk_bf16_f32 on gfx950)
 __device__ inline uint32_t pack2_bf16(float lo, float hi) {

@@ -18,7 +18,8 @@ F32, BF16 = 0, 1
 E_STATIC_LIMIT = -8
 STATIC_WORKSPACE_BYTES = 256 << 20
 ACT = {'relu': 0, 'gelu': 1, 'tanh': 2, 'leaky_relu': 3, 'gelu_tanh': 4, 'silu': 5, 'identity': 6, 'abs': 7}
-PATH = {'auto': 0, 'generic': 1, 'mfma_dense': 2, 'mfma_sparse': 3, 'mfma_decode': 4, 'mfma_gemm': 5}
+PATH = {'auto': 0, 'generic': 1, 'mfma_dense': 2, 'mfma_sparse': 3, 'mfma_decode': 4, 'mfma_gemm': 5,
+        'mfma_mid': 6}
 
 # every extern "C" symbol the header declares
 EXPORTS = (
