@@ -47,14 +47,24 @@ WORKLOADS = {
     # the CPU baseline's own case (8 x 197 tokens, float32) on the GPU: float32 storage and float32 matrix arithmetic
     'vit_b_1576_f32': (8, 197, 768, 128, 24, 128, 'relu'),
 }
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (profiles/), scaled by
-# the factors a plain copy kernel of known size gives for the same counters (2.0 and 1.0); None = not measured
-MEASURED_TRAFFIC = {
-    'vit_b_50k': 468.0e6,     # experts_mfma_dense_kernel
-    'gemma_16': 207.1e6,      # decode_hidden_kernel + decode_out_kernel
-    'gemma_1': 163.7e6,
-    'gemma_4096': 2169.8e6,   # up product + down product + finish
-}
+TRAFFIC_TABLE = os.path.join(ROOT, 'profiles', 'traffic_per_launch.md')
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch of the workload's dominant kernel(s), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: read from
+    the table committed under profiles/ (one row per workload: bytes, the summary it comes from, the commit it was taken
+    at).  Returns (bytes or None, source or None); nothing is assumed when the table or the row is missing."""
+    try:
+        with open(TRAFFIC_TABLE) as f:
+            for row in f:
+                cells = [c.strip().strip('`') for c in row.strip().strip('|').split('|')]
+                if len(cells) >= 5 and cells[0] == workload:
+                    return float(cells[2]) * 1e6, {'file': 'profiles/' + cells[3], 'kernels': cells[1], 'commit': cells[4]}
+    except (OSError, ValueError):
+        pass
+    return None, None
+
+
 # Gemma-2B-shape gated layer: (tokens, D, E, Ed, W, activation)
 GATED_WORKLOADS = {
     'gemma_1': (1, 2048, 256, 64, 256, 'gelu_tanh'),
@@ -203,9 +213,14 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, pa
 
 
 def run_gated(args, ops, dev):
+    print(json.dumps(gated_record(args, ops, dev, args.workload)))
+
+
+def gated_record(args, ops, dev, workload):
     """Gemma-shape gated layer: whole-layer time and the HBM rate over the bytes that have to move (router weights,
     the weights of every expert some token routes to, token input/output)."""
-    N, D, E, Ed, W, act = GATED_WORKLOADS[args.workload]
+    N, D, E, Ed, W, act = GATED_WORKLOADS[workload]
+    traffic, traffic_src = measured_traffic(workload)
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(0)
 
@@ -232,11 +247,11 @@ def run_gated(args, ops, dev):
     s = x.element_size()
     algo_bytes = (W * D + E * W) * s + union * 3 * D * Ed * s + 2 * N * D * s + N * E * s
     line = {
-        'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
+        'metric': f'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, Gemma-2B-shape gated layer tau={args.tau}',
         'value': N / ms_layer * 1e3, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': ms_layer, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16',
         'data': 'synthetic',
-        'config': {'workload': f'{args.workload}: {N} tokens, D={D}, {E} gated experts x {Ed}, {act}, router {D}->{W}->{E}, '
+        'config': {'workload': f'{workload}: {N} tokens, D={D}, {E} gated experts x {Ed}, {act}, router {D}->{W}->{E}, '
                                f'module tau={args.tau}, whole layer', 'experts_routed_to': union,
                    'mean_active_experts': pairs / N, 'mfma_kernels': packed is not None},
         'active_tflops': pairs * 6.0 * D * Ed / ms_layer / 1e9, 'hbm_gbps': algo_bytes / ms_layer / 1e6,
@@ -244,7 +259,7 @@ def run_gated(args, ops, dev):
                      'achieved': (union * 3 * D * Ed * s + 2 * N * D * s) / ms_experts / 1e6,
                      'peak': PEAK_HBM_GBPS, 'unit': 'GB/s',
                      'frac': (union * 3 * D * Ed * s + 2 * N * D * s) / ms_experts / 1e6 / PEAK_HBM_GBPS,
-                     'traffic': MEASURED_TRAFFIC.get(args.workload),
+                     'traffic': traffic, 'traffic_source': traffic_src,
                      'kernel_ms': ms_experts, 'algorithmic_bytes_layer': algo_bytes,
                      'layer_frac': algo_bytes / ms_layer / 1e6 / PEAK_HBM_GBPS},
     }
@@ -256,7 +271,7 @@ def run_gated(args, ops, dev):
         line['roofline'] = {'bound': 'mfma', 'kernel': 'experts (up + down products + finish)',
                             'achieved': active / ms_experts / 1e9, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
                             'frac': active / ms_experts / 1e9 / PEAK_BF16_TFLOPS,
-                            'traffic': MEASURED_TRAFFIC.get(args.workload), 'kernel_ms': ms_experts,
+                            'traffic': traffic, 'traffic_source': traffic_src, 'kernel_ms': ms_experts,
                             'executed_tflops': executed / ms_experts / 1e9}
         # the literal reading of the same number (keep norm >= tau * max): a few experts per token, the layer is bound by
         # the weight stream again and takes the expert-major path
@@ -276,7 +291,7 @@ def run_gated(args, ops, dev):
                                 'roofline': {'bound': 'hbm', 'achieved': bytes_lit / ms_lit / 1e6, 'peak': PEAK_HBM_GBPS,
                                              'unit': 'GB/s', 'frac': bytes_lit / ms_lit / 1e6 / PEAK_HBM_GBPS,
                                              'algorithmic_bytes': bytes_lit}}
-    print(json.dumps(line))
+    return line
 
 
 def run_gpt2(args, dev):
@@ -443,28 +458,110 @@ def run_norms(args, ops, dev):
     print(json.dumps(line))
 
 
-def cpu_baseline(D, E, Ed, W, act, tau, budget_s=12.0):
+def cpu_baseline(D, E, Ed, W, act, tau, budget_s=16.0):
     """The oracle's restatement of the reference CPU path (router -> dynk_max gate -> per-expert loop), float32,
-    8 x 197 tokens of the same layer shape, repeated until about budget_s seconds have been spent."""
+    8 x 197 tokens of the same layer shape, under both readings of the threshold number: the module's (keep norm >=
+    (1 - tau) * max, the headline's) and the literal one (keep norm >= tau * max, i.e. module tau 1 - tau).  Each is
+    repeated until its half of budget_s seconds has been spent."""
     from oracle import d2dmoe_oracle as O
     threads = os.cpu_count() or 1
     threads = min(threads, 16)   # the box's CPU share for one GPU
     torch.set_num_threads(threads)
     p = O.make_layer_params(D, E, Ed, W, seed=0)
     x = torch.randn(8, 197, D, generator=torch.Generator().manual_seed(1))
-    with torch.no_grad():
-        O.moe_layer_forward(x, p, tau, act, 'naive')
-        times = []
-        t_start = time.perf_counter()
-        while (time.perf_counter() - t_start < budget_s and len(times) < 400) or len(times) < 3:
-            t0 = time.perf_counter()
-            O.moe_layer_forward(x, p, tau, act, 'naive')
-            times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
+
+    def timed(module_tau, budget):
+        with torch.no_grad():
+            _, gating, _ = O.moe_layer_forward(x, p, module_tau, act, 'naive')
+            times = []
+            t_start = time.perf_counter()
+            while (time.perf_counter() - t_start < budget and len(times) < 400) or len(times) < 3:
+                t0 = time.perf_counter()
+                O.moe_layer_forward(x, p, module_tau, act, 'naive')
+                times.append(time.perf_counter() - t0)
+        times.sort()
+        return times[len(times) // 2], len(times), gating.float().sum(-1).mean().item()
+
+    med, reps, k = timed(tau, budget_s / 2)
+    med_lit, reps_lit, k_lit = timed(1.0 - tau, budget_s / 2)
     return dict(value=8 * 197 / med, unit='tokens/s', cores=threads, kind='port',
-                sample=f'8x197=1576 tokens of the same layer (D={D}, {E}x{Ed} experts), float32, module tau={tau}, '
-                       f'{len(times)} repetitions, median {med * 1e3:.1f} ms per pass')
+                sample=f'8x197=1576 tokens of the same layer (D={D}, {E}x{Ed} experts), float32, module tau={tau} '
+                       f'({k:.1f} experts per token), {reps} repetitions, median {med * 1e3:.1f} ms per pass',
+                literal_rule=dict(value=8 * 197 / med_lit, unit='tokens/s', rule=f'keep norm >= {tau}*max',
+                                  sample=f'the same 1576 tokens, module tau={1.0 - tau:.2f} ({k_lit:.1f} experts per token), '
+                                         f'{reps_lit} repetitions, median {med_lit * 1e3:.1f} ms per pass'))
+
+
+def compact_gated(line):
+    """The fields of a gated workload's line that matter inside another line."""
+    keep = {'workload': line['config']['workload'], 'ms_per_step': line['ms_per_step'], 'tokens_per_s': line['value'],
+            'mean_active_experts': line['config']['mean_active_experts'],
+            'experts_routed_to': line['config']['experts_routed_to'], 'roofline': line['roofline']}
+    if 'literal_rule' in line:
+        keep['literal_rule'] = line['literal_rule']
+    return keep
+
+
+def skew_norms(N, E, dtype, dev):
+    """Norms that bypass the router: |randn| * w_e with w_e = rank_e^-1.2 over a random ranking of the experts."""
+    g = torch.Generator().manual_seed(2)
+    ranks = torch.randperm(E, generator=g).float() + 1.0
+    wts = ranks ** -1.2
+    return (torch.randn(N, E, generator=g).abs() * (wts / wts.max())).to(dtype).to(dev)
+
+
+def regime_roofline(r, N, peak):
+    """The experts call of one regime against both ceilings: active-pair FLOPs over the MFMA peak and the layer's
+    algorithmic bytes over the HBM peak; the bound named is the one the larger fraction belongs to."""
+    f_mfma = r['active_tflops_kernel'] / peak
+    f_hbm = r['algo_bytes'] / r['ms_experts'] / 1e6 / PEAK_HBM_GBPS
+    if f_mfma >= f_hbm:
+        return {'bound': 'mfma', 'achieved': r['active_tflops_kernel'], 'peak': peak, 'unit': 'TFLOP/s', 'frac': f_mfma,
+                'kernel_ms': r['ms_experts']}
+    return {'bound': 'hbm', 'achieved': r['algo_bytes'] / r['ms_experts'] / 1e6, 'peak': PEAK_HBM_GBPS, 'unit': 'GB/s',
+            'frac': f_hbm, 'kernel_ms': r['ms_experts']}
+
+
+def skew_record(args, ops, dev, steps, warmup):
+    """vit_b_skew inside the default line: both readings of the threshold number on the skewed norms."""
+    B, T, D, E, Ed, W, act = WORKLOADS['vit_b_skew']
+    N = B * T
+    p = make_params(D, E, Ed, W, seed=0, dtype=torch.bfloat16, device=dev)
+    x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(dev)
+    packed = ops.pack_weights(ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x), act), p['w1'], p['b1'], p['w2'], None,
+                              p['router_w1'], p['router_w2'])
+    norms_in = skew_norms(N, E, torch.bfloat16, dev)
+    rec = {'workload': f'vit_b_skew: {N} tokens, D={D}, {E} experts x {Ed}, {act}, norms |randn| * rank^-1.2 in place of the router'}
+    for key, thr in (('module_tau', 1.0 - args.tau), ('literal_rule', args.tau)):
+        r = run_regime(ops, x, p, packed, float(thr), act, steps, warmup, D, E, Ed, W, norms_in=norms_in)
+        rec[key] = {'keep_norm_ge_frac_of_max': round(thr, 4), 'ms_per_step': r['ms_layer'], 'tokens_per_s': r['tokens_per_s'],
+                    'mean_active_experts': r['mean_active'], 'p99_active_experts': r['p99_active'],
+                    'expert_load_max_over_mean': r['expert_load_max_over_mean'],
+                    'roofline': regime_roofline(r, N, PEAK_BF16_TFLOPS)}
+    return rec
+
+
+def reference_shape_record(ops, dev, steps, warmup):
+    """The shape and sweep of the reference's own micro-benchmark (scripts/test_moe_implementations.py:109-142, 214-285):
+    hidden 768, 24 experts x 128 neurons, ReLU, 256 x 197 tokens; the router's output is overridden by Bernoulli(k_frac)
+    draws and the layer runs dynk_max with tau = 0.99, so a token keeps exactly the experts that drew 1 (every expert
+    when a token drew none: all norms equal the maximum 0).  The draws enter through norms_in."""
+    B, T, D, E, Ed, W, act = 256, 197, 768, 24, 128, 128, 'relu'
+    N = B * T
+    p = make_params(D, E, Ed, W, seed=0, dtype=torch.bfloat16, device=dev)
+    x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(dev)
+    packed = ops.pack_weights(ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x), act), p['w1'], p['b1'], p['w2'], None,
+                              p['router_w1'], p['router_w2'])
+    rows = []
+    for k_frac in (1.0, 0.5, 0.1):
+        g = torch.Generator().manual_seed(int(k_frac * 100))
+        norms_in = (torch.rand(N, E, generator=g) < k_frac).to(torch.bfloat16).to(dev)
+        r = run_regime(ops, x, p, packed, 0.01, act, steps, warmup, D, E, Ed, W, norms_in=norms_in)
+        rows.append({'k_frac': k_frac, 'ms_per_step': r['ms_layer'], 'tokens_per_s': r['tokens_per_s'],
+                     'mean_active_experts': r['mean_active'], 'roofline': regime_roofline(r, N, PEAK_BF16_TFLOPS)})
+    dense_ms = dense_mlp_ms(x, D, E * Ed, act, steps, warmup)
+    return {'workload': f'reference micro-benchmark shape: {B}x{T}={N} tokens, D={D}, {E} experts x {Ed}, {act}, bf16, '
+                        f'Bernoulli(k_frac) router override, tau=0.99', 'dense_mlp_ms': dense_ms, 'rows': rows}
 
 
 def main():
@@ -476,6 +573,8 @@ def main():
     ap.add_argument('--tau', type=float, default=0.9, help='module tau (keep expert when norm >= (1 - tau) * max)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-sweep', action='store_true', help='skip the threshold sweep (5 values x 2 readings)')
+    ap.add_argument('--no-sub-records', action='store_true',
+                    help='skip the other workloads the default line carries (gemma_1/16/4096, vit_b_skew, reference shape)')
     ap.add_argument('--quantile-iters', type=int, default=200,
                     help='per-call timed launches of the experts kernel for median / 2.5 % / 97.5 % (0 = skip)')
     ap.add_argument('--copy-probe', action='store_true',
@@ -523,12 +622,8 @@ def main():
     x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
     shape = ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x), act)
     packed = ops.pack_weights(shape, p['w1'], p['b1'], p['w2'], None, p['router_w1'], p['router_w2'])
-    norms_in = None
-    if args.workload == 'vit_b_skew':
-        g = torch.Generator().manual_seed(2)
-        ranks = torch.randperm(E, generator=g).float() + 1.0
-        wts = ranks ** -1.2
-        norms_in = (torch.randn(N, E, generator=g).abs() * (wts / wts.max())).to(dtype).to(dev)
+    traffic, traffic_src = measured_traffic(args.workload)
+    norms_in = skew_norms(N, E, dtype, dev) if args.workload == 'vit_b_skew' else None
     with torch.no_grad():
         main_r = run_regime(ops, x, p, packed, float(1.0 - args.tau), act, args.steps, args.warmup, D, E, Ed, W,
                             quantile_iters=args.quantile_iters, norms_in=norms_in)
@@ -557,7 +652,7 @@ def main():
         'active_tflops': main_r['active_tflops_layer'], 'hbm_gbps': main_r['hbm_gbps_layer'],
         'roofline': {'bound': 'mfma', 'kernel': 'experts', 'achieved': main_r['active_tflops_kernel'],
                      'peak': peak, 'unit': 'TFLOP/s', 'frac': main_r['active_tflops_kernel'] / peak,
-                     'traffic': MEASURED_TRAFFIC.get(args.workload), 'kernel_ms': main_r['ms_experts'],
+                     'traffic': traffic, 'traffic_source': traffic_src, 'kernel_ms': main_r['ms_experts'],
                      'kernel_quantiles': main_r['experts_quantiles'], 'router_select_ms': main_r['ms_router'],
                      'frac_of_library_gemm': main_r['active_tflops_kernel'] / ceil['library_gemm_bf16_8192_tflops']},
         'measured_ceilings': ceil,
@@ -571,6 +666,20 @@ def main():
                                       'algorithmic_bytes': lit_r['algo_bytes'], 'kernel_ms': lit_r['ms_experts']}},
         'sweep': sweep,
     }
+    if args.workload == 'vit_b_50k' and not args.no_sub_records:
+        # the other workloads this library is measured on, each with its own roofline, so that one run shows them all
+        del x, p, packed
+        sub_steps, sub_warmup = max(args.steps // 2, 10), max(args.warmup // 2, 3)
+        sub = {}
+        with torch.no_grad():
+            saved = args.steps, args.warmup
+            args.steps, args.warmup = sub_steps, sub_warmup
+            for w in ('gemma_1', 'gemma_16', 'gemma_4096'):
+                sub[w] = compact_gated(gated_record(args, ops, dev, w))
+            args.steps, args.warmup = saved
+            sub['vit_b_skew'] = skew_record(args, ops, dev, sub_steps, sub_warmup)
+            sub['reference_shape'] = reference_shape_record(ops, dev, sub_steps, sub_warmup)
+        line['sub_records'] = sub
     if not args.no_cpu_baseline:
         line['cpu_baseline'] = cpu_baseline(D, E, Ed, W, act, args.tau)
     print(json.dumps(line))
