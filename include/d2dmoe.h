@@ -77,12 +77,13 @@ enum {
   D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 MFMA for a handful of tokens: per pass of 16 tokens one workgroup per expert streams
                                  that expert's packed weights once (gated or ungated experts); at most 48 tokens (three
                                  passes).  AUTO picks it up to 16 tokens, for gated experts up to 48 */
-  D2DMOE_PATH_MFMA_MID = 6,   /* bf16 MFMA, ungated experts of at most 32 neurons at D = 768: work follows the routed pairs.
-                                 An expert-stationary first product gathers each expert's routed tokens from token tiles held
-                                 in LDS and keeps 64 bytes of hidden activations per pair; an output-stationary second
-                                 product adds every expert's contribution, in ascending expert order, to float32 token
-                                 rows held in LDS.  Taken when at most 48 experts per token are routed on average (checked
-                                 on the device), else the dense sweep runs */
+  D2DMOE_PATH_MFMA_MID = 6,   /* bf16 MFMA, ungated experts of at most 31 neurons at D = 768, at most 256 experts: work follows
+                                 the routed pairs.  An expert-stationary first product gathers each expert's routed tokens
+                                 (16 at a time, straight into registers) and keeps 64 bytes of hidden activations per pair;
+                                 an output-stationary second product adds every expert's contribution, in ascending expert
+                                 order, to float32 token rows held in LDS.  Runs when at most 48 experts per token are
+                                 routed on average (checked on the device), else the dense sweep does.  Never picked by
+                                 AUTO: it is ahead of the other paths only between about 6 and 9 experts per token */
   D2DMOE_PATH_MFMA_GEMM = 5   /* bf16 or f32 MFMA, D a multiple of 256, gated or ungated experts: two tiled products over all
                                  experts with the routing value as a factor of the hidden activations, which stay in
                                  the workspace between them; AUTO picks it for more than 16 tokens when the dense sweep

@@ -30,7 +30,7 @@ def _packed(d, act='relu', E=128, Ed=24, with_router=False):
 
 @pytest.mark.parametrize('N,E,Ed,density', [(1, 128, 24, 0.2), (31, 128, 24, 0.2), (32, 128, 24, 0.2), (33, 128, 24, 0.3),
                                             (197, 128, 24, 0.18), (300, 128, 24, 0.02), (300, 128, 24, 0.36), (1576, 128, 24, 0.18),
-                                            (1576, 128, 24, 0.06), (700, 96, 30, 0.25), (520, 16, 32, 0.5), (260, 8, 5, 0.6),
+                                            (1576, 128, 24, 0.06), (700, 96, 30, 0.25), (520, 16, 31, 0.5), (700, 100, 24, 0.2), (1000, 40, 7, 0.4), (260, 8, 5, 0.6),
                                             (4100, 128, 24, 0.3), (2048, 144, 16, 0.1)])
 def test_mid_path_matches_oracle(N, E, Ed, density):
     _say('mid', N, E, Ed, density)
