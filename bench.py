@@ -100,6 +100,28 @@ def time_events(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+def time_graph(fn, steps, warmup):
+    """Mean milliseconds per call of fn when the call is captured once into a HIP graph and replayed (the C ABI calls neither
+    allocate nor synchronise, so a whole layer captures): wall clock over `steps` replays, bracketed by synchronize."""
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        fn()
+    for _ in range(warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
 def time_quantiles(fn, iters, warmup):
     """Per-call durations of fn from one HIP event pair per call on the launch stream: median, 2.5 % and 97.5 %
     quantiles in milliseconds (the reference's own bench reports the same three, test_moe_implementations.py:171-175)."""
@@ -168,25 +190,8 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, pa
         layer()
     torch.cuda.synchronize()
     ms_layer_eager = (time.perf_counter() - t0) * 1e3 / steps
-    # the same step replayed from a HIP graph (the C ABI calls neither allocate nor synchronise, so the whole layer
-    # captures): removes the host's launch latency between the dependent kernels
-    graph = torch.cuda.CUDAGraph()
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        layer()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    with torch.cuda.graph(graph):
-        layer()
-    for _ in range(warmup):
-        graph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        graph.replay()
-    torch.cuda.synchronize()
-    ms_layer = (time.perf_counter() - t0) * 1e3 / steps
+    # the same step replayed from a HIP graph: removes the host's launch latency between the dependent kernels
+    ms_layer = time_graph(layer, steps, warmup)
     # dominant kernel alone (same routing), HIP events on the launch stream
     # the experts call the layer makes: under AUTO d2dmoe_forward takes the expert-major path for high thresholds (bf16)
     experts_path = path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 and x.dtype == torch.bfloat16 else 'auto')
@@ -241,7 +246,8 @@ def gated_record(args, ops, dev, workload):
     torch.cuda.synchronize()
     union = int((routing.float().sum(0) > 0).sum().item())
     pairs = int(routing.float().sum().item())
-    ms_layer = time_events(layer, args.steps, args.warmup)
+    ms_layer_eager = time_events(layer, args.steps, args.warmup)
+    ms_layer = time_graph(layer, args.steps, args.warmup)     # as for the headline: replays of a HIP graph of one layer call
     ms_experts = time_events(lambda: ops.experts(x, routing, wg, None, wd, wu, None, act, False, 'auto', packed),
                              args.steps, args.warmup)
     s = x.element_size()
@@ -254,6 +260,7 @@ def gated_record(args, ops, dev, workload):
         'config': {'workload': f'{workload}: {N} tokens, D={D}, {E} gated experts x {Ed}, {act}, router {D}->{W}->{E}, '
                                f'module tau={args.tau}, whole layer', 'experts_routed_to': union,
                    'mean_active_experts': pairs / N, 'mfma_kernels': packed is not None},
+        'ms_per_step_eager_launches': ms_layer_eager,
         'active_tflops': pairs * 6.0 * D * Ed / ms_layer / 1e9, 'hbm_gbps': algo_bytes / ms_layer / 1e6,
         'roofline': {'bound': 'hbm', 'kernel': 'experts (hidden + out kernels)',
                      'achieved': (union * 3 * D * Ed * s + 2 * N * D * s) / ms_experts / 1e6,
@@ -282,7 +289,7 @@ def gated_record(args, ops, dev, workload):
 
         _, r_lit, _, _ = layer_lit()
         torch.cuda.synchronize()
-        ms_lit = time_events(layer_lit, args.steps, args.warmup)
+        ms_lit = time_graph(layer_lit, args.steps, args.warmup)
         union_lit = int((r_lit.float().sum(0) > 0).sum().item())
         pairs_lit = int(r_lit.float().sum().item())
         bytes_lit = (W * D + E * W) * s + union_lit * 3 * D * Ed * s + 2 * N * D * s + N * E * s
@@ -494,7 +501,8 @@ def cpu_baseline(D, E, Ed, W, act, tau, budget_s=16.0):
 
 def compact_gated(line):
     """The fields of a gated workload's line that matter inside another line."""
-    keep = {'workload': line['config']['workload'], 'ms_per_step': line['ms_per_step'], 'tokens_per_s': line['value'],
+    keep = {'workload': line['config']['workload'], 'ms_per_step': line['ms_per_step'],
+            'ms_per_step_eager_launches': line['ms_per_step_eager_launches'], 'tokens_per_s': line['value'],
             'mean_active_experts': line['config']['mean_active_experts'],
             'experts_routed_to': line['config']['experts_routed_to'], 'roofline': line['roofline']}
     if 'literal_rule' in line:

@@ -340,6 +340,16 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   const ForwardWorkspace plan = plan_workspace(sh);
   if (!workspace || workspace_bytes < plan.total || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
   char* ws = (char*)workspace;
+  if (norms_in == nullptr && (path == D2DMOE_PATH_AUTO || path == D2DMOE_PATH_MFMA_DECODE) && packed != nullptr &&
+      mfma_decode_layer_supported(sh) && router_w1 && router_w2 && w1 && w2 && (sh.gated ? (w_up && !b1) : !w_up) &&
+      aligned16(x) && aligned16(out) && aligned16(routing) && aligned16(router_w1) && aligned16(router_w2) &&
+      (!norms_out || aligned16(norms_out))) {
+    // a handful of tokens: three launches for the whole layer, the router running beside the experts' first layer
+    void* nbuf = norms_out ? norms_out : (void*)(ws + plan.norms_off);
+    return (int)launch_mfma_decode_layer(sh, x, router_w1, router_w2, thr_scale,
+                                         (const char*)packed + mfma_decode_section_offset(sh), last_bias, ws + plan.hidden_off,
+                                         nbuf, routing, counts, out, ws + plan.perm_off, (hipStream_t)stream);
+  }
   if (norms_in == nullptr) {
     st = d2dmoe_router_select(shape, x, router_w1, router_w2, packed, thr_scale, norms_out, routing, counts, workspace,
                               workspace_bytes, stream);

@@ -140,24 +140,85 @@ hipError_t launch_decode_pack(const d2dmoe_shape& sh, const void* w1, const void
 struct DecodeArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* wgu; const bf16x8* wd; const bf16_t* bias;
   bf16x8* hfrag; int* active; const bf16_t* last_bias; bf16_t* out; int N; int D; int E; int nt16; int act; int add_residual;
+  // Whole layer in three launches (fused != 0): the hidden kernel computes every expert (it does not wait for the routing)
+  // and its extra workgroups compute the first router layer; the output kernel derives the routing from the norms itself.
+  int fused;
+  const bf16_t* rw1; bf16_t* rhidden; int rwidth; int ract;     // first router layer: [rwidth, D] -> rhidden [N, rwidth]
+  const bf16_t* norms; bf16_t* routing_out; int32_t* counts; float thr_scale;
 };
+
+// First router layer inside the hidden kernel's launch: 4 features per workgroup of 4 waves.  K is cut into the same parts
+// as by linear_skinny_kernel (16 where K is long, else 4), each part accumulated on its own in K order and the parts
+// summed in order, so the result has the bits that kernel produces.
+__device__ __forceinline__ void decode_router_l1_block(const DecodeArgs& A, int blk, float (*part)[4][64]) {
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  const int gq = lane >> 4, c16 = lane & 15;
+  const int K = A.D, Nout = A.rwidth, N = A.N;
+  const int P = (K % 512 == 0 && K >= 1024) ? 16 : 4;   // parts of K
+  const int KQ = K / P;                                   // a multiple of 32
+  const int f0 = blk * 4;
+  const int fr = f0 + (c16 & 3);
+  const int frow = (fr < Nout) ? fr : (Nout - 1);
+  const int trow = (c16 < N) ? c16 : (N - 1);
+  for (int p = w * (P / 4); p < (w + 1) * (P / 4); ++p) {
+    const bf16x8* bp = (const bf16x8*)(A.rw1 + (int64_t)frow * K + p * KQ) + gq;
+    const bf16x8* ap = (const bf16x8*)(A.x + (int64_t)trow * K + p * KQ) + gq;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int ks0 = 0; ks0 < KQ / 32; ks0 += 4) {
+      bf16x8 bv[4], av[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int ks = (ks0 + u < KQ / 32) ? (ks0 + u) : ks0;
+        bv[u] = bp[ks * 4];
+        av[u] = ap[ks * 4];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (ks0 + u < KQ / 32) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv[u], av[u], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) part[p][r][lane] = acc[r];
+  }
+  __syncthreads();
+  if (w == 0 && gq == 0 && c16 < N) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float v = part[0][r][lane];
+      for (int pp = 1; pp < P; ++pp) v += part[pp][r][lane];
+      const int f = f0 + r;
+      if (f < Nout) {
+        const float vr = bf16_to_f32(f32_to_bf16(v));
+        A.rhidden[(int64_t)c16 * Nout + f] = f32_to_bf16(apply_act(A.ract, vr));
+      }
+    }
+  }
+}
 
 template <bool GATED, int U1>
 __global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) {
-  __shared__ float part[4][(GATED ? 2 : 1) * 8][64];
+  __shared__ float part_raw[16 * 4 * 64];          // [4][NM * 8][64] here, [16][4][64] for the router workgroups
+  float (*part)[(GATED ? 2 : 1) * 8][64] = (float (*)[(GATED ? 2 : 1) * 8][64])part_raw;
   const int D = A.D, N = A.N, E = A.E, NT16 = A.nt16;
+  // fused: the first workgroups of the grid are the router's (they start first, so the second router layer's input is
+  // ready long before the grid has drained)
+  const int n_router = A.fused ? (A.rwidth + 3) / 4 : 0;
+  if ((int)blockIdx.x < n_router) {
+    decode_router_l1_block(A, (int)blockIdx.x, (float (*)[4][64])part_raw);
+    return;
+  }
+  const int hb = (int)blockIdx.x - n_router;
   const int KS = D / 32;          // K steps of GEMM1
   const int KQ = KS / 4;          // per wave
   constexpr int NM = GATED ? 2 : 1;
   constexpr int FPS = NM * 2;     // fragments per K step
   const int KS2 = NT16 / 2;
-  const int e = blockIdx.x / KS2, k2 = blockIdx.x % KS2;
+  const int e = hb / KS2, k2 = hb % KS2;
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
   const int gq = lane >> 4, c16 = lane & 15;
   const int tc = (c16 < N) ? c16 : (N - 1);
-  const bf16_t rbits = A.routing[(int64_t)tc * E + e];
+  const bf16_t rbits = A.fused ? (bf16_t)0x3f80 : A.routing[(int64_t)tc * E + e];   // fused: the routing is applied later
   const bool any = __ballot((rbits & 0x7fff) != 0) != 0ull;
-  if (k2 == 0 && t == 0) A.active[e] = any ? 1 : 0;
+  if (!A.fused && k2 == 0 && t == 0) A.active[e] = any ? 1 : 0;
   if (!any) return;   // nobody routes to this expert: its fragments are never read
 
   f32x4 acc1[NM][2];
@@ -166,7 +227,7 @@ __global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) 
 #pragma unroll
     for (int a = 0; a < 2; ++a) acc1[m][a] = f32x4{0.f, 0.f, 0.f, 0.f};
   // this workgroup's stream is contiguous: KS steps of FPS fragments; wave w takes steps [w*KQ, (w+1)*KQ)
-  const bf16x8* wf = A.wgu + ((int64_t)blockIdx.x * KS + (int64_t)w * KQ) * FPS * 64 + lane;
+  const bf16x8* wf = A.wgu + ((int64_t)hb * KS + (int64_t)w * KQ) * FPS * 64 + lane;
   const bf16x8* xf = (const bf16x8*)(A.x + (int64_t)tc * D + (int64_t)w * KQ * 32) + gq;   // + 4 per K step
   // Two register buffers of U1 K steps each: while one is multiplied the other is being filled.  KQ is a multiple of
   // 2*U1 (the launcher picks U1 that way).
@@ -239,26 +300,63 @@ template <int KS2>
 __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeArgs A) {
   constexpr int UB = 8 / KS2;                  // experts per load batch (8 fragments of each operand)
   __shared__ float part[DO_WAVES][4][64];
+  __shared__ float s_thr[16];                  // fused: the tokens' thresholds
+  __shared__ unsigned short s_bits[DO_WAVES * 64];   // fused: per expert, bit t = token t routes to it
   const int D = A.D, N = A.N, E = A.E;
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
   const int gq = lane >> 4, c16 = lane & 15;
   const int cb = blockIdx.x;                   // 8-column block
   const int EW = (E + DO_WAVES - 1) / DO_WAVES;
   const int e_lo = w * EW, e_hi = (e_lo + EW < E) ? (e_lo + EW) : E;
+  if (A.fused) {
+    // Dynamic-k selection from the norms (moefication.py:80-85), by every workgroup for itself (8 KB out of L2): wave 0
+    // takes the maximum of every token's row, then a lane per expert compares its column with the thresholds.  Same
+    // arithmetic as select_kernel: m NaN-propagating, thr = round(m * thr_scale), on = norm >= thr.
+    // (E <= 512 here: one expert per thread; its column is requested before the maxima are worked out)
+    const int ecol = (t < E) ? t : (E - 1);
+    bf16_t colv[DC_MAX_TOKENS];
+#pragma unroll
+    for (int tk = 0; tk < DC_MAX_TOKENS; ++tk) colv[tk] = A.norms[(int64_t)(tk < N ? tk : N - 1) * E + ecol];
+    if (w == 0) {
+      const int tc = (c16 < N) ? c16 : (N - 1);
+      float m = -INFINITY;
+      for (int e8 = gq * 8; e8 < E; e8 += 32) {          // E is a multiple of 32 here
+        const u32x4 v = *(const u32x4*)(A.norms + (int64_t)tc * E + e8);
+        const uint32_t vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) m = nanmax(m, __uint_as_float((i & 1) ? (vw[i >> 1] & 0xffff0000u) : (vw[i >> 1] << 16)));
+      }
+      m = nanmax(m, __shfl_xor(m, 16, 64));
+      m = nanmax(m, __shfl_xor(m, 32, 64));
+      if (gq == 0) s_thr[c16] = bf16_to_f32(f32_to_bf16(m * A.thr_scale));
+    }
+    __syncthreads();
+    if (t < E) {
+      unsigned bits = 0u;
+#pragma unroll
+      for (int tk = 0; tk < DC_MAX_TOKENS; ++tk) bits |= ((tk < N && bf16_to_f32(colv[tk]) >= s_thr[tk]) ? 1u : 0u) << tk;
+      s_bits[t] = (unsigned short)bits;
+      if (cb == 0) {                                      // one workgroup also leaves the routing tensor and the counts
+        for (int tk = 0; tk < N; ++tk) A.routing_out[(int64_t)tk * E + t] = ((bits >> tk) & 1u) ? (bf16_t)0x3f80 : (bf16_t)0;
+        if (A.counts != nullptr) A.counts[t] = __popc(bits);
+      }
+    }
+    __syncthreads();
+  }
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   // A fragment rows 0..7 only (lanes c16 >= 8 repeat them); result rows 8..15 are dropped
   const bf16x8* wdf = A.wd + (int64_t)cb * E * KS2 * 32 + gq * 8 + (c16 & 7);
   const bf16x8* hf = A.hfrag + lane;
   bf16x8 aA[UB][KS2], bA[UB][KS2], aB[UB][KS2], bB[UB][KS2];
+  int esA[UB], esB[UB];
   for (int e0 = e_lo; e0 < e_hi; e0 += 64) {   // 64 experts per pass: one flag per lane
-    const bool on = (e0 + lane < e_hi) && (A.active[e0 + lane] != 0);
+    const bool on = (e0 + lane < e_hi) && (A.fused ? (s_bits[e0 + lane] != 0) : (A.active[e0 + lane] != 0));
     unsigned long long mask = __ballot(on);
     int cntA = 0, cntB = 0;
     // take the next up to UB routed experts off the mask and request their fragments; unused slots repeat the last one
-    auto fill = [&](bf16x8 (&a)[UB][KS2], bf16x8 (&b)[UB][KS2], int& cnt) __attribute__((always_inline)) {
+    auto fill = [&](bf16x8 (&a)[UB][KS2], bf16x8 (&b)[UB][KS2], int (&es)[UB], int& cnt) __attribute__((always_inline)) {
       cnt = 0;
       int e = e0;
-      int es[UB];
 #pragma unroll
       for (int j = 0; j < UB; ++j) {
         if (mask != 0ull) {
@@ -277,24 +375,30 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
 #pragma unroll
         for (int k2 = 0; k2 < KS2; ++k2) a[j][k2] = wdf[((int64_t)es[j] * KS2 + k2) * 32];
     };
-    auto multiply = [&](bf16x8 (&a)[UB][KS2], bf16x8 (&b)[UB][KS2], int cnt) __attribute__((always_inline)) {
+    auto multiply = [&](bf16x8 (&a)[UB][KS2], bf16x8 (&b)[UB][KS2], int (&es)[UB], int cnt) __attribute__((always_inline)) {
 #pragma unroll
       for (int j = 0; j < UB; ++j) {
         if (j < cnt) {
+          // fused: the hidden fragment holds every token; the columns of tokens that do not route here are cleared
+          const bool keep = A.fused ? (((s_bits[es[j]] >> c16) & 1u) != 0u) : true;
 #pragma unroll
-          for (int k2 = 0; k2 < KS2; ++k2) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][k2], b[j][k2], acc, 0, 0, 0);
+          for (int k2 = 0; k2 < KS2; ++k2) {
+            u32x4 bm = __builtin_bit_cast(u32x4, b[j][k2]);
+            bm.x = keep ? bm.x : 0u; bm.y = keep ? bm.y : 0u; bm.z = keep ? bm.z : 0u; bm.w = keep ? bm.w : 0u;
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][k2], __builtin_bit_cast(bf16x8, bm), acc, 0, 0, 0);
+          }
         }
       }
     };
     if (mask != 0ull) {
-      fill(aA, bA, cntA);
+      fill(aA, bA, esA, cntA);
       while (cntA > 0) {
         cntB = 0;
-        if (mask != 0ull) fill(aB, bB, cntB);
-        multiply(aA, bA, cntA);
+        if (mask != 0ull) fill(aB, bB, esB, cntB);
+        multiply(aA, bA, esA, cntA);
         cntA = 0;
-        if (mask != 0ull) fill(aA, bA, cntA);
-        multiply(aB, bB, cntB);
+        if (mask != 0ull) fill(aA, bA, esA, cntA);
+        multiply(aB, bB, esB, cntB);
       }
     }
   }
@@ -331,7 +435,7 @@ template <bool GATED>
 static hipError_t launch_hidden(const DecodeArgs& A, hipStream_t s) {
   // K steps per wave (D/128) must be a multiple of 2*U1; D is a multiple of 256, so U1 = 1 always fits.
   const int KQ = A.D / 128;
-  const dim3 grid((unsigned)(A.E * (A.nt16 / 2)));
+  const dim3 grid((unsigned)(A.E * (A.nt16 / 2) + (A.fused ? (A.rwidth + 3) / 4 : 0)));
   if (KQ % 8 == 0) hipLaunchKernelGGL((decode_hidden_kernel<GATED, 4>), grid, dim3(256), 0, s, A);
   else if (KQ % 4 == 0) hipLaunchKernelGGL((decode_hidden_kernel<GATED, 2>), grid, dim3(256), 0, s, A);
   else hipLaunchKernelGGL((decode_hidden_kernel<GATED, 1>), grid, dim3(256), 0, s, A);
@@ -350,7 +454,44 @@ hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void*
   A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out;
   A.N = (int)sh.n_tokens; A.D = sh.d_model; A.E = sh.n_experts; A.nt16 = L.nt16; A.act = sh.activation;
   A.add_residual = sh.add_residual;
+  A.fused = 0; A.rw1 = nullptr; A.rhidden = nullptr; A.rwidth = 0; A.ract = 0; A.norms = nullptr; A.routing_out = nullptr;
+  A.counts = nullptr; A.thr_scale = 0.f;
   const hipError_t e = sh.gated ? launch_hidden<true>(A, s) : launch_hidden<false>(A, s);
+  if (e != hipSuccess) return e;
+  const dim3 grid((unsigned)(sh.d_model / 8));
+  if (L.nt16 == 2) hipLaunchKernelGGL(decode_out_kernel<1>, grid, dim3(DO_WAVES * 64), 0, s, A);
+  else if (L.nt16 == 4) hipLaunchKernelGGL(decode_out_kernel<2>, grid, dim3(DO_WAVES * 64), 0, s, A);
+  else hipLaunchKernelGGL(decode_out_kernel<4>, grid, dim3(DO_WAVES * 64), 0, s, A);
+  return hipGetLastError();
+}
+
+// The whole layer for at most 16 tokens in three launches: hidden activations of every expert + first router layer (one
+// launch: neither waits for the other), second router layer (norms), output kernel with the selection inside.
+bool mfma_decode_layer_supported(const d2dmoe_shape& sh) {
+  return mfma_decode_supported(sh) && sh.n_tokens >= 1 && sh.n_tokens <= DC_MAX_TOKENS && sh.n_experts % 32 == 0 &&
+         sh.n_experts <= DO_WAVES * 64 && sh.router_width > 0 && linear_skinny_supported(sh.n_tokens, sh.d_model, sh.dtype) &&
+         linear_skinny_supported(sh.n_tokens, sh.router_width, sh.dtype);
+}
+
+hipError_t launch_mfma_decode_layer(const d2dmoe_shape& sh, const void* x, const void* router_w1, const void* router_w2,
+                                    float thr_scale, const void* packed_section, const void* last_bias, void* router_hidden,
+                                    void* norms, void* routing, int32_t* counts, void* out, void* workspace, hipStream_t s) {
+  const DecodeLayout L = decode_layout(sh);
+  const char* pk = (const char*)packed_section;
+  DecodeArgs A;
+  A.x = (const bf16_t*)x; A.routing = nullptr; A.wgu = (const bf16x8*)(pk + L.gu_off);
+  A.wd = (const bf16x8*)(pk + L.d_off); A.bias = (const bf16_t*)(pk + L.b_off);
+  A.hfrag = (bf16x8*)workspace; A.active = nullptr;
+  A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out;
+  A.N = (int)sh.n_tokens; A.D = sh.d_model; A.E = sh.n_experts; A.nt16 = L.nt16; A.act = sh.activation;
+  A.add_residual = sh.add_residual;
+  A.fused = 1; A.rw1 = (const bf16_t*)router_w1; A.rhidden = (bf16_t*)router_hidden; A.rwidth = sh.router_width;
+  A.ract = sh.router_activation; A.norms = (const bf16_t*)norms; A.routing_out = (bf16_t*)routing; A.counts = counts;
+  A.thr_scale = thr_scale;
+  hipError_t e = sh.gated ? launch_hidden<true>(A, s) : launch_hidden<false>(A, s);
+  if (e != hipSuccess) return e;
+  e = launch_linear_skinny(router_hidden, router_w2, norms, (int)sh.n_tokens, sh.router_width, sh.n_experts,
+                           sh.router_output_activation, s);
   if (e != hipSuccess) return e;
   const dim3 grid((unsigned)(sh.d_model / 8));
   if (L.nt16 == 2) hipLaunchKernelGGL(decode_out_kernel<1>, grid, dim3(DO_WAVES * 64), 0, s, A);
@@ -361,18 +502,21 @@ hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void*
 
 // ---------------------------------------------------------------------------------------------------
 // Skinny Linear for <= 16 rows: C[N, Nout] = round(act(round(A[N,K] . B[Nout,K]^T))), bf16.
-// Both operands are read straight from their row-major layouts (K contiguous in each): a workgroup owns 16 output features,
-// its 4 or 16 waves share K; partial tiles are summed through LDS in wave order.  Used for the router layers at small N.
+// Both operands are read straight from their row-major layouts (K contiguous in each): a workgroup owns 16 output features
+// (4 where K is long and the features few, so that more than a handful of CUs pull on the weights), its 4 or 16 waves
+// share K; partial tiles are summed through LDS in wave order.  Used for the router layers at small N.
 // ---------------------------------------------------------------------------------------------------
-template <int NW>
+template <int NW, int FPB>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
                                                                bf16_t* __restrict__ C, int N, int K, int Nout, int act) {
   __shared__ float part[NW][4][64];
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
   const int gq = lane >> 4, c16 = lane & 15;
-  const int f0 = blockIdx.x * 16;                 // first output feature of this workgroup
+  const int f0 = blockIdx.x * FPB;                // first output feature of this workgroup
   const int KQ = K / NW;                          // per wave, a multiple of 32
-  const int frow = (f0 + c16 < Nout) ? (f0 + c16) : (Nout - 1);
+  // FPB < 16: the rows of the 16-row tile past the workgroup's features repeat them (no extra traffic) and are dropped
+  const int fr = f0 + (c16 & (FPB - 1));
+  const int frow = (fr < Nout) ? fr : (Nout - 1);
   const int trow = (c16 < N) ? c16 : (N - 1);
   const bf16x8* bp = (const bf16x8*)(B + (int64_t)frow * K + w * KQ) + gq;
   const bf16x8* ap = (const bf16x8*)(A + (int64_t)trow * K + w * KQ) + gq;
@@ -400,7 +544,7 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
 #pragma unroll
       for (int ww = 1; ww < NW; ++ww) v += part[ww][r][lane];
       const int f = f0 + 4 * gq + r;
-      if (c16 < N && f < Nout) {
+      if (c16 < N && f < Nout && 4 * gq + r < FPB) {
         const float vr = bf16_to_f32(f32_to_bf16(v));
         C[(int64_t)c16 * Nout + f] = f32_to_bf16(apply_act(act, vr));
       }
@@ -411,12 +555,17 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
 bool linear_skinny_supported(int64_t N, int K, int dtype) { return dtype == D2DMOE_BF16 && N >= 1 && N <= 16 && K % 128 == 0; }
 
 hipError_t launch_linear_skinny(const void* A, const void* B, void* C, int N, int K, int Nout, int act, hipStream_t s) {
-  if (K % 512 == 0 && K >= 1024)   // long rows: 16 waves share K so that each requests its part in one go
-    hipLaunchKernelGGL(linear_skinny_kernel<16>, dim3((Nout + 15) / 16), dim3(1024), 0, s, (const bf16_t*)A, (const bf16_t*)B,
+  if (K % 512 == 0 && K >= 1024) {   // long rows: 16 waves share K so that each requests its part in one go
+    if (Nout <= 1024)
+      hipLaunchKernelGGL((linear_skinny_kernel<16, 4>), dim3((Nout + 3) / 4), dim3(1024), 0, s, (const bf16_t*)A,
+                         (const bf16_t*)B, (bf16_t*)C, N, K, Nout, act);
+    else
+      hipLaunchKernelGGL((linear_skinny_kernel<16, 16>), dim3((Nout + 15) / 16), dim3(1024), 0, s, (const bf16_t*)A,
+                         (const bf16_t*)B, (bf16_t*)C, N, K, Nout, act);
+  } else {
+    hipLaunchKernelGGL((linear_skinny_kernel<4, 16>), dim3((Nout + 15) / 16), dim3(256), 0, s, (const bf16_t*)A, (const bf16_t*)B,
                        (bf16_t*)C, N, K, Nout, act);
-  else
-    hipLaunchKernelGGL(linear_skinny_kernel<4>, dim3((Nout + 15) / 16), dim3(256), 0, s, (const bf16_t*)A, (const bf16_t*)B,
-                       (bf16_t*)C, N, K, Nout, act);
+  }
   return hipGetLastError();
 }
 
