@@ -583,6 +583,8 @@ def main():
     ap.add_argument('--no-sweep', action='store_true', help='skip the threshold sweep (5 values x 2 readings)')
     ap.add_argument('--no-sub-records', action='store_true',
                     help='skip the other workloads the default line carries (gemma_1/16/4096, vit_b_skew, reference shape)')
+    ap.add_argument('--path', default='auto', choices=['auto', 'mfma_dense', 'mfma_sparse', 'mfma_mid', 'generic'],
+                    help='force the experts path of the ungated workloads (default: the library chooses)')
     ap.add_argument('--quantile-iters', type=int, default=200,
                     help='per-call timed launches of the experts kernel for median / 2.5 % / 97.5 % (0 = skip)')
     ap.add_argument('--copy-probe', action='store_true',
@@ -634,14 +636,16 @@ def main():
     norms_in = skew_norms(N, E, dtype, dev) if args.workload == 'vit_b_skew' else None
     with torch.no_grad():
         main_r = run_regime(ops, x, p, packed, float(1.0 - args.tau), act, args.steps, args.warmup, D, E, Ed, W,
-                            quantile_iters=args.quantile_iters, norms_in=norms_in)
-        lit_r = run_regime(ops, x, p, packed, float(args.tau), act, args.steps, args.warmup, D, E, Ed, W, norms_in=norms_in)
+                            path=args.path, quantile_iters=args.quantile_iters, norms_in=norms_in)
+        lit_r = run_regime(ops, x, p, packed, float(args.tau), act, args.steps, args.warmup, D, E, Ed, W, path=args.path,
+                           norms_in=norms_in)
         sweep = []
         if not args.no_sweep:
             # the threshold number under both readings
             for v in (0.5, 0.8, 0.9, 0.95, 0.99):
                 for rule, thr in (('module_tau', 1.0 - v), ('literal', v)):
-                    r = run_regime(ops, x, p, packed, float(thr), act, max(args.steps // 5, 5), 3, D, E, Ed, W, norms_in=norms_in)
+                    r = run_regime(ops, x, p, packed, float(thr), act, max(args.steps // 5, 5), 3, D, E, Ed, W, path=args.path,
+                                   norms_in=norms_in)
                     sweep.append({'v': v, 'rule': rule, 'keep_norm_ge_frac_of_max': round(thr, 4), 'ms_per_step': r['ms_layer'],
                                   'tokens_per_s': r['tokens_per_s'], 'mean_active_experts': r['mean_active'],
                                   'p99_active_experts': r['p99_active'], 'active_tflops': r['active_tflops_layer']})
@@ -655,7 +659,7 @@ def main():
         'config': {'workload': f'{args.workload}: {B}x{T}={N} tokens, D={D}, {E} experts x {Ed}, {act}, router {D}->{W}->{E}, '
                                f'module tau={args.tau} (keep norm >= {1 - args.tau:.2f}*max), whole layer',
                    'mean_active_experts': main_r['mean_active'], 'p99_active_experts': main_r['p99_active'],
-                   'mfma_kernels': packed is not None},
+                   'mfma_kernels': packed is not None, 'experts_path': args.path},
         'ms_per_step_eager_launches': main_r['ms_layer_eager'],
         'active_tflops': main_r['active_tflops_layer'], 'hbm_gbps': main_r['hbm_gbps_layer'],
         'roofline': {'bound': 'mfma', 'kernel': 'experts', 'achieved': main_r['active_tflops_kernel'],
@@ -674,7 +678,7 @@ def main():
                                       'algorithmic_bytes': lit_r['algo_bytes'], 'kernel_ms': lit_r['ms_experts']}},
         'sweep': sweep,
     }
-    if args.workload == 'vit_b_50k' and not args.no_sub_records:
+    if args.workload == 'vit_b_50k' and args.path == 'auto' and not args.no_sub_records:
         # the other workloads this library is measured on, each with its own roofline, so that one run shows them all
         del x, p, packed
         sub_steps, sub_warmup = max(args.steps // 2, 10), max(args.warmup // 2, 3)
