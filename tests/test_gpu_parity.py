@@ -437,6 +437,33 @@ def test_decode_path_matches_oracle(N, D, E, Ed, W, gated, act):
     assert H.rel_err(out.cpu(), want) < H.TOL_BF16
 
 
+@pytest.mark.parametrize('N', [1, 7, 16])
+@pytest.mark.parametrize('D,E,Ed,W,gated,act', [(2048, 256, 64, 256, True, 'gelu_tanh'), (768, 128, 24, 128, False, 'relu')])
+@pytest.mark.parametrize('tau', [0.9, 0.1])
+def test_small_batch_layer_equals_staged_calls(N, D, E, Ed, W, gated, act, tau):
+    """d2dmoe_forward runs a layer of at most 16 tokens as three launches (first router layer beside the experts' first
+    layer, selection inside the output kernel).  Norms, routing, counts and outputs must be the bits the stand-alone
+    entry points produce: router -> select -> experts."""
+    _say('small batch layer vs staged', N, D, E, gated, tau)
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=3 * N + E, dtype=torch.bfloat16, gated=gated, bias=not gated)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, W, 1, act, gated=gated)
+    if gated:
+        packed = _ops().pack_weights(sh, d['w_gate'], None, d['w_down'], d['w_up'], d['router_w1'], d['router_w2'])
+    else:
+        packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, d['router_w1'], d['router_w2'])
+    out, routing, norms, counts = _forward(x, p, tau, act, packed=packed, residual=True)
+    xd = x.to(DEV)
+    norms2 = _ops().router(xd, d['router_w1'], d['router_w2'])
+    routing2, counts2 = _ops().select(norms2, float(1.0 - tau), want_counts=True)
+    assert torch.equal(norms, norms2)
+    assert torch.equal(routing, routing2)
+    assert torch.equal(counts, counts2)
+    out2 = _experts_got(x, routing2.cpu(), p, act, residual=True, path='mfma_decode', packed=packed)
+    assert torch.equal(out.cpu(), out2)
+    assert torch.equal(routing.cpu(), O.gate_dynk_max(norms.cpu(), tau))
+
+
 # =================================================================== tiled products (gated, or ungated at other widths) ===
 @pytest.mark.parametrize('N,D,E,Ed,W,act,gated', [(300, 256, 6, 24, 128, 'silu', True), (700, 512, 16, 64, 128, 'relu', True),
                                                   (257, 1024, 5, 128, 128, 'gelu', True), (9000, 256, 4, 32, 128, 'gelu_tanh', True),
