@@ -298,7 +298,8 @@ constexpr int DO_WAVES = 8;
 // most per pass, and walks the routed ones among them in ascending order.
 template <int KS2>
 __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeArgs A) {
-  constexpr int UB = 8 / KS2;                  // experts per load batch (8 fragments of each operand)
+  constexpr int UB = 8 / KS2;                  // experts per load batch (8 hidden fragments, half as many weight loads;
+                                               // twice as many in flight was slower: 18.7 against 16.7 us at 16 tokens)
   __shared__ float part[DO_WAVES][4][64];
   __shared__ float s_thr[16];                  // fused: the tokens' thresholds
   __shared__ unsigned short s_bits[DO_WAVES * 64];   // fused: per expert, bit t = token t routes to it
@@ -347,14 +348,16 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
   // A fragment rows 0..7 only (lanes c16 >= 8 repeat them); result rows 8..15 are dropped
   const bf16x8* wdf = A.wd + (int64_t)cb * E * KS2 * 32 + gq * 8 + (c16 & 7);
   const bf16x8* hf = A.hfrag + lane;
-  bf16x8 aA[UB][KS2], bA[UB][KS2], aB[UB][KS2], bB[UB][KS2];
+  constexpr int KP = (KS2 + 1) / 2;            // weight loads per expert: two K steps each
+  const int khalf = (KS2 > 1) ? (c16 >> 3) : 0;
+  bf16x8 aA[UB][KP], bA[UB][KS2], aB[UB][KP], bB[UB][KS2];
   int esA[UB], esB[UB];
   for (int e0 = e_lo; e0 < e_hi; e0 += 64) {   // 64 experts per pass: one flag per lane
     const bool on = (e0 + lane < e_hi) && (A.fused ? (s_bits[e0 + lane] != 0) : (A.active[e0 + lane] != 0));
     unsigned long long mask = __ballot(on);
     int cntA = 0, cntB = 0;
     // take the next up to UB routed experts off the mask and request their fragments; unused slots repeat the last one
-    auto fill = [&](bf16x8 (&a)[UB][KS2], bf16x8 (&b)[UB][KS2], int (&es)[UB], int& cnt) __attribute__((always_inline)) {
+    auto fill = [&](bf16x8 (&a)[UB][KP], bf16x8 (&b)[UB][KS2], int (&es)[UB], int& cnt) __attribute__((always_inline)) {
       cnt = 0;
       int e = e0;
 #pragma unroll
@@ -368,14 +371,16 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
         for (int k2 = 0; k2 < KS2; ++k2) b[j][k2] = hf[((int64_t)e * KS2 + k2) * 64];
         es[j] = e;
       }
-      // rows 8..15 of the A tile are not needed: their lanes read the same 16 bytes as rows 0..7 (no extra traffic, and
-      // no load under a lane-dependent branch), and the result rows they produce are dropped
+      // Rows 8..15 of the A tile are not needed (the result rows they produce are dropped), so their lanes fetch the
+      // fragment of the NEXT K step instead of repeating rows 0..7: one load brings two K steps, and the second one's
+      // MFMA takes the register rotated by 8 lanes inside every row of 16 (a DPP move).  No load sits under a
+      // lane-dependent branch.  (KS2 == 1: nothing to pair, the upper lanes repeat the lower ones.)
 #pragma unroll
       for (int j = 0; j < UB; ++j)
 #pragma unroll
-        for (int k2 = 0; k2 < KS2; ++k2) a[j][k2] = wdf[((int64_t)es[j] * KS2 + k2) * 32];
+        for (int kp = 0; kp < KP; ++kp) a[j][kp] = wdf[((int64_t)es[j] * KS2 + 2 * kp + khalf) * 32];
     };
-    auto multiply = [&](bf16x8 (&a)[UB][KS2], bf16x8 (&b)[UB][KS2], int (&es)[UB], int cnt) __attribute__((always_inline)) {
+    auto multiply = [&](bf16x8 (&a)[UB][KP], bf16x8 (&b)[UB][KS2], int (&es)[UB], int cnt) __attribute__((always_inline)) {
 #pragma unroll
       for (int j = 0; j < UB; ++j) {
         if (j < cnt) {
@@ -385,7 +390,16 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
           for (int k2 = 0; k2 < KS2; ++k2) {
             u32x4 bm = __builtin_bit_cast(u32x4, b[j][k2]);
             bm.x = keep ? bm.x : 0u; bm.y = keep ? bm.y : 0u; bm.z = keep ? bm.z : 0u; bm.w = keep ? bm.w : 0u;
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][k2], __builtin_bit_cast(bf16x8, bm), acc, 0, 0, 0);
+            bf16x8 av = a[j][k2 / 2];
+            if (KS2 > 1 && (k2 & 1)) {       // the odd K step sits in the upper 8 lanes of every row: rotate it down
+              u32x4 aw = __builtin_bit_cast(u32x4, av);
+              aw.x = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)aw.x, 0x128, 0xf, 0xf, false);
+              aw.y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)aw.y, 0x128, 0xf, 0xf, false);
+              aw.z = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)aw.z, 0x128, 0xf, 0xf, false);
+              aw.w = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)aw.w, 0x128, 0xf, 0xf, false);
+              av = __builtin_bit_cast(bf16x8, aw);
+            }
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, bm), acc, 0, 0, 0);
           }
         }
       }
