@@ -43,7 +43,7 @@ int static_scratch(void** out) {
 
 inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 inline size_t elem_size(int dtype) { return dtype == D2DMOE_F32 ? 4 : 2; }
-inline bool dtype_ok(int dtype) { return dtype == D2DMOE_F32 || dtype == D2DMOE_BF16; }
+inline bool dtype_ok(int dtype) { return dtype == D2DMOE_F32 || dtype == D2DMOE_BF16 || dtype == D2DMOE_F16; }
 inline bool act_ok(int a) { return a >= D2DMOE_ACT_RELU && a <= D2DMOE_ACT_ABS; }
 inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
 
@@ -139,6 +139,14 @@ int d2dmoe_router(const void* x, const void* router_w1, const void* router_w2, v
     if (e == hipSuccess)
       e = m2 ? launch_linear_mfma_f32(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s)
              : launch_linear_act<float>(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s);
+  } else if (dtype == D2DMOE_F16) {
+    const bool m1 = linear_mfma_f16_supported(n_tokens, d_model, router_width) && aligned16(x) && aligned16(router_w1);
+    const bool m2 = linear_mfma_f16_supported(n_tokens, router_width, n_experts) && aligned16(router_w2);
+    e = m1 ? launch_linear_mfma_f16(x, router_w1, workspace, n_tokens, d_model, router_width, activation, s)
+           : launch_linear_act<f16_t>(x, router_w1, workspace, n_tokens, d_model, router_width, activation, s);
+    if (e == hipSuccess)
+      e = m2 ? launch_linear_mfma_f16(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s)
+             : launch_linear_act<f16_t>(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s);
   } else {
     e = launch_linear_act<bf16_t>(x, router_w1, workspace, n_tokens, d_model, router_width, activation, s);
     if (e == hipSuccess) e = launch_linear_act<bf16_t>(workspace, router_w2, norms, n_tokens, router_width, n_experts, output_activation, s);
@@ -156,6 +164,7 @@ int d2dmoe_select(const void* norms, void* routing, int32_t* counts, int64_t n_t
     if (counts) return (int)launch_fill_i32(counts, n_experts, 0, s);
     return D2DMOE_OK;
   }
+  if (dtype == D2DMOE_F16) return (int)launch_select<f16_t>(norms, routing, counts, n_tokens, n_experts, thr_scale, s);
   hipError_t e = (dtype == D2DMOE_F32) ? launch_select<float>(norms, routing, counts, n_tokens, n_experts, thr_scale, s)
                                        : launch_select<bf16_t>(norms, routing, counts, n_tokens, n_experts, thr_scale, s);
   return (int)e;
@@ -177,6 +186,9 @@ int d2dmoe_build_permutation(const void* routing, int64_t n_tokens, int32_t n_ex
   if (!routing) return D2DMOE_E_NULL;
   if (!workspace || workspace_bytes < perm_workspace_bytes(n_tokens, n_experts) || !aligned16(workspace))
     return D2DMOE_E_WORKSPACE;
+  if (dtype == D2DMOE_F16)
+    return (int)launch_build_permutation<f16_t>(routing, n_tokens, n_experts, offsets, token_idx, sort_indices, unsort_indices,
+                                                bincounts, workspace, s);
   hipError_t e = (dtype == D2DMOE_F32)
                      ? launch_build_permutation<float>(routing, n_tokens, n_experts, offsets, token_idx, sort_indices,
                                                        unsort_indices, bincounts, workspace, s)
@@ -232,6 +244,8 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
   switch (path) {
     case D2DMOE_PATH_GENERIC: {
       if (!experts_generic_supported(sh)) return D2DMOE_E_UNSUPPORTED;
+      if (sh.dtype == D2DMOE_F16)
+        return (int)launch_experts_generic<f16_t>(sh, x, routing, w1, b1, w2, w_up, last_bias, out, s);
       hipError_t e = (sh.dtype == D2DMOE_F32)
                          ? launch_experts_generic<float>(sh, x, routing, w1, b1, w2, w_up, last_bias, out, s)
                          : launch_experts_generic<bf16_t>(sh, x, routing, w1, b1, w2, w_up, last_bias, out, s);

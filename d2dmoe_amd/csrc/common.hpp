@@ -42,6 +42,17 @@ template <> struct Elem<bf16_t> {
   __device__ static inline void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
   __device__ static inline float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
 };
+// IEEE half precision (the reference benches float32 and float16, test_moe_implementations.py:223-228): a type of its
+// own, so that it selects its own kernels; conversions round to nearest even, as torch.float16 does
+typedef _Float16 f16_t;
+template <> struct Elem<f16_t> {
+  static constexpr int dtype = D2DMOE_F16;
+  __device__ static inline float load(const f16_t* p) { return (float)*p; }
+  __device__ static inline void store(f16_t* p, float v) { *p = (f16_t)v; }
+  __device__ static inline float round(float v) { return (float)(f16_t)v; }
+};
+// two values rounded to the 16-bit storage type and packed, low half first
+template <typename T> __device__ inline uint32_t pack2_16(float lo, float hi);
 
 // ---------------------------------------------------------------- activations ------------------
 // Definitions follow the reference's kernel-side helpers (utils.py:730-756).

@@ -44,6 +44,7 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 template <typename T> struct GemmElem;
 template <> struct GemmElem<bf16_t> { static constexpr int KPF = 16, EPP = 8; };
 template <> struct GemmElem<float> { static constexpr int KPF = 8, EPP = 4; };
+template <> struct GemmElem<f16_t> { static constexpr int KPF = 16, EPP = 8; };   // v_mfma_f32_32x32x16_f16: bf16's shapes
 
 static inline int gemm_kpf(const d2dmoe_shape& sh) { return sh.dtype == D2DMOE_F32 ? 8 : 16; }
 static inline size_t gemm_esize(const d2dmoe_shape& sh) { return sh.dtype == D2DMOE_F32 ? 4 : 2; }
@@ -69,7 +70,8 @@ static GemmLayout gemm_layout(const d2dmoe_shape& sh) {
 }
 
 bool mfma_gemm_supported(const d2dmoe_shape& sh) {
-  return (sh.dtype == D2DMOE_BF16 || sh.dtype == D2DMOE_F32) && sh.d_model % 256 == 0 && sh.d_model >= 256;
+  return (sh.dtype == D2DMOE_BF16 || sh.dtype == D2DMOE_F32 || sh.dtype == D2DMOE_F16) && sh.d_model % 256 == 0 &&
+         sh.d_model >= 256;
 }
 
 size_t mfma_gemm_packed_bytes(const d2dmoe_shape& sh) { return mfma_gemm_supported(sh) ? gemm_layout(sh).total : 0; }
@@ -179,6 +181,7 @@ static hipError_t launch_gemm_pack_t(const d2dmoe_shape& sh, const void* w1, con
 hipError_t launch_gemm_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                             void* packed_section, hipStream_t s) {
   if (sh.dtype == D2DMOE_F32) return launch_gemm_pack_t<float>(sh, w1, b1, w2, w_up, packed_section, s);
+  if (sh.dtype == D2DMOE_F16) return launch_gemm_pack_t<f16_t>(sh, w1, b1, w2, w_up, packed_section, s);
   return launch_gemm_pack_t<bf16_t>(sh, w1, b1, w2, w_up, packed_section, s);
 }
 
@@ -201,7 +204,13 @@ struct GemmArgs {
 // one fragment pair into a 32 x 32 accumulator tile
 template <typename T>
 __device__ __forceinline__ void frag_mfma(const u32x4& a, const u32x4& b, f32x16& c) {
-  if constexpr (sizeof(T) == 2) {
+  if constexpr (sizeof(T) == 2 && Elem<T>::dtype == D2DMOE_F16) {
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    f16x8 av, bv;
+    __builtin_memcpy(&av, &a, 16);
+    __builtin_memcpy(&bv, &b, 16);
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, c, 0, 0, 0);
+  } else if constexpr (sizeof(T) == 2) {
     bf16x8 av, bv;
     __builtin_memcpy(&av, &a, 16);
     __builtin_memcpy(&bv, &b, 16);
@@ -380,8 +389,8 @@ __global__ __launch_bounds__(256, 1) void gated_gemm_kernel(const GemmArgs<T> A)
 #pragma unroll
           for (int k = 0; k < 2; ++k) {
             u32x4 pk;
-            pk.x = pack2_bf16(hv[8 * k + 0], hv[8 * k + 1]); pk.y = pack2_bf16(hv[8 * k + 2], hv[8 * k + 3]);
-            pk.z = pack2_bf16(hv[8 * k + 4], hv[8 * k + 5]); pk.w = pack2_bf16(hv[8 * k + 6], hv[8 * k + 7]);
+            pk.x = pack2_16<T>(hv[8 * k + 0], hv[8 * k + 1]); pk.y = pack2_16<T>(hv[8 * k + 2], hv[8 * k + 3]);
+            pk.z = pack2_16<T>(hv[8 * k + 4], hv[8 * k + 5]); pk.w = pack2_16<T>(hv[8 * k + 6], hv[8 * k + 7]);
             hdst[k * 64] = pk;
           }
         } else {
@@ -443,8 +452,8 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* __restric
   }
   if constexpr (sizeof(T) == 2) {
     uint4 o;
-    o.x = pack2_bf16(v[0], v[1]); o.y = pack2_bf16(v[2], v[3]);
-    o.z = pack2_bf16(v[4], v[5]); o.w = pack2_bf16(v[6], v[7]);
+    o.x = pack2_16<T>(v[0], v[1]); o.y = pack2_16<T>(v[2], v[3]);
+    o.z = pack2_16<T>(v[4], v[5]); o.w = pack2_16<T>(v[6], v[7]);
     *(uint4*)(out + n * D + col) = o;
   } else {
     *(float4*)(out + n * D + col) = float4{v[0], v[1], v[2], v[3]};
@@ -520,6 +529,10 @@ hipError_t launch_mfma_gemm(const d2dmoe_shape& sh, const void* x, const void* r
   if (sh.dtype == D2DMOE_F32) {
     if (sh.gated) return launch_gemm_gated<float, true>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
     return launch_gemm_gated<float, false>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
+  }
+  if (sh.dtype == D2DMOE_F16) {
+    if (sh.gated) return launch_gemm_gated<f16_t, true>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
+    return launch_gemm_gated<f16_t, false>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
   }
   if (sh.gated) return launch_gemm_gated<bf16_t, true>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);
   return launch_gemm_gated<bf16_t, false>(sh, x, routing, packed_section, last_bias, out, workspace, s, skip_flag);

@@ -73,6 +73,7 @@ hipError_t launch_linear_act(const void* A, const void* B, void* C, int64_t M, i
 }
 template hipError_t launch_linear_act<float>(const void*, const void*, void*, int64_t, int, int, int, hipStream_t);
 template hipError_t launch_linear_act<bf16_t>(const void*, const void*, void*, int64_t, int, int, int, hipStream_t);
+template hipError_t launch_linear_act<f16_t>(const void*, const void*, void*, int64_t, int, int, int, hipStream_t);
 
 // The same layer in float32 on the matrix cores (v_mfma_f32_32x32x2_f32: float32 operands, products and sums), for
 // K a multiple of 32 and Nout a multiple of 32.  Workgroup = 32 rows x 128 columns, one 32 x 32 tile per wave, no LDS:
@@ -136,6 +137,63 @@ hipError_t launch_linear_mfma_f32(const void* A, const void* B, void* C, int64_t
   return hipGetLastError();
 }
 
+// The same layer for float16 storage on the matrix cores (v_mfma_f32_32x32x16_f16: float32 sums), for K a multiple of
+// 64 and Nout a multiple of 32; the arrangement of the float32 kernel above with 8 K values per lane and step of 16.
+// The output is rounded to float16, then the activation is applied and rounded again, as the scalar kernel does.
+typedef _Float16 f16x8_g __attribute__((ext_vector_type(8)));
+
+__global__ __launch_bounds__(256) void linear_act_mfma_f16_kernel(const f16_t* __restrict__ A, const f16_t* __restrict__ B,
+                                                                  f16_t* __restrict__ C, int64_t M, int K, int Nout, int act) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int c32 = lane & 31, kh = lane >> 5;
+  const int64_t row0 = (int64_t)blockIdx.x * 32;
+  const int col0 = (blockIdx.y * 4 + w) * 32;
+  if (col0 >= Nout) return;   // whole waves leave; the kernel has no barrier
+  int64_t ar = row0 + c32;
+  ar = ar < M ? ar : (M - 1);   // rows beyond M repeat the last row and are not stored
+  const f16x8_g* ap = (const f16x8_g*)(A + ar * K) + kh;
+  const f16x8_g* bp = (const f16x8_g*)(B + (int64_t)(col0 + c32) * K) + kh;
+  f32x16_g acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  f16x8_g a0[4], b0[4], a1[4], b1[4];   // two buffers of 64 K values
+  auto fill = [&](f16x8_g (&a)[4], f16x8_g (&b)[4], int k0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      a[u] = ap[(k0 >> 3) + 2 * u];
+      b[u] = bp[(k0 >> 3) + 2 * u];
+    }
+  };
+  auto multiply = [&](const f16x8_g (&a)[4], const f16x8_g (&b)[4]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[u], b[u], acc, 0, 0, 0);
+  };
+  const int k_last = K - 64;
+  fill(a0, b0, 0);
+  for (int k0 = 0; k0 < K; k0 += 128) {
+    fill(a1, b1, (k0 + 64 < K) ? (k0 + 64) : k_last);   // past the end: an in-bounds re-read that is not multiplied
+    multiply(a0, b0);
+    if (k0 + 64 < K) {
+      fill(a0, b0, (k0 + 128 < K) ? (k0 + 128) : k_last);
+      multiply(a1, b1);
+    }
+  }
+  // lane = column c32; accumulator r = row 8*(r/4) + 4*kh + r%4
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int64_t row = row0 + 8 * (r / 4) + 4 * kh + (r % 4);
+    if (row < M) Elem<f16_t>::store(C + row * Nout + col0 + c32, apply_act(act, Elem<f16_t>::round(acc[r])));
+  }
+}
+
+bool linear_mfma_f16_supported(int64_t M, int K, int Nout) { return M > 0 && K >= 64 && K % 64 == 0 && Nout % 32 == 0; }
+
+hipError_t launch_linear_mfma_f16(const void* A, const void* B, void* C, int64_t M, int K, int Nout, int act, hipStream_t s) {
+  dim3 grid((unsigned)cdiv64(M, 32), (unsigned)((Nout + 127) / 128));
+  hipLaunchKernelGGL(linear_act_mfma_f16_kernel, grid, dim3(256), 0, s, (const f16_t*)A, (const f16_t*)B, (f16_t*)C, M, K, Nout, act);
+  return hipGetLastError();
+}
+
 // =====================================================================================================
 // small fill kernel (used instead of a memset node so the path stays graph-capture friendly)
 // =====================================================================================================
@@ -182,7 +240,12 @@ __global__ __launch_bounds__(256) void select_kernel(const T* __restrict__ norms
       }
     }
     m = wave_nanmax(m);
-    const float thr = Elem<T>::round(m * thr_scale);
+    // the product is rounded to float32 first, then to T, as the reference's tensor expression does on a GPU; without the
+    // empty asm the compiler folds multiply and conversion to float16 into one mixed-precision instruction with a
+    // single rounding, which differs when the float32 product is an exact tie of the float16 grid
+    float prod = m * thr_scale;
+    asm volatile("" : "+v"(prod));
+    const float thr = Elem<T>::round(prod);
 #pragma unroll
     for (int k = 0; k < SEL_MAX_VPT; ++k) {
       if (k < vpt) {
@@ -221,6 +284,7 @@ hipError_t launch_select(const void* norms, void* routing, int32_t* counts, int6
 }
 template hipError_t launch_select<float>(const void*, void*, int32_t*, int64_t, int, float, hipStream_t);
 template hipError_t launch_select<bf16_t>(const void*, void*, int32_t*, int64_t, int, float, hipStream_t);
+template hipError_t launch_select<f16_t>(const void*, void*, int32_t*, int64_t, int, float, hipStream_t);
 
 // =====================================================================================================
 // Token -> expert permutation (moe_layers.py:213-224, 241-249), canonical stable order.
@@ -438,6 +502,8 @@ template hipError_t launch_build_permutation<float>(const void*, int64_t, int, i
                                                     int64_t*, void*, hipStream_t);
 template hipError_t launch_build_permutation<bf16_t>(const void*, int64_t, int, int32_t*, int32_t*, int64_t*, int64_t*,
                                                      int64_t*, void*, hipStream_t);
+template hipError_t launch_build_permutation<f16_t>(const void*, int64_t, int, int32_t*, int32_t*, int64_t*, int64_t*,
+                                                     int64_t*, void*, hipStream_t);
 
 // =====================================================================================================
 // Experts, generic token-tile-major kernel.
@@ -575,6 +641,8 @@ hipError_t launch_experts_generic(const d2dmoe_shape& sh, const void* x, const v
 template hipError_t launch_experts_generic<float>(const d2dmoe_shape&, const void*, const void*, const void*, const void*,
                                                   const void*, const void*, const void*, void*, hipStream_t);
 template hipError_t launch_experts_generic<bf16_t>(const d2dmoe_shape&, const void*, const void*, const void*, const void*,
+                                                   const void*, const void*, const void*, void*, hipStream_t);
+template hipError_t launch_experts_generic<f16_t>(const d2dmoe_shape&, const void*, const void*, const void*, const void*,
                                                    const void*, const void*, const void*, void*, hipStream_t);
 
 }  // namespace d2dmoe

@@ -14,6 +14,9 @@ template <typename T>
 hipError_t launch_linear_act(const void* A, const void* B, void* C, int64_t M, int K, int Nout, int act, hipStream_t s);
 bool linear_mfma_f32_supported(int64_t M, int K, int Nout);
 hipError_t launch_linear_mfma_f32(const void* A, const void* B, void* C, int64_t M, int K, int Nout, int act, hipStream_t s);
+// float16 storage on the matrix cores: K a multiple of 64, Nout a multiple of 32
+bool linear_mfma_f16_supported(int64_t M, int K, int Nout);
+hipError_t launch_linear_mfma_f16(const void* A, const void* B, void* C, int64_t M, int K, int Nout, int act, hipStream_t s);
 
 hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s);
 

@@ -69,6 +69,15 @@ __device__ inline uint32_t pack2_bf16(float lo, float hi) {
   return u;
 }
 
+template <> __device__ inline uint32_t pack2_16<bf16_t>(float lo, float hi) { return pack2_bf16(lo, hi); }
+template <> __device__ inline uint32_t pack2_16<f16_t>(float lo, float hi) {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  const f16x2 h = {(_Float16)lo, (_Float16)hi};   // round-to-nearest-even each
+  uint32_t u;
+  __builtin_memcpy(&u, &h, 4);
+  return u;
+}
+
 // LDS-only workgroup barrier: waits for this wave's LDS operations, not for its outstanding global loads.
 __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 

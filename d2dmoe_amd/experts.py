@@ -109,7 +109,7 @@ class _HipContainer(ExpertsLayer):
 
     def packed_weights(self, router_w1=None, router_w2=None, router_activation='relu', router_output_activation='abs'):
         w1, b1, w2, w_up, act = self.hip_operands()
-        if not w1.is_cuda or w1.dtype not in (torch.bfloat16, torch.float32):
+        if not w1.is_cuda or w1.dtype not in (torch.bfloat16, torch.float32, torch.float16):
             return None
         sh = ops.make_shape(0, w1.size(1), w1.size(0), w1.size(2), router_w1.size(0) if router_w1 is not None else 0,
                             ops._dtype_code(w1), act, gated=w_up is not None, router_activation=router_activation,
@@ -190,7 +190,7 @@ class HipKernelExperts(_HipContainer):
         assert x.dim() == 2, f'{x.size()=}'
         if x.is_cuda and not (torch.is_grad_enabled() and (x.requires_grad or self.w1.requires_grad)):
             sh = ops.make_shape(0, self.hidden_dim, self.num_experts, self.expert_dim, 0, ops._dtype_code(x),
-                                self.activation_str) if x.dtype in (torch.bfloat16, torch.float32) else None
+                                self.activation_str) if x.dtype in (torch.bfloat16, torch.float32, torch.float16) else None
             if sh is not None and x.dtype == self.w1.dtype:
                 key = tuple((t.data_ptr(), t._version, t.dtype, t.device) for t in (self.w1, self.b1, self.w2))
                 if self._norms_packed is None or self._norms_packed[0] != key:

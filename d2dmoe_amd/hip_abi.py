@@ -14,7 +14,7 @@ LIB_NAME = 'libd2dmoe_hip.so'
 LIB_PATH = os.environ.get('D2DMOE_LIB') or os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 # enums of include/d2dmoe.h
-F32, BF16 = 0, 1
+F32, BF16, F16 = 0, 1, 2
 E_STATIC_LIMIT = -8
 STATIC_WORKSPACE_BYTES = 256 << 20
 ACT = {'relu': 0, 'gelu': 1, 'tanh': 2, 'leaky_relu': 3, 'gelu_tanh': 4, 'silu': 5, 'identity': 6, 'abs': 7}

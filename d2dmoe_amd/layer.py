@@ -94,7 +94,7 @@ class MoeficationRouter(nn.Module):
 
     def forward(self, x):
         if (x.is_cuda and not torch.is_grad_enabled() and self.hip_compatible()
-                and x.dtype in (torch.float32, torch.bfloat16)):
+                and x.dtype in (torch.float32, torch.bfloat16, torch.float16)):
             lead = x.shape[:-1]
             x = ops.router(x.reshape(-1, x.size(-1)).contiguous(), self.layers[0].weight, self.layers[2].weight,
                            self.activation, self.output_activation).view(*lead, -1)
@@ -161,7 +161,7 @@ class MoeficationMoE(MoELayer):
             return keep.gather(dim=-1, index=order.argsort(dim=-1)).to(x.dtype)
         if mode == 'dynk_max':
             norms = self.router(x)
-            if norms.is_cuda and norms.dtype in (torch.float32, torch.bfloat16):
+            if norms.is_cuda and norms.dtype in (torch.float32, torch.bfloat16, torch.float16):
                 routing, _ = ops.select(norms.reshape(-1, norms.size(-1)).contiguous(), float(1.0 - self.tau))
                 return routing.view(norms.shape)
             max_norms, _ = norms.max(dim=-1, keepdim=True)
@@ -177,7 +177,7 @@ class MoeficationMoE(MoELayer):
         call would be taken under autograd with a tensor that asks for a gradient: the kernels have no backward
         (the reference's wrappers raise there too, moe_impls.py:60-64), and an output silently cut off from the graph
         would leave the parameters without gradients."""
-        if self.forward_mode != 'dynk_max' or not x.is_cuda or x.dtype not in (torch.float32, torch.bfloat16):
+        if self.forward_mode != 'dynk_max' or not x.is_cuda or x.dtype not in (torch.float32, torch.bfloat16, torch.float16):
             return False
         ex = self.experts
         if not isinstance(ex, _HipContainer) or ex.forward_mode not in ex.HIP_MODES:

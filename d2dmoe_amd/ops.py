@@ -12,7 +12,7 @@ import torch
 
 from . import hip_abi as abi
 
-_DTYPES = {torch.float32: abi.F32, torch.bfloat16: abi.BF16}
+_DTYPES = {torch.float32: abi.F32, torch.bfloat16: abi.BF16, torch.float16: abi.F16}
 _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
@@ -20,7 +20,7 @@ def _dtype_code(t: torch.Tensor) -> int:
     try:
         return _DTYPES[t.dtype]
     except KeyError:
-        raise abi.D2DMoEError(f'unsupported dtype {t.dtype}: the HIP path handles float32 and bfloat16') from None
+        raise abi.D2DMoEError(f'unsupported dtype {t.dtype}: the HIP path handles float32, bfloat16 and float16') from None
 
 
 def _require_same_dtype(what: str, ref: torch.Tensor, **tensors: Optional[torch.Tensor]) -> None:
@@ -259,7 +259,7 @@ class PreparedForward:
         self.dtype = dtype
         self.code = _DTYPES.get(dtype)
         if self.code is None:
-            raise abi.D2DMoEError(f'unsupported dtype {dtype}: the HIP path handles float32 and bfloat16')
+            raise abi.D2DMoEError(f'unsupported dtype {dtype}: the HIP path handles float32, bfloat16 and float16')
         self.dev = _require_gpu(*self.tensors)
         self.lib = abi.load()
         self.d = d_model

@@ -50,7 +50,7 @@ enum {
 };
 
 /* element types */
-enum { D2DMOE_F32 = 0, D2DMOE_BF16 = 1 };
+enum { D2DMOE_F32 = 0, D2DMOE_BF16 = 1, D2DMOE_F16 = 2 };   /* F16: the generic kernels and the tiled MFMA products */
 
 /* activations.  Reference: utils.py:730-756 (kernel-side definitions), common.py:159-169 (names). */
 enum {
@@ -98,7 +98,7 @@ typedef struct d2dmoe_shape {
   int32_t n_experts;    /* E */
   int32_t expert_dim;   /* Ed, neurons per expert */
   int32_t router_width; /* W */
-  int32_t dtype;        /* D2DMOE_F32 | D2DMOE_BF16 (activations, weights, routing all share it) */
+  int32_t dtype;        /* D2DMOE_F32 | D2DMOE_BF16 | D2DMOE_F16 (activations, weights, routing all share it) */
   int32_t activation;   /* expert activation, D2DMOE_ACT_* */
   int32_t gated;        /* 0: out = act(x w1 + b1) w2 ; 1: out = (act(x w1) * (x w_up)) w2 */
   int32_t add_residual; /* 1: out += x  (moefication.py:98-99) */

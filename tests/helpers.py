@@ -13,6 +13,7 @@ GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden')
 # the oracle on the same stored inputs.
 TOL_F32 = 1e-5
 TOL_BF16 = 2e-2
+TOL_F16 = 4e-3     # float16 keeps 11 significant bits where bfloat16 keeps 8
 
 
 class GELUTanh(torch.nn.GELU):
@@ -33,7 +34,7 @@ def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
 
 
 def tol_for(dtype) -> float:
-    return TOL_F32 if dtype == torch.float32 else TOL_BF16
+    return {torch.float32: TOL_F32, torch.bfloat16: TOL_BF16, torch.float16: TOL_F16}[dtype]
 
 
 def load_fixture(name):

@@ -108,7 +108,7 @@ def test_gated_module_reaches_the_product_kernels(N, tau):
 
 
 # =================================================================== every container in its 'hip' mode =================
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('experts_class,gated', [('custom_kernel', False), ('execute_all', False), ('execute_all', True),
                                                  ('module', False), ('module', True), ('batched', False)])
 def test_every_container_runs_the_hip_kernels(experts_class, gated, dtype):
