@@ -46,6 +46,8 @@ WORKLOADS = {
     'vit_b_skew': (256, 197, 768, 128, 24, 128, 'relu'),
     # the CPU baseline's own case (8 x 197 tokens, float32) on the GPU: float32 storage and float32 matrix arithmetic
     'vit_b_1576_f32': (8, 197, 768, 128, 24, 128, 'relu'),
+    # float16 storage (the reference benches float32 and float16): router on an MFMA linear kernel, experts on the tiled products
+    'vit_b_50k_f16': (256, 197, 768, 128, 24, 128, 'relu'),
 }
 TRAFFIC_TABLE = os.path.join(ROOT, 'profiles', 'traffic_per_launch.md')
 
@@ -630,7 +632,8 @@ def main():
     B, T, D, E, Ed, W, act = WORKLOADS[args.workload]
     N = B * T
     f32 = args.workload.endswith('_f32')
-    dtype = torch.float32 if f32 else torch.bfloat16
+    f16 = args.workload.endswith('_f16')
+    dtype = torch.float32 if f32 else (torch.float16 if f16 else torch.bfloat16)
     peak = PEAK_F32_TFLOPS if f32 else PEAK_BF16_TFLOPS
     p = make_params(D, E, Ed, W, seed=0, dtype=dtype, device=dev)
     x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
@@ -659,7 +662,7 @@ def main():
         'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
         'value': main_r['tokens_per_s'], 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': main_r['ms_layer'], 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
-        'dtype': 'f32' if f32 else 'bf16', 'data': 'synthetic',
+        'dtype': 'f32' if f32 else ('f16' if f16 else 'bf16'), 'data': 'synthetic',
         'config': {'workload': f'{args.workload}: {B}x{T}={N} tokens, D={D}, {E} experts x {Ed}, {act}, router {D}->{W}->{E}, '
                                f'module tau={args.tau} (keep norm >= {1 - args.tau:.2f}*max), whole layer',
                    'mean_active_experts': main_r['mean_active'], 'p99_active_experts': main_r['p99_active'],
