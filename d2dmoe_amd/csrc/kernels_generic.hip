@@ -452,6 +452,24 @@ __global__ __launch_bounds__(256) void perm_scatter_kernel(const T* __restrict__
       for (int i = 0; i < PERM_SEG; ++i) onbits[k] |= (unsigned long long)(v[i] > 0.f ? 1 : 0) << i;
     }
   }
+  if (sort_indices == nullptr && unsort_indices == nullptr) {
+    // only the per-expert token lists are wanted: a lane walks the set bits of its experts' masks (the routed tokens, in
+    // ascending order) instead of all the segment's tokens
+#pragma unroll
+    for (int k = 0; k < PERM_MAX_VPT; ++k) {
+      if (k < vpt) {
+        // (rows past the end of the batch and lanes past the last expert hold copies of clamped loads: masked here)
+        const unsigned long long live = (rows >= 64) ? ~0ull : ((1ull << rows) - 1ull);
+        unsigned long long bits = (lane + k * kWave < E) ? (onbits[k] & live) : 0ull;
+        int64_t pos = (int64_t)base[k] + run[k];
+        while (bits != 0ull) {
+          token_idx[pos++] = (int32_t)(t0 + __builtin_ctzll(bits));
+          bits &= bits - 1ull;
+        }
+      }
+    }
+    return;
+  }
   for (int i = 0; i < rows; ++i) {
     const int64_t tok = t0 + i;
 #pragma unroll
