@@ -27,7 +27,7 @@ static size_t dense_lds_bytes(const d2dmoe_shape& sh) {
 
 // The fused experts kernel is instantiated for D = 768 (ViT-B, GPT-2 small, BERT-base), ungated experts, bf16.
 bool mfma_dense_supported(const d2dmoe_shape& sh) {
-  if (sh.dtype != D2DMOE_BF16 || sh.gated) return false;
+  if ((sh.dtype != D2DMOE_BF16 && sh.dtype != D2DMOE_F16) || sh.gated) return false;
   if (sh.d_model != 768) return false;
   if (sh.n_experts > 256) return false;          // expert indices are staged as uint8
   if (sh.expert_dim > MD_HC) return false;       // an expert spans at most two chunks
@@ -236,6 +236,29 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
 // on LDS traffic only, so the global loads in flight survive them; GEMM2 of one chunk and GEMM1 of the next run
 // back to back between barriers.
 // ---------------------------------------------------------------------------------------------------
+// 16-bit storage of the sweep: bf16 (F16 = false) or IEEE half (F16 = true).  Both keep the same fragment layouts; what
+// differs is the MFMA instruction, the decoding of stored values and the final rounding.
+template <bool F16> __device__ __forceinline__ float dec16(uint32_t bits16) {       // low 16 bits -> float
+  if constexpr (F16) { _Float16 h; const uint16_t u = (uint16_t)bits16; __builtin_memcpy(&h, &u, 2); return (float)h; }
+  else return __uint_as_float(bits16 << 16);
+}
+template <bool F16> __device__ __forceinline__ float dec16_hi(uint32_t word) {      // high 16 bits -> float
+  if constexpr (F16) return dec16<true>(word >> 16);
+  else return __uint_as_float(word & 0xffff0000u);
+}
+template <bool F16> __device__ __forceinline__ uint32_t enc16x2(float lo, float hi) {
+  if constexpr (F16) return pack2_16<f16_t>(lo, hi);
+  else return pack2_bf16(lo, hi);
+}
+template <bool F16> __device__ __forceinline__ f32x16 mfma_32x32x16(const bf16x8& a, const bf16x8& b, const f32x16& c) {
+  if constexpr (F16) {
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+}
+
 struct DenseArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* wp; const bf16_t* b1p; const uint8_t* eidx;
   const bf16_t* last_bias; bf16_t* out;
@@ -247,7 +270,7 @@ struct DenseArgs {
 
 // SPLIT: the workgroup handles only chunks [c_begin, c_end) of its tile and leaves its float32 sums, without bias or
 // residual, in A.partial[split]; a finishing kernel adds the splits in ascending order.
-template <int D, int ACT, bool ED8, int TT, bool SPLIT = false>
+template <int D, int ACT, bool ED8, int TT, bool SPLIT = false, bool F16 = false>
 __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw,
                                            const int c_begin = 0, const int c_end = 1 << 30, const int split = 0) {
   constexpr int KS1 = D / 16;          // K steps of GEMM1
@@ -450,17 +473,17 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             if (ED8) {
-              e_rq[tt][q] = bf16_to_f32(rrow[e_idx[q]]);
+              e_rq[tt][q] = dec16<F16>(rrow[e_idx[q]]);
             } else {
 #pragma unroll
-              for (int i = 0; i < 4; ++i) e_rq[tt][q * 4 + i] = bf16_to_f32(rrow[(e_idx[q] >> (8 * i)) & 0xff]);
+              for (int i = 0; i < 4; ++i) e_rq[tt][q * 4 + i] = dec16<F16>(rrow[(e_idx[q] >> (8 * i)) & 0xff]);
             }
           }
         }
       };
       auto epi_math = [&](int rt, int q) __attribute__((always_inline)) {
-        const float b0 = __uint_as_float(e_bias[q].x << 16), b1 = __uint_as_float(e_bias[q].x & 0xffff0000u);
-        const float b2 = __uint_as_float(e_bias[q].y << 16), b3 = __uint_as_float(e_bias[q].y & 0xffff0000u);
+        const float b0 = dec16<F16>(e_bias[q].x & 0xffffu), b1 = dec16_hi<F16>(e_bias[q].x);
+        const float b2 = dec16<F16>(e_bias[q].y & 0xffffu), b3 = dec16_hi<F16>(e_bias[q].y);
         const float bias[4] = {b0, b1, b2, b3};
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
@@ -479,10 +502,10 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             uint4 pk;
-            pk.x = pack2_bf16(e_hv[tt][half * 8 + 0], e_hv[tt][half * 8 + 1]);
-            pk.y = pack2_bf16(e_hv[tt][half * 8 + 2], e_hv[tt][half * 8 + 3]);
-            pk.z = pack2_bf16(e_hv[tt][half * 8 + 4], e_hv[tt][half * 8 + 5]);
-            pk.w = pack2_bf16(e_hv[tt][half * 8 + 6], e_hv[tt][half * 8 + 7]);
+            pk.x = enc16x2<F16>(e_hv[tt][half * 8 + 0], e_hv[tt][half * 8 + 1]);
+            pk.y = enc16x2<F16>(e_hv[tt][half * 8 + 2], e_hv[tt][half * 8 + 3]);
+            pk.z = enc16x2<F16>(e_hv[tt][half * 8 + 4], e_hv[tt][half * 8 + 5]);
+            pk.w = enc16x2<F16>(e_hv[tt][half * 8 + 6], e_hv[tt][half * 8 + 7]);
             const int ks2 = (w * 2 + rt) * 2 + half;
             ((uint4*)hs)[(tt * MD_KS2 + ks2) * 64 + lane] = pk;
           }
@@ -511,8 +534,8 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
           for (int tt = 0; tt < TT; ++tt) nxb[tt] = xs[(tt * KS1 + kn) * 64 + lane];
 #pragma unroll
           for (int tt = 0; tt < TT; ++tt) {
-            acc1[0][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, xb[tt], acc1[0][tt], 0, 0, 0);
-            acc1[1][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, xb[tt], acc1[1][tt], 0, 0, 0);
+            acc1[0][tt] = mfma_32x32x16<F16>(a0, xb[tt], acc1[0][tt]);
+            acc1[1][tt] = mfma_32x32x16<F16>(a1, xb[tt], acc1[1][tt]);
           }
 #pragma unroll
           for (int tt = 0; tt < TT; ++tt) xb[tt] = nxb[tt];
@@ -537,7 +560,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
             ring[s % R] = (s + R < NW2) ? cur[(NW1 + s + R) * 64] : nxt[(s + R - NW2) * 64];
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt)
-              acc2[tt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ha[tt], b, acc2[tt][ct], 0, 0, 0);
+              acc2[tt][ct] = mfma_32x32x16<F16>(ha[tt], b, acc2[tt][ct]);
           });
 #pragma unroll
           for (int tt = 0; tt < TT; ++tt) ha[tt] = nha[tt];
@@ -578,7 +601,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     float lb[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
-      lb[ct] = with_bias ? bf16_to_f32(A.last_bias[w * (D / 4) + ct * 32 + c32]) : 0.f;
+      lb[ct] = with_bias ? dec16<F16>(A.last_bias[w * (D / 4) + ct * 32 + c32]) : 0.f;
     const int row = w * 8 + r8;                     // row of the pass this thread finishes
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
@@ -611,10 +634,10 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
           if (with_res) {
             const uint32_t xw[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] += __uint_as_float((i & 1) ? (xw[i >> 1] & 0xffff0000u) : (xw[i >> 1] << 16));
+            for (int i = 0; i < 8; ++i) v[i] += (i & 1) ? dec16_hi<F16>(xw[i >> 1]) : dec16<F16>(xw[i >> 1] & 0xffffu);
           }
-          o[k].x = pack2_bf16(v[0], v[1]); o[k].y = pack2_bf16(v[2], v[3]);
-          o[k].z = pack2_bf16(v[4], v[5]); o[k].w = pack2_bf16(v[6], v[7]);
+          o[k].x = enc16x2<F16>(v[0], v[1]); o[k].y = enc16x2<F16>(v[2], v[3]);
+          o[k].z = enc16x2<F16>(v[4], v[5]); o[k].w = enc16x2<F16>(v[6], v[7]);
         }
       }
       if (live) {
@@ -636,23 +659,23 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
 }
 
 // Out-of-line copy of the tile routine for the variant below (keeps its register allocation apart from the loop).
-template <int D, int ACT, bool ED8, int TT>
+template <int D, int ACT, bool ED8, int TT, bool F16>
 __device__ __attribute__((noinline)) void dense_tile_call(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw) {
-  dense_tile<D, ACT, ED8, TT>(A, tok0, smem_raw);
+  dense_tile<D, ACT, ED8, TT, false, F16>(A, tok0, smem_raw);
 }
 
 // The same sweep launched as one workgroup per CU that walks the tiles in launch order.  Used where the launch is
 // usually a no-op (the fall-back behind the expert-major path): a skipped call then retires after one round of empty
 // workgroups instead of one per tile.
-template <int D, int ACT, bool ED8>
+template <int D, int ACT, bool ED8, bool F16 = false>
 __global__ __launch_bounds__(256, 1) void experts_mfma_dense_walk_kernel(const DenseArgs A) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
   for (int b = blockIdx.x; b < A.n_tiles; b += gridDim.x) {
     if (b < A.n_full)
-      dense_tile_call<D, ACT, ED8, 2>(A, (int64_t)b * 64, smem_raw);
+      dense_tile_call<D, ACT, ED8, 2, F16>(A, (int64_t)b * 64, smem_raw);
     else
-      dense_tile_call<D, ACT, ED8, 1>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
+      dense_tile_call<D, ACT, ED8, 1, F16>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
     __syncthreads();   // the next tile's staging overwrites the LDS the final epilogue just read
   }
 }
@@ -660,20 +683,20 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_dense_walk_kernel(const D
 // Workgroups [0, n_full) take tiles of 64 tokens.  The tokens left over after the last full round of the machine go to
 // tiles of 32; if those would still leave most CUs idle, each of them is dealt to csplit workgroups by chunk ranges,
 // which leave float32 sums in A.partial for the finishing kernel.
-template <int D, int ACT, bool ED8>
+template <int D, int ACT, bool ED8, bool F16 = false>
 __global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
   const int b = blockIdx.x;
   if (b < A.n_full) {
-    dense_tile<D, ACT, ED8, 2>(A, (int64_t)b * 64, smem_raw);
+    dense_tile<D, ACT, ED8, 2, false, F16>(A, (int64_t)b * 64, smem_raw);
   } else if (A.csplit <= 1) {
-    dense_tile<D, ACT, ED8, 1>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
+    dense_tile<D, ACT, ED8, 1, false, F16>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
   } else {
     const int idx = b - A.n_full;
     const int tile = idx / A.csplit, split = idx % A.csplit;
     const int c_begin = split * A.chunks_per_split;
-    dense_tile<D, ACT, ED8, 1, true>(A, (int64_t)A.n_full * 64 + (int64_t)tile * 32, smem_raw, c_begin,
+    dense_tile<D, ACT, ED8, 1, true, F16>(A, (int64_t)A.n_full * 64 + (int64_t)tile * 32, smem_raw, c_begin,
                                      c_begin + A.chunks_per_split, split);
   }
 }
@@ -730,7 +753,7 @@ size_t mfma_dense_workspace_bytes(const d2dmoe_shape& sh) {
   return T.csplit > 1 ? (size_t)T.csplit * T.part_rows * sh.d_model * 4 : 0;
 }
 
-template <int D, int ACT, bool ED8>
+template <int D, int ACT, bool ED8, bool F16>
 static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                                    const void* last_bias, void* out, const int* skip_flag, void* workspace,
                                    size_t workspace_bytes, hipStream_t s) {
@@ -741,7 +764,7 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   const int cus = device_cu_count();
   const bool allow_split = skip_flag == nullptr && workspace != nullptr && workspace_bytes >= mfma_dense_workspace_bytes(sh);
   const DenseTiling T = dense_tiling(sh, allow_split);
-  auto kern = (skip_flag != nullptr) ? experts_mfma_dense_walk_kernel<D, ACT, ED8> : experts_mfma_dense_kernel<D, ACT, ED8>;
+  auto kern = (skip_flag != nullptr) ? experts_mfma_dense_walk_kernel<D, ACT, ED8, F16> : experts_mfma_dense_kernel<D, ACT, ED8, F16>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   DenseArgs A;
@@ -758,16 +781,22 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   e = hipGetLastError();
   if (e != hipSuccess || T.csplit <= 1) return e;
   return launch_sum_partials(A.partial, last_bias, (const bf16_t*)x + T.part_base * sh.d_model,
-                             (bf16_t*)out + T.part_base * sh.d_model, T.part_rows, sh.d_model, T.csplit, sh.add_residual, s);
+                             (bf16_t*)out + T.part_base * sh.d_model, T.part_rows, sh.d_model, T.csplit, sh.add_residual, s,
+                             sh.dtype);
 }
 
 template <int D, int ACT>
 static hipError_t launch_dense_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                                    const void* last_bias, void* out, const int* skip_flag, void* workspace,
                                    size_t workspace_bytes, hipStream_t s) {
+  if (sh.dtype == D2DMOE_F16) {
+    if (sh.expert_dim % 8 == 0)
+      return launch_dense_cfg<D, ACT, true, true>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+    return launch_dense_cfg<D, ACT, false, true>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+  }
   if (sh.expert_dim % 8 == 0)
-    return launch_dense_cfg<D, ACT, true>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
-  return launch_dense_cfg<D, ACT, false>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+    return launch_dense_cfg<D, ACT, true, false>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+  return launch_dense_cfg<D, ACT, false, false>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
 }
 
 hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,

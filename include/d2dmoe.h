@@ -50,7 +50,7 @@ enum {
 };
 
 /* element types */
-enum { D2DMOE_F32 = 0, D2DMOE_BF16 = 1, D2DMOE_F16 = 2 };   /* F16: the generic kernels and the tiled MFMA products */
+enum { D2DMOE_F32 = 0, D2DMOE_BF16 = 1, D2DMOE_F16 = 2 };   /* F16: generic kernels, the fused sweep, the tiled MFMA products */
 
 /* activations.  Reference: utils.py:730-756 (kernel-side definitions), common.py:159-169 (names). */
 enum {

@@ -117,7 +117,8 @@ def test_tiled_products_f16(N, D, E, Ed, W, gated, act, density):
     got = _got(x, routing, p, act, path='mfma_gemm', packed=packed)
     assert H.rel_err(got, _want(x, routing, p, act)) < TOL_F16
     assert H.rel_err(got, _got(x, routing, p, act, path='generic')) < TOL_F16
-    assert torch.equal(got, _got(x, routing, p, act, path='auto', packed=packed))        # AUTO takes the MFMA path
+    if gated or D != 768:
+        assert torch.equal(got, _got(x, routing, p, act, path='auto', packed=packed))    # AUTO takes the tiled products
     assert torch.equal(got, _got(x, routing, p, act, path='mfma_gemm', packed=packed))   # run to run
     g = torch.Generator().manual_seed(3)
     weights = (routing.float() * (torch.rand(N, E, generator=g) + 0.5)).half()
@@ -126,6 +127,30 @@ def test_tiled_products_f16(N, D, E, Ed, W, gated, act, density):
     zero = _got(x, torch.zeros_like(routing), p, act, path='mfma_gemm', packed=packed)
     lbias = p['last_bias'].expand(N, -1).float() if 'last_bias' in p else torch.zeros(N, D)
     assert torch.equal(zero.float(), lbias)
+
+
+@pytest.mark.parametrize('N,E,Ed,density,act', [(197, 128, 24, 0.8, 'relu'), (1576, 128, 24, 0.79, 'gelu'), (65, 128, 24, 0.05, 'relu'),
+                                                (1, 128, 24, 0.5, 'relu'), (300, 24, 128, 0.5, 'relu'), (700, 100, 30, 0.3, 'tanh'),
+                                                (9000, 128, 24, 0.6, 'relu')])
+def test_dense_sweep_f16(N, E, Ed, density, act):
+    """The fused sweep (D = 768) with v_mfma_f32_32x32x16_f16: against the float64 oracle, against the tiled products,
+    weighted routing + residual, zero routing, run-to-run bit equality; AUTO takes it."""
+    _say('f16 dense sweep', N, E, Ed, density, act)
+    D, W = 768, 128
+    x, routing, p = H.random_case(N, D, E, Ed, W, seed=N + E, dtype=F16, density=density)
+    packed = _pack(p, D, E, Ed, W, act, False)
+    got = _got(x, routing, p, act, path='mfma_dense', packed=packed)
+    assert H.rel_err(got, _want(x, routing, p, act)) < TOL_F16
+    assert H.rel_err(got, _got(x, routing, p, act, path='mfma_gemm', packed=packed)) < TOL_F16
+    assert torch.equal(got, _got(x, routing, p, act, path='mfma_dense', packed=packed))
+    if N > 16:
+        assert torch.equal(got, _got(x, routing, p, act, path='auto', packed=packed))
+    g = torch.Generator().manual_seed(3)
+    weights = (routing.float() * (torch.rand(N, E, generator=g) + 0.5)).half()
+    got = _got(x, weights, p, act, residual=True, path='mfma_dense', packed=packed)
+    assert H.rel_err(got, _want(x, weights, p, act, True)) < TOL_F16
+    zero = _got(x, torch.zeros_like(routing), p, act, path='mfma_dense', packed=packed)
+    assert torch.equal(zero.float(), p['last_bias'].expand(N, -1).float())
 
 
 @pytest.mark.parametrize('tau', [0.9, 0.1])
@@ -150,6 +175,6 @@ def test_bf16_only_paths_refuse_f16():
     from d2dmoe_amd.hip_abi import D2DMoEError
     x, routing, p = H.random_case(64, 768, 128, 24, 128, seed=1, dtype=F16)
     packed = _pack(p, 768, 128, 24, 128, 'relu', False)
-    for path in ('mfma_dense', 'mfma_sparse', 'mfma_decode', 'mfma_mid'):
+    for path in ('mfma_sparse', 'mfma_decode', 'mfma_mid'):
         with pytest.raises(D2DMoEError):
             _got(x, routing, p, 'relu', path=path, packed=packed)
