@@ -38,7 +38,7 @@ bool mfma_dense_supported(const d2dmoe_shape& sh) {
 // The fused router+select kernel covers the D2DMoE router: bf16, depth 2, ReLU hidden / abs output activation,
 // width and expert count both 128 or both 256, D a multiple of 64.
 bool mfma_router_supported(const d2dmoe_shape& sh) {
-  if (sh.dtype != D2DMOE_BF16 || sh.router_width <= 0) return false;
+  if ((sh.dtype != D2DMOE_BF16 && sh.dtype != D2DMOE_F16) || sh.router_width <= 0) return false;
   if (sh.router_activation != D2DMOE_ACT_RELU || sh.router_output_activation != D2DMOE_ACT_ABS) return false;
   if (sh.d_model % 64 != 0) return false;
   return (sh.router_width == 128 && sh.n_experts == 128) || (sh.router_width == 256 && sh.n_experts == 256);
@@ -823,11 +823,12 @@ hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* 
 // A lane ends up with one token and 4 consecutive experts per accumulator quad, stored as 8-byte pieces.
 // Optional outputs: the norms, and per-expert token counts (wave ballots + one integer atomic per expert).
 // ---------------------------------------------------------------------------------------------------
-template <int WT, int ET, int U>
+template <int WT, int ET, int U, bool F16 = false>
 __global__ __launch_bounds__(256) void router_select_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16x8* __restrict__ w1f, const bf16x8* __restrict__ w2f,
     bf16_t* __restrict__ routing, bf16_t* __restrict__ norms_out, int32_t* __restrict__ counts, int64_t N, int D,
     float thr_scale) {
+  constexpr uint32_t ONE = F16 ? 0x3C00u : 0x3F80u;   // 1.0 in the storage type
   constexpr int E = ET * 32;
   __shared__ __attribute__((aligned(16))) unsigned char stage_all[4 * 32 * E * 2];   // per wave: 32 rows of routing
   const int lane = threadIdx.x & 63;
@@ -859,7 +860,7 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int rt = 0; rt < WT; ++rt) acc1[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wr[u][rt], xb[u], acc1[rt], 0, 0, 0);
+      for (int rt = 0; rt < WT; ++rt) acc1[rt] = mfma_32x32x16<F16>(wr[u][rt], xb[u], acc1[rt]);
   };
   fill(xA, wA, 0);
   for (int ks0 = 0; ks0 < KS1; ks0 += 2 * U) {
@@ -875,10 +876,10 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       uint4 pk;
-      pk.x = pack2_bf16(fmaxf(acc1[rt][half * 8 + 0], 0.f), fmaxf(acc1[rt][half * 8 + 1], 0.f));
-      pk.y = pack2_bf16(fmaxf(acc1[rt][half * 8 + 2], 0.f), fmaxf(acc1[rt][half * 8 + 3], 0.f));
-      pk.z = pack2_bf16(fmaxf(acc1[rt][half * 8 + 4], 0.f), fmaxf(acc1[rt][half * 8 + 5], 0.f));
-      pk.w = pack2_bf16(fmaxf(acc1[rt][half * 8 + 6], 0.f), fmaxf(acc1[rt][half * 8 + 7], 0.f));
+      pk.x = enc16x2<F16>(fmaxf(acc1[rt][half * 8 + 0], 0.f), fmaxf(acc1[rt][half * 8 + 1], 0.f));
+      pk.y = enc16x2<F16>(fmaxf(acc1[rt][half * 8 + 2], 0.f), fmaxf(acc1[rt][half * 8 + 3], 0.f));
+      pk.z = enc16x2<F16>(fmaxf(acc1[rt][half * 8 + 4], 0.f), fmaxf(acc1[rt][half * 8 + 5], 0.f));
+      pk.w = enc16x2<F16>(fmaxf(acc1[rt][half * 8 + 6], 0.f), fmaxf(acc1[rt][half * 8 + 7], 0.f));
       __builtin_memcpy(&hb[rt * 2 + half], &pk, 16);
     }
   f32x16 acc2[ET];
@@ -891,7 +892,7 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
 #pragma unroll
     for (int et = 0; et < ET; ++et) {
       const bf16x8 a = w2f[(int64_t)(ks2 * ET + et) * 64 + lane];
-      acc2[et] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, hb[ks2], acc2[et], 0, 0, 0);
+      acc2[et] = mfma_32x32x16<F16>(a, hb[ks2], acc2[et]);
     }
   }
   // norms (bf16 values held as float), per-token maximum
@@ -900,13 +901,17 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
   for (int et = 0; et < ET; ++et)
 #pragma unroll
     for (int r = 0; r < 16; r += 2) {
-      const uint32_t pk = pack2_bf16(fabsf(acc2[et][r]), fabsf(acc2[et][r + 1]));
-      acc2[et][r] = __uint_as_float(pk << 16);
-      acc2[et][r + 1] = __uint_as_float(pk & 0xffff0000u);
+      const uint32_t pk = enc16x2<F16>(fabsf(acc2[et][r]), fabsf(acc2[et][r + 1]));
+      acc2[et][r] = dec16<F16>(pk & 0xffffu);
+      acc2[et][r + 1] = dec16_hi<F16>(pk);
       m = nanmax(m, nanmax(acc2[et][r], acc2[et][r + 1]));
     }
   m = nanmax(m, __shfl_xor(m, 32, kWave));
-  const float thr = __uint_as_float(pack2_bf16(m * thr_scale, 0.f) << 16);
+  // (the product is rounded to float32 before it is rounded to the storage type: kept apart by the empty asm, or the
+  // compiler folds multiply and float16 conversion into one instruction with a single rounding)
+  float thr_prod = m * thr_scale;
+  asm volatile("" : "+v"(thr_prod));
+  const float thr = dec16<F16>(enc16x2<F16>(thr_prod, 0.f) & 0xffffu);
   // A lane holds 4 consecutive experts of one token per accumulator quad.  The rows go through a wave-private LDS tile
   // (16-byte pieces XORed with the row, so both directions spread over the banks) and leave as whole rows: CH lanes
   // write the E * 2 contiguous bytes of a token's routing (or norms) row.
@@ -933,8 +938,8 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
 #pragma unroll
       for (int s = 0; s < 4; ++s) on[et][q * 4 + s] = acc2[et][q * 4 + s] >= thr;
       uint2 rv;
-      rv.x = (on[et][q * 4 + 0] ? 0x3F80u : 0u) | (on[et][q * 4 + 1] ? 0x3F800000u : 0u);   // bf16 1.0 = 0x3F80
-      rv.y = (on[et][q * 4 + 2] ? 0x3F80u : 0u) | (on[et][q * 4 + 3] ? 0x3F800000u : 0u);
+      rv.x = (on[et][q * 4 + 0] ? ONE : 0u) | (on[et][q * 4 + 1] ? (ONE << 16) : 0u);   // 1.0 in the storage type
+      rv.y = (on[et][q * 4 + 2] ? ONE : 0u) | (on[et][q * 4 + 3] ? (ONE << 16) : 0u);
       srow_w[(((et * 4 + q) ^ (c32 & (CH - 1))) << 1) + g] = rv;
     }
   }
@@ -945,8 +950,8 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         uint2 nv;
-        nv.x = (__float_as_uint(acc2[et][q * 4 + 0]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 1]) & 0xffff0000u);
-        nv.y = (__float_as_uint(acc2[et][q * 4 + 2]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 3]) & 0xffff0000u);
+        nv.x = enc16x2<F16>(acc2[et][q * 4 + 0], acc2[et][q * 4 + 1]);   // exact: the values are representable
+        nv.y = enc16x2<F16>(acc2[et][q * 4 + 2], acc2[et][q * 4 + 3]);
         srow_w[(((et * 4 + q) ^ (c32 & (CH - 1))) << 1) + g] = nv;
       }
     flush(norms_out);
@@ -974,11 +979,12 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
 // wave w computes expert tiles [w*TE, (w+1)*TE); the per-token maximum is completed through LDS.  No partial sums are
 // exchanged, so every value is bit-identical to the one-wave kernel's.  Loads run U K steps ahead in two register
 // buffers.
-template <int TW, int TE, int U>
+template <int TW, int TE, int U, bool F16 = false>
 __global__ __launch_bounds__(256) void router_select_split_kernel(
     const bf16_t* __restrict__ x, const bf16x8* __restrict__ w1f, const bf16x8* __restrict__ w2f,
     bf16_t* __restrict__ routing, bf16_t* __restrict__ norms_out, int32_t* __restrict__ counts, int64_t N, int D,
     float thr_scale) {
+  constexpr uint32_t ONE = F16 ? 0x3C00u : 0x3F80u;   // 1.0 in the storage type
   constexpr int WT = 4 * TW, ET = 4 * TE, E = ET * 32;
   __shared__ bf16x8 hs[2 * WT][64];
   __shared__ float smax[4][32];
@@ -1009,7 +1015,7 @@ __global__ __launch_bounds__(256) void router_select_split_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int a = 0; a < TW; ++a) acc1[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wr[u][a], xb[u], acc1[a], 0, 0, 0);
+      for (int a = 0; a < TW; ++a) acc1[a] = mfma_32x32x16<F16>(wr[u][a], xb[u], acc1[a]);
   };
   fill(xA, wA, 0);
   for (int ks0 = 0; ks0 < KS1; ks0 += 2 * U) {
@@ -1026,10 +1032,10 @@ __global__ __launch_bounds__(256) void router_select_split_kernel(
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       uint4 pk;
-      pk.x = pack2_bf16(fmaxf(acc1[a][half * 8 + 0], 0.f), fmaxf(acc1[a][half * 8 + 1], 0.f));
-      pk.y = pack2_bf16(fmaxf(acc1[a][half * 8 + 2], 0.f), fmaxf(acc1[a][half * 8 + 3], 0.f));
-      pk.z = pack2_bf16(fmaxf(acc1[a][half * 8 + 4], 0.f), fmaxf(acc1[a][half * 8 + 5], 0.f));
-      pk.w = pack2_bf16(fmaxf(acc1[a][half * 8 + 6], 0.f), fmaxf(acc1[a][half * 8 + 7], 0.f));
+      pk.x = enc16x2<F16>(fmaxf(acc1[a][half * 8 + 0], 0.f), fmaxf(acc1[a][half * 8 + 1], 0.f));
+      pk.y = enc16x2<F16>(fmaxf(acc1[a][half * 8 + 2], 0.f), fmaxf(acc1[a][half * 8 + 3], 0.f));
+      pk.z = enc16x2<F16>(fmaxf(acc1[a][half * 8 + 4], 0.f), fmaxf(acc1[a][half * 8 + 5], 0.f));
+      pk.w = enc16x2<F16>(fmaxf(acc1[a][half * 8 + 6], 0.f), fmaxf(acc1[a][half * 8 + 7], 0.f));
       ((uint4*)hs)[((w * TW + a) * 2 + half) * 64 + lane] = pk;
     }
   __syncthreads();
@@ -1048,7 +1054,7 @@ __global__ __launch_bounds__(256) void router_select_split_kernel(
     for (int k = 0; k < 8; ++k) {
       const bf16x8 hb = hs[k0 + k][lane];
 #pragma unroll
-      for (int et = 0; et < TE; ++et) acc2[et] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2[k][et], hb, acc2[et], 0, 0, 0);
+      for (int et = 0; et < TE; ++et) acc2[et] = mfma_32x32x16<F16>(a2[k][et], hb, acc2[et]);
     }
   }
   // norms (bf16 values held as float), per-token maximum over this wave's experts, then over the four waves
@@ -1057,16 +1063,20 @@ __global__ __launch_bounds__(256) void router_select_split_kernel(
   for (int et = 0; et < TE; ++et)
 #pragma unroll
     for (int r = 0; r < 16; r += 2) {
-      const uint32_t pk = pack2_bf16(fabsf(acc2[et][r]), fabsf(acc2[et][r + 1]));
-      acc2[et][r] = __uint_as_float(pk << 16);
-      acc2[et][r + 1] = __uint_as_float(pk & 0xffff0000u);
+      const uint32_t pk = enc16x2<F16>(fabsf(acc2[et][r]), fabsf(acc2[et][r + 1]));
+      acc2[et][r] = dec16<F16>(pk & 0xffffu);
+      acc2[et][r + 1] = dec16_hi<F16>(pk);
       m = nanmax(m, nanmax(acc2[et][r], acc2[et][r + 1]));
     }
   m = nanmax(m, __shfl_xor(m, 32, kWave));
   if (g == 0) smax[w][c32] = m;
   __syncthreads();
   m = nanmax(nanmax(smax[0][c32], smax[1][c32]), nanmax(smax[2][c32], smax[3][c32]));
-  const float thr = __uint_as_float(pack2_bf16(m * thr_scale, 0.f) << 16);
+  // (the product is rounded to float32 before it is rounded to the storage type: kept apart by the empty asm, or the
+  // compiler folds multiply and float16 conversion into one instruction with a single rounding)
+  float thr_prod = m * thr_scale;
+  asm volatile("" : "+v"(thr_prod));
+  const float thr = dec16<F16>(enc16x2<F16>(thr_prod, 0.f) & 0xffffu);
 #pragma unroll
   for (int et = 0; et < TE; ++et) {
     const int etg = w * TE + et;
@@ -1078,13 +1088,13 @@ __global__ __launch_bounds__(256) void router_select_split_kernel(
       for (int s = 0; s < 4; ++s) on[s] = acc2[et][q * 4 + s] >= thr;
       if (valid) {
         uint2 rv;
-        rv.x = (on[0] ? 0x3F80u : 0u) | (on[1] ? 0x3F800000u : 0u);   // bf16 1.0 = 0x3F80
-        rv.y = (on[2] ? 0x3F80u : 0u) | (on[3] ? 0x3F800000u : 0u);
+        rv.x = (on[0] ? ONE : 0u) | (on[1] ? (ONE << 16) : 0u);   // 1.0 in the storage type
+        rv.y = (on[2] ? ONE : 0u) | (on[3] ? (ONE << 16) : 0u);
         *(uint2*)(routing + token * E + e0) = rv;
         if (norms_out != nullptr) {
           uint2 nv;
-          nv.x = (__float_as_uint(acc2[et][q * 4 + 0]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 1]) & 0xffff0000u);
-          nv.y = (__float_as_uint(acc2[et][q * 4 + 2]) >> 16) | (__float_as_uint(acc2[et][q * 4 + 3]) & 0xffff0000u);
+          nv.x = enc16x2<F16>(acc2[et][q * 4 + 0], acc2[et][q * 4 + 1]);   // exact: the values are representable
+          nv.y = enc16x2<F16>(acc2[et][q * 4 + 2], acc2[et][q * 4 + 3]);
           *(uint2*)(norms_out + token * E + e0) = nv;
         }
       }
@@ -1103,7 +1113,8 @@ __global__ __launch_bounds__(256) void router_select_split_kernel(
   }
 }
 
-hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
+template <bool F16>
+static hipError_t launch_mfma_router_select_t(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
                                      void* norms_out, int32_t* counts, float thr_scale, hipStream_t s) {
   const PackedLayout L = packed_layout(sh);
   if (!L.has_router) return hipErrorInvalidValue;
@@ -1122,14 +1133,14 @@ hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, cons
     const unsigned grid = (unsigned)cdiv64(sh.n_tokens, 32);
     const bool deep = (sh.d_model / 16) % 8 == 0;
     if (sh.router_width == 128) {
-      if (deep) hipLaunchKernelGGL((router_select_split_kernel<1, 1, 4>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+      if (deep) hipLaunchKernelGGL((router_select_split_kernel<1, 1, 4, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
                                    (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
-      else hipLaunchKernelGGL((router_select_split_kernel<1, 1, 2>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+      else hipLaunchKernelGGL((router_select_split_kernel<1, 1, 2, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
                               (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
     } else {
-      if (deep) hipLaunchKernelGGL((router_select_split_kernel<2, 2, 4>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+      if (deep) hipLaunchKernelGGL((router_select_split_kernel<2, 2, 4, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
                                    (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
-      else hipLaunchKernelGGL((router_select_split_kernel<2, 2, 2>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+      else hipLaunchKernelGGL((router_select_split_kernel<2, 2, 2, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
                               (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
     }
     return hipGetLastError();
@@ -1137,16 +1148,22 @@ hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, cons
   const unsigned grid = (unsigned)cdiv64(sh.n_tokens, 128);
   if (sh.router_width == 128) {
     if ((sh.d_model / 16) % 8 == 0)
-      hipLaunchKernelGGL((router_select_mfma_kernel<4, 4, 4>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+      hipLaunchKernelGGL((router_select_mfma_kernel<4, 4, 4, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
                          (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
     else
-      hipLaunchKernelGGL((router_select_mfma_kernel<4, 4, 2>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+      hipLaunchKernelGGL((router_select_mfma_kernel<4, 4, 2, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
                          (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
   } else {
-    hipLaunchKernelGGL((router_select_mfma_kernel<8, 8, 2>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
+    hipLaunchKernelGGL((router_select_mfma_kernel<8, 8, 2, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
                        (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
   }
   return hipGetLastError();
+}
+
+hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
+                                     void* norms_out, int32_t* counts, float thr_scale, hipStream_t s) {
+  if (sh.dtype == D2DMOE_F16) return launch_mfma_router_select_t<true>(sh, x, packed, routing, norms_out, counts, thr_scale, s);
+  return launch_mfma_router_select_t<false>(sh, x, packed, routing, norms_out, counts, thr_scale, s);
 }
 
 }  // namespace d2dmoe

@@ -63,6 +63,26 @@ def test_router_and_select_f16(N, D, W, E):
         assert torch.equal(counts.cpu().long(), (want > 0).sum(0))
 
 
+@pytest.mark.parametrize('N,D,W,E', [(197, 768, 128, 128), (50432, 768, 128, 128), (4096, 2048, 256, 256), (33, 768, 128, 128)])
+def test_fused_router_select_f16(N, D, W, E):
+    """The fused router + selection kernels with float16 storage: norms against the float64 oracle, the mask bit-exact with
+    the oracle's gate on the kernel's own norms (thresholds 0.1, 0.5 and 0.9 of the maximum), counts."""
+    _say('f16 fused router', N, D, W, E)
+    Ed = 24 if D == 768 else 8
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=N + D, dtype=F16)
+    d = H.to_dev(p, DEV)
+    packed = _pack(p, D, E, Ed, W, 'relu', False)
+    assert packed is not None
+    want64 = O.router_forward(x.double(), p['router_w1'].double(), p['router_w2'].double())
+    for tau in (0.9, 0.5, 0.1):
+        routing, norms, counts = _ops().router_select(x.to(DEV), d['router_w1'], d['router_w2'], float(1.0 - tau), packed, E,
+                                                      Ed, want_norms=True, want_counts=True)
+        assert H.rel_err(norms.cpu(), want64) < TOL_F16
+        want = O.gate_dynk_max(norms.cpu(), tau)
+        assert torch.equal(routing.cpu(), want)
+        assert torch.equal(counts.cpu().long(), (want > 0).sum(0))
+
+
 def test_select_special_rows_f16():
     norms = torch.rand(64, 32).half()
     norms[3] = 0.0                       # all-zero row: every expert kept
