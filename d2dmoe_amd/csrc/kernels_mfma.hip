@@ -1113,6 +1113,227 @@ __global__ __launch_bounds__(256) void router_select_split_kernel(
   }
 }
 
+// The same computation for many tokens of a router whose first layer fits the register file (D = 768, width 128:
+// 192 registers per lane): one workgroup per CU walks the tiles of 32 tokens, wave w keeps the A fragments of hidden
+// tile w (all of K) and of expert tile w in registers for the whole launch, so the only stream through the CU is x itself
+// (the kernels above fetch the 196 KB of first-layer fragments from L2 for every 32 tokens, four times the bytes of x).
+// The x tiles go from global memory straight into LDS (global_load_lds: a wave instruction moves 64 x 16 bytes to 1 KB
+// of consecutive LDS, whatever the lanes' global addresses), two tiles ahead of the one being multiplied, into three
+// buffers.  A 1 KB block holds 128 bytes (8 pieces of 16) of each of 8 rows; piece pp of row r of row group R sits at
+// position 16*(pp/2) + 2r + ((pp ^ R) & 1): two neighbouring lanes fetch 32 contiguous bytes, and the 16 tokens a quarter
+// wave reads for one B fragment (same piece, rows of two row groups) fall into 16 different 16-byte bank groups.
+// Hidden activations, row maxima and the routing / norms rows are exchanged through LDS as in the split kernel (the
+// rows where the hidden activations were); every accumulator chain runs over K in
+// ascending order, so all three kernels give the same bits.  Per-expert counts are kept in registers over the tiles
+// and added once per wave.
+typedef __attribute__((address_space(3))) void rr_lds_void;
+constexpr int RR_D = 768;
+constexpr int RR_TILE_BYTES = 32 * RR_D * 2;
+constexpr size_t RR_LDS = (size_t)3 * RR_TILE_BYTES + 8 * 64 * 16 + 4 * 32 * sizeof(float);
+
+template <int D, bool F16 = false>
+__global__ __launch_bounds__(256, 1) void router_select_resident_kernel(
+    const bf16_t* __restrict__ x, const bf16x8* __restrict__ w1f, const bf16x8* __restrict__ w2f,
+    bf16_t* __restrict__ routing, bf16_t* __restrict__ norms_out, int32_t* __restrict__ counts, int64_t N,
+    float thr_scale) {
+  constexpr uint32_t ONE = F16 ? 0x3C00u : 0x3F80u;   // 1.0 in the storage type
+  constexpr int KS1 = D / 16, E = 128, CH = 16;
+  constexpr int XP = KS1 / 4;                          // 1 KB blocks per wave and tile (groups of 8 pieces per row)
+  constexpr int TB = RR_TILE_BYTES / 16;               // tile buffer in 16-byte units
+  static_assert(D == RR_D, "the LDS budget is written for D = 768");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* xs = (u32x4*)smem_raw;                        // [3][4 row groups][XP blocks][64]
+  u32x4* hs = xs + 3 * TB;                             // [8][64]
+  float* smax = (float*)(hs + 8 * 64);                 // [4][32]
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int g = lane >> 5, c32 = lane & 31;
+  const int64_t n_tiles = (N + 31) / 32;
+  const int64_t G = gridDim.x;
+
+  // x rows -> LDS: wave w moves row group w (rows 8w .. 8w+7); lane = 16a + 2r + par fetches piece 2a + (par ^ (w & 1))
+  // of the block's 8, of row r
+  const int dr = (lane >> 1) & 7, dpp = 2 * (lane >> 4) + ((lane ^ w) & 1);
+  auto issue_part = [&](int64_t t, int buf, int j0, int j1) __attribute__((always_inline)) {
+    int64_t row = t * 32 + 8 * w + dr;
+    row = row < N ? row : N - 1;                       // rows past the end: the last row again (unused)
+    const bf16_t* src = x + row * D + dpp * 8;
+    unsigned char* dst = smem_raw + (size_t)buf * RR_TILE_BYTES + (size_t)w * XP * 1024;
+#pragma unroll
+    for (int j = j0; j < j1; ++j)
+      __builtin_amdgcn_global_load_lds(src + j * 64, (rr_lds_void*)(dst + j * 1024), 16, 0, 0);
+  };
+  auto issue = [&](int64_t t, int buf) __attribute__((always_inline)) { issue_part(t, buf, 0, XP); };
+  int64_t tile = blockIdx.x;
+  issue(tile, 0);
+  issue(tile + G < n_tiles ? tile + G : tile, 1);
+
+  bf16x8 w1r[KS1], w2r[8];
+#pragma unroll
+  for (int ks = 0; ks < KS1; ++ks) w1r[ks] = w1f[(int64_t)(ks * 4 + w) * 64 + lane];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) w2r[k] = w2f[(int64_t)(k * 4 + w) * 64 + lane];
+  // the weights are waited for here, once: left pending into the loop, every trip would wait for them again
+#pragma unroll
+  for (int ks = 0; ks < KS1; ++ks) asm volatile("" : "+v"(w1r[ks]));
+#pragma unroll
+  for (int k = 0; k < 8; ++k) asm volatile("" : "+v"(w2r[k]));
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // ... and with them the first two tiles
+
+  // B fragment of K step ks, half g, token c32 = row c32 % 8 of row group c32 / 8: block ks / 4 of the group, position
+  // 16*(ks % 4) + 2r + ((g ^ R) & 1)
+  const int xrd = (c32 >> 3) * XP * 64 + 2 * (c32 & 7) + ((g ^ (c32 >> 3)) & 1);
+  int cnt[32];
+#pragma unroll
+  for (int i = 0; i < 32; ++i) cnt[i] = 0;
+  const int frow = threadIdx.x >> 4, fpc = threadIdx.x & 15;   // flush: 16 lanes write one 256-byte row
+
+  for (int it = 0; tile < n_tiles; tile += G, ++it) {
+    const int buf = it % 3;
+    const int64_t tok0 = tile * 32;
+    const bool valid = tok0 + c32 < N;
+    lds_barrier();                                     // every wave's pieces of this tile have landed (it waited for its
+                                                       // own below), and the buffer of the tile before is free
+    // the tile after next is requested two blocks at a time between the groups of products below (all twelve at once
+    // keep the wave at the issue of its loads for longer than the first products take)
+    const int64_t ahead = tile + 2 * G < n_tiles ? tile + 2 * G : tile;   // past the end: this tile's rows again, unused
+    constexpr int XI = XP / (KS1 / 8);                 // blocks per group of 8 K steps
+    static_assert(XI * (KS1 / 8) == XP, "the requests are dealt evenly over the groups of products");
+    f32x16 acc1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc1[r] = 0.f;
+    // fragments are read a group of XG K steps ahead of the products that use them (two register groups)
+    constexpr int XG = 8;
+    static_assert(KS1 % (2 * XG) == 0, "K steps come in pairs of groups");
+    u32x4 fa[XG], fb[XG];
+    const u32x4* xt = xs + buf * TB + xrd;
+    auto fetch = [&](u32x4 (&f)[XG], int ks0) __attribute__((always_inline)) {
+#pragma unroll
+      for (int u = 0; u < XG; ++u) f[u] = xt[((ks0 + u) >> 2) * 64 + ((ks0 + u) & 3) * 16];
+    };
+    auto product = [&](u32x4 (&f)[XG], int ks0) __attribute__((always_inline)) {
+#pragma unroll
+      for (int u = 0; u < XG; ++u) {
+        bf16x8 b;
+        __builtin_memcpy(&b, &f[u], 16);
+        acc1 = mfma_32x32x16<F16>(w1r[ks0 + u], b, acc1);
+      }
+    };
+    fetch(fa, 0);
+#pragma unroll
+    for (int ks0 = 0; ks0 < KS1; ks0 += 2 * XG) {
+      fetch(fb, ks0 + XG);
+      __builtin_amdgcn_sched_barrier(0);
+      product(fa, ks0);
+      __builtin_amdgcn_sched_barrier(0);
+      issue_part(ahead, (it + 2) % 3, (ks0 / XG) * XI, (ks0 / XG + 1) * XI);
+      __builtin_amdgcn_sched_barrier(0);
+      if (ks0 + 2 * XG < KS1) fetch(fa, ks0 + 2 * XG);
+      __builtin_amdgcn_sched_barrier(0);
+      product(fb, ks0 + XG);
+      __builtin_amdgcn_sched_barrier(0);
+      issue_part(ahead, (it + 2) % 3, (ks0 / XG + 1) * XI, (ks0 / XG + 2) * XI);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      u32x4 pk;
+      pk.x = enc16x2<F16>(fmaxf(acc1[half * 8 + 0], 0.f), fmaxf(acc1[half * 8 + 1], 0.f));
+      pk.y = enc16x2<F16>(fmaxf(acc1[half * 8 + 2], 0.f), fmaxf(acc1[half * 8 + 3], 0.f));
+      pk.z = enc16x2<F16>(fmaxf(acc1[half * 8 + 4], 0.f), fmaxf(acc1[half * 8 + 5], 0.f));
+      pk.w = enc16x2<F16>(fmaxf(acc1[half * 8 + 6], 0.f), fmaxf(acc1[half * 8 + 7], 0.f));
+      hs[(w * 2 + half) * 64 + lane] = pk;
+    }
+    lds_barrier();                                     // from here on nobody reads this tile's x buffer
+    f32x16 acc2;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc2[r] = 0.f;
+    u32x4 hv[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) hv[k] = hs[k * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      bf16x8 hb;
+      __builtin_memcpy(&hb, &hv[k], 16);
+      acc2 = mfma_32x32x16<F16>(w2r[k], hb, acc2);
+    }
+    // norms (storage-type values held as float), per-token maximum over this wave's experts, then over the four waves
+    float m = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      const uint32_t pk = enc16x2<F16>(fabsf(acc2[r]), fabsf(acc2[r + 1]));
+      acc2[r] = dec16<F16>(pk & 0xffffu);
+      acc2[r + 1] = dec16_hi<F16>(pk);
+      m = nanmax(m, nanmax(acc2[r], acc2[r + 1]));
+    }
+    m = nanmax(m, __shfl_xor(m, 32, kWave));
+    if (g == 0) smax[w * 32 + c32] = m;
+    lds_barrier();
+    m = nanmax(nanmax(smax[c32], smax[32 + c32]), nanmax(smax[64 + c32], smax[96 + c32]));
+    // (the product is rounded to float32 before it is rounded to the storage type: kept apart by the empty asm, or the
+    // compiler folds multiply and float16 conversion into one instruction with a single rounding)
+    float thr_prod = m * thr_scale;
+    asm volatile("" : "+v"(thr_prod));
+    const float thr = dec16<F16>(enc16x2<F16>(thr_prod, 0.f) & 0xffffu);
+    // routing rows (then norms rows): 32 rows of 16 pieces each, where the hidden activations were
+    // (written with ds_write_b64 spelled out: before an ordinary LDS store the compiler waits for every global_load_lds
+    // in flight, the tile after next included; the barriers below wait for these writes like for any other)
+    const uint32_t srow = (uint32_t)(uintptr_t)(rr_lds_void*)(hs + c32 * CH);   // this lane's row; piece p, half g at
+    auto put = [&](int piece, const uint2& v) __attribute__((always_inline)) {  // byte ((p ^ (c32 & 15)) * 2 + g) * 8
+      asm volatile("ds_write_b64 %0, %1" :: "v"(srow + (uint32_t)((((piece ^ (c32 & (CH - 1))) << 1) + g) << 3)), "v"(v) : "memory");
+    };
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      bool on[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) on[s] = acc2[q * 4 + s] >= thr;
+      uint2 rv;
+      rv.x = (on[0] ? ONE : 0u) | (on[1] ? (ONE << 16) : 0u);
+      rv.y = (on[2] ? ONE : 0u) | (on[3] ? (ONE << 16) : 0u);
+      put(w * 4 + q, rv);
+      if (counts != nullptr) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const unsigned long long bal = __ballot(on[s] && valid);
+          cnt[8 * q + s] += __popcll(bal & 0xffffffffull);
+          cnt[8 * q + 4 + s] += __popcll(bal >> 32);
+        }
+      }
+    }
+    lds_barrier();
+    // This wave's pieces of the NEXT tile have landed once only the XP loads issued in this trip are still in flight
+    // (the stores below come after the wait, the ones of the trip before are older than those loads).
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(XP) : "memory");
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = frow + 16 * i;
+      if (tok0 + row < N) *(u32x4*)(routing + (tok0 + row) * E + fpc * 8) = hs[row * CH + (fpc ^ (row & (CH - 1)))];
+    }
+    if (norms_out != nullptr) {                        // uniform
+      lds_barrier();
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        uint2 nv;
+        nv.x = enc16x2<F16>(acc2[q * 4 + 0], acc2[q * 4 + 1]);   // exact: the values are representable
+        nv.y = enc16x2<F16>(acc2[q * 4 + 2], acc2[q * 4 + 3]);
+        put(w * 4 + q, nv);
+      }
+      lds_barrier();
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int row = frow + 16 * i;
+        if (tok0 + row < N) *(u32x4*)(norms_out + (tok0 + row) * E + fpc * 8) = hs[row * CH + (fpc ^ (row & (CH - 1)))];
+      }
+    }
+  }
+  if (counts != nullptr) {
+    int mine = 0;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) mine = (lane == i) ? cnt[i] : mine;
+    if (lane < 32 && mine != 0) atomicAdd(counts + w * 32 + lane, mine);
+  }
+}
+
 template <bool F16>
 static hipError_t launch_mfma_router_select_t(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
                                      void* norms_out, int32_t* counts, float thr_scale, hipStream_t s) {
@@ -1128,7 +1349,17 @@ static hipError_t launch_mfma_router_select_t(const d2dmoe_shape& sh, const void
   const bf16x8* r2 = (const bf16x8*)(base + L.r2_off);
   // One wave per 32 tokens fills the machine from about 4 * 32 * CUs tokens on; below that (or with long rows, where a
   // wave's K loop is the critical path) a workgroup per 32 tokens shares the output features among its waves.
-  const bool split = (sh.n_tokens < (int64_t)128 * device_cu_count() || sh.d_model >= 2048) && (sh.d_model / 16) % 4 == 0;
+  const int cus = device_cu_count();
+  if (sh.d_model == RR_D && sh.router_width == 128 && sh.n_tokens >= (int64_t)64 * cus) {
+    auto kern = router_select_resident_kernel<RR_D, F16>;
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RR_LDS);
+    if (e != hipSuccess) return e;
+    const int64_t n_tiles = cdiv64(sh.n_tokens, 32);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(n_tiles < cus ? n_tiles : cus)), dim3(256), RR_LDS, s, xp, r1, r2, (bf16_t*)routing,
+                       (bf16_t*)norms_out, counts, sh.n_tokens, thr_scale);
+    return hipGetLastError();
+  }
+  const bool split = (sh.n_tokens < (int64_t)128 * cus || sh.d_model >= 2048) && (sh.d_model / 16) % 4 == 0;
   if (split) {
     const unsigned grid = (unsigned)cdiv64(sh.n_tokens, 32);
     const bool deep = (sh.d_model / 16) % 8 == 0;

@@ -361,6 +361,38 @@ def test_packed_weights_cache_tracks_parameter_updates():
 
 
 # =================================================================== fused router + select (MFMA) =====
+@pytest.mark.parametrize('N', [16384, 16385, 50432, 50401])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_router_select_resident(N, dtype):
+    """From 16 384 tokens on, the ViT-B router runs with its weights resident in registers and x staged through LDS
+    (one workgroup per CU walking the tiles).  Checked: the mask is the oracle's gate applied to the kernel's own
+    norms; the counts are the column sums of the mask; a token's result does not depend on where it stands in the
+    batch (bit-exact under a permutation of the tokens); and, since every kernel accumulates over K in ascending order,
+    the rows equal, bit for bit, what the tiled kernels (one wave or one workgroup per 32 tokens) give on slices."""
+    _say('router resident', N, dtype)
+    D, W, E, Ed = 768, 128, 128, 24
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=N, dtype=dtype)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, W, 1 if dtype == torch.bfloat16 else 2, 'relu')
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, d['router_w1'], d['router_w2'])
+    xd = x.to(DEV)
+    want64 = O.router_forward(x[:4096].double(), p['router_w1'].double(), p['router_w2'].double())
+    perm = torch.randperm(N, generator=torch.Generator().manual_seed(N)).to(DEV)
+    for thr in (0.1, 0.9):
+        r, n, c = _ops().router_select(xd, d['router_w1'], d['router_w2'], thr, packed, E, Ed, True, True)
+        assert torch.equal(c.long(), (r > 0).sum(0))
+        assert torch.equal(r.cpu(), O.gate_dynk_max(n.cpu(), 1.0 - thr))
+        assert H.rel_err(n[:4096].cpu(), want64) < (H.TOL_BF16 if dtype == torch.bfloat16 else H.TOL_F16)
+        rp, np_, cp = _ops().router_select(xd[perm].contiguous(), d['router_w1'], d['router_w2'], thr, packed, E, Ed, True, True)
+        assert torch.equal(np_, n[perm]) and torch.equal(rp, r[perm]) and torch.equal(cp, c)
+        for lo, hi in ((0, 4096), (N - 12001, N), (5000, 5033)):
+            r2, n2, _ = _ops().router_select(xd[lo:hi].contiguous(), d['router_w1'], d['router_w2'], thr, packed, E, Ed, True, True)
+            assert torch.equal(n[lo:hi], n2) and torch.equal(r[lo:hi], r2), (lo, hi)
+    # without the optional outputs
+    r3, n3, c3 = _ops().router_select(xd, d['router_w1'], d['router_w2'], 0.9, packed, E, Ed, False, False)
+    assert n3 is None and c3 is None and torch.equal(r3, r)
+
+
 @pytest.mark.parametrize('N,D,W,E', [(197, 768, 128, 128), (1, 768, 128, 128), (33, 768, 128, 128), (1576, 768, 128, 128),
                                      (50432, 768, 128, 128), (16, 2048, 256, 256), (300, 2048, 256, 256)])
 @pytest.mark.parametrize('tau', [0.1, 0.9])
