@@ -1334,6 +1334,44 @@ __global__ __launch_bounds__(256, 1) void router_select_resident_kernel(
   }
 }
 
+// Per-expert token counts of a routing mask [N, E] in 16-bit storage, E = 64 * EPL: column sums of the non-zero entries.
+// Behind the split kernel, whose workgroups own 32 tokens each: one integer atomic per expert and workgroup from a few
+// hundred workgroups queues up on the four cache lines of the counters (8192 tokens: 16 -> 95 us); here a workgroup
+// takes a long run of rows, lanes = experts, and adds once.
+template <int EPL>
+__global__ __launch_bounds__(256) void routing_counts_kernel(const bf16_t* __restrict__ routing, int32_t* __restrict__ counts,
+                                                             int64_t N, int64_t rows_per_wg) {
+  constexpr int E = 64 * EPL;
+  typedef uint16_t row_piece __attribute__((ext_vector_type(EPL)));
+  __shared__ int part[4][E];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_wg;
+  const int64_t r1 = (r0 + rows_per_wg < N) ? (r0 + rows_per_wg) : N;
+  int cnt[EPL];
+#pragma unroll
+  for (int k = 0; k < EPL; ++k) cnt[k] = 0;
+  constexpr int UN = 8;
+  for (int64_t r = r0 + w; r < r1; r += 4 * UN) {
+    row_piece v[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int64_t rr = (r + 4 * u < r1) ? (r + 4 * u) : (r1 - 1);   // clamped: the loads go out together
+      v[u] = *(const row_piece*)(routing + rr * E + lane * EPL);
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+#pragma unroll
+      for (int k = 0; k < EPL; ++k) cnt[k] += (r + 4 * u < r1 && (v[u][k] & 0x7fff) != 0) ? 1 : 0;
+  }
+#pragma unroll
+  for (int k = 0; k < EPL; ++k) part[w][lane * EPL + k] = cnt[k];
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256) {
+    const int t = part[0][e] + part[1][e] + part[2][e] + part[3][e];
+    if (t != 0) atomicAdd(counts + e, t);
+  }
+}
+
 template <bool F16>
 static hipError_t launch_mfma_router_select_t(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
                                      void* norms_out, int32_t* counts, float thr_scale, hipStream_t s) {
@@ -1363,16 +1401,27 @@ static hipError_t launch_mfma_router_select_t(const d2dmoe_shape& sh, const void
   if (split) {
     const unsigned grid = (unsigned)cdiv64(sh.n_tokens, 32);
     const bool deep = (sh.d_model / 16) % 8 == 0;
+    // from a few hundred workgroups on, the counts are taken from the finished mask by a kernel of their own
+    const bool count_after = counts != nullptr && grid > 64;
+    int32_t* kc = count_after ? nullptr : counts;
     if (sh.router_width == 128) {
       if (deep) hipLaunchKernelGGL((router_select_split_kernel<1, 1, 4, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
-                                   (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+                                   (bf16_t*)norms_out, kc, sh.n_tokens, sh.d_model, thr_scale);
       else hipLaunchKernelGGL((router_select_split_kernel<1, 1, 2, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
-                              (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+                              (bf16_t*)norms_out, kc, sh.n_tokens, sh.d_model, thr_scale);
     } else {
       if (deep) hipLaunchKernelGGL((router_select_split_kernel<2, 2, 4, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
-                                   (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+                                   (bf16_t*)norms_out, kc, sh.n_tokens, sh.d_model, thr_scale);
       else hipLaunchKernelGGL((router_select_split_kernel<2, 2, 2, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
-                              (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+                              (bf16_t*)norms_out, kc, sh.n_tokens, sh.d_model, thr_scale);
+    }
+    if (count_after) {
+      const int64_t rows_per_wg = cdiv64(sh.n_tokens, 32);   // 32 workgroups
+      const unsigned cgrid = (unsigned)cdiv64(sh.n_tokens, rows_per_wg);
+      if (sh.n_experts == 128)
+        hipLaunchKernelGGL(routing_counts_kernel<2>, dim3(cgrid), dim3(256), 0, s, (const bf16_t*)routing, counts, sh.n_tokens, rows_per_wg);
+      else
+        hipLaunchKernelGGL(routing_counts_kernel<4>, dim3(cgrid), dim3(256), 0, s, (const bf16_t*)routing, counts, sh.n_tokens, rows_per_wg);
     }
     return hipGetLastError();
   }

@@ -394,7 +394,8 @@ def test_router_select_resident(N, dtype):
 
 
 @pytest.mark.parametrize('N,D,W,E', [(197, 768, 128, 128), (1, 768, 128, 128), (33, 768, 128, 128), (1576, 768, 128, 128),
-                                     (50432, 768, 128, 128), (16, 2048, 256, 256), (300, 2048, 256, 256)])
+                                     (50432, 768, 128, 128), (16, 2048, 256, 256), (300, 2048, 256, 256),
+                                     (8191, 768, 128, 128), (4100, 2048, 256, 256)])
 @pytest.mark.parametrize('tau', [0.1, 0.9])
 def test_router_select_mfma(N, D, W, E, tau):
     """Fused router + selection: norms within tolerance of the float64 router, mask bit-exact for the kernel's own
