@@ -218,9 +218,11 @@ int d2dmoe_pack_weights(const d2dmoe_shape* shape, const void* w1, const void* b
   return (int)launch_mfma_pack(*shape, w1, b1, w2, w_up, router_w1, router_w2, packed, (hipStream_t)stream);
 }
 
-int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing, const void* w1, const void* b1,
-                   const void* w2, const void* w_up, const void* last_bias, const void* packed, void* out,
-                   int32_t path, void* workspace, size_t workspace_bytes, void* stream) {
+// plan_counts_ready: the router kernel of this call has already left the expert-major plan's per-segment counts in
+// the workspace (d2dmoe_forward only)
+static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* routing, const void* w1, const void* b1,
+                        const void* w2, const void* w_up, const void* last_bias, const void* packed, void* out,
+                        int32_t path, void* workspace, size_t workspace_bytes, void* stream, bool plan_counts_ready) {
   int st = check_shape(shape);
   if (st != D2DMOE_OK) return st;
   const d2dmoe_shape& sh = *shape;
@@ -264,7 +266,8 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
       const size_t need = mfma_sparse_workspace_bytes(sh);
       if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
       const int* flag = nullptr;
-      hipError_t e = launch_mfma_sparse(sh, x, routing, packed, last_bias, out, workspace, mfma_sparse_capacity_k(sh), &flag, s);
+      hipError_t e = launch_mfma_sparse(sh, x, routing, packed, last_bias, out, workspace, mfma_sparse_capacity_k(sh), &flag, s,
+                                        plan_counts_ready);
       if (e != hipSuccess) return (int)e;
       // with every expert routed to by every token the pairs still fit: the fall-back can never be needed
       if (sh.n_tokens * (int64_t)sh.n_experts <= mfma_sparse_capacity_pairs(sh)) return D2DMOE_OK;
@@ -315,9 +318,18 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
   }
 }
 
-int d2dmoe_router_select(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
-                         const void* packed, float thr_scale, void* norms_out, void* routing, int32_t* counts,
-                         void* workspace, size_t workspace_bytes, void* stream) {
+int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing, const void* w1, const void* b1,
+                   const void* w2, const void* w_up, const void* last_bias, const void* packed, void* out,
+                   int32_t path, void* workspace, size_t workspace_bytes, void* stream) {
+  return experts_impl(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, workspace, workspace_bytes, stream,
+                      false);
+}
+
+// seg_counts / seg_pairs: see launch_mfma_router_select
+static int router_select_impl(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
+                              const void* packed, float thr_scale, void* norms_out, void* routing, int32_t* counts,
+                              void* workspace, size_t workspace_bytes, void* stream, int32_t* seg_counts,
+                              int32_t* seg_pairs) {
   int st = check_shape(shape);
   if (st != D2DMOE_OK) return st;
   const d2dmoe_shape& sh = *shape;
@@ -327,7 +339,8 @@ int d2dmoe_router_select(const d2dmoe_shape* shape, const void* x, const void* r
   if (!x) return D2DMOE_E_NULL;
   if (packed != nullptr && mfma_router_supported(sh) && sh.n_tokens > 16) {
     if (!aligned16(x) || !aligned16(routing) || (norms_out && !aligned16(norms_out))) return D2DMOE_E_ALIGN;
-    return (int)launch_mfma_router_select(sh, x, packed, routing, norms_out, counts, thr_scale, (hipStream_t)stream);
+    return (int)launch_mfma_router_select(sh, x, packed, routing, norms_out, counts, thr_scale, (hipStream_t)stream,
+                                          seg_counts, seg_pairs);
   }
   if (!router_w1 || !router_w2) return D2DMOE_E_NULL;
   const ForwardWorkspace plan = plan_workspace(sh);
@@ -339,6 +352,13 @@ int d2dmoe_router_select(const d2dmoe_shape* shape, const void* x, const void* r
                      plan.norms_off - plan.hidden_off, stream);
   if (st != D2DMOE_OK) return st;
   return d2dmoe_select(nbuf, routing, counts, sh.n_tokens, sh.n_experts, sh.dtype, thr_scale, stream);
+}
+
+int d2dmoe_router_select(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
+                         const void* packed, float thr_scale, void* norms_out, void* routing, int32_t* counts,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+  return router_select_impl(shape, x, router_w1, router_w2, packed, thr_scale, norms_out, routing, counts, workspace,
+                            workspace_bytes, stream, nullptr, nullptr);
 }
 
 int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
@@ -364,13 +384,6 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
                                          (const char*)packed + mfma_decode_section_offset(sh), last_bias, ws + plan.hidden_off,
                                          nbuf, routing, counts, out, ws + plan.perm_off, (hipStream_t)stream);
   }
-  if (norms_in == nullptr) {
-    st = d2dmoe_router_select(shape, x, router_w1, router_w2, packed, thr_scale, norms_out, routing, counts, workspace,
-                              workspace_bytes, stream);
-  } else {
-    st = d2dmoe_select(norms_in, routing, counts, sh.n_tokens, sh.n_experts, sh.dtype, thr_scale, stream);
-  }
-  if (st != D2DMOE_OK) return st;
   // A high threshold fraction keeps few experts per token: take the expert-major path (it falls back to the dense
   // sweep on the device if the routing turns out dense after all).
   // (gated experts: from a lower fraction on -- their dense alternative costs ten times the expert-major path at few
@@ -381,8 +394,24 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
       (thr_scale >= (sh.gated ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128)) && mfma_sparse_supported(sh) &&
       (sh.gated ? mfma_gemm_supported(sh) : mfma_dense_supported(sh)))
     path = D2DMOE_PATH_MFMA_SPARSE;
-  return d2dmoe_experts(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,
-                        plan.total - plan.perm_off, stream);
+  // ... and when the router kernel of this call is the one that walks the 32-token segments of that path's plan, it
+  // leaves the plan's per-segment counts in the workspace on its way
+  bool plan_counts_ready = false;
+  if (norms_in == nullptr) {
+    int32_t *seg_counts = nullptr, *seg_pairs = nullptr;
+    if (path == D2DMOE_PATH_MFMA_SPARSE && packed != nullptr && mfma_sparse_supported(sh) && mfma_router_writes_plan_counts(sh) &&
+        plan.total - plan.perm_off >= mfma_sparse_workspace_bytes(sh)) {
+      mfma_sparse_plan_counts(sh, ws + plan.perm_off, &seg_counts, &seg_pairs);
+      plan_counts_ready = true;
+    }
+    st = router_select_impl(shape, x, router_w1, router_w2, packed, thr_scale, norms_out, routing, counts, workspace,
+                            workspace_bytes, stream, seg_counts, seg_pairs);
+  } else {
+    st = d2dmoe_select(norms_in, routing, counts, sh.n_tokens, sh.n_experts, sh.dtype, thr_scale, stream);
+  }
+  if (st != D2DMOE_OK) return st;
+  return experts_impl(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,
+                      plan.total - plan.perm_off, stream, plan_counts_ready);
 }
 
 int d2dmoe_forward_static(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,

@@ -1129,13 +1129,13 @@ __global__ __launch_bounds__(256) void router_select_split_kernel(
 typedef __attribute__((address_space(3))) void rr_lds_void;
 constexpr int RR_D = 768;
 constexpr int RR_TILE_BYTES = 32 * RR_D * 2;
-constexpr size_t RR_LDS = (size_t)3 * RR_TILE_BYTES + 8 * 64 * 16 + 4 * 32 * sizeof(float);
+constexpr size_t RR_LDS = (size_t)3 * RR_TILE_BYTES + 8 * 64 * 16 + 4 * 32 * sizeof(float) + 4 * sizeof(int);
 
 template <int D, bool F16 = false>
 __global__ __launch_bounds__(256, 1) void router_select_resident_kernel(
     const bf16_t* __restrict__ x, const bf16x8* __restrict__ w1f, const bf16x8* __restrict__ w2f,
-    bf16_t* __restrict__ routing, bf16_t* __restrict__ norms_out, int32_t* __restrict__ counts, int64_t N,
-    float thr_scale) {
+    bf16_t* __restrict__ routing, bf16_t* __restrict__ norms_out, int32_t* __restrict__ counts,
+    int32_t* __restrict__ seg_counts, int32_t* __restrict__ seg_pairs, int64_t N, float thr_scale) {
   constexpr uint32_t ONE = F16 ? 0x3C00u : 0x3F80u;   // 1.0 in the storage type
   constexpr int KS1 = D / 16, E = 128, CH = 16;
   constexpr int XP = KS1 / 4;                          // 1 KB blocks per wave and tile (groups of 8 pieces per row)
@@ -1145,10 +1145,12 @@ __global__ __launch_bounds__(256, 1) void router_select_resident_kernel(
   u32x4* xs = (u32x4*)smem_raw;                        // [3][4 row groups][XP blocks][64]
   u32x4* hs = xs + 3 * TB;                             // [8][64]
   float* smax = (float*)(hs + 8 * 64);                 // [4][32]
+  int* spair = (int*)(smax + 4 * 32);                  // [4]: the waves' routed pairs of the tile
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int g = lane >> 5, c32 = lane & 31;
   const int64_t n_tiles = (N + 31) / 32;
   const int64_t G = gridDim.x;
+  const bool counting = counts != nullptr || seg_counts != nullptr;   // uniform
 
   // x rows -> LDS: wave w moves row group w (rows 8w .. 8w+7); lane = 16a + 2r + par fetches piece 2a + (par ^ (w & 1))
   // of the block's 8, of row r
@@ -1182,9 +1184,7 @@ __global__ __launch_bounds__(256, 1) void router_select_resident_kernel(
   // B fragment of K step ks, half g, token c32 = row c32 % 8 of row group c32 / 8: block ks / 4 of the group, position
   // 16*(ks % 4) + 2r + ((g ^ R) & 1)
   const int xrd = (c32 >> 3) * XP * 64 + 2 * (c32 & 7) + ((g ^ (c32 >> 3)) & 1);
-  int cnt[32];
-#pragma unroll
-  for (int i = 0; i < 32; ++i) cnt[i] = 0;
+  int cnt = 0;                                         // lanes 0..31: tokens routed to expert 32w + lane so far
   const int frow = threadIdx.x >> 4, fpc = threadIdx.x & 15;   // flush: 16 lanes write one 256-byte row
 
   for (int it = 0; tile < n_tiles; tile += G, ++it) {
@@ -1282,6 +1282,7 @@ __global__ __launch_bounds__(256, 1) void router_select_resident_kernel(
     auto put = [&](int piece, const uint2& v) __attribute__((always_inline)) {  // byte ((p ^ (c32 & 15)) * 2 + g) * 8
       asm volatile("ds_write_b64 %0, %1" :: "v"(srow + (uint32_t)((((piece ^ (c32 & (CH - 1))) << 1) + g) << 3)), "v"(v) : "memory");
     };
+    int tcnt = 0;                                      // lanes 0..31: this tile's tokens routed to expert 32w + lane
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       bool on[4];
@@ -1291,16 +1292,24 @@ __global__ __launch_bounds__(256, 1) void router_select_resident_kernel(
       rv.x = (on[0] ? ONE : 0u) | (on[1] ? (ONE << 16) : 0u);
       rv.y = (on[2] ? ONE : 0u) | (on[3] ? (ONE << 16) : 0u);
       put(w * 4 + q, rv);
-      if (counts != nullptr) {
+      if (counting) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-          const unsigned long long bal = __ballot(on[s] && valid);
-          cnt[8 * q + s] += __popcll(bal & 0xffffffffull);
-          cnt[8 * q + 4 + s] += __popcll(bal >> 32);
+          const unsigned long long bal = __ballot(on[s] && valid);   // low half: expert 8q + s, high half: 8q + 4 + s
+          tcnt = (lane == 8 * q + s) ? __popcll(bal & 0xffffffffull) : tcnt;
+          tcnt = (lane == 8 * q + 4 + s) ? __popcll(bal >> 32) : tcnt;
         }
       }
     }
+    cnt += tcnt;
+    if (seg_counts != nullptr) {
+      // the expert-major plan's first pass, for the segment of 32 tokens this tile is: tokens per expert, pairs in all
+      if (lane < 32) seg_counts[tile * E + w * 32 + lane] = tcnt;
+      const int wp = wave_sum_i32(tcnt);
+      if (lane == 0) spair[w] = wp;
+    }
     lds_barrier();
+    if (seg_counts != nullptr && threadIdx.x == 0) seg_pairs[tile] = spair[0] + spair[1] + spair[2] + spair[3];
     // This wave's pieces of the NEXT tile have landed once only the XP loads issued in this trip are still in flight
     // (the stores below come after the wait, the ones of the trip before are older than those loads).
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(XP) : "memory");
@@ -1326,12 +1335,7 @@ __global__ __launch_bounds__(256, 1) void router_select_resident_kernel(
       }
     }
   }
-  if (counts != nullptr) {
-    int mine = 0;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) mine = (lane == i) ? cnt[i] : mine;
-    if (lane < 32 && mine != 0) atomicAdd(counts + w * 32 + lane, mine);
-  }
+  if (counts != nullptr && lane < 32 && cnt != 0) atomicAdd(counts + w * 32 + lane, cnt);
 }
 
 // Per-expert token counts of a routing mask [N, E] in 16-bit storage, E = 64 * EPL: column sums of the non-zero entries.
@@ -1372,9 +1376,15 @@ __global__ __launch_bounds__(256) void routing_counts_kernel(const bf16_t* __res
   }
 }
 
+bool mfma_router_writes_plan_counts(const d2dmoe_shape& sh) {
+  return mfma_router_supported(sh) && sh.d_model == RR_D && sh.router_width == 128 &&
+         sh.n_tokens >= (int64_t)64 * device_cu_count();
+}
+
 template <bool F16>
 static hipError_t launch_mfma_router_select_t(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
-                                     void* norms_out, int32_t* counts, float thr_scale, hipStream_t s) {
+                                     void* norms_out, int32_t* counts, float thr_scale, int32_t* seg_counts,
+                                     int32_t* seg_pairs, hipStream_t s) {
   const PackedLayout L = packed_layout(sh);
   if (!L.has_router) return hipErrorInvalidValue;
   const char* base = (const char*)packed;
@@ -1388,13 +1398,13 @@ static hipError_t launch_mfma_router_select_t(const d2dmoe_shape& sh, const void
   // One wave per 32 tokens fills the machine from about 4 * 32 * CUs tokens on; below that (or with long rows, where a
   // wave's K loop is the critical path) a workgroup per 32 tokens shares the output features among its waves.
   const int cus = device_cu_count();
-  if (sh.d_model == RR_D && sh.router_width == 128 && sh.n_tokens >= (int64_t)64 * cus) {
+  if (mfma_router_writes_plan_counts(sh)) {
     auto kern = router_select_resident_kernel<RR_D, F16>;
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RR_LDS);
     if (e != hipSuccess) return e;
     const int64_t n_tiles = cdiv64(sh.n_tokens, 32);
     hipLaunchKernelGGL(kern, dim3((unsigned)(n_tiles < cus ? n_tiles : cus)), dim3(256), RR_LDS, s, xp, r1, r2, (bf16_t*)routing,
-                       (bf16_t*)norms_out, counts, sh.n_tokens, thr_scale);
+                       (bf16_t*)norms_out, counts, seg_counts, seg_pairs, sh.n_tokens, thr_scale);
     return hipGetLastError();
   }
   const bool split = (sh.n_tokens < (int64_t)128 * cus || sh.d_model >= 2048) && (sh.d_model / 16) % 4 == 0;
@@ -1440,10 +1450,14 @@ static hipError_t launch_mfma_router_select_t(const d2dmoe_shape& sh, const void
   return hipGetLastError();
 }
 
+// seg_counts / seg_pairs (optional): the expert-major plan's per-segment counts, written by the kernel when
+// mfma_router_writes_plan_counts(sh) holds and ignored otherwise.
 hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
-                                     void* norms_out, int32_t* counts, float thr_scale, hipStream_t s) {
-  if (sh.dtype == D2DMOE_F16) return launch_mfma_router_select_t<true>(sh, x, packed, routing, norms_out, counts, thr_scale, s);
-  return launch_mfma_router_select_t<false>(sh, x, packed, routing, norms_out, counts, thr_scale, s);
+                                     void* norms_out, int32_t* counts, float thr_scale, hipStream_t s, int32_t* seg_counts,
+                                     int32_t* seg_pairs) {
+  if (sh.dtype == D2DMOE_F16)
+    return launch_mfma_router_select_t<true>(sh, x, packed, routing, norms_out, counts, thr_scale, seg_counts, seg_pairs, s);
+  return launch_mfma_router_select_t<false>(sh, x, packed, routing, norms_out, counts, thr_scale, seg_counts, seg_pairs, s);
 }
 
 }  // namespace d2dmoe

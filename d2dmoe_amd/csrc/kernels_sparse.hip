@@ -790,22 +790,29 @@ static void launch_sparse_experts(const SparseArgs& A, int act, unsigned grid, h
 }
 
 void launch_plan_count_scan(const void* routing, int64_t N, int E, int32_t* seg_counts, int32_t* seg_pairs,
-                            int32_t* seg_offsets, int32_t* totals, hipStream_t s) {
+                            int32_t* seg_offsets, int32_t* totals, hipStream_t s, bool counts_ready) {
   const int64_t n_seg = cdiv64(N, SP_SEG);
   const unsigned seg_blocks = (unsigned)cdiv64(n_seg, 4);
   const int vpt = (E + 63) / 64;
 #define D2DMOE_PLAN_DISPATCH(V)                                                                                          \
   hipLaunchKernelGGL(plan_count_kernel<V>, dim3(seg_blocks), dim3(256), 0, s, (const bf16_t*)routing, seg_counts, seg_pairs, N, \
                      E, n_seg)
-  if (vpt <= 1) D2DMOE_PLAN_DISPATCH(1); else if (vpt <= 2) D2DMOE_PLAN_DISPATCH(2); else if (vpt <= 4) D2DMOE_PLAN_DISPATCH(4);
+  if (counts_ready) {}   // the router kernel has left them there
+  else if (vpt <= 1) D2DMOE_PLAN_DISPATCH(1); else if (vpt <= 2) D2DMOE_PLAN_DISPATCH(2); else if (vpt <= 4) D2DMOE_PLAN_DISPATCH(4);
   else if (vpt <= 8) D2DMOE_PLAN_DISPATCH(8); else D2DMOE_PLAN_DISPATCH(16);
 #undef D2DMOE_PLAN_DISPATCH
   launch_perm_scan(seg_counts, seg_offsets, totals, E, n_seg, s);
 }
 
+void mfma_sparse_plan_counts(const d2dmoe_shape& sh, void* workspace, int32_t** seg_counts, int32_t** seg_pairs) {
+  const SparseWorkspace W = sparse_workspace(sh, mfma_sparse_capacity_k(sh));
+  *seg_counts = (int32_t*)((char*)workspace + W.seg_counts);
+  *seg_pairs = (int32_t*)((char*)workspace + W.seg_pairs);
+}
+
 hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                               const void* last_bias, void* out, void* workspace, int max_mean_k, const int** flag_out,
-                              hipStream_t s) {
+                              hipStream_t s, bool counts_ready) {
   const int cap_k = mfma_sparse_capacity_k(sh);
   if (max_mean_k > cap_k) max_mean_k = cap_k;
   const SparseWorkspace W = sparse_workspace(sh, cap_k);   // sized for the maximum; the flag uses max_mean_k
@@ -831,7 +838,7 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   // at 50 432)
   const bool split_seg = W.n_seg <= 512;
   const int vpt = (E + 63) / 64;
-  launch_plan_count_scan(routing, N, E, seg_counts, seg_pairs, seg_offsets, totals, s);
+  launch_plan_count_scan(routing, N, E, seg_counts, seg_pairs, seg_offsets, totals, s, counts_ready);
 #define D2DMOE_PLAN_DISPATCH(V)                                                                                          \
   hipLaunchKernelGGL(plan_scatter_kernel<V>, dim3(split_seg ? (unsigned)W.n_seg : seg_blocks), dim3(256), 0, s,          \
                      (const bf16_t*)routing, seg_offsets,                                                                \

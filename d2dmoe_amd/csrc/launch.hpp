@@ -44,8 +44,12 @@ bool mfma_router_supported(const d2dmoe_shape& sh);
 size_t mfma_packed_bytes(const d2dmoe_shape& sh);
 hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                             const void* router_w1, const void* router_w2, void* packed, hipStream_t s);
+// seg_counts / seg_pairs (optional): where the expert-major plan keeps its per-segment counts; written by the router
+// kernel itself iff mfma_router_writes_plan_counts(sh), which saves that plan its first pass.
+bool mfma_router_writes_plan_counts(const d2dmoe_shape& sh);
 hipError_t launch_mfma_router_select(const d2dmoe_shape& sh, const void* x, const void* packed, void* routing,
-                                     void* norms_out, int32_t* counts, float thr_scale, hipStream_t s);
+                                     void* norms_out, int32_t* counts, float thr_scale, hipStream_t s,
+                                     int32_t* seg_counts = nullptr, int32_t* seg_pairs = nullptr);
 // With few tokens the sweep deals each tile's chunks to several workgroups and needs mfma_dense_workspace_bytes() of
 // workspace for their float32 sums (without it, or with skip_flag, it runs one workgroup per tile).
 size_t mfma_dense_workspace_bytes(const d2dmoe_shape& sh);
@@ -67,9 +71,11 @@ size_t mfma_sparse_fallback_offset(const d2dmoe_shape& sh);
 // Plans the call on the device (permutation, tiles, path flag), runs the expert-major kernels when the number of routed
 // pairs is at most n_tokens * max_mean_k, and leaves *flag == 0 otherwise so that the dense sweep (launched by the
 // caller with skip_flag = the returned pointer) does the work instead.
+// counts_ready: the per-segment counts are already in the workspace (mfma_sparse_plan_counts names the place).
 hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                               const void* last_bias, void* out, void* workspace, int max_mean_k, const int** flag_out,
-                              hipStream_t s);
+                              hipStream_t s, bool counts_ready = false);
+void mfma_sparse_plan_counts(const d2dmoe_shape& sh, void* workspace, int32_t** seg_counts, int32_t** seg_pairs);
 // ---- compacted two-kernel bf16 MFMA path for middling routing density (kernels_mid.hip) ----
 bool mfma_mid_supported(const d2dmoe_shape& sh);
 size_t mfma_mid_workspace_bytes(const d2dmoe_shape& sh);

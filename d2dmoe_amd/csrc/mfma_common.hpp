@@ -56,7 +56,7 @@ hipError_t launch_sparse_pack(const d2dmoe_shape& sh, const PackedLayout& L, con
 // Per-segment routed-token counts and their per-expert prefix over segments (plan passes 1 and 2 of the expert-major
 // paths): seg_counts[seg][e], seg_pairs[seg], then seg_offsets[seg][e] and totals[e].
 void launch_plan_count_scan(const void* routing, int64_t N, int E, int32_t* seg_counts, int32_t* seg_pairs,
-                            int32_t* seg_offsets, int32_t* totals, hipStream_t s);
+                            int32_t* seg_offsets, int32_t* totals, hipStream_t s, bool counts_ready = false);
 hipError_t launch_mid_pack(const d2dmoe_shape& sh, const PackedLayout& L, const void* w1, const void* w2, void* packed,
                            hipStream_t s);
 
