@@ -47,8 +47,8 @@ bool mfma_router_supported(const d2dmoe_shape& sh) {
 // The expert-major kernel covers the same layers as the dense sweep with experts of at most 128 neurons.
 // Gated experts have their own expert-major kernel, instantiated for D = 2048 and experts of at most 64 neurons (Gemma).
 bool mfma_sparse_supported(const d2dmoe_shape& sh) {
-  if (sh.dtype != D2DMOE_BF16) return false;
-  if (sh.gated) return sh.d_model == 2048 && sh.expert_dim <= 64 && sh.n_experts <= 1024;
+  if (sh.gated) return sh.dtype == D2DMOE_BF16 && sh.d_model == 2048 && sh.expert_dim <= 64 && sh.n_experts <= 1024;
+  if (sh.dtype != D2DMOE_BF16 && sh.dtype != D2DMOE_F16) return false;
   if (sh.d_model != 768) return false;
   return sh.expert_dim <= 128 && sh.n_experts <= 1024;
 }
@@ -236,29 +236,6 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
 // on LDS traffic only, so the global loads in flight survive them; GEMM2 of one chunk and GEMM1 of the next run
 // back to back between barriers.
 // ---------------------------------------------------------------------------------------------------
-// 16-bit storage of the sweep: bf16 (F16 = false) or IEEE half (F16 = true).  Both keep the same fragment layouts; what
-// differs is the MFMA instruction, the decoding of stored values and the final rounding.
-template <bool F16> __device__ __forceinline__ float dec16(uint32_t bits16) {       // low 16 bits -> float
-  if constexpr (F16) { _Float16 h; const uint16_t u = (uint16_t)bits16; __builtin_memcpy(&h, &u, 2); return (float)h; }
-  else return __uint_as_float(bits16 << 16);
-}
-template <bool F16> __device__ __forceinline__ float dec16_hi(uint32_t word) {      // high 16 bits -> float
-  if constexpr (F16) return dec16<true>(word >> 16);
-  else return __uint_as_float(word & 0xffff0000u);
-}
-template <bool F16> __device__ __forceinline__ uint32_t enc16x2(float lo, float hi) {
-  if constexpr (F16) return pack2_16<f16_t>(lo, hi);
-  else return pack2_bf16(lo, hi);
-}
-template <bool F16> __device__ __forceinline__ f32x16 mfma_32x32x16(const bf16x8& a, const bf16x8& b, const f32x16& c) {
-  if constexpr (F16) {
-    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  } else {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-}
-
 struct DenseArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* wp; const bf16_t* b1p; const uint8_t* eidx;
   const bf16_t* last_bias; bf16_t* out;

@@ -333,7 +333,7 @@ struct SparseArgs {
   const int32_t* tok_off; const bf16_t* last_bias; bf16_t* out; int add_residual;   // tokens with ONE routed expert
 };
 
-template <int D, int NT, int ACT>
+template <int D, int NT, int ACT, bool F16 = false>
 __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const SparseArgs A) {
   constexpr int KS1 = D / 16;
   constexpr int KQ = KS1 / 4;    // K steps per wave
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
     // A token with a single routed expert has nothing to be summed with: its row leaves this kernel as the finished
     // output row (float32 accumulator + last_bias (+ x), one rounding) and the combine kernel skips the token.
     const bool single = valid && (cur.t1 - cur.t0 == 1);
-    const float rw = bf16_to_f32(cur.rbits);
+    const float rw = dec16<F16>(cur.rbits);
     const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)tok * D) + 2 * w * KQ + g;
 
     // GEMM1, this wave's quarter of K: all loads are issued before the first MFMA
@@ -418,7 +418,7 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
     for (int ks = 0; ks < KQ; ++ks)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        acc1[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1f[(ks * NT + t) * 64], xb[ks], acc1[t], 0, 0, 0);
+        acc1[t] = mfma_32x32x16<F16>(w1f[(ks * NT + t) * 64], xb[ks], acc1[t]);
     // W2^T fragments of this wave's columns: requested now, used after the reduction
     const bf16x8* w2f = A.w2s + ((int64_t)e * (D / 32) + w * CTW) * (2 * NT) * 64 + lane;
     bf16x8 w2r[CTW * 2 * NT];
@@ -441,8 +441,7 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const uint2 bq = *(const uint2*)(bias_e + t * 32 + 8 * q + 4 * g);
-        const float bias[4] = {__uint_as_float(bq.x << 16), __uint_as_float(bq.x & 0xffff0000u),
-                               __uint_as_float(bq.y << 16), __uint_as_float(bq.y & 0xffff0000u)};
+        const float bias[4] = {dec16<F16>(bq.x & 0xffffu), dec16_hi<F16>(bq.x), dec16<F16>(bq.y & 0xffffu), dec16_hi<F16>(bq.y)};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int r = q * 4 + i;
@@ -456,10 +455,10 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         uint4 pk;
-        pk.x = pack2_bf16(hv[half * 8 + 0], hv[half * 8 + 1]);
-        pk.y = pack2_bf16(hv[half * 8 + 2], hv[half * 8 + 3]);
-        pk.z = pack2_bf16(hv[half * 8 + 4], hv[half * 8 + 5]);
-        pk.w = pack2_bf16(hv[half * 8 + 6], hv[half * 8 + 7]);
+        pk.x = enc16x2<F16>(hv[half * 8 + 0], hv[half * 8 + 1]);
+        pk.y = enc16x2<F16>(hv[half * 8 + 2], hv[half * 8 + 3]);
+        pk.z = enc16x2<F16>(hv[half * 8 + 4], hv[half * 8 + 5]);
+        pk.w = enc16x2<F16>(hv[half * 8 + 6], hv[half * 8 + 7]);
         __builtin_memcpy(&hb[t * 2 + half], &pk, 16);
       }
     }
@@ -474,7 +473,7 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
     for (int ct = 0; ct < CTW; ++ct)
 #pragma unroll
       for (int ks2 = 0; ks2 < 2 * NT; ++ks2)
-        acc2[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w2r[ct * 2 * NT + ks2], hb[ks2], acc2[ct], 0, 0, 0);
+        acc2[ct] = mfma_32x32x16<F16>(w2r[ct * 2 * NT + ks2], hb[ks2], acc2[ct]);
     const bool any_single = __ballot(single) != 0ull;   // uniform
     const int col0 = w * (D / 4) + 4 * g;
     if (any_single) {
@@ -487,17 +486,17 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
         for (int q = 0; q < 4; ++q) {
           uint2 lb = *(const uint2*)(s_last_bias + col0 + ct * 32 + 8 * q);
           lb.x &= keep; lb.y &= keep;
-          acc2[ct][q * 4 + 0] += __uint_as_float(lb.x << 16);
-          acc2[ct][q * 4 + 1] += __uint_as_float(lb.x & 0xffff0000u);
-          acc2[ct][q * 4 + 2] += __uint_as_float(lb.y << 16);
-          acc2[ct][q * 4 + 3] += __uint_as_float(lb.y & 0xffff0000u);
+          acc2[ct][q * 4 + 0] += dec16<F16>(lb.x & 0xffffu);
+          acc2[ct][q * 4 + 1] += dec16_hi<F16>(lb.x);
+          acc2[ct][q * 4 + 2] += dec16<F16>(lb.y & 0xffffu);
+          acc2[ct][q * 4 + 3] += dec16_hi<F16>(lb.y);
           if (A.add_residual) {   // uniform
             uint2 xv = *(const uint2*)(xres + ct * 32 + 8 * q);
             xv.x &= keep; xv.y &= keep;
-            acc2[ct][q * 4 + 0] += __uint_as_float(xv.x << 16);
-            acc2[ct][q * 4 + 1] += __uint_as_float(xv.x & 0xffff0000u);
-            acc2[ct][q * 4 + 2] += __uint_as_float(xv.y << 16);
-            acc2[ct][q * 4 + 3] += __uint_as_float(xv.y & 0xffff0000u);
+            acc2[ct][q * 4 + 0] += dec16<F16>(xv.x & 0xffffu);
+            acc2[ct][q * 4 + 1] += dec16_hi<F16>(xv.x);
+            acc2[ct][q * 4 + 2] += dec16<F16>(xv.y & 0xffffu);
+            acc2[ct][q * 4 + 3] += dec16_hi<F16>(xv.y);
           }
         }
     }
@@ -527,8 +526,8 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             uint2 o;
-            o.x = pack2_bf16(acc2[2 * ps + cta][q * 4 + 0], acc2[2 * ps + cta][q * 4 + 1]);
-            o.y = pack2_bf16(acc2[2 * ps + cta][q * 4 + 2], acc2[2 * ps + cta][q * 4 + 3]);
+            o.x = enc16x2<F16>(acc2[2 * ps + cta][q * 4 + 0], acc2[2 * ps + cta][q * 4 + 1]);
+            o.y = enc16x2<F16>(acc2[2 * ps + cta][q * 4 + 2], acc2[2 * ps + cta][q * 4 + 3]);
             *(uint2*)(stage + c32 * 128 + (((cta * 4 + q) ^ (c32 & 7)) * 16) + 8 * g) = o;
           }
         __builtin_amdgcn_wave_barrier();
@@ -546,6 +545,7 @@ __global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const Spars
 }
 
 // Ordered combine: thread = (token, 8 columns); the token's result rows are contiguous, experts ascending.
+template <bool F16 = false>
 __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__ y, const int32_t* __restrict__ tok_off,
                                                       const int32_t* __restrict__ flag, const bf16_t* __restrict__ x,
                                                       const bf16_t* __restrict__ last_bias, bf16_t* __restrict__ out, int64_t N,
@@ -572,30 +572,30 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__
     for (int u = 0; u < 8; ++u) {
       const uint32_t wd[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+      for (int i = 0; i < 8; ++i) acc[i] += (i & 1) ? dec16_hi<F16>(wd[i >> 1]) : dec16<F16>(wd[i >> 1] & 0xffffu);
     }
   }
   for (; q < q1; ++q) {
     const uint4 v = *(const uint4*)(y + (int64_t)q * D + col);
     const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+    for (int i = 0; i < 8; ++i) acc[i] += (i & 1) ? dec16_hi<F16>(wd[i >> 1]) : dec16<F16>(wd[i >> 1] & 0xffffu);
   }
   if (last_bias != nullptr) {
     const uint4 v = *(const uint4*)(last_bias + col);
     const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+    for (int i = 0; i < 8; ++i) acc[i] += (i & 1) ? dec16_hi<F16>(wd[i >> 1]) : dec16<F16>(wd[i >> 1] & 0xffffu);
   }
   if (add_residual) {
     const uint4 v = *(const uint4*)(x + n * D + col);
     const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += __uint_as_float((i & 1) ? (wd[i >> 1] & 0xffff0000u) : (wd[i >> 1] << 16));
+    for (int i = 0; i < 8; ++i) acc[i] += (i & 1) ? dec16_hi<F16>(wd[i >> 1]) : dec16<F16>(wd[i >> 1] & 0xffffu);
   }
   uint4 o;
-  o.x = pack2_bf16(acc[0], acc[1]); o.y = pack2_bf16(acc[2], acc[3]);
-  o.z = pack2_bf16(acc[4], acc[5]); o.w = pack2_bf16(acc[6], acc[7]);
+  o.x = enc16x2<F16>(acc[0], acc[1]); o.y = enc16x2<F16>(acc[2], acc[3]);
+  o.z = enc16x2<F16>(acc[4], acc[5]); o.w = enc16x2<F16>(acc[6], acc[7]);
   *(uint4*)(out + n * D + col) = o;
 }
 
@@ -777,15 +777,15 @@ static void launch_gated_sparse_experts(const SparseArgs& A, int act, unsigned g
   }
 }
 
-template <int NT>
+template <int NT, bool F16>
 static void launch_sparse_experts(const SparseArgs& A, int act, unsigned grid, hipStream_t s) {
   switch (act) {
     case D2DMOE_ACT_RELU:
-      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, D2DMOE_ACT_RELU>), dim3(grid), dim3(256), 0, s, A); break;
+      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, D2DMOE_ACT_RELU, F16>), dim3(grid), dim3(256), 0, s, A); break;
     case D2DMOE_ACT_GELU:
-      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, D2DMOE_ACT_GELU>), dim3(grid), dim3(256), 0, s, A); break;
+      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, D2DMOE_ACT_GELU, F16>), dim3(grid), dim3(256), 0, s, A); break;
     default:
-      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, -1>), dim3(grid), dim3(256), 0, s, A); break;
+      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, -1, F16>), dim3(grid), dim3(256), 0, s, A); break;
   }
 }
 
@@ -855,13 +855,18 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   A.tok_off = tok_off; A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.add_residual = sh.add_residual;
   A.wus = (const bf16x8*)(pk + L.su_off);
   const unsigned grid = (unsigned)(8 * device_cu_count());
+  const bool f16 = sh.dtype == D2DMOE_F16;   // ungated layers only (mfma_sparse_supported)
   if (sh.gated) launch_gated_sparse_experts(A, sh.activation, grid, s);
-  else if (L.nt == 1) launch_sparse_experts<1>(A, sh.activation, grid, s);
-  else if (L.nt == 2) launch_sparse_experts<2>(A, sh.activation, grid, s);
-  else launch_sparse_experts<4>(A, sh.activation, grid, s);
+  else if (L.nt == 1) { if (f16) launch_sparse_experts<1, true>(A, sh.activation, grid, s); else launch_sparse_experts<1, false>(A, sh.activation, grid, s); }
+  else if (L.nt == 2) { if (f16) launch_sparse_experts<2, true>(A, sh.activation, grid, s); else launch_sparse_experts<2, false>(A, sh.activation, grid, s); }
+  else { if (f16) launch_sparse_experts<4, true>(A, sh.activation, grid, s); else launch_sparse_experts<4, false>(A, sh.activation, grid, s); }
   const int64_t n_threads = N * (sh.d_model / 8);
-  hipLaunchKernelGGL(combine_kernel, dim3((unsigned)cdiv64(n_threads, 256)), dim3(256), 0, s, y, tok_off, flag, (const bf16_t*)x,
-                     (const bf16_t*)last_bias, (bf16_t*)out, N, sh.d_model, sh.add_residual, sh.gated ? 0 : 1);
+  if (f16)
+    hipLaunchKernelGGL(combine_kernel<true>, dim3((unsigned)cdiv64(n_threads, 256)), dim3(256), 0, s, y, tok_off, flag, (const bf16_t*)x,
+                       (const bf16_t*)last_bias, (bf16_t*)out, N, sh.d_model, sh.add_residual, sh.gated ? 0 : 1);
+  else
+    hipLaunchKernelGGL(combine_kernel<false>, dim3((unsigned)cdiv64(n_threads, 256)), dim3(256), 0, s, y, tok_off, flag, (const bf16_t*)x,
+                       (const bf16_t*)last_bias, (bf16_t*)out, N, sh.d_model, sh.add_residual, sh.gated ? 0 : 1);
   *flag_out = flag;
   return hipGetLastError();
 }

@@ -78,6 +78,29 @@ template <> __device__ inline uint32_t pack2_16<f16_t>(float lo, float hi) {
   return u;
 }
 
+// 16-bit storage of the MFMA kernels that take both: bf16 (F16 = false) or IEEE half (F16 = true).  Fragment layouts are
+// the same; what differs is the MFMA instruction, the decoding of stored values and the final rounding.
+template <bool F16> __device__ __forceinline__ float dec16(uint32_t bits16) {       // low 16 bits -> float
+  if constexpr (F16) { _Float16 h; const uint16_t u = (uint16_t)bits16; __builtin_memcpy(&h, &u, 2); return (float)h; }
+  else return __uint_as_float(bits16 << 16);
+}
+template <bool F16> __device__ __forceinline__ float dec16_hi(uint32_t word) {      // high 16 bits -> float
+  if constexpr (F16) return dec16<true>(word >> 16);
+  else return __uint_as_float(word & 0xffff0000u);
+}
+template <bool F16> __device__ __forceinline__ uint32_t enc16x2(float lo, float hi) {
+  if constexpr (F16) return pack2_16<f16_t>(lo, hi);
+  else return pack2_bf16(lo, hi);
+}
+template <bool F16> __device__ __forceinline__ f32x16 mfma_32x32x16(const bf16x8& a, const bf16x8& b, const f32x16& c) {
+  if constexpr (F16) {
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+}
+
 // LDS-only workgroup barrier: waits for this wave's LDS operations, not for its outstanding global loads.
 __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 

@@ -173,6 +173,38 @@ def test_dense_sweep_f16(N, E, Ed, density, act):
     assert torch.equal(zero.float(), p['last_bias'].expand(N, -1).float())
 
 
+@pytest.mark.parametrize('N,E,Ed,density,act', [(197, 128, 24, 0.02, 'relu'), (1576, 128, 24, 0.03, 'gelu'), (65, 128, 24, 0.05, 'relu'),
+                                                (1, 128, 24, 0.2, 'relu'), (300, 24, 128, 0.2, 'relu'), (700, 100, 30, 0.06, 'tanh'),
+                                                (600, 64, 40, 0.1, 'relu'), (50432, 128, 24, 0.017, 'relu')])
+def test_expert_major_f16(N, E, Ed, density, act):
+    """The expert-major path (plan, experts, ordered combine) with float16 storage: against the float64 oracle (on row
+    slices at 50 432 tokens), single-expert and no-expert tokens, weighted routing + residual, the over-capacity
+    fall-back to the sweep, run-to-run bit equality."""
+    _say('f16 expert-major', N, E, Ed, density, act)
+    D, W = 768, 128
+    x, routing, p = H.random_case(N, D, E, Ed, W, seed=N + E, dtype=F16, density=density)
+    if N > 4:
+        routing[1] = 0
+        routing[2] = 0
+        routing[2, E // 2] = 1      # one expert: finished inside the experts kernel
+        routing[3] = 1              # every expert
+    packed = _pack(p, D, E, Ed, W, act, False)
+    got = _got(x, routing, p, act, path='mfma_sparse', packed=packed)
+    rows = slice(0, N) if N <= 4096 else slice(N - 3000, N)
+    pr = {k: v for k, v in p.items()}
+    assert H.rel_err(got[rows], _want(x[rows], routing[rows], pr, act)) < TOL_F16
+    assert torch.equal(got, _got(x, routing, p, act, path='mfma_sparse', packed=packed))
+    assert H.rel_err(got, _got(x, routing, p, act, path='mfma_dense', packed=packed)) < TOL_F16
+    if N <= 4096:
+        g = torch.Generator().manual_seed(3)
+        weights = (routing.float() * (torch.rand(N, E, generator=g) + 0.5)).half()
+        got = _got(x, weights, p, act, residual=True, path='mfma_sparse', packed=packed)
+        assert H.rel_err(got, _want(x, weights, p, act, True)) < TOL_F16
+        dense_routing = (torch.rand(N, E, generator=g) < 0.9).half()     # beyond the capacity: the sweep does the work
+        got = _got(x, dense_routing, p, act, path='mfma_sparse', packed=packed)
+        assert H.rel_err(got, _want(x, dense_routing, p, act)) < TOL_F16
+
+
 @pytest.mark.parametrize('tau', [0.9, 0.1])
 def test_layer_f16_vit_shape(tau):
     """Whole layer (router -> dynamic-k selection -> experts) at the ViT-B shape, 1576 tokens, float16 storage."""
@@ -195,6 +227,6 @@ def test_bf16_only_paths_refuse_f16():
     from d2dmoe_amd.hip_abi import D2DMoEError
     x, routing, p = H.random_case(64, 768, 128, 24, 128, seed=1, dtype=F16)
     packed = _pack(p, 768, 128, 24, 128, 'relu', False)
-    for path in ('mfma_sparse', 'mfma_decode', 'mfma_mid'):
+    for path in ('mfma_decode', 'mfma_mid'):
         with pytest.raises(D2DMoEError):
             _got(x, routing, p, 'relu', path=path, packed=packed)
