@@ -174,8 +174,8 @@ def test_dense_sweep_f16(N, E, Ed, density, act):
 
 
 @pytest.mark.parametrize('N,E,Ed,density,act', [(197, 128, 24, 0.02, 'relu'), (1576, 128, 24, 0.03, 'gelu'), (65, 128, 24, 0.05, 'relu'),
-                                                (1, 128, 24, 0.2, 'relu'), (300, 24, 128, 0.2, 'relu'), (700, 100, 30, 0.06, 'tanh'),
-                                                (600, 64, 40, 0.1, 'relu'), (50432, 128, 24, 0.017, 'relu')])
+                                                (1, 128, 24, 0.2, 'relu'), (300, 24, 128, 0.1, 'relu'), (700, 100, 30, 0.06, 'tanh'),
+                                                (600, 64, 40, 0.06, 'relu'), (50432, 128, 24, 0.017, 'relu')])
 def test_expert_major_f16(N, E, Ed, density, act):
     """The expert-major path (plan, experts, ordered combine) with float16 storage: against the float64 oracle (on row
     slices at 50 432 tokens), single-expert and no-expert tokens, weighted routing + residual, the over-capacity
