@@ -261,7 +261,9 @@ static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* ro
     case D2DMOE_PATH_MFMA_SPARSE: {
       // expert-major when the routed pairs fit the provisioned capacity, else the dense sweep: decided on the device
       if (!mfma_sparse_supported(sh)) return D2DMOE_E_UNSUPPORTED;
-      if (sh.gated ? !mfma_gemm_supported(sh) : !mfma_dense_supported(sh)) return D2DMOE_E_UNSUPPORTED;
+      // the fall-back: the dense sweep where it exists (ungated, D = 768), else the tiled products
+      const bool fb_gemm = sh.gated || !mfma_dense_supported(sh);
+      if (fb_gemm && !mfma_gemm_supported(sh)) return D2DMOE_E_UNSUPPORTED;
       if (!packed) return D2DMOE_E_NULL;
       const size_t need = mfma_sparse_workspace_bytes(sh);
       if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
@@ -271,7 +273,7 @@ static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* ro
       if (e != hipSuccess) return (int)e;
       // with every expert routed to by every token the pairs still fit: the fall-back can never be needed
       if (sh.n_tokens * (int64_t)sh.n_experts <= mfma_sparse_capacity_pairs(sh)) return D2DMOE_OK;
-      if (sh.gated)   // gated layers fall back to the tiled products, which work behind the plan in the same workspace
+      if (fb_gemm)   // the tiled products work behind the plan in the same workspace
         return (int)launch_mfma_gemm(sh, x, routing, (const char*)packed + mfma_gemm_section_offset(sh), last_bias, out,
                                      (char*)workspace + mfma_sparse_fallback_offset(sh), s, flag);
       return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, nullptr, 0, s);
@@ -392,7 +394,7 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   // products pay for with whole 256-token tiles)
   if (path == D2DMOE_PATH_AUTO && sh.n_tokens > (sh.gated && mfma_decode_supported(sh) ? 48 : 16) && packed != nullptr &&
       (thr_scale >= (sh.gated ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128)) && mfma_sparse_supported(sh) &&
-      (sh.gated ? mfma_gemm_supported(sh) : mfma_dense_supported(sh)))
+      ((!sh.gated && mfma_dense_supported(sh)) || mfma_gemm_supported(sh)))
     path = D2DMOE_PATH_MFMA_SPARSE;
   // ... and when the router kernel of this call is the one that walks the 32-token segments of that path's plan, it
   // leaves the plan's per-segment counts in the workspace on its way

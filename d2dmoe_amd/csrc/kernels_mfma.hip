@@ -49,8 +49,12 @@ bool mfma_router_supported(const d2dmoe_shape& sh) {
 bool mfma_sparse_supported(const d2dmoe_shape& sh) {
   if (sh.gated) return sh.dtype == D2DMOE_BF16 && sh.d_model == 2048 && sh.expert_dim <= 64 && sh.n_experts <= 1024;
   if (sh.dtype != D2DMOE_BF16 && sh.dtype != D2DMOE_F16) return false;
-  if (sh.d_model != 768) return false;
-  return sh.expert_dim <= 128 && sh.n_experts <= 1024;
+  if (sh.n_experts > 1024) return false;
+  if (sh.d_model == 768) return sh.expert_dim <= 128;
+  // wider models: the registers a wave needs grow with D and with the expert's row tiles
+  if (sh.d_model == 1024) return sh.expert_dim <= 64;
+  if (sh.d_model == 1280) return sh.expert_dim <= 32;
+  return false;
 }
 
 PackedLayout packed_layout(const d2dmoe_shape& sh) {

@@ -32,6 +32,9 @@ struct SparseWorkspace {
 // 64 x 48, 48 x 64, 32 x 96 and 24 x 128 experts at D = 768).
 int mfma_sparse_capacity_k(const d2dmoe_shape& sh) {
   if (sh.gated) return (sh.n_tokens <= 16384) ? SP_MAX_MEAN_K_GATED : SP_MAX_MEAN_K;
+  // D = 1024 / 1280: the alternative is the tiled products (1.3 ms at 50 432 tokens, 128 experts x 32, against 0.19 ms +
+  // 0.085 ms per routed expert per token here): equal at about 13
+  if (sh.d_model != 768) return sh.expert_dim <= 32 ? 12 : 6;
   return sh.expert_dim <= 32 ? SP_MAX_MEAN_K : (sh.expert_dim <= 64 ? 5 : 3);
 }
 
@@ -57,7 +60,7 @@ static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) 
   W.token_idx = take((size_t)W.cap * 4);
   W.pair_dst = take((size_t)W.cap * 4);
   size_t ybytes = (size_t)W.cap * sh.d_model * 2;
-  if (sh.gated) {   // the fall-back of a gated layer (tiled products) works in the same region
+  if (sh.gated || sh.d_model != 768) {   // where the fall-back is the tiled products, they work in the same region
     const size_t g = mfma_gemm_workspace_bytes(sh);
     if (g > ybytes) ybytes = g;
   }
@@ -338,7 +341,7 @@ struct SparseArgs {
 };
 
 template <int D, int NT, int ACT, bool F16 = false>
-__global__ __launch_bounds__(256, 3) void experts_mfma_sparse_kernel(const SparseArgs A) {
+__global__ __launch_bounds__(256, ((D <= 768 && NT < 4) ? 3 : 1)) void experts_mfma_sparse_kernel(const SparseArgs A) {
   constexpr int KS1 = D / 16;
   constexpr int KQ = KS1 / 4;    // K steps per wave
   constexpr int CTW = D / 128;   // column tiles per wave
@@ -793,6 +796,14 @@ static void launch_sparse_experts(const SparseArgs& A, int act, unsigned grid, h
   }
 }
 
+// The wider models (D = 1024: GPT-2 medium, BERT-large, ViT-L; D = 1280: GPT-2 large): the same kernel with the
+// activation chosen at run time, at one workgroup per CU (a wave's x fragments, W2^T fragments and output accumulators
+// grow with D: 300 - 370 registers).
+template <int D, int NT, bool F16>
+static void launch_sparse_experts_wide(const SparseArgs& A, unsigned grid, hipStream_t s) {
+  hipLaunchKernelGGL((experts_mfma_sparse_kernel<D, NT, -1, F16>), dim3(grid), dim3(256), 0, s, A);
+}
+
 void launch_plan_count_scan(const void* routing, int64_t N, int E, int32_t* seg_counts, int32_t* seg_pairs,
                             int32_t* seg_offsets, int32_t* totals, hipStream_t s, bool counts_ready) {
   const int64_t n_seg = cdiv64(N, SP_SEG);
@@ -861,6 +872,12 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   const unsigned grid = (unsigned)(8 * device_cu_count());
   const bool f16 = sh.dtype == D2DMOE_F16;   // ungated layers only (mfma_sparse_supported)
   if (sh.gated) launch_gated_sparse_experts(A, sh.activation, grid, s);
+  else if (sh.d_model == 1024) {
+    if (L.nt == 1) { if (f16) launch_sparse_experts_wide<1024, 1, true>(A, grid, s); else launch_sparse_experts_wide<1024, 1, false>(A, grid, s); }
+    else { if (f16) launch_sparse_experts_wide<1024, 2, true>(A, grid, s); else launch_sparse_experts_wide<1024, 2, false>(A, grid, s); }
+  } else if (sh.d_model == 1280) {
+    if (f16) launch_sparse_experts_wide<1280, 1, true>(A, grid, s); else launch_sparse_experts_wide<1280, 1, false>(A, grid, s);
+  }
   else if (L.nt == 1) { if (f16) launch_sparse_experts<1, true>(A, sh.activation, grid, s); else launch_sparse_experts<1, false>(A, sh.activation, grid, s); }
   else if (L.nt == 2) { if (f16) launch_sparse_experts<2, true>(A, sh.activation, grid, s); else launch_sparse_experts<2, false>(A, sh.activation, grid, s); }
   else { if (f16) launch_sparse_experts<4, true>(A, sh.activation, grid, s); else launch_sparse_experts<4, false>(A, sh.activation, grid, s); }

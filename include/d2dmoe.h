@@ -71,7 +71,8 @@ enum {
   D2DMOE_PATH_MFMA_DENSE = 2, /* bf16 or f16 MFMA, token-tile-major, masked dense sweep over all experts */
   D2DMOE_PATH_MFMA_SPARSE = 3, /* bf16 (ungated: or f16) MFMA, expert-major over the permutation, then ordered combine; taken when at most
                                  8 experts per token are routed on average (checked on the device), else the dense
-                                 sweep runs.  Ungated experts at D = 768.  Gated experts at D = 2048 with at most 64
+                                 sweep runs.  Ungated experts at D = 768 (also D = 1024 with at most 64 neurons and D = 1280 with at
+                                 most 32: up to 12 / 6 experts per token, tiled products as fall-back).  Gated experts at D = 2048 with at most 64
                                  neurons: up to 32 experts per token (8 beyond 16 384 tokens), else the tiled products
                                  run.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 (gated: >= 0.5) */
   D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 MFMA for a handful of tokens: per pass of 16 tokens one workgroup per expert streams

@@ -265,6 +265,62 @@ def test_experts_mfma_sparse_matches_oracle(N, E, Ed, density):
     assert torch.equal(got, _experts_got(x, routing, p, 'relu', path='mfma_sparse', packed=packed))   # deterministic
 
 
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('N,D,E,Ed,density,act', [(300, 1024, 128, 32, 0.03, 'gelu'), (1576, 1024, 128, 32, 0.02, 'relu'),
+                                                  (700, 1024, 64, 64, 0.05, 'relu'), (333, 1024, 100, 20, 0.04, 'tanh'),
+                                                  (1, 1024, 128, 32, 0.05, 'relu'), (900, 1280, 160, 32, 0.03, 'gelu'),
+                                                  (20000, 1024, 128, 32, 0.017, 'gelu')])
+def test_experts_mfma_sparse_wide_models(N, D, E, Ed, density, act, dtype):
+    """The expert-major path at the widths of GPT-2 medium / BERT-large / ViT-L (D = 1024) and GPT-2 large (D = 1280): against
+    the float64 oracle (row slices at 20 000 tokens) and the tiled products, single-expert / no-expert / all-expert
+    tokens, weighted routing + residual, run-to-run bit equality, and the over-capacity fall-back, which at these widths
+    is the tiled products working behind the plan in the same workspace."""
+    _say('experts sparse wide', N, D, E, Ed, density, act, dtype)
+    tol = H.tol_for(dtype)
+    x, routing, p = H.random_case(N, D, E, Ed, 8, seed=N + D + E, dtype=dtype, density=density)
+    if N > 4:
+        routing[1] = 0
+        routing[2] = 0
+        routing[2, E // 2] = 1
+        routing[3] = 1
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, 0, 1 if dtype == torch.bfloat16 else 2, act)
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, None, None)
+    assert packed is not None
+    got = _experts_got(x, routing, p, act, path='mfma_sparse', packed=packed)
+    rows = slice(0, N) if N <= 4096 else slice(N - 2500, N)
+    assert H.rel_err(got[rows], _experts_want(x[rows], routing[rows], p, act)) < tol
+    assert torch.equal(got, _experts_got(x, routing, p, act, path='mfma_sparse', packed=packed))
+    if N > 16:
+        assert H.rel_err(got, _experts_got(x, routing, p, act, path='mfma_gemm', packed=packed)) < tol
+    if N <= 4096:
+        g = torch.Generator().manual_seed(5)
+        weights = (routing.float() * (torch.rand(N, E, generator=g) + 0.5)).to(dtype)
+        got = _experts_got(x, weights, p, act, residual=True, path='mfma_sparse', packed=packed)
+        assert H.rel_err(got, _experts_want(x, weights, p, act, True)) < tol
+        dense_routing = (torch.rand(N, E, generator=g) < 0.6).to(dtype)   # beyond the capacity
+        got = _experts_got(x, dense_routing, p, act, path='mfma_sparse', packed=packed)
+        assert H.rel_err(got, _experts_want(x, dense_routing, p, act)) < tol
+
+
+@pytest.mark.parametrize('tau', [0.9, 0.1])
+def test_layer_wide_model_auto(tau):
+    """Whole layer at D = 1024 (128 experts x 32, GELU) under AUTO at 2000 tokens: the literal rule takes the expert-major
+    path, the module reading the tiled products; mask exact for the kernel's own norms, output against the oracle."""
+    N, D, E, Ed, W = 2000, 1024, 128, 32, 128
+    _say('layer wide', tau)
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=21, dtype=torch.bfloat16)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, W, 1, 'gelu')
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, d['router_w1'], d['router_w2'])
+    out, routing, norms, counts = _ops().forward(x.to(DEV), d['router_w1'], d['router_w2'], float(1.0 - tau), d['w1'], d['b1'],
+                                                 d['w2'], None, d['last_bias'].view(-1), 'gelu', False, None, True, True, 'auto',
+                                                 packed)
+    assert torch.equal(routing.cpu(), O.gate_dynk_max(norms.cpu(), tau))
+    assert torch.equal(counts.cpu().long(), (routing.cpu() > 0).sum(0))
+    assert H.rel_err(out.cpu(), _experts_want(x, routing.cpu(), p, 'gelu')) < H.TOL_BF16
+
+
 @pytest.mark.parametrize('act', ['relu', 'gelu', 'tanh'])
 def test_experts_mfma_sparse_activations_weights_edges(act):
     x, routing, p = H.random_case(500, 768, 128, 24, 8, seed=41, dtype=torch.bfloat16, density=0.03)
