@@ -46,8 +46,11 @@ WORKLOADS = {
     'vit_b_skew': (256, 197, 768, 128, 24, 128, 'relu'),
     # the CPU baseline's own case (8 x 197 tokens, float32) on the GPU: float32 storage and float32 matrix arithmetic
     'vit_b_1576_f32': (8, 197, 768, 128, 24, 128, 'relu'),
-    # float16 storage (the reference benches float32 and float16): router on an MFMA linear kernel, experts on the tiled products
+    # float16 storage (the reference benches float32 and float16): same kernel families as bf16
     'vit_b_50k_f16': (256, 197, 768, 128, 24, 128, 'relu'),
+    # one FFN layer of a GPT-2-medium-sized model (D = 1024, d_ff = 4096 as 128 experts x 32, GELU), 16 x 1024 tokens:
+    # tiled products under module tau 0.9, expert-major kernels under the literal rule
+    'gpt2_medium_layer': (16, 1024, 1024, 128, 32, 128, 'gelu'),
 }
 TRAFFIC_TABLE = os.path.join(ROOT, 'profiles', 'traffic_per_launch.md')
 
@@ -195,8 +198,8 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, pa
     # the same step replayed from a HIP graph: removes the host's launch latency between the dependent kernels
     ms_layer = time_graph(layer, steps, warmup)
     # dominant kernel alone (same routing), HIP events on the launch stream
-    # the experts call the layer makes: under AUTO d2dmoe_forward takes the expert-major path for high thresholds (bf16)
-    experts_path = path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 and x.dtype == torch.bfloat16 else 'auto')
+    # the experts call the layer makes: under AUTO d2dmoe_forward takes the expert-major path for high thresholds
+    experts_path = path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 and x.dtype in (torch.bfloat16, torch.float16) else 'auto')
     ms_experts = time_events(lambda: ops.experts(x, routing, p['w1'], p['b1'], p['w2'], None, p['last_bias'], act, False,
                                                  experts_path, packed), steps, warmup)
     quant = None
