@@ -3,7 +3,8 @@
 Called through the C ABI; its outputs are compared bit for bit with d2dmoe_forward's (same kernels, caller-owned
 workspace) on two calls in a row, the second with a smaller input, so that whatever the first call left in the array is
 there when the second runs.  Covers a path per workspace use: dense sweep with chunk-split tail (float32 partial sums),
-expert-major (plan, per-pair rows, device flag), small batch (hidden fragments, expert flags), tiled products.
+expert-major (plan, per-pair rows, device flag; also with the plan's first pass written by the router kernel, and at
+D = 1024 with the tiled products' region behind it), small batch (hidden fragments, expert flags), tiled products.
 """
 import ctypes
 
@@ -32,6 +33,9 @@ def _call(static, x, d, tau, act, gated, packed, bufs=None):
     ('gemma small batch', 2048, 256, 64, 256, 'gelu_tanh', True, 0.9, (16, 5)),
     ('gemma tiled products', 2048, 256, 64, 256, 'gelu_tanh', True, 0.9, (600, 200)),
     ('gemma expert-major', 2048, 256, 64, 256, 'gelu_tanh', True, 0.1, (300, 100)),
+    # from 16 384 tokens on the router kernel also writes the expert-major plan's per-segment counts into the workspace
+    ('vit expert-major, resident router', 768, 128, 24, 128, 'relu', False, 0.1, (16500, 16390)),
+    ('gpt2-medium width expert-major', 1024, 128, 32, 128, 'gelu', False, 0.1, (2000, 700)),
 ])
 def test_static_workspace_forward_equals_forward(name, D, E, Ed, W, act, gated, tau, sizes):
     from d2dmoe_amd import ops
