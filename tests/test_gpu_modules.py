@@ -143,6 +143,39 @@ def test_every_container_runs_the_hip_kernels(experts_class, gated, dtype):
         assert 0 < routing.sum() < routing.numel()
 
 
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('tau', [0.9, 0.1])
+def test_wide_model_layer_through_the_module(tau, dtype):
+    """A converted FFN of GPT-2-medium / BERT-large width (D = 1024, 128 experts x 32, GELU) through MoeficationMoE in 'hip'
+    mode, 2 x 1000 tokens: under the literal reading the fused call takes the expert-major kernels, under module tau 0.9
+    the tiled products; mask from the oracle gate on the module's own norms, output against the float64 oracle."""
+    from d2dmoe_amd import MoeficationMoE, MoeficationRouter
+    _say('wide module', tau, dtype)
+    D, E, Ed = 1024, 128, 32
+    torch.manual_seed(9)
+    moe = MoeficationMoE('m', D, E, True, Ed, nn.GELU, experts_class='custom_kernel')
+    with torch.no_grad():
+        moe.last_bias.normal_(0, 0.05)
+    moe.router = MoeficationRouter(D, E, width=128, depth=2, bias=False, activation='relu', output_activation='abs')
+    moe = moe.to(DEV).to(dtype).eval()
+    moe.forward_mode, moe.tau = 'dynk_max', tau
+    moe.experts.forward_mode = 'hip'
+    x = torch.randn(2, 1000, D, generator=torch.Generator().manual_seed(2)).to(dtype).to(DEV)
+    with torch.no_grad():
+        moe.collect_counts = True
+        out, gating = moe(x)
+    routing = gating['m'][0].reshape(-1, E).cpu()
+    assert torch.equal(moe.last_expert_counts.cpu().long(), routing.float().sum(0).long())
+    p, act = _layer_params(moe)
+    norms = O.router_forward(x.reshape(-1, D).cpu(), p['router_w1'], p['router_w2'])
+    flips = (routing != O.gate_dynk_max(norms, tau)).float().mean().item()
+    assert flips < 2e-3
+    want = O.layer_from_routing(x.reshape(-1, D).cpu().double(), O.upcast(p), routing.double(), act, 'all')
+    assert H.rel_err(out.reshape(-1, D).cpu(), want) < H.tol_for(dtype)
+    k = routing.sum(1).mean().item()
+    assert (k < 8) if tau < 0.5 else (k > 50)
+
+
 # =================================================================== the other gates feed the HIP experts (a3) ============
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('mode', ['all', 'topk', 'dynk'])
