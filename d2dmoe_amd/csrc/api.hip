@@ -128,8 +128,9 @@ int d2dmoe_router(const void* x, const void* router_w1, const void* router_w2, v
   hipError_t e;
   if (linear_skinny_supported(n_tokens, d_model, dtype) && linear_skinny_supported(n_tokens, router_width, dtype)) {
     // a handful of tokens: MFMA kernels that spread the output features over the machine
-    e = launch_linear_skinny(x, router_w1, workspace, (int)n_tokens, d_model, router_width, activation, s);
-    if (e == hipSuccess) e = launch_linear_skinny(workspace, router_w2, norms, (int)n_tokens, router_width, n_experts, output_activation, s);
+    e = launch_linear_skinny(x, router_w1, workspace, (int)n_tokens, d_model, router_width, activation, s, dtype);
+    if (e == hipSuccess)
+      e = launch_linear_skinny(workspace, router_w2, norms, (int)n_tokens, router_width, n_experts, output_activation, s, dtype);
   } else if (dtype == D2DMOE_F32) {
     // float32 on the matrix cores where the widths allow 16-byte operand loads and whole 32-column tiles
     const bool m1 = linear_mfma_f32_supported(n_tokens, d_model, router_width) && aligned16(x) && aligned16(router_w1);

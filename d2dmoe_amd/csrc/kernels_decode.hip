@@ -40,7 +40,7 @@ static DecodeLayout decode_layout(const d2dmoe_shape& sh) {
 }
 
 bool mfma_decode_supported(const d2dmoe_shape& sh) {
-  if (sh.dtype != D2DMOE_BF16) return false;
+  if (sh.dtype != D2DMOE_BF16 && sh.dtype != D2DMOE_F16) return false;
   if (sh.d_model % 256 != 0 || sh.d_model > 4096) return false;   // an even number of whole 32-steps per wave
   const int edp = (sh.expert_dim + 31) / 32 * 32;
   return edp == 32 || edp == 64 || edp == 128;
@@ -150,6 +150,7 @@ struct DecodeArgs {
 // First router layer inside the hidden kernel's launch: 4 features per workgroup of 4 waves.  K is cut into the same parts
 // as by linear_skinny_kernel (16 where K is long, else 4), each part accumulated on its own in K order and the parts
 // summed in order, so the result has the bits that kernel produces.
+template <bool F16>
 __device__ __forceinline__ void decode_router_l1_block(const DecodeArgs& A, int blk, float (*part)[4][64]) {
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
   const int gq = lane >> 4, c16 = lane & 15;
@@ -174,7 +175,7 @@ __device__ __forceinline__ void decode_router_l1_block(const DecodeArgs& A, int 
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
-        if (ks0 + u < KQ / 32) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv[u], av[u], acc, 0, 0, 0);
+        if (ks0 + u < KQ / 32) acc = mfma_16x16x32<F16>(bv[u], av[u], acc);
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) part[p][r][lane] = acc[r];
@@ -187,14 +188,14 @@ __device__ __forceinline__ void decode_router_l1_block(const DecodeArgs& A, int 
       for (int pp = 1; pp < P; ++pp) v += part[pp][r][lane];
       const int f = f0 + r;
       if (f < Nout) {
-        const float vr = bf16_to_f32(f32_to_bf16(v));
-        A.rhidden[(int64_t)c16 * Nout + f] = f32_to_bf16(apply_act(A.ract, vr));
+        const float vr = round16<F16>(v);
+        A.rhidden[(int64_t)c16 * Nout + f] = enc16<F16>(apply_act(A.ract, vr));
       }
     }
   }
 }
 
-template <bool GATED, int U1>
+template <bool GATED, int U1, bool F16 = false>
 __global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) {
   __shared__ float part_raw[16 * 4 * 64];          // [4][NM * 8][64] here, [16][4][64] for the router workgroups
   float (*part)[(GATED ? 2 : 1) * 8][64] = (float (*)[(GATED ? 2 : 1) * 8][64])part_raw;
@@ -203,7 +204,7 @@ __global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) 
   // ready long before the grid has drained)
   const int n_router = A.fused ? (A.rwidth + 3) / 4 : 0;
   if ((int)blockIdx.x < n_router) {
-    decode_router_l1_block(A, (int)blockIdx.x, (float (*)[4][64])part_raw);
+    decode_router_l1_block<F16>(A, (int)blockIdx.x, (float (*)[4][64])part_raw);
     return;
   }
   const int hb = (int)blockIdx.x - n_router;
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) 
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
   const int gq = lane >> 4, c16 = lane & 15;
   const int tc = (c16 < N) ? c16 : (N - 1);
-  const bf16_t rbits = A.fused ? (bf16_t)0x3f80 : A.routing[(int64_t)tc * E + e];   // fused: the routing is applied later
+  const bf16_t rbits = A.fused ? (bf16_t)(F16 ? 0x3c00 : 0x3f80) : A.routing[(int64_t)tc * E + e];   // fused: the routing is applied later
   const bool any = __ballot((rbits & 0x7fff) != 0) != 0ull;
   if (!A.fused && k2 == 0 && t == 0) A.active[e] = any ? 1 : 0;
   if (!any) return;   // nobody routes to this expert: its fragments are never read
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) 
       for (int m = 0; m < NM; ++m)
 #pragma unroll
         for (int a = 0; a < 2; ++a)
-          acc1[m][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wr[u][m * 2 + a], xb[u], acc1[m][a], 0, 0, 0);
+          acc1[m][a] = mfma_16x16x32<F16>(wr[u][m * 2 + a], xb[u], acc1[m][a]);
   };
   fill(wA, xA, 0);
   for (int ks0 = 0; ks0 < KQ; ks0 += 2 * U1) {
@@ -266,7 +267,7 @@ __global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) 
   if (w != 0) return;
   // ---- hidden activations -> the block's B fragment of GEMM2.  Rows of x beyond N were copies of row N-1; their
   // columns are zeroed here and never stored by the output kernel.
-  const float rw = (c16 < N) ? bf16_to_f32(rbits) : 0.f;
+  const float rw = (c16 < N) ? dec16<F16>(rbits) : 0.f;
   const bf16_t* bias_e = A.bias + (int64_t)e * NT16 * 16 + k2 * 32;
   float hv[8];
 #pragma unroll
@@ -282,13 +283,13 @@ __global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) 
     if (GATED) {
       v = apply_act(A.act, gsum) * usum;
     } else {
-      v = apply_act(A.act, gsum + bf16_to_f32(bias_e[a * 16 + 4 * gq + r]));
+      v = apply_act(A.act, gsum + dec16<F16>(bias_e[a * 16 + 4 * gq + r]));
     }
     hv[i] = (c16 < N) ? v * rw : 0.f;
   }
   uint4 pk;
-  pk.x = pack2_bf16(hv[0], hv[1]); pk.y = pack2_bf16(hv[2], hv[3]);
-  pk.z = pack2_bf16(hv[4], hv[5]); pk.w = pack2_bf16(hv[6], hv[7]);
+  pk.x = enc16x2<F16>(hv[0], hv[1]); pk.y = enc16x2<F16>(hv[2], hv[3]);
+  pk.z = enc16x2<F16>(hv[4], hv[5]); pk.w = enc16x2<F16>(hv[6], hv[7]);
   ((uint4*)A.hfrag)[((int64_t)e * KS2 + k2) * 64 + lane] = pk;
 }
 
@@ -296,7 +297,7 @@ constexpr int DO_WAVES = 8;
 
 // Workgroup = 8 output columns, 8 waves; wave w owns experts [w*EW, (w+1)*EW) with EW = ceil(E/8) rounded up to 64 at
 // most per pass, and walks the routed ones among them in ascending order.
-template <int KS2>
+template <int KS2, bool F16 = false>
 __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeArgs A) {
   constexpr int UB = 8 / KS2;                  // experts per load batch (8 hidden fragments, half as many weight loads;
                                                // twice as many in flight was slower: 18.7 against 16.7 us at 16 tokens)
@@ -325,20 +326,24 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
         const u32x4 v = *(const u32x4*)(A.norms + (int64_t)tc * E + e8);
         const uint32_t vw[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int i = 0; i < 8; ++i) m = nanmax(m, __uint_as_float((i & 1) ? (vw[i >> 1] & 0xffff0000u) : (vw[i >> 1] << 16)));
+        for (int i = 0; i < 8; ++i) m = nanmax(m, (i & 1) ? dec16_hi<F16>(vw[i >> 1]) : dec16<F16>(vw[i >> 1] & 0xffffu));
       }
       m = nanmax(m, __shfl_xor(m, 16, 64));
       m = nanmax(m, __shfl_xor(m, 32, 64));
-      if (gq == 0) s_thr[c16] = bf16_to_f32(f32_to_bf16(m * A.thr_scale));
+      // (the product is rounded to float32 before it is rounded to the storage type: kept apart by the empty asm, or the
+      // compiler folds multiply and float16 conversion into one instruction with a single rounding)
+      float thr_prod = m * A.thr_scale;
+      asm volatile("" : "+v"(thr_prod));
+      if (gq == 0) s_thr[c16] = round16<F16>(thr_prod);
     }
     __syncthreads();
     if (t < E) {
       unsigned bits = 0u;
 #pragma unroll
-      for (int tk = 0; tk < DC_MAX_TOKENS; ++tk) bits |= ((tk < N && bf16_to_f32(colv[tk]) >= s_thr[tk]) ? 1u : 0u) << tk;
+      for (int tk = 0; tk < DC_MAX_TOKENS; ++tk) bits |= ((tk < N && dec16<F16>(colv[tk]) >= s_thr[tk]) ? 1u : 0u) << tk;
       s_bits[t] = (unsigned short)bits;
       if (cb == 0) {                                      // one workgroup also leaves the routing tensor and the counts
-        for (int tk = 0; tk < N; ++tk) A.routing_out[(int64_t)tk * E + t] = ((bits >> tk) & 1u) ? (bf16_t)0x3f80 : (bf16_t)0;
+        for (int tk = 0; tk < N; ++tk) A.routing_out[(int64_t)tk * E + t] = ((bits >> tk) & 1u) ? (bf16_t)(F16 ? 0x3c00 : 0x3f80) : (bf16_t)0;
         if (A.counts != nullptr) A.counts[t] = __popc(bits);
       }
     }
@@ -399,7 +404,7 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
               aw.w = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)aw.w, 0x128, 0xf, 0xf, false);
               av = __builtin_bit_cast(bf16x8, aw);
             }
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, bm), acc, 0, 0, 0);
+            acc = mfma_16x16x32<F16>(av, __builtin_bit_cast(bf16x8, bm), acc);
           }
         }
       }
@@ -432,28 +437,40 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
     const int col = cb * 8 + 4 * gq;
     if (A.last_bias != nullptr) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[r] += bf16_to_f32(A.last_bias[col + r]);
+      for (int r = 0; r < 4; ++r) o[r] += dec16<F16>(A.last_bias[col + r]);
     }
     if (A.add_residual) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[r] += bf16_to_f32(A.x[(int64_t)c16 * D + col + r]);
+      for (int r = 0; r < 4; ++r) o[r] += dec16<F16>(A.x[(int64_t)c16 * D + col + r]);
     }
     uint2 ov;
-    ov.x = pack2_bf16(o[0], o[1]);
-    ov.y = pack2_bf16(o[2], o[3]);
+    ov.x = enc16x2<F16>(o[0], o[1]);
+    ov.y = enc16x2<F16>(o[2], o[3]);
     *(uint2*)(A.out + (int64_t)c16 * D + col) = ov;
   }
 }
 
-template <bool GATED>
+template <bool GATED, bool F16>
 static hipError_t launch_hidden(const DecodeArgs& A, hipStream_t s) {
   // K steps per wave (D/128) must be a multiple of 2*U1; D is a multiple of 256, so U1 = 1 always fits.
   const int KQ = A.D / 128;
   const dim3 grid((unsigned)(A.E * (A.nt16 / 2) + (A.fused ? (A.rwidth + 3) / 4 : 0)));
-  if (KQ % 8 == 0) hipLaunchKernelGGL((decode_hidden_kernel<GATED, 4>), grid, dim3(256), 0, s, A);
-  else if (KQ % 4 == 0) hipLaunchKernelGGL((decode_hidden_kernel<GATED, 2>), grid, dim3(256), 0, s, A);
-  else hipLaunchKernelGGL((decode_hidden_kernel<GATED, 1>), grid, dim3(256), 0, s, A);
+  if (KQ % 8 == 0) hipLaunchKernelGGL((decode_hidden_kernel<GATED, 4, F16>), grid, dim3(256), 0, s, A);
+  else if (KQ % 4 == 0) hipLaunchKernelGGL((decode_hidden_kernel<GATED, 2, F16>), grid, dim3(256), 0, s, A);
+  else hipLaunchKernelGGL((decode_hidden_kernel<GATED, 1, F16>), grid, dim3(256), 0, s, A);
   return hipGetLastError();
+}
+
+// both kernels of the experts for one storage type
+template <bool F16>
+static hipError_t launch_hidden_t(const DecodeArgs& A, bool gated, hipStream_t s) {
+  return gated ? launch_hidden<true, F16>(A, s) : launch_hidden<false, F16>(A, s);
+}
+template <bool F16>
+static void launch_out_t(const DecodeArgs& A, int nt16, unsigned grid, hipStream_t s) {
+  if (nt16 == 2) hipLaunchKernelGGL((decode_out_kernel<1, F16>), dim3(grid), dim3(DO_WAVES * 64), 0, s, A);
+  else if (nt16 == 4) hipLaunchKernelGGL((decode_out_kernel<2, F16>), dim3(grid), dim3(DO_WAVES * 64), 0, s, A);
+  else hipLaunchKernelGGL((decode_out_kernel<4, F16>), dim3(grid), dim3(DO_WAVES * 64), 0, s, A);
 }
 
 hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
@@ -470,12 +487,11 @@ hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void*
   A.add_residual = sh.add_residual;
   A.fused = 0; A.rw1 = nullptr; A.rhidden = nullptr; A.rwidth = 0; A.ract = 0; A.norms = nullptr; A.routing_out = nullptr;
   A.counts = nullptr; A.thr_scale = 0.f;
-  const hipError_t e = sh.gated ? launch_hidden<true>(A, s) : launch_hidden<false>(A, s);
+  const bool f16 = sh.dtype == D2DMOE_F16;
+  const hipError_t e = f16 ? launch_hidden_t<true>(A, sh.gated != 0, s) : launch_hidden_t<false>(A, sh.gated != 0, s);
   if (e != hipSuccess) return e;
-  const dim3 grid((unsigned)(sh.d_model / 8));
-  if (L.nt16 == 2) hipLaunchKernelGGL(decode_out_kernel<1>, grid, dim3(DO_WAVES * 64), 0, s, A);
-  else if (L.nt16 == 4) hipLaunchKernelGGL(decode_out_kernel<2>, grid, dim3(DO_WAVES * 64), 0, s, A);
-  else hipLaunchKernelGGL(decode_out_kernel<4>, grid, dim3(DO_WAVES * 64), 0, s, A);
+  if (f16) launch_out_t<true>(A, L.nt16, (unsigned)(sh.d_model / 8), s);
+  else launch_out_t<false>(A, L.nt16, (unsigned)(sh.d_model / 8), s);
   return hipGetLastError();
 }
 
@@ -502,15 +518,14 @@ hipError_t launch_mfma_decode_layer(const d2dmoe_shape& sh, const void* x, const
   A.fused = 1; A.rw1 = (const bf16_t*)router_w1; A.rhidden = (bf16_t*)router_hidden; A.rwidth = sh.router_width;
   A.ract = sh.router_activation; A.norms = (const bf16_t*)norms; A.routing_out = (bf16_t*)routing; A.counts = counts;
   A.thr_scale = thr_scale;
-  hipError_t e = sh.gated ? launch_hidden<true>(A, s) : launch_hidden<false>(A, s);
+  const bool f16 = sh.dtype == D2DMOE_F16;
+  hipError_t e = f16 ? launch_hidden_t<true>(A, sh.gated != 0, s) : launch_hidden_t<false>(A, sh.gated != 0, s);
   if (e != hipSuccess) return e;
   e = launch_linear_skinny(router_hidden, router_w2, norms, (int)sh.n_tokens, sh.router_width, sh.n_experts,
-                           sh.router_output_activation, s);
+                           sh.router_output_activation, s, sh.dtype);
   if (e != hipSuccess) return e;
-  const dim3 grid((unsigned)(sh.d_model / 8));
-  if (L.nt16 == 2) hipLaunchKernelGGL(decode_out_kernel<1>, grid, dim3(DO_WAVES * 64), 0, s, A);
-  else if (L.nt16 == 4) hipLaunchKernelGGL(decode_out_kernel<2>, grid, dim3(DO_WAVES * 64), 0, s, A);
-  else hipLaunchKernelGGL(decode_out_kernel<4>, grid, dim3(DO_WAVES * 64), 0, s, A);
+  if (f16) launch_out_t<true>(A, L.nt16, (unsigned)(sh.d_model / 8), s);
+  else launch_out_t<false>(A, L.nt16, (unsigned)(sh.d_model / 8), s);
   return hipGetLastError();
 }
 
@@ -520,7 +535,7 @@ hipError_t launch_mfma_decode_layer(const d2dmoe_shape& sh, const void* x, const
 // (4 where K is long and the features few, so that more than a handful of CUs pull on the weights), its 4 or 16 waves
 // share K; partial tiles are summed through LDS in wave order.  Used for the router layers at small N.
 // ---------------------------------------------------------------------------------------------------
-template <int NW, int FPB>
+template <int NW, int FPB, bool F16 = false>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
                                                                bf16_t* __restrict__ C, int N, int K, int Nout, int act) {
   __shared__ float part[NW][4][64];
@@ -545,7 +560,7 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u)
-      if (ks0 + u < KQ / 32) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv[u], av[u], acc, 0, 0, 0);
+      if (ks0 + u < KQ / 32) acc = mfma_16x16x32<F16>(bv[u], av[u], acc);
   }
 #pragma unroll
   for (int r = 0; r < 4; ++r) part[w][r][lane] = acc[r];
@@ -559,27 +574,35 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
       for (int ww = 1; ww < NW; ++ww) v += part[ww][r][lane];
       const int f = f0 + 4 * gq + r;
       if (c16 < N && f < Nout && 4 * gq + r < FPB) {
-        const float vr = bf16_to_f32(f32_to_bf16(v));
-        C[(int64_t)c16 * Nout + f] = f32_to_bf16(apply_act(act, vr));
+        const float vr = round16<F16>(v);
+        C[(int64_t)c16 * Nout + f] = enc16<F16>(apply_act(act, vr));
       }
     }
   }
 }
 
-bool linear_skinny_supported(int64_t N, int K, int dtype) { return dtype == D2DMOE_BF16 && N >= 1 && N <= 16 && K % 128 == 0; }
+bool linear_skinny_supported(int64_t N, int K, int dtype) {
+  return (dtype == D2DMOE_BF16 || dtype == D2DMOE_F16) && N >= 1 && N <= 16 && K % 128 == 0;
+}
 
-hipError_t launch_linear_skinny(const void* A, const void* B, void* C, int N, int K, int Nout, int act, hipStream_t s) {
+template <bool F16>
+static void launch_linear_skinny_t(const void* A, const void* B, void* C, int N, int K, int Nout, int act, hipStream_t s) {
   if (K % 512 == 0 && K >= 1024) {   // long rows: 16 waves share K so that each requests its part in one go
     if (Nout <= 1024)
-      hipLaunchKernelGGL((linear_skinny_kernel<16, 4>), dim3((Nout + 3) / 4), dim3(1024), 0, s, (const bf16_t*)A,
+      hipLaunchKernelGGL((linear_skinny_kernel<16, 4, F16>), dim3((Nout + 3) / 4), dim3(1024), 0, s, (const bf16_t*)A,
                          (const bf16_t*)B, (bf16_t*)C, N, K, Nout, act);
     else
-      hipLaunchKernelGGL((linear_skinny_kernel<16, 16>), dim3((Nout + 15) / 16), dim3(1024), 0, s, (const bf16_t*)A,
+      hipLaunchKernelGGL((linear_skinny_kernel<16, 16, F16>), dim3((Nout + 15) / 16), dim3(1024), 0, s, (const bf16_t*)A,
                          (const bf16_t*)B, (bf16_t*)C, N, K, Nout, act);
   } else {
-    hipLaunchKernelGGL((linear_skinny_kernel<4, 16>), dim3((Nout + 15) / 16), dim3(256), 0, s, (const bf16_t*)A, (const bf16_t*)B,
-                       (bf16_t*)C, N, K, Nout, act);
+    hipLaunchKernelGGL((linear_skinny_kernel<4, 16, F16>), dim3((Nout + 15) / 16), dim3(256), 0, s, (const bf16_t*)A,
+                       (const bf16_t*)B, (bf16_t*)C, N, K, Nout, act);
   }
+}
+
+hipError_t launch_linear_skinny(const void* A, const void* B, void* C, int N, int K, int Nout, int act, hipStream_t s, int dtype) {
+  if (dtype == D2DMOE_F16) launch_linear_skinny_t<true>(A, B, C, N, K, Nout, act, s);
+  else launch_linear_skinny_t<false>(A, B, C, N, K, Nout, act, s);
   return hipGetLastError();
 }
 

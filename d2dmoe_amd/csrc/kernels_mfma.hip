@@ -47,8 +47,8 @@ bool mfma_router_supported(const d2dmoe_shape& sh) {
 // The expert-major kernel covers the same layers as the dense sweep with experts of at most 128 neurons.
 // Gated experts have their own expert-major kernel, instantiated for D = 2048 and experts of at most 64 neurons (Gemma).
 bool mfma_sparse_supported(const d2dmoe_shape& sh) {
-  if (sh.gated) return sh.dtype == D2DMOE_BF16 && sh.d_model == 2048 && sh.expert_dim <= 64 && sh.n_experts <= 1024;
   if (sh.dtype != D2DMOE_BF16 && sh.dtype != D2DMOE_F16) return false;
+  if (sh.gated) return sh.d_model == 2048 && sh.expert_dim <= 64 && sh.n_experts <= 1024;
   if (sh.n_experts > 1024) return false;
   if (sh.d_model == 768) return sh.expert_dim <= 128;
   // wider models: the registers a wave needs grow with D and with the expert's row tiles

@@ -618,7 +618,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__
 // four in flight while the current are multiplied; rows leave through a wave-private LDS tile as whole 256-byte
 // segments.  Every pair's row goes to y, tokens with one expert included; the combine kernel sums them.
 // ---------------------------------------------------------------------------------------------------
-template <int D, int ACT>
+template <int D, int ACT, bool F16 = false>
 __global__ __launch_bounds__(256, 2) void experts_gated_sparse_kernel(const SparseArgs A) {
   constexpr int KS1 = D / 16;
   constexpr int NT = 2;          // 32-neuron tiles per projection (expert size <= 64)
@@ -656,7 +656,7 @@ __global__ __launch_bounds__(256, 2) void experts_gated_sparse_kernel(const Spar
     const int pj = base + j0 + (c32 < rows ? c32 : rows - 1);
     const int tok = A.token_idx[pj];
     const int dst = A.pair_dst[pj];
-    const float rw = bf16_to_f32(A.routing[(int64_t)tok * E + e]);
+    const float rw = dec16<F16>(A.routing[(int64_t)tok * E + e]);
 
     // ---- first products: this wave's tile over all of K
     const bf16x8* wf = ((w >> 1) ? A.wus : A.w1s) + ((int64_t)e * KS1 * NT + (w & 1)) * 64 + lane;   // + NT * 64 per K step
@@ -674,7 +674,7 @@ __global__ __launch_bounds__(256, 2) void experts_gated_sparse_kernel(const Spar
     };
     auto multiply = [&](bf16x8 (&xb)[U], bf16x8 (&wb)[U]) __attribute__((always_inline)) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[u], xb[u], acc1, 0, 0, 0);
+      for (int u = 0; u < U; ++u) acc1 = mfma_32x32x16<F16>(wb[u], xb[u], acc1);
     };
     fill(xA, wA, 0);
     for (int ks0 = 0; ks0 < KS1; ks0 += 2 * U) {
@@ -708,10 +708,10 @@ __global__ __launch_bounds__(256, 2) void experts_gated_sparse_kernel(const Spar
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         uint4 pk;
-        pk.x = pack2_bf16(hv[half * 8 + 0], hv[half * 8 + 1]);
-        pk.y = pack2_bf16(hv[half * 8 + 2], hv[half * 8 + 3]);
-        pk.z = pack2_bf16(hv[half * 8 + 4], hv[half * 8 + 5]);
-        pk.w = pack2_bf16(hv[half * 8 + 6], hv[half * 8 + 7]);
+        pk.x = enc16x2<F16>(hv[half * 8 + 0], hv[half * 8 + 1]);
+        pk.y = enc16x2<F16>(hv[half * 8 + 2], hv[half * 8 + 3]);
+        pk.z = enc16x2<F16>(hv[half * 8 + 4], hv[half * 8 + 5]);
+        pk.w = enc16x2<F16>(hv[half * 8 + 6], hv[half * 8 + 7]);
         ((uint4*)hs)[(w * 2 + half) * 64 + lane] = pk;
       }
     }
@@ -739,7 +739,7 @@ __global__ __launch_bounds__(256, 2) void experts_gated_sparse_kernel(const Spar
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc2[ct][r] = 0.f;
 #pragma unroll
-        for (int k = 0; k < 2 * NT; ++k) acc2[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[ct][k], hb[k], acc2[ct], 0, 0, 0);
+        for (int k = 0; k < 2 * NT; ++k) acc2[ct] = mfma_32x32x16<F16>(f[ct][k], hb[k], acc2[ct]);
       }
       // lane = pair c32, accumulator r = column 8*(r/4) + 4g + r%4 of the tile -> 16-byte piece ct*4 + r/4, half g
       uint2* srow = (uint2*)(stage + c32 * 16);
@@ -748,8 +748,8 @@ __global__ __launch_bounds__(256, 2) void experts_gated_sparse_kernel(const Spar
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           uint2 o;
-          o.x = pack2_bf16(acc2[ct][q * 4 + 0], acc2[ct][q * 4 + 1]);
-          o.y = pack2_bf16(acc2[ct][q * 4 + 2], acc2[ct][q * 4 + 3]);
+          o.x = enc16x2<F16>(acc2[ct][q * 4 + 0], acc2[ct][q * 4 + 1]);
+          o.y = enc16x2<F16>(acc2[ct][q * 4 + 2], acc2[ct][q * 4 + 3]);
           srow[(((ct * 4 + q) ^ (c32 & 15)) << 1) + g] = o;
         }
       __builtin_amdgcn_wave_barrier();
@@ -773,14 +773,15 @@ __global__ __launch_bounds__(256, 2) void experts_gated_sparse_kernel(const Spar
   }
 }
 
+template <bool F16>
 static void launch_gated_sparse_experts(const SparseArgs& A, int act, unsigned grid, hipStream_t s) {
   switch (act) {
     case D2DMOE_ACT_GELU_TANH:
-      hipLaunchKernelGGL((experts_gated_sparse_kernel<2048, D2DMOE_ACT_GELU_TANH>), dim3(grid), dim3(256), 0, s, A); break;
+      hipLaunchKernelGGL((experts_gated_sparse_kernel<2048, D2DMOE_ACT_GELU_TANH, F16>), dim3(grid), dim3(256), 0, s, A); break;
     case D2DMOE_ACT_RELU:
-      hipLaunchKernelGGL((experts_gated_sparse_kernel<2048, D2DMOE_ACT_RELU>), dim3(grid), dim3(256), 0, s, A); break;
+      hipLaunchKernelGGL((experts_gated_sparse_kernel<2048, D2DMOE_ACT_RELU, F16>), dim3(grid), dim3(256), 0, s, A); break;
     default:
-      hipLaunchKernelGGL((experts_gated_sparse_kernel<2048, -1>), dim3(grid), dim3(256), 0, s, A); break;
+      hipLaunchKernelGGL((experts_gated_sparse_kernel<2048, -1, F16>), dim3(grid), dim3(256), 0, s, A); break;
   }
 }
 
@@ -870,8 +871,8 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   A.tok_off = tok_off; A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.add_residual = sh.add_residual;
   A.wus = (const bf16x8*)(pk + L.su_off);
   const unsigned grid = (unsigned)(8 * device_cu_count());
-  const bool f16 = sh.dtype == D2DMOE_F16;   // ungated layers only (mfma_sparse_supported)
-  if (sh.gated) launch_gated_sparse_experts(A, sh.activation, grid, s);
+  const bool f16 = sh.dtype == D2DMOE_F16;
+  if (sh.gated) { if (f16) launch_gated_sparse_experts<true>(A, sh.activation, grid, s); else launch_gated_sparse_experts<false>(A, sh.activation, grid, s); }
   else if (sh.d_model == 1024) {
     if (L.nt == 1) { if (f16) launch_sparse_experts_wide<1024, 1, true>(A, grid, s); else launch_sparse_experts_wide<1024, 1, false>(A, grid, s); }
     else { if (f16) launch_sparse_experts_wide<1024, 2, true>(A, grid, s); else launch_sparse_experts_wide<1024, 2, false>(A, grid, s); }

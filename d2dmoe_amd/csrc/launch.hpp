@@ -91,7 +91,8 @@ hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void*
                               const void* last_bias, void* out, void* workspace, hipStream_t s);
 size_t mfma_decode_section_offset(const d2dmoe_shape& sh);
 bool linear_skinny_supported(int64_t N, int K, int dtype);
-hipError_t launch_linear_skinny(const void* A, const void* B, void* C, int N, int K, int Nout, int act, hipStream_t s);
+hipError_t launch_linear_skinny(const void* A, const void* B, void* C, int N, int K, int Nout, int act, hipStream_t s,
+                                int dtype = D2DMOE_BF16);
 // whole layer for at most 16 tokens in three launches (router included; the routing is derived inside the output kernel)
 bool mfma_decode_layer_supported(const d2dmoe_shape& sh);
 hipError_t launch_mfma_decode_layer(const d2dmoe_shape& sh, const void* x, const void* router_w1, const void* router_w2,

@@ -11,6 +11,7 @@ namespace d2dmoe {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // 16 raw bytes that stay in registers
@@ -101,6 +102,17 @@ template <bool F16> __device__ __forceinline__ f32x16 mfma_32x32x16(const bf16x8
   }
 }
 
+template <bool F16> __device__ __forceinline__ f32x4_t mfma_16x16x32(const bf16x8& a, const bf16x8& b, const f32x4_t& c) {
+  if constexpr (F16) {
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+}
+// one value: rounded to the storage type (bits), and rounded and decoded again
+template <bool F16> __device__ __forceinline__ uint16_t enc16(float v) { return (uint16_t)(enc16x2<F16>(v, 0.f) & 0xffffu); }
+template <bool F16> __device__ __forceinline__ float round16(float v) { return dec16<F16>(enc16x2<F16>(v, 0.f) & 0xffffu); }
 // LDS-only workgroup barrier: waits for this wave's LDS operations, not for its outstanding global loads.
 __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 

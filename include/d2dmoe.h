@@ -50,7 +50,7 @@ enum {
 };
 
 /* element types */
-enum { D2DMOE_F32 = 0, D2DMOE_BF16 = 1, D2DMOE_F16 = 2 };   /* F16: every kernel family but the small-batch, gated expert-major and compacted ones */
+enum { D2DMOE_F32 = 0, D2DMOE_BF16 = 1, D2DMOE_F16 = 2 };   /* F16: every kernel family but the opt-in compacted one */
 
 /* activations.  Reference: utils.py:730-756 (kernel-side definitions), common.py:159-169 (names). */
 enum {
@@ -69,13 +69,13 @@ enum {
   D2DMOE_PATH_AUTO = 0,       /* MFMA kernels when the shape and dtype have one, else the generic kernel */
   D2DMOE_PATH_GENERIC = 1,    /* token-tile-major scalar-FMA kernel: any shape, f32, bf16 or f16 storage, f32 math */
   D2DMOE_PATH_MFMA_DENSE = 2, /* bf16 or f16 MFMA, token-tile-major, masked dense sweep over all experts */
-  D2DMOE_PATH_MFMA_SPARSE = 3, /* bf16 (ungated: or f16) MFMA, expert-major over the permutation, then ordered combine; taken when at most
+  D2DMOE_PATH_MFMA_SPARSE = 3, /* bf16 or f16 MFMA, expert-major over the permutation, then ordered combine; taken when at most
                                  8 experts per token are routed on average (checked on the device), else the dense
                                  sweep runs.  Ungated experts at D = 768 (also D = 1024 with at most 64 neurons and D = 1280 with at
                                  most 32: up to 12 / 6 experts per token, tiled products as fall-back).  Gated experts at D = 2048 with at most 64
                                  neurons: up to 32 experts per token (8 beyond 16 384 tokens), else the tiled products
                                  run.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 (gated: >= 0.5) */
-  D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 MFMA for a handful of tokens: per pass of 16 tokens one workgroup per expert streams
+  D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 or f16 MFMA for a handful of tokens: per pass of 16 tokens one workgroup per expert streams
                                  that expert's packed weights once (gated or ungated experts); at most 48 tokens (three
                                  passes).  AUTO picks it up to 16 tokens, for gated experts up to 48 */
   D2DMOE_PATH_MFMA_MID = 6,   /* bf16 MFMA, ungated experts of at most 31 neurons at D = 768, at most 256 experts: work follows
@@ -183,8 +183,9 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
                    void* workspace, size_t workspace_bytes, void* stream);
 
 /* Bytes of the derived weight buffer for the MFMA kernels (0 when `shape` has no MFMA kernel).  The buffer has one
- * section per kernel family that covers the shape (dense sweep and expert-major: bf16 or f16, D = 768, ungated; gated expert-major: bf16,
- * D = 2048; small batch: bf16, D a multiple of 256; tiled products: bf16, f16 or f32, D a multiple of 256) and a router
+ * section per kernel family that covers the shape (16-bit storage, i.e. bf16 or f16 -- dense sweep: D = 768, ungated;
+ * expert-major: ungated at D = 768 / 1024 / 1280, gated at D = 2048; small batch: D a multiple of 256 -- and tiled
+ * products: bf16, f16 or f32, D a multiple of 256) and a router
  * section (when shape.router_width > 0 and the fused router+selection kernel covers the router: bf16 or f16, ReLU/abs,
  * width = experts = 128 or 256). */
 size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape);

@@ -223,10 +223,75 @@ def test_layer_f16_vit_shape(tau):
     assert H.rel_err(out.cpu(), _want(x, routing.cpu(), p, 'relu')) < TOL_F16
 
 
+_GEMMA = (2048, 256, 64, 256, True, 'gelu_tanh')
+_VITB = (768, 128, 24, 128, False, 'relu')
+_WIDE = (1024, 64, 40, 128, False, 'gelu')
+
+
+@pytest.mark.parametrize('N,D,E,Ed,W,gated,act', [(n,) + c for c in (_GEMMA, _VITB, _WIDE) for n in (1, 7, 16)] + [(40,) + _GEMMA])
+def test_small_batch_path_f16(N, D, E, Ed, W, gated, act):
+    """The small-batch kernels (at most 16 tokens per pass, gated experts up to 48 tokens) with float16 storage: experts
+    against the float64 oracle with weighted routing and residual; the whole layer (three launches) bit-equal to the staged
+    entry points router -> select -> experts under both tau readings, mask exact for its own norms."""
+    _say('f16 small batch', N, D, E, Ed, gated, act)
+    x, routing, p = H.random_case(N, D, E, Ed, W, seed=5 * N + E, dtype=F16, gated=gated, bias=not gated, density=0.6)
+    packed = _pack(p, D, E, Ed, W, act, gated)
+    g = torch.Generator().manual_seed(4)
+    weights = (routing.float() * (torch.rand(N, E, generator=g) + 0.5)).half()
+    got = _got(x, weights, p, act, residual=True, path='mfma_decode', packed=packed)
+    assert H.rel_err(got, _want(x, weights, p, act, True)) < TOL_F16
+    assert torch.equal(got, _got(x, weights, p, act, residual=True, path='auto', packed=packed))
+    if N > 16:
+        return
+    d = H.to_dev(p, DEV)
+    lb = d['last_bias'].view(-1) if 'last_bias' in d else None
+    ew = (d['w_gate'], None, d['w_down'], d['w_up']) if gated else (d['w1'], d['b1'], d['w2'], None)
+    xd = x.to(DEV)
+    for tau in (0.9, 0.1):
+        out, r, norms, counts = _ops().forward(xd, d['router_w1'], d['router_w2'], float(1.0 - tau), *ew, lb, act, True, None,
+                                               True, True, 'auto', packed)
+        norms2 = _ops().router(xd, d['router_w1'], d['router_w2'])
+        r2, counts2 = _ops().select(norms2, float(1.0 - tau), want_counts=True)
+        assert torch.equal(norms, norms2) and torch.equal(r, r2) and torch.equal(counts, counts2)
+        assert torch.equal(r.cpu(), O.gate_dynk_max(norms.cpu(), tau))
+        out2 = _got(x, r2.cpu(), p, act, residual=True, path='mfma_decode', packed=packed)
+        assert torch.equal(out.cpu(), out2)
+        assert H.rel_err(out.cpu(), _want(x, r2.cpu(), p, act, True)) < TOL_F16
+
+
+@pytest.mark.parametrize('N,E,Ed,density', [(100, 256, 64, 0.01), (1030, 256, 64, 0.009), (300, 64, 40, 0.1), (1, 256, 64, 0.02)])
+def test_gated_expert_major_f16(N, E, Ed, density):
+    """The gated expert-major path (Gemma shape, D = 2048) with float16 storage: against the float64 oracle and the tiled
+    products, weighted routing + residual, run-to-run bit equality; and the whole layer under the literal rule."""
+    _say('f16 gated expert-major', N, E, Ed, density)
+    D, W, act = 2048, 256, 'gelu_tanh'
+    x, routing, p = H.random_case(N, D, E, Ed, W, seed=N + E, dtype=F16, gated=True, bias=False, density=density)
+    if N > 4:
+        routing[1] = 0
+        routing[2] = 0
+        routing[2, E // 2] = 1
+    packed = _pack(p, D, E, Ed, W, act, True)
+    got = _got(x, routing, p, act, path='mfma_sparse', packed=packed)
+    assert H.rel_err(got, _want(x, routing, p, act)) < TOL_F16
+    assert torch.equal(got, _got(x, routing, p, act, path='mfma_sparse', packed=packed))
+    if N > 16:
+        assert H.rel_err(got, _got(x, routing, p, act, path='mfma_gemm', packed=packed)) < TOL_F16
+    g = torch.Generator().manual_seed(6)
+    weights = (routing.float() * (torch.rand(N, E, generator=g) + 0.5)).half()
+    got = _got(x, weights, p, act, residual=True, path='mfma_sparse', packed=packed)
+    assert H.rel_err(got, _want(x, weights, p, act, True)) < TOL_F16
+    if E == 256 and N > 16:
+        d = H.to_dev(p, DEV)
+        out, r, norms, counts = _ops().forward(x.to(DEV), d['router_w1'], d['router_w2'], 0.9, d['w_gate'], None, d['w_down'],
+                                               d['w_up'], None, act, False, None, True, True, 'auto', packed)
+        assert torch.equal(r.cpu(), O.gate_dynk_max(norms.cpu(), 0.1))
+        assert H.rel_err(out.cpu(), _want(x, r.cpu(), p, act)) < TOL_F16
+
+
 def test_bf16_only_paths_refuse_f16():
     from d2dmoe_amd.hip_abi import D2DMoEError
     x, routing, p = H.random_case(64, 768, 128, 24, 128, seed=1, dtype=F16)
     packed = _pack(p, 768, 128, 24, 128, 'relu', False)
-    for path in ('mfma_decode', 'mfma_mid'):
+    for path in ('mfma_mid',):
         with pytest.raises(D2DMoEError):
             _got(x, routing, p, 'relu', path=path, packed=packed)
