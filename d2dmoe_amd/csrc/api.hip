@@ -389,12 +389,14 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   }
   // A high threshold fraction keeps few experts per token: take the expert-major path (it falls back to the dense
   // sweep on the device if the routing turns out dense after all).
-  // (gated experts: from a lower fraction on -- their dense alternative costs ten times the expert-major path at few
-  // experts per token and the device-side switch is cheap next to it;
+  // (gated experts, and ungated ones at the widths without a fused sweep: from a lower fraction on -- their dense
+  // alternative costs several times the expert-major path at few experts per token and the device-side switch is cheap
+  // next to it;
   // and with at most 128 tokens whatever the fraction -- the layer is bound by the weight stream there, which the tiled
   // products pay for with whole 256-token tiles)
   if (path == D2DMOE_PATH_AUTO && sh.n_tokens > (sh.gated && mfma_decode_supported(sh) ? 48 : 16) && packed != nullptr &&
-      (thr_scale >= (sh.gated ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128)) && mfma_sparse_supported(sh) &&
+      (thr_scale >= ((sh.gated || !mfma_dense_supported(sh)) ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128)) &&
+      mfma_sparse_supported(sh) &&
       ((!sh.gated && mfma_dense_supported(sh)) || mfma_gemm_supported(sh)))
     path = D2DMOE_PATH_MFMA_SPARSE;
   // ... and when the router kernel of this call is the one that walks the 32-token segments of that path's plan, it
