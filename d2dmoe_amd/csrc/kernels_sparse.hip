@@ -35,7 +35,7 @@ int mfma_sparse_capacity_k(const d2dmoe_shape& sh) {
   // D = 1024 / 1280: the alternative is the tiled products (1.3 ms at 50 432 tokens, 128 experts x 32, against 0.19 ms +
   // 0.085 ms per routed expert per token here): equal at about 13
   if (sh.d_model != 768) return sh.expert_dim <= 32 ? 12 : 6;
-  return sh.expert_dim <= 32 ? SP_MAX_MEAN_K : (sh.expert_dim <= 64 ? 5 : 3);
+  return sh.expert_dim <= 32 ? SP_MAX_MEAN_K : (sh.expert_dim <= 64 ? 5 : 8);
 }
 
 static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) {
@@ -431,6 +431,12 @@ __global__ __launch_bounds__(256, ((D <= 768 && NT < 4) ? 3 : 1)) void experts_m
     bf16x8 w2r[CTW * 2 * NT];
 #pragma unroll
     for (int i = 0; i < CTW * 2 * NT; ++i) w2r[i] = w2f[i * 64];
+    const bf16_t* bias_e = A.b1s + (int64_t)e * NT * 32;
+    uint2 bqr[NT][4];   // requested ahead of the barrier, like the W2^T fragments
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) bqr[t][q] = *(const uint2*)(bias_e + t * 32 + 8 * q + 4 * g);
     __builtin_amdgcn_sched_barrier(0);
     if (has_next) tile_token(nxt);
     __builtin_amdgcn_sched_barrier(0);
@@ -441,13 +447,12 @@ __global__ __launch_bounds__(256, ((D <= 768 && NT < 4) ? 3 : 1)) void experts_m
     __syncthreads();
     // bias, activation, routing weight, round to bf16 -> B fragments of the second product
     bf16x8 hb[2 * NT];
-    const bf16_t* bias_e = A.b1s + (int64_t)e * NT * 32;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       float hv[16];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const uint2 bq = *(const uint2*)(bias_e + t * 32 + 8 * q + 4 * g);
+        const uint2 bq = bqr[t][q];
         const float bias[4] = {dec16<F16>(bq.x & 0xffffu), dec16_hi<F16>(bq.x), dec16<F16>(bq.y & 0xffffu), dec16_hi<F16>(bq.y)};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -487,25 +492,42 @@ __global__ __launch_bounds__(256, ((D <= 768 && NT < 4) ? 3 : 1)) void experts_m
       // the bias (and residual) pieces are fetched by every lane, unconditionally, and added under a mask
       const uint32_t keep = single ? 0xffffffffu : 0u;
       const bf16_t* xres = A.x + (int64_t)tok * D + col0;
+      // + last_bias on the rows of those pairs, by the matrix unit: one more K step whose only non-zero entries are
+      // the bias (k = 0 of the column's A fragment) and 1.0 for such a pair (k = 0 of its B fragment) -- an exact product,
+      // added to the accumulator with the one rounding a float addition has.  (A bias that is not finite would spread to
+      // the other pairs' rows as NaN; their tokens' results carry that bias anyway.)
+      {
+        const uint32_t one16 = F16 ? 0x3c00u : 0x3f80u;
+        const u32x4 kb = {(g == 0 && single) ? one16 : 0u, 0u, 0u, 0u};
+        bf16x8 keep_b;
+        __builtin_memcpy(&keep_b, &kb, 16);
+        uint32_t lbv[CTW];
 #pragma unroll
-      for (int ct = 0; ct < CTW; ++ct)
+        for (int ct = 0; ct < CTW; ++ct) lbv[ct] = s_last_bias[w * (D / 4) + ct * 32 + c32];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          uint2 lb = *(const uint2*)(s_last_bias + col0 + ct * 32 + 8 * q);
-          lb.x &= keep; lb.y &= keep;
-          acc2[ct][q * 4 + 0] += dec16<F16>(lb.x & 0xffffu);
-          acc2[ct][q * 4 + 1] += dec16_hi<F16>(lb.x);
-          acc2[ct][q * 4 + 2] += dec16<F16>(lb.y & 0xffffu);
-          acc2[ct][q * 4 + 3] += dec16_hi<F16>(lb.y);
-          if (A.add_residual) {   // uniform
-            uint2 xv = *(const uint2*)(xres + ct * 32 + 8 * q);
-            xv.x &= keep; xv.y &= keep;
-            acc2[ct][q * 4 + 0] += dec16<F16>(xv.x & 0xffffu);
-            acc2[ct][q * 4 + 1] += dec16_hi<F16>(xv.x);
-            acc2[ct][q * 4 + 2] += dec16<F16>(xv.y & 0xffffu);
-            acc2[ct][q * 4 + 3] += dec16_hi<F16>(xv.y);
+        for (int ct = 0; ct < CTW; ++ct) {
+          const u32x4 ab = {(g == 0) ? lbv[ct] : 0u, 0u, 0u, 0u};
+          bf16x8 bias_a;
+          __builtin_memcpy(&bias_a, &ab, 16);
+          acc2[ct] = mfma_32x32x16<F16>(bias_a, keep_b, acc2[ct]);
+        }
+      }
+      if (A.add_residual) {   // uniform; after the bias, as in the combine kernel
+#pragma unroll
+        for (int ct = 0; ct < CTW; ++ct) {
+          uint2 xv[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) xv[q] = *(const uint2*)(xres + ct * 32 + 8 * q);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint32_t vx = xv[q].x & keep, vy = xv[q].y & keep;
+            acc2[ct][q * 4 + 0] += dec16<F16>(vx & 0xffffu);
+            acc2[ct][q * 4 + 1] += dec16_hi<F16>(vx);
+            acc2[ct][q * 4 + 2] += dec16<F16>(vy & 0xffffu);
+            acc2[ct][q * 4 + 3] += dec16_hi<F16>(vy);
           }
         }
+      }
     }
     // The rows leave through this wave's slice of the partial-sum buffer (idle until the next tile, and touched by no
     // other wave outside the two barriers above), two column tiles at a time: a lane holds 4 columns of one row, the
@@ -548,6 +570,291 @@ __global__ __launch_bounds__(256, ((D <= 768 && NT < 4) ? 3 : 1)) void experts_m
       }
     }
     cur = nxt;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Expert-major kernel for big experts (more than 64 neurons): a workgroup takes a GROUP of up to SG_MAX tiles of 32
+// pairs of one expert and keeps the expert's weights in registers while the tiles pass -- W1 (this wave's quarter of
+// the model dimension, NT row tiles) through the first product of every tile of the group, then W2^T (this wave's
+// quarter of the output columns) in the same registers through the second product of every tile.  With one tile per
+// weight load (the kernel above) an expert of 128 neurons costs 12 KB of weight traffic per pair; here 1.5 - 3 KB.
+//   first product: as above (split over K, partial tiles summed through LDS in wave order), but wave w finishes row
+//   tiles w, w + 4, ... only and leaves the rounded hidden values in LDS as B fragments of the second product;
+//   second product and the row stores: as above.
+// The group size is chosen per launch from the number of tiles (whole rounds over the grid, overhead per group), the
+// same value in every workgroup.
+// ---------------------------------------------------------------------------------------------------
+constexpr int SG_MAX = 8;
+template <int NT> constexpr size_t sg_lds_bytes(int D) {
+  return (size_t)4 * NT * 16 * 64 * 4 + (size_t)SG_MAX * 2 * NT * 64 * 16 + (size_t)2 * 1025 * 4 + (size_t)4 * SG_MAX * 32 * 4 + (size_t)D * 2;
+}
+
+template <int D, int NT, int ACT, bool F16 = false>
+__global__ __launch_bounds__(256, 1) void experts_mfma_group_kernel(const SparseArgs A) {
+  constexpr int KS1 = D / 16;
+  constexpr int KQ = KS1 / 4;    // K steps per wave
+  constexpr int CTW = D / 128;   // column tiles per wave
+  static_assert(KS1 % 4 == 0 && CTW % 2 == 0, "the model dimension must split over four waves");
+  extern __shared__ __attribute__((aligned(16))) unsigned char sg_smem[];
+  typedef float PartT[NT * 16][64];
+  PartT* part = (PartT*)sg_smem;                                     // [4][NT*16][64]
+  uint4* hbs = (uint4*)(sg_smem + (size_t)4 * NT * 16 * 64 * 4);     // [SG_MAX][2 NT][64]: hidden values, B fragments
+  int32_t* s_goff = (int32_t*)(hbs + SG_MAX * 2 * NT * 64);          // [1025] groups before expert e
+  int32_t* s_offsets = s_goff + 1025;                                // [1025]
+  int32_t* s_tok = s_offsets + 1025;                                 // [SG_MAX][32] the group's pairs: token,
+  int32_t* s_dst = s_tok + SG_MAX * 32;                              //   row of y,
+  float* s_rw = (float*)(s_dst + SG_MAX * 32);                       //   routing weight,
+  int32_t* s_single = (int32_t*)(s_rw + SG_MAX * 32);                //   whether it is its token's only pair
+  bf16_t* s_last_bias = (bf16_t*)(s_single + SG_MAX * 32);           // [D]
+  if (A.flag[0] == 0) return;
+  const int E = A.E;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int g = lane >> 5, c32 = lane & 31;
+  for (int i = threadIdx.x; i <= E; i += 256) s_offsets[i] = A.offsets[i];
+  for (int i = threadIdx.x; i < D; i += 256) s_last_bias[i] = (A.last_bias != nullptr) ? A.last_bias[i] : (bf16_t)0;
+  // group size: whole rounds over the grid cost (tiles per group + about 3 tile times of weight loads and waits) each
+  const int n_tiles = A.tile_off[E];
+  int gs = 1;
+  {
+    int64_t best = -1;
+    for (int c = 1; c <= SG_MAX; ++c) {
+      const int groups = (n_tiles + c - 1) / c + E / 2;
+      const int64_t cost = (int64_t)((groups + (int)gridDim.x - 1) / (int)gridDim.x) * (c + 3);
+      if (best < 0 || cost <= best) { best = cost; gs = c; }
+    }
+  }
+  __syncthreads();
+  if (w == 0) {   // groups before each expert: inclusive scan, 64 experts at a time
+    int carry = 0;
+    for (int b = 0; b < E; b += 64) {
+      const int e = b + lane;
+      int v = 0;
+      if (e < E) {
+        const int tiles = (s_offsets[e + 1] - s_offsets[e] + SP_BT - 1) / SP_BT;
+        v = (tiles + gs - 1) / gs;
+      }
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(v, d, kWave);
+        if (lane >= d) v += o;
+      }
+      if (e < E) s_goff[e + 1] = carry + v;
+      carry += __shfl(v, 63, kWave);
+    }
+    if (lane == 0) s_goff[0] = 0;
+  }
+  __syncthreads();
+  const int n_groups = s_goff[E];
+
+  for (int G = blockIdx.x; G < n_groups; G += gridDim.x) {
+    int lo = 0, hi = E;   // largest e with goff[e] <= G (experts without groups share their successor's offset)
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (s_goff[mid] <= G) lo = mid; else hi = mid;
+    }
+    const int e = lo;
+    const int base = s_offsets[e] + (G - s_goff[e]) * gs * SP_BT;
+    int np = s_offsets[e + 1] - base;
+    if (np > gs * SP_BT) np = gs * SP_BT;
+    const int nsub = (np + SP_BT - 1) / SP_BT;
+
+    // W1 fragments of this wave's quarter of K: requested first, the pairs' records travel at the same time
+    const bf16x8* w1f = A.w1s + ((int64_t)e * KS1 + w * KQ) * NT * 64 + lane;
+    bf16x8 wr[KQ * NT];
+    static_assert(KQ * NT == CTW * 2 * NT, "both weight sets fill the same registers");
+#pragma unroll
+    for (int i = 0; i < KQ * NT; ++i) wr[i] = w1f[i * 64];
+    {
+      const int j = threadIdx.x;             // pair j of the group (sub-tile j / 32); short sub-tiles repeat their last pair
+      const int jj = (j < np) ? j : (((j >> 5) < nsub) ? np - 1 : 0);
+      if ((j >> 5) < nsub) {
+        const int tok = A.token_idx[base + jj];
+        s_tok[j] = tok;
+        s_dst[j] = A.pair_dst[base + jj];
+        s_single[j] = (A.tok_off[tok + 1] - A.tok_off[tok] == 1) ? 1 : 0;
+        s_rw[j] = dec16<F16>(A.routing[(int64_t)tok * E + e]);
+      }
+    }
+    __syncthreads();
+
+    // ---- first product of every tile of the group
+    const bf16_t* bias_e = A.b1s + (int64_t)e * NT * 32;
+    constexpr int TW = (NT + 3) / 4;   // row tiles a wave finishes
+    uint2 bqr[TW][4];                  // their biases: fetched once per group, ahead of the barriers
+#pragma unroll
+    for (int i = 0; i < TW; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) bqr[i][q] = *(const uint2*)(bias_e + (((4 * i + w) < NT) ? (4 * i + w) : 0) * 32 + 8 * q + 4 * g);
+    bf16x8 xb[KQ];
+    {
+      const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)s_tok[c32] * D) + 2 * w * KQ + g;
+#pragma unroll
+      for (int ks = 0; ks < KQ; ++ks) xb[ks] = xrow[2 * ks];
+    }
+    for (int sb = 0; sb < nsub; ++sb) {
+      bf16x8 xn[KQ];
+      {   // the next tile's x rows (the last trip re-reads its own)
+        const int sn = (sb + 1 < nsub) ? sb + 1 : sb;
+        const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)s_tok[sn * 32 + c32] * D) + 2 * w * KQ + g;
+#pragma unroll
+        for (int ks = 0; ks < KQ; ++ks) xn[ks] = xrow[2 * ks];
+      }
+      f32x16 acc1[NT];
+#pragma unroll
+      for (int a = 0; a < NT; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc1[a][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KQ; ++ks)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc1[t] = mfma_32x32x16<F16>(wr[ks * NT + t], xb[ks], acc1[t]);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) part[w][t * 16 + r][lane] = acc1[t][r];
+      __syncthreads();
+      const float rw = s_rw[sb * 32 + c32];
+#pragma unroll
+      for (int t0 = 0; t0 < NT; t0 += 4) {
+        const int t = t0 + w;
+        if (t < NT) {   // uniform per wave
+          float hv[16];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint2 bq = bqr[t0 / 4][q];
+            const float bias[4] = {dec16<F16>(bq.x & 0xffffu), dec16_hi<F16>(bq.x), dec16<F16>(bq.y & 0xffffu), dec16_hi<F16>(bq.y)};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int r = q * 4 + i;
+              float v = ((part[0][t * 16 + r][lane] + part[1][t * 16 + r][lane]) + part[2][t * 16 + r][lane]) +
+                        part[3][t * 16 + r][lane];
+              v += bias[i];
+              v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(A.act_rt, v);
+              hv[r] = v * rw;
+            }
+          }
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            uint4 pk;
+            pk.x = enc16x2<F16>(hv[half * 8 + 0], hv[half * 8 + 1]);
+            pk.y = enc16x2<F16>(hv[half * 8 + 2], hv[half * 8 + 3]);
+            pk.z = enc16x2<F16>(hv[half * 8 + 4], hv[half * 8 + 5]);
+            pk.w = enc16x2<F16>(hv[half * 8 + 6], hv[half * 8 + 7]);
+            hbs[(sb * 2 * NT + t * 2 + half) * 64 + lane] = pk;
+          }
+        }
+      }
+      __syncthreads();   // partial tiles are rewritten by the next tile; the hidden fragments are complete
+#pragma unroll
+      for (int ks = 0; ks < KQ; ++ks) xb[ks] = xn[ks];
+    }
+
+    // ---- second product of every tile of the group: W2^T fragments of this wave's columns take the registers over
+    const bf16x8* w2f = A.w2s + ((int64_t)e * (D / 32) + w * CTW) * (2 * NT) * 64 + lane;
+#pragma unroll
+    for (int i = 0; i < CTW * 2 * NT; ++i) wr[i] = w2f[i * 64];
+    const int col0 = w * (D / 4) + 4 * g;
+    for (int sb = 0; sb < nsub; ++sb) {
+      const int rows = (np - sb * SP_BT < SP_BT) ? (np - sb * SP_BT) : SP_BT;
+      const int tok = s_tok[sb * 32 + c32], dst = s_dst[sb * 32 + c32];
+      const bool single = (c32 < rows) && s_single[sb * 32 + c32] != 0;
+      bf16x8 hb[2 * NT];
+#pragma unroll
+      for (int k2 = 0; k2 < 2 * NT; ++k2) {
+        const uint4 v = hbs[(sb * 2 * NT + k2) * 64 + lane];
+        __builtin_memcpy(&hb[k2], &v, 16);
+      }
+      f32x16 acc2[CTW];
+#pragma unroll
+      for (int a = 0; a < CTW; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc2[a][r] = 0.f;
+#pragma unroll
+      for (int ks2 = 0; ks2 < 2 * NT; ++ks2) {   // K outside: CTW independent accumulators between dependent MFMAs
+#pragma unroll
+        for (int ct = 0; ct < CTW; ++ct) acc2[ct] = mfma_32x32x16<F16>(wr[ct * 2 * NT + ks2], hb[ks2], acc2[ct]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      const bool any_single = __ballot(single) != 0ull;   // uniform
+      if (any_single) {
+        const uint32_t keep = single ? 0xffffffffu : 0u;
+        const bf16_t* xres = A.x + (int64_t)tok * D + col0;
+        // + last_bias on the rows of those pairs, by the matrix unit: one more K step whose only non-zero entries are
+        // the bias (k = 0 of the column's A fragment) and 1.0 for such a pair (k = 0 of its B fragment) -- an exact product,
+        // added to the accumulator with the one rounding a float addition has.  (A bias that is not finite would spread to
+        // the other pairs' rows as NaN; their tokens' results carry that bias anyway.)
+        {
+          const uint32_t one16 = F16 ? 0x3c00u : 0x3f80u;
+          const u32x4 kb = {(g == 0 && single) ? one16 : 0u, 0u, 0u, 0u};
+          bf16x8 keep_b;
+          __builtin_memcpy(&keep_b, &kb, 16);
+          uint32_t lbv[CTW];
+#pragma unroll
+          for (int ct = 0; ct < CTW; ++ct) lbv[ct] = s_last_bias[w * (D / 4) + ct * 32 + c32];
+#pragma unroll
+          for (int ct = 0; ct < CTW; ++ct) {
+            const u32x4 ab = {(g == 0) ? lbv[ct] : 0u, 0u, 0u, 0u};
+            bf16x8 bias_a;
+            __builtin_memcpy(&bias_a, &ab, 16);
+            acc2[ct] = mfma_32x32x16<F16>(bias_a, keep_b, acc2[ct]);
+          }
+        }
+        if (A.add_residual) {   // uniform; after the bias, as in the combine kernel
+#pragma unroll
+          for (int ct = 0; ct < CTW; ++ct) {
+            uint2 xv[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xv[q] = *(const uint2*)(xres + ct * 32 + 8 * q);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const uint32_t vx = xv[q].x & keep, vy = xv[q].y & keep;
+              acc2[ct][q * 4 + 0] += dec16<F16>(vx & 0xffffu);
+              acc2[ct][q * 4 + 1] += dec16_hi<F16>(vx);
+              acc2[ct][q * 4 + 2] += dec16<F16>(vy & 0xffffu);
+              acc2[ct][q * 4 + 3] += dec16_hi<F16>(vy);
+            }
+          }
+        }
+      }
+      // rows leave through this wave's slice of the partial-sum buffer (no other wave touches it in this phase)
+      {
+        unsigned char* stage = (unsigned char*)&part[w][0][0];   // 32 rows x 128 bytes
+        const int ridx = single ? tok : dst;
+        const int rl = lane >> 3, pc = lane & 7;
+        bf16_t* rptr[4];
+        bool rlive[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int R = rl + 8 * i;
+          const int idx = __shfl(ridx, R, kWave);
+          const int sg = __shfl((int)single, R, kWave);
+          rptr[i] = (sg ? A.out : A.y) + (int64_t)idx * D + w * (D / 4) + pc * 8;
+          rlive[i] = R < rows;
+        }
+#pragma unroll
+        for (int ps = 0; ps < CTW / 2; ++ps) {
+#pragma unroll
+          for (int cta = 0; cta < 2; ++cta)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              uint2 o;
+              o.x = enc16x2<F16>(acc2[2 * ps + cta][q * 4 + 0], acc2[2 * ps + cta][q * 4 + 1]);
+              o.y = enc16x2<F16>(acc2[2 * ps + cta][q * 4 + 2], acc2[2 * ps + cta][q * 4 + 3]);
+              *(uint2*)(stage + c32 * 128 + (((cta * 4 + q) ^ (c32 & 7)) * 16) + 8 * g) = o;
+            }
+          __builtin_amdgcn_wave_barrier();
+          u32x4 rowv[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) rowv[i] = *(const u32x4*)(stage + (rl + 8 * i) * 128 + ((pc ^ rl) * 16));
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (rlive[i]) *(u32x4*)(rptr[i] + ps * 64) = rowv[i];
+        }
+      }
+    }
+    __syncthreads();   // the pairs' records and the staging slices are rewritten by the next group
   }
 }
 
@@ -797,6 +1104,26 @@ static void launch_sparse_experts(const SparseArgs& A, int act, unsigned grid, h
   }
 }
 
+template <int D, int NT, bool F16>
+static hipError_t launch_group_experts(const SparseArgs& A, int act, hipStream_t s) {
+  const size_t lds = sg_lds_bytes<NT>(D);
+  const unsigned grid = (unsigned)device_cu_count();   // one workgroup per CU (390 registers per lane)
+#define D2DMOE_GROUP_LAUNCH(ACTV)                                                                                \
+  {                                                                                                              \
+    auto kern = experts_mfma_group_kernel<D, NT, ACTV, F16>;                                                     \
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+    if (e != hipSuccess) return e;                                                                               \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, s, A);                                                  \
+  }
+  switch (act) {
+    case D2DMOE_ACT_RELU: D2DMOE_GROUP_LAUNCH(D2DMOE_ACT_RELU) break;
+    case D2DMOE_ACT_GELU: D2DMOE_GROUP_LAUNCH(D2DMOE_ACT_GELU) break;
+    default: D2DMOE_GROUP_LAUNCH(-1) break;
+  }
+#undef D2DMOE_GROUP_LAUNCH
+  return hipSuccess;
+}
+
 // The wider models (D = 1024: GPT-2 medium, BERT-large, ViT-L; D = 1280: GPT-2 large): the same kernel with the
 // activation chosen at run time, at one workgroup per CU (a wave's x fragments, W2^T fragments and output accumulators
 // grow with D: 300 - 370 registers).
@@ -881,7 +1208,10 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   }
   else if (L.nt == 1) { if (f16) launch_sparse_experts<1, true>(A, sh.activation, grid, s); else launch_sparse_experts<1, false>(A, sh.activation, grid, s); }
   else if (L.nt == 2) { if (f16) launch_sparse_experts<2, true>(A, sh.activation, grid, s); else launch_sparse_experts<2, false>(A, sh.activation, grid, s); }
-  else { if (f16) launch_sparse_experts<4, true>(A, sh.activation, grid, s); else launch_sparse_experts<4, false>(A, sh.activation, grid, s); }
+  else {
+    hipError_t ge = f16 ? launch_group_experts<768, 4, true>(A, sh.activation, s) : launch_group_experts<768, 4, false>(A, sh.activation, s);
+    if (ge != hipSuccess) return ge;
+  }
   const int64_t n_threads = N * (sh.d_model / 8);
   if (f16)
     hipLaunchKernelGGL(combine_kernel<true>, dim3((unsigned)cdiv64(n_threads, 256)), dim3(256), 0, s, y, tok_off, flag, (const bf16_t*)x,
