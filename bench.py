@@ -570,7 +570,7 @@ def reference_shape_record(ops, dev, steps, warmup):
     packed = ops.pack_weights(ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x), act), p['w1'], p['b1'], p['w2'], None,
                               p['router_w1'], p['router_w2'])
     rows = []
-    for k_frac in (1.0, 0.5, 0.1):
+    for k_frac in (1.0, 0.5, 0.3, 0.2, 0.1):
         g = torch.Generator().manual_seed(int(k_frac * 100))
         norms_in = (torch.rand(N, E, generator=g) < k_frac).to(torch.bfloat16).to(dev)
         r = run_regime(ops, x, p, packed, 0.01, act, steps, warmup, D, E, Ed, W, norms_in=norms_in)

@@ -240,6 +240,11 @@ static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* ro
     if (packed != nullptr && sh.n_tokens <= (sh.gated ? 48 : 16) && mfma_decode_supported(sh)) path = D2DMOE_PATH_MFMA_DECODE;
     else if (packed != nullptr && sh.gated && sh.n_tokens <= 128 && mfma_sparse_supported(sh) && mfma_gemm_supported(sh))
       path = D2DMOE_PATH_MFMA_SPARSE;   // still bound by the weight stream: expert-major whatever the routing
+    // big experts: the dense sweep cannot skip anything (a chunk of 256 neurons is two experts), so the expert-major
+    // path is tried whatever the threshold; it hands over to the sweep on the device when the routing is dense
+    else if (packed != nullptr && !sh.gated && sh.expert_dim > 64 && mfma_sparse_supported(sh) && mfma_dense_supported(sh) &&
+             workspace != nullptr && workspace_bytes >= mfma_sparse_workspace_bytes(sh))
+      path = D2DMOE_PATH_MFMA_SPARSE;
     else if (packed != nullptr && mfma_dense_supported(sh)) path = D2DMOE_PATH_MFMA_DENSE;
     else if (packed != nullptr && mfma_gemm_supported(sh)) path = D2DMOE_PATH_MFMA_GEMM;
     else path = D2DMOE_PATH_GENERIC;
@@ -277,7 +282,10 @@ static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* ro
       if (fb_gemm)   // the tiled products work behind the plan in the same workspace
         return (int)launch_mfma_gemm(sh, x, routing, (const char*)packed + mfma_gemm_section_offset(sh), last_bias, out,
                                      (char*)workspace + mfma_sparse_fallback_offset(sh), s, flag);
-      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, nullptr, 0, s);
+      // (the sweep's split tail tiles leave their partial sums in the pair rows' region, idle when the sweep runs)
+      const size_t fb_off = mfma_sparse_fallback_offset(sh);
+      return (int)launch_mfma_dense(sh, x, routing, packed, last_bias, out, flag, (char*)workspace + fb_off,
+                                    workspace_bytes - fb_off, s);
     }
     case D2DMOE_PATH_MFMA_MID: {
       // compacted two-kernel path when the routed pairs fit the provisioned capacity, else the dense sweep: decided on
@@ -393,9 +401,11 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   // alternative costs several times the expert-major path at few experts per token and the device-side switch is cheap
   // next to it;
   // and with at most 128 tokens whatever the fraction -- the layer is bound by the weight stream there, which the tiled
-  // products pay for with whole 256-token tiles)
+  // products pay for with whole 256-token tiles;
+  // big ungated experts whatever the fraction: the dense sweep cannot skip at their granularity)
   if (path == D2DMOE_PATH_AUTO && sh.n_tokens > (sh.gated && mfma_decode_supported(sh) ? 48 : 16) && packed != nullptr &&
-      (thr_scale >= ((sh.gated || !mfma_dense_supported(sh)) ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128)) &&
+      (thr_scale >= ((sh.gated || !mfma_dense_supported(sh)) ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128) ||
+       (!sh.gated && sh.expert_dim > 64)) &&
       mfma_sparse_supported(sh) &&
       ((!sh.gated && mfma_dense_supported(sh)) || mfma_gemm_supported(sh)))
     path = D2DMOE_PATH_MFMA_SPARSE;

@@ -471,9 +471,10 @@ static hipError_t launch_sum_partials_t(const float* partial, const void* last_b
 }
 
 hipError_t launch_sum_partials(const float* partial, const void* last_bias, const void* x, void* out, int64_t N, int D,
-                               int n_splits, int add_residual, hipStream_t s, int dtype) {
-  if (dtype == D2DMOE_F16) return launch_sum_partials_t<f16_t>(partial, last_bias, x, out, N, D, n_splits, add_residual, s);
-  return launch_sum_partials_t<bf16_t>(partial, last_bias, x, out, N, D, n_splits, add_residual, s);
+                               int n_splits, int add_residual, hipStream_t s, int dtype, const int* skip_flag) {
+  if (dtype == D2DMOE_F16)
+    return launch_sum_partials_t<f16_t>(partial, last_bias, x, out, N, D, n_splits, add_residual, s, skip_flag);
+  return launch_sum_partials_t<bf16_t>(partial, last_bias, x, out, N, D, n_splits, add_residual, s, skip_flag);
 }
 
 template <typename T, int ACT, bool GATED>

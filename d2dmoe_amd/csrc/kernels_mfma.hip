@@ -743,9 +743,13 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   const size_t lds = dense_lds_bytes(sh);
   if (lds > 160 * 1024) return hipErrorInvalidValue;
   const int cus = device_cu_count();
-  const bool allow_split = skip_flag == nullptr && workspace != nullptr && workspace_bytes >= mfma_dense_workspace_bytes(sh);
+  // Behind the expert-major path the launch is usually a no-op: one workgroup per CU walks the tiles, so a skipped call
+  // retires after one round of empty workgroups.  With big experts (the reference's benchmark shape, swept over
+  // densities) the fall-back runs as often as not, and the walk costs 15 % per tile: the ordinary grid there.
+  const bool walk = skip_flag != nullptr && sh.expert_dim <= 64;
+  const bool allow_split = !walk && workspace != nullptr && workspace_bytes >= mfma_dense_workspace_bytes(sh);
   const DenseTiling T = dense_tiling(sh, allow_split);
-  auto kern = (skip_flag != nullptr) ? experts_mfma_dense_walk_kernel<D, ACT, ED8, F16> : experts_mfma_dense_kernel<D, ACT, ED8, F16>;
+  auto kern = walk ? experts_mfma_dense_walk_kernel<D, ACT, ED8, F16> : experts_mfma_dense_kernel<D, ACT, ED8, F16>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   DenseArgs A;
@@ -757,13 +761,13 @@ static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const 
   A.partial = (float*)workspace; A.csplit = T.csplit; A.chunks_per_split = T.per;
   A.part_base = T.part_base; A.part_rows = T.part_rows;
   int64_t grid = T.n_full + T.n_half * T.csplit;
-  if (skip_flag != nullptr && A.n_tiles > cus) grid = cus;
+  if (walk && A.n_tiles > cus) grid = cus;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, s, A);
   e = hipGetLastError();
   if (e != hipSuccess || T.csplit <= 1) return e;
   return launch_sum_partials(A.partial, last_bias, (const bf16_t*)x + T.part_base * sh.d_model,
                              (bf16_t*)out + T.part_base * sh.d_model, T.part_rows, sh.d_model, T.csplit, sh.add_residual, s,
-                             sh.dtype);
+                             sh.dtype, skip_flag);
 }
 
 template <int D, int ACT>

@@ -58,7 +58,7 @@ hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* 
                              hipStream_t s);
 // out = round(sum over splits (ascending) of partial[split] + last_bias (+ x)); partial is [n_splits][N][D] float32
 hipError_t launch_sum_partials(const float* partial, const void* last_bias, const void* x, void* out, int64_t N, int D,
-                               int n_splits, int add_residual, hipStream_t s, int dtype = D2DMOE_BF16);
+                               int n_splits, int add_residual, hipStream_t s, int dtype = D2DMOE_BF16, const int* skip_flag = nullptr);
 
 // ---- bf16 MFMA expert-major path (kernels_sparse.hip) ----
 bool mfma_sparse_supported(const d2dmoe_shape& sh);
