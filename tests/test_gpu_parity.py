@@ -266,6 +266,47 @@ def test_experts_mfma_sparse_matches_oracle(N, E, Ed, density):
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('N,E,Ed,density,act', [(5000, 24, 128, 0.1, 'relu'), (2000, 10, 100, 0.3, 'gelu'), (33, 24, 128, 0.2, 'relu'),
+                                                (1, 24, 128, 0.5, 'relu'), (9000, 3, 128, 0.5, 'tanh'),
+                                                (50432, 24, 128, 0.1, 'relu'), (50432, 24, 128, 0.5, 'relu')])
+def test_experts_mfma_sparse_big_experts(N, E, Ed, density, act, dtype):
+    """Expert-major path for experts of more than 64 neurons (the reference's own benchmark shape, 24 experts x 128:
+    scripts/test_moe_implementations.py:109-126): groups of up to 8 tiles of 32 pairs per weight load.  Against the
+    float64 oracle (row slices at 50 432 tokens) and the dense sweep; tokens with no / one / every expert; weighted
+    routing + residual; run-to-run bit equality; AUTO takes this path for such experts; at density 0.5 the pairs exceed
+    the provisioned capacity and the device-side flag hands over to the sweep, whose result must then be the sweep's
+    own, bit for bit."""
+    _say('experts sparse big', N, E, Ed, density, act, dtype)
+    tol = H.tol_for(dtype)
+    x, routing, p = H.random_case(N, 768, E, Ed, 8, seed=N + E + Ed, dtype=dtype, density=density)
+    if N > 4:
+        routing[1] = 0
+        routing[2] = 0
+        routing[2, E // 2] = 1
+        routing[3] = 1
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, 768, E, Ed, 0, 1 if dtype == torch.bfloat16 else 2, act)
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, None, None)
+    assert packed is not None
+    got = _experts_got(x, routing, p, act, path='mfma_sparse', packed=packed)
+    rows = slice(0, N) if N <= 5000 else slice(N - 2500, N)
+    assert H.rel_err(got[rows], _experts_want(x[rows], routing[rows], p, act)) < tol
+    assert torch.equal(got, _experts_got(x, routing, p, act, path='mfma_sparse', packed=packed))
+    if N > 16:
+        assert torch.equal(got, _experts_got(x, routing, p, act, path='auto', packed=packed))
+    dense = _experts_got(x, routing, p, act, path='mfma_dense', packed=packed)
+    if routing.float().sum().item() > 8 * N:
+        assert torch.equal(got, dense)          # over capacity: the sweep ran
+    else:
+        assert H.rel_err(got, dense) < tol
+    if N <= 5000:
+        g = torch.Generator().manual_seed(5)
+        weights = (routing.float() * (torch.rand(N, E, generator=g) + 0.5)).to(dtype)
+        got = _experts_got(x, weights, p, act, residual=True, path='mfma_sparse', packed=packed)
+        assert H.rel_err(got, _experts_want(x, weights, p, act, True)) < tol
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('N,D,E,Ed,density,act', [(300, 1024, 128, 32, 0.03, 'gelu'), (1576, 1024, 128, 32, 0.02, 'relu'),
                                                   (700, 1024, 64, 64, 0.05, 'relu'), (333, 1024, 100, 20, 0.04, 'tanh'),
                                                   (1, 1024, 128, 32, 0.05, 'relu'), (900, 1280, 160, 32, 0.03, 'gelu'),
