@@ -70,11 +70,12 @@ enum {
   D2DMOE_PATH_GENERIC = 1,    /* token-tile-major scalar-FMA kernel: any shape, f32, bf16 or f16 storage, f32 math */
   D2DMOE_PATH_MFMA_DENSE = 2, /* bf16 or f16 MFMA, token-tile-major, masked dense sweep over all experts */
   D2DMOE_PATH_MFMA_SPARSE = 3, /* bf16 or f16 MFMA, expert-major over the permutation, then ordered combine; taken when at most
-                                 8 experts per token are routed on average (checked on the device), else the dense
-                                 sweep runs.  Ungated experts at D = 768 (also D = 1024 with at most 64 neurons and D = 1280 with at
+                                 8 experts per token are routed on average (5 for experts of 33 - 64 neurons; checked on the
+                                 device), else the dense sweep runs.  Ungated experts at D = 768 (also D = 1024 with at most 64 neurons and D = 1280 with at
                                  most 32: up to 12 / 6 experts per token, tiled products as fall-back).  Gated experts at D = 2048 with at most 64
                                  neurons: up to 32 experts per token (8 beyond 16 384 tokens), else the tiled products
-                                 run.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 (gated: >= 0.5) */
+                                 run.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 (gated: >= 0.5); for ungated
+                                 experts of more than 64 neurons AUTO picks it whatever the threshold, in d2dmoe_experts too */
   D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 or f16 MFMA for a handful of tokens: per pass of 16 tokens one workgroup per expert streams
                                  that expert's packed weights once (gated or ungated experts); at most 48 tokens (three
                                  passes).  AUTO picks it up to 16 tokens, for gated experts up to 48 */
