@@ -27,15 +27,12 @@ struct SparseWorkspace {
 // sweep is as fast from about 7 on.  Gated experts at the Gemma shape (786 KB each): the tiled products cost 0.8 ms per
 // 4096 tokens whatever the routing and the expert-major kernels stay below that up to about 40 pairs per token, so the
 // capacity is 32 -- up to 16 384 tokens, where the per-pair rows (4 KB each) take 2 GB; beyond that 8.
-// Ungated experts of more than 32 neurons: the experts kernel works on 2 or 4 row tiles per expert at lower occupancy and
-// costs 80 / 135 us per routed expert per token at 50 432 tokens instead of 55; it meets the sweep at 5 / 3 (measured:
-// 64 x 48, 48 x 64, 32 x 96 and 24 x 128 experts at D = 768).
 int mfma_sparse_capacity_k(const d2dmoe_shape& sh) {
   if (sh.gated) return (sh.n_tokens <= 16384) ? SP_MAX_MEAN_K_GATED : SP_MAX_MEAN_K;
-  // D = 1024 / 1280: the alternative is the tiled products (1.3 ms at 50 432 tokens, 128 experts x 32, against 0.19 ms +
-  // 0.085 ms per routed expert per token here): equal at about 13
+  // D = 1024 / 1280: the alternative is the tiled products (1.3 ms at 50 432 tokens, 128 experts x 32, against 0.15 ms +
+  // 0.07 ms per routed expert per token here)
   if (sh.d_model != 768) return sh.expert_dim <= 32 ? 12 : 6;
-  return sh.expert_dim <= 32 ? SP_MAX_MEAN_K : (sh.expert_dim <= 64 ? 5 : 8);
+  return SP_MAX_MEAN_K;   // ~45 us + 40 - 52 us per routed expert per token against 0.44 - 0.49 ms for the sweep
 }
 
 static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) {
@@ -322,16 +319,7 @@ __global__ __launch_bounds__(256) void plan_scatter_kernel(const bf16_t* __restr
   }
 }
 
-// ---------------------------------------------------------------------------------------------------
-// Expert-major fused experts kernel.  256 threads = 4 waves per tile of 32 pairs of one expert.
-//   GEMM1 (transposed, H^T = W1^T . X^T) is split over K: wave w multiplies its quarter of the model dimension, reading
-//   the x rows straight from their gathered positions as B fragments; the four partial tiles are summed through LDS
-//   in wave order, so every wave ends up with the same complete H^T.
-//   Bias, activation, routing weight and the rounding to bf16 happen in registers, which already sit in B-fragment
-//   position for GEMM2 (also transposed: OUT^T = W2^T . H^T), of which wave w owns D/4 output columns.  A lane ends
-//   with ONE pair and 4 consecutive columns per accumulator quad: 8-byte stores into the pair's token-major slot.
-// A fixed grid loops over the tiles listed by tile_off; the expert of a tile is found by bisection.
-// ---------------------------------------------------------------------------------------------------
+// Arguments of the expert-major experts kernels.
 struct SparseArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* w1s; const bf16x8* w2s; const bf16_t* b1s;
   const bf16x8* wus;   // gated experts: fragments of the up projection, arranged like w1s
@@ -340,258 +328,34 @@ struct SparseArgs {
   const int32_t* tok_off; const bf16_t* last_bias; bf16_t* out; int add_residual;   // tokens with ONE routed expert
 };
 
-template <int D, int NT, int ACT, bool F16 = false>
-__global__ __launch_bounds__(256, ((D <= 768 && NT < 4) ? 3 : 1)) void experts_mfma_sparse_kernel(const SparseArgs A) {
-  constexpr int KS1 = D / 16;
-  constexpr int KQ = KS1 / 4;    // K steps per wave
-  constexpr int CTW = D / 128;   // column tiles per wave
-  static_assert(KS1 % 4 == 0, "the model dimension must split over four waves");
-  __shared__ int32_t s_tile_off[1025];
-  __shared__ int32_t s_offsets[1025];
-  __shared__ float part[4][NT * 16][64];
-  __shared__ __attribute__((aligned(16))) bf16_t s_last_bias[D];
-  if (A.flag[0] == 0) return;
-  const int E = A.E;
-  for (int i = threadIdx.x; i <= E; i += 256) {
-    s_tile_off[i] = A.tile_off[i];
-    s_offsets[i] = A.offsets[i];
-  }
-  for (int i = threadIdx.x; i < D; i += 256) s_last_bias[i] = (A.last_bias != nullptr) ? A.last_bias[i] : (bf16_t)0;
-  __syncthreads();
-  const int n_tiles = s_tile_off[E];
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int g = lane >> 5, c32 = lane & 31;
-  // Workgroups are dealt to the 8 XCDs round-robin.  Each XCD takes one contiguous eighth of the tiles (tiles are in
-  // expert order), so an expert's weights pass through one L2, or two, instead of all eight.
-  const int xcd = blockIdx.x & 7, wg = blockIdx.x >> 3, nwg = gridDim.x >> 3;   // the grid is a multiple of 8
-  const int t_lo = (int)((int64_t)n_tiles * xcd / 8), t_hi = (int)((int64_t)n_tiles * (xcd + 1) / 8);
-  // What a tile needs before its first x load hangs on two dependent global reads (pair -> token -> that token's pair
-  // range and routing value).  They are made one tile ahead, in stages placed between the phases of the current tile,
-  // so that each has returned long before its result is used.
-  struct TileInfo {
-    int e, rows, tok, dst, t0, t1;
-    bf16_t rbits;
-  };
-  auto tile_begin = [&](int T, TileInfo& ti) __attribute__((always_inline)) {   // LDS lookups, then the pair's token and row
-    int lo = 0, hi = E;   // largest e with tile_off[e] <= T (experts without tiles share their successor's offset)
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (s_tile_off[mid] <= T) lo = mid; else hi = mid;
-    }
-    ti.e = lo;
-    const int base = s_offsets[lo];
-    const int cnt = s_offsets[lo + 1] - base;
-    const int j0 = (T - s_tile_off[lo]) * SP_BT;
-    ti.rows = (cnt - j0 < SP_BT) ? (cnt - j0) : SP_BT;
-    const int pj = base + j0 + (c32 < ti.rows ? c32 : ti.rows - 1);
-    ti.tok = A.token_idx[pj];
-    ti.dst = A.pair_dst[pj];
-  };
-  auto tile_token = [&](TileInfo& ti) __attribute__((always_inline)) {          // the token's pair range and routing value
-    ti.t0 = A.tok_off[ti.tok];
-    ti.t1 = A.tok_off[ti.tok + 1];
-    ti.rbits = A.routing[(int64_t)ti.tok * E + ti.e];
-  };
-  int T = t_lo + wg;
-  TileInfo cur = {0, 1, 0, 0, 0, 0, 0}, nxt = {0, 1, 0, 0, 0, 0, 0};
-  if (T < t_hi) {
-    tile_begin(T, cur);
-    tile_token(cur);
-  }
-  for (; T < t_hi; T += nwg) {
-    const bool has_next = T + nwg < t_hi;   // uniform
-    const int e = cur.e, rows = cur.rows, tok = cur.tok, dst = cur.dst;
-    const bool valid = c32 < rows;
-    // A token with a single routed expert has nothing to be summed with: its row leaves this kernel as the finished
-    // output row (float32 accumulator + last_bias (+ x), one rounding) and the combine kernel skips the token.
-    const bool single = valid && (cur.t1 - cur.t0 == 1);
-    const float rw = dec16<F16>(cur.rbits);
-    const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)tok * D) + 2 * w * KQ + g;
-
-    // GEMM1, this wave's quarter of K: all loads are issued before the first MFMA
-    const bf16x8* w1f = A.w1s + ((int64_t)e * KS1 + w * KQ) * NT * 64 + lane;
-    bf16x8 xb[KQ];
-#pragma unroll
-    for (int ks = 0; ks < KQ; ++ks) xb[ks] = xrow[2 * ks];
-    __builtin_amdgcn_sched_barrier(0);
-    if (has_next) tile_begin(T + nwg, nxt);
-    __builtin_amdgcn_sched_barrier(0);
-    f32x16 acc1[NT];
-#pragma unroll
-    for (int a = 0; a < NT; ++a)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc1[a][r] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KQ; ++ks)
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-        acc1[t] = mfma_32x32x16<F16>(w1f[(ks * NT + t) * 64], xb[ks], acc1[t]);
-    // W2^T fragments of this wave's columns: requested now, used after the reduction
-    const bf16x8* w2f = A.w2s + ((int64_t)e * (D / 32) + w * CTW) * (2 * NT) * 64 + lane;
-    bf16x8 w2r[CTW * 2 * NT];
-#pragma unroll
-    for (int i = 0; i < CTW * 2 * NT; ++i) w2r[i] = w2f[i * 64];
-    const bf16_t* bias_e = A.b1s + (int64_t)e * NT * 32;
-    uint2 bqr[NT][4];   // requested ahead of the barrier, like the W2^T fragments
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) bqr[t][q] = *(const uint2*)(bias_e + t * 32 + 8 * q + 4 * g);
-    __builtin_amdgcn_sched_barrier(0);
-    if (has_next) tile_token(nxt);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) part[w][t * 16 + r][lane] = acc1[t][r];
-    __syncthreads();
-    // bias, activation, routing weight, round to bf16 -> B fragments of the second product
-    bf16x8 hb[2 * NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      float hv[16];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint2 bq = bqr[t][q];
-        const float bias[4] = {dec16<F16>(bq.x & 0xffffu), dec16_hi<F16>(bq.x), dec16<F16>(bq.y & 0xffffu), dec16_hi<F16>(bq.y)};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int r = q * 4 + i;
-          float v = ((part[0][t * 16 + r][lane] + part[1][t * 16 + r][lane]) + part[2][t * 16 + r][lane]) +
-                    part[3][t * 16 + r][lane];
-          v += bias[i];
-          v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(A.act_rt, v);
-          hv[r] = v * rw;
-        }
-      }
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        uint4 pk;
-        pk.x = enc16x2<F16>(hv[half * 8 + 0], hv[half * 8 + 1]);
-        pk.y = enc16x2<F16>(hv[half * 8 + 2], hv[half * 8 + 3]);
-        pk.z = enc16x2<F16>(hv[half * 8 + 4], hv[half * 8 + 5]);
-        pk.w = enc16x2<F16>(hv[half * 8 + 6], hv[half * 8 + 7]);
-        __builtin_memcpy(&hb[t * 2 + half], &pk, 16);
-      }
-    }
-    __syncthreads();   // partial tiles are rewritten by the next tile
-    // GEMM2 (transposed): OUT^T[D/4 columns of this wave, 32 pairs]
-    f32x16 acc2[CTW];
-#pragma unroll
-    for (int a = 0; a < CTW; ++a)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc2[a][r] = 0.f;
-#pragma unroll
-    for (int ct = 0; ct < CTW; ++ct)
-#pragma unroll
-      for (int ks2 = 0; ks2 < 2 * NT; ++ks2)
-        acc2[ct] = mfma_32x32x16<F16>(w2r[ct * 2 * NT + ks2], hb[ks2], acc2[ct]);
-    const bool any_single = __ballot(single) != 0ull;   // uniform
-    const int col0 = w * (D / 4) + 4 * g;
-    if (any_single) {
-      // the bias (and residual) pieces are fetched by every lane, unconditionally, and added under a mask
-      const uint32_t keep = single ? 0xffffffffu : 0u;
-      const bf16_t* xres = A.x + (int64_t)tok * D + col0;
-      // + last_bias on the rows of those pairs, by the matrix unit: one more K step whose only non-zero entries are
-      // the bias (k = 0 of the column's A fragment) and 1.0 for such a pair (k = 0 of its B fragment) -- an exact product,
-      // added to the accumulator with the one rounding a float addition has.  (A bias that is not finite would spread to
-      // the other pairs' rows as NaN; their tokens' results carry that bias anyway.)
-      {
-        const uint32_t one16 = F16 ? 0x3c00u : 0x3f80u;
-        const u32x4 kb = {(g == 0 && single) ? one16 : 0u, 0u, 0u, 0u};
-        bf16x8 keep_b;
-        __builtin_memcpy(&keep_b, &kb, 16);
-        uint32_t lbv[CTW];
-#pragma unroll
-        for (int ct = 0; ct < CTW; ++ct) lbv[ct] = s_last_bias[w * (D / 4) + ct * 32 + c32];
-#pragma unroll
-        for (int ct = 0; ct < CTW; ++ct) {
-          const u32x4 ab = {(g == 0) ? lbv[ct] : 0u, 0u, 0u, 0u};
-          bf16x8 bias_a;
-          __builtin_memcpy(&bias_a, &ab, 16);
-          acc2[ct] = mfma_32x32x16<F16>(bias_a, keep_b, acc2[ct]);
-        }
-      }
-      if (A.add_residual) {   // uniform; after the bias, as in the combine kernel
-#pragma unroll
-        for (int ct = 0; ct < CTW; ++ct) {
-          uint2 xv[4];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) xv[q] = *(const uint2*)(xres + ct * 32 + 8 * q);
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const uint32_t vx = xv[q].x & keep, vy = xv[q].y & keep;
-            acc2[ct][q * 4 + 0] += dec16<F16>(vx & 0xffffu);
-            acc2[ct][q * 4 + 1] += dec16_hi<F16>(vx);
-            acc2[ct][q * 4 + 2] += dec16<F16>(vy & 0xffffu);
-            acc2[ct][q * 4 + 3] += dec16_hi<F16>(vy);
-          }
-        }
-      }
-    }
-    // The rows leave through this wave's slice of the partial-sum buffer (idle until the next tile, and touched by no
-    // other wave outside the two barriers above), two column tiles at a time: a lane holds 4 columns of one row, the
-    // transposed read gives 8 lanes 128 contiguous bytes of a row.  16-byte pieces are XORed with the row so that both
-    // directions spread over the banks.
-    {
-      static_assert(CTW % 2 == 0, "column tiles are written in pairs");
-      unsigned char* stage = (unsigned char*)&part[w][0][0];   // 32 rows x 128 bytes
-      const int ridx = single ? tok : dst;
-      const int rl = lane >> 3, pc = lane & 7;
-      bf16_t* rptr[4];   // where row rl + 8 i goes: a finished row of out, or a row of y for the combine kernel
-      bool rlive[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int R = rl + 8 * i;
-        const int idx = __shfl(ridx, R, kWave);
-        const int sg = __shfl((int)single, R, kWave);
-        rptr[i] = (sg ? A.out : A.y) + (int64_t)idx * D + w * (D / 4) + pc * 8;
-        rlive[i] = R < rows;
-      }
-#pragma unroll
-      for (int ps = 0; ps < CTW / 2; ++ps) {
-#pragma unroll
-        for (int cta = 0; cta < 2; ++cta)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            uint2 o;
-            o.x = enc16x2<F16>(acc2[2 * ps + cta][q * 4 + 0], acc2[2 * ps + cta][q * 4 + 1]);
-            o.y = enc16x2<F16>(acc2[2 * ps + cta][q * 4 + 2], acc2[2 * ps + cta][q * 4 + 3]);
-            *(uint2*)(stage + c32 * 128 + (((cta * 4 + q) ^ (c32 & 7)) * 16) + 8 * g) = o;
-          }
-        __builtin_amdgcn_wave_barrier();
-        u32x4 rowv[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) rowv[i] = *(const u32x4*)(stage + (rl + 8 * i) * 128 + ((pc ^ rl) * 16));
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (rlive[i]) *(u32x4*)(rptr[i] + ps * 64) = rowv[i];
-      }
-    }
-    cur = nxt;
-  }
-}
-
 // ---------------------------------------------------------------------------------------------------
-// Expert-major kernel for big experts (more than 64 neurons): a workgroup takes a GROUP of up to SG_MAX tiles of 32
+// Expert-major fused experts kernel.  256 threads = 4 waves; a workgroup takes a GROUP of up to SG_MAX tiles of 32
 // pairs of one expert and keeps the expert's weights in registers while the tiles pass -- W1 (this wave's quarter of
-// the model dimension, NT row tiles) through the first product of every tile of the group, then W2^T (this wave's
-// quarter of the output columns) in the same registers through the second product of every tile.  With one tile per
-// weight load (the kernel above) an expert of 128 neurons costs 12 KB of weight traffic per pair; here 1.5 - 3 KB.
-//   first product: as above (split over K, partial tiles summed through LDS in wave order), but wave w finishes row
-//   tiles w, w + 4, ... only and leaves the rounded hidden values in LDS as B fragments of the second product;
-//   second product and the row stores: as above.
+// the model dimension, NT row tiles of 32 neurons) through the first product of every tile of the group, then W2^T
+// (this wave's quarter of the output columns) in the same registers through the second product of every tile.  (With
+// one tile per weight load an expert of 128 neurons costs 12 KB of weight traffic per pair; here 1.5 - 3 KB.)
+//   First product (transposed, H^T = W1^T . X^T), split over K: wave w multiplies its quarter of the model dimension,
+//   reading the x rows straight from their gathered positions as B fragments, one tile ahead; the four partial tiles
+//   are summed through LDS in wave order.  Wave w finishes accumulator quad w of every row tile -- bias, activation,
+//   routing weight, rounding to 16 bits -- and leaves the values in LDS in B-fragment position for the second product.
+//   Second product (also transposed: OUT^T = W2^T . H^T), K outside so that D / 128 accumulators sit between
+//   dependent MFMAs.  A lane ends with ONE pair and 4 consecutive columns per accumulator quad; rows leave through the
+//   wave's slice of the partial-sum buffer, two column tiles at a time, so that 8 lanes write 128 contiguous bytes of
+//   a row: into the pair's token-major slot of y, or, for a token with a single routed expert, finished
+//   (+ last_bias (+ x), one rounding) into out.
 // The group size is chosen per launch from the number of tiles (whole rounds over the grid, overhead per group), the
-// same value in every workgroup.
+// same value in every workgroup; the expert of a group is found by bisection over the groups-per-expert prefix sums.
 // ---------------------------------------------------------------------------------------------------
 constexpr int SG_MAX = 8;
+// workgroups per CU: the weights a wave keeps (D / 64 * NT fragments) and its output accumulators (D / 8 registers)
+// leave room for two at D = 768 with one or two row tiles and at D = 1024 with one
+constexpr int sg_wgs_per_cu(int D, int NT) { return (D <= 1024 && D * NT <= 1536) ? 2 : 1; }
 template <int NT> constexpr size_t sg_lds_bytes(int D) {
   return (size_t)4 * NT * 16 * 64 * 4 + (size_t)SG_MAX * 2 * NT * 64 * 16 + (size_t)2 * 1025 * 4 + (size_t)4 * SG_MAX * 32 * 4 + (size_t)D * 2;
 }
 
 template <int D, int NT, int ACT, bool F16 = false>
-__global__ __launch_bounds__(256, 1) void experts_mfma_group_kernel(const SparseArgs A) {
+__global__ __launch_bounds__(256, sg_wgs_per_cu(D, NT)) void experts_mfma_group_kernel(const SparseArgs A) {
   constexpr int KS1 = D / 16;
   constexpr int KQ = KS1 / 4;    // K steps per wave
   constexpr int CTW = D / 128;   // column tiles per wave
@@ -680,25 +444,29 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_group_kernel(const Sparse
 
     // ---- first product of every tile of the group
     const bf16_t* bias_e = A.b1s + (int64_t)e * NT * 32;
-    constexpr int TW = (NT + 3) / 4;   // row tiles a wave finishes
-    uint2 bqr[TW][4];                  // their biases: fetched once per group, ahead of the barriers
+    uint2 bqr[NT];   // biases of the rows this wave finishes (quad w of every row tile): fetched once per group
 #pragma unroll
-    for (int i = 0; i < TW; ++i)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) bqr[i][q] = *(const uint2*)(bias_e + (((4 * i + w) < NT) ? (4 * i + w) : 0) * 32 + 8 * q + 4 * g);
+    for (int t = 0; t < NT; ++t) bqr[t] = *(const uint2*)(bias_e + t * 32 + 8 * w + 4 * g);
+    // x rows: one tile ahead (at three workgroups per CU, where the registers of a second set are not there, the
+    // kernel spills and runs slower than at two)
+    constexpr bool XPRE = true;
     bf16x8 xb[KQ];
-    {
+    if constexpr (XPRE) {
       const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)s_tok[c32] * D) + 2 * w * KQ + g;
 #pragma unroll
       for (int ks = 0; ks < KQ; ++ks) xb[ks] = xrow[2 * ks];
     }
     for (int sb = 0; sb < nsub; ++sb) {
-      bf16x8 xn[KQ];
-      {   // the next tile's x rows (the last trip re-reads its own)
+      bf16x8 xn[XPRE ? KQ : 1];
+      if constexpr (XPRE) {   // the next tile's x rows (the last trip re-reads its own)
         const int sn = (sb + 1 < nsub) ? sb + 1 : sb;
         const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)s_tok[sn * 32 + c32] * D) + 2 * w * KQ + g;
 #pragma unroll
         for (int ks = 0; ks < KQ; ++ks) xn[ks] = xrow[2 * ks];
+      } else {
+        const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)s_tok[sb * 32 + c32] * D) + 2 * w * KQ + g;
+#pragma unroll
+        for (int ks = 0; ks < KQ; ++ks) xb[ks] = xrow[2 * ks];
       }
       f32x16 acc1[NT];
 #pragma unroll
@@ -715,39 +483,31 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_group_kernel(const Sparse
         for (int r = 0; r < 16; ++r) part[w][t * 16 + r][lane] = acc1[t][r];
       __syncthreads();
       const float rw = s_rw[sb * 32 + c32];
+      // wave w finishes accumulator quad w (4 neurons per lane) of every row tile: 8 bytes of a B fragment each
 #pragma unroll
-      for (int t0 = 0; t0 < NT; t0 += 4) {
-        const int t = t0 + w;
-        if (t < NT) {   // uniform per wave
-          float hv[16];
+      for (int t = 0; t < NT; ++t) {
+        const uint2 bq = bqr[t];
+        const float bias[4] = {dec16<F16>(bq.x & 0xffffu), dec16_hi<F16>(bq.x), dec16<F16>(bq.y & 0xffffu), dec16_hi<F16>(bq.y)};
+        float hv[4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const uint2 bq = bqr[t0 / 4][q];
-            const float bias[4] = {dec16<F16>(bq.x & 0xffffu), dec16_hi<F16>(bq.x), dec16<F16>(bq.y & 0xffffu), dec16_hi<F16>(bq.y)};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int r = q * 4 + i;
-              float v = ((part[0][t * 16 + r][lane] + part[1][t * 16 + r][lane]) + part[2][t * 16 + r][lane]) +
-                        part[3][t * 16 + r][lane];
-              v += bias[i];
-              v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(A.act_rt, v);
-              hv[r] = v * rw;
-            }
-          }
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            uint4 pk;
-            pk.x = enc16x2<F16>(hv[half * 8 + 0], hv[half * 8 + 1]);
-            pk.y = enc16x2<F16>(hv[half * 8 + 2], hv[half * 8 + 3]);
-            pk.z = enc16x2<F16>(hv[half * 8 + 4], hv[half * 8 + 5]);
-            pk.w = enc16x2<F16>(hv[half * 8 + 6], hv[half * 8 + 7]);
-            hbs[(sb * 2 * NT + t * 2 + half) * 64 + lane] = pk;
-          }
+        for (int i = 0; i < 4; ++i) {
+          const int r = w * 4 + i;
+          float v = ((part[0][t * 16 + r][lane] + part[1][t * 16 + r][lane]) + part[2][t * 16 + r][lane]) +
+                    part[3][t * 16 + r][lane];
+          v += bias[i];
+          v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(A.act_rt, v);
+          hv[i] = v * rw;
         }
+        uint2 pk;
+        pk.x = enc16x2<F16>(hv[0], hv[1]);
+        pk.y = enc16x2<F16>(hv[2], hv[3]);
+        ((uint2*)(hbs + (sb * 2 * NT + t * 2 + (w >> 1)) * 64 + lane))[w & 1] = pk;
       }
       __syncthreads();   // partial tiles are rewritten by the next tile; the hidden fragments are complete
+      if constexpr (XPRE) {
 #pragma unroll
-      for (int ks = 0; ks < KQ; ++ks) xb[ks] = xn[ks];
+        for (int ks = 0; ks < KQ; ++ks) xb[ks] = xn[ks];
+      }
     }
 
     // ---- second product of every tile of the group: W2^T fragments of this wave's columns take the registers over
@@ -1092,22 +852,10 @@ static void launch_gated_sparse_experts(const SparseArgs& A, int act, unsigned g
   }
 }
 
-template <int NT, bool F16>
-static void launch_sparse_experts(const SparseArgs& A, int act, unsigned grid, hipStream_t s) {
-  switch (act) {
-    case D2DMOE_ACT_RELU:
-      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, D2DMOE_ACT_RELU, F16>), dim3(grid), dim3(256), 0, s, A); break;
-    case D2DMOE_ACT_GELU:
-      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, D2DMOE_ACT_GELU, F16>), dim3(grid), dim3(256), 0, s, A); break;
-    default:
-      hipLaunchKernelGGL((experts_mfma_sparse_kernel<768, NT, -1, F16>), dim3(grid), dim3(256), 0, s, A); break;
-  }
-}
-
-template <int D, int NT, bool F16>
+template <int D, int NT, bool F16, bool RT_ACT = false>   // RT_ACT: only the variant with the activation chosen at run time
 static hipError_t launch_group_experts(const SparseArgs& A, int act, hipStream_t s) {
   const size_t lds = sg_lds_bytes<NT>(D);
-  const unsigned grid = (unsigned)device_cu_count();   // one workgroup per CU (390 registers per lane)
+  const unsigned grid = (unsigned)(device_cu_count() * sg_wgs_per_cu(D, NT));
 #define D2DMOE_GROUP_LAUNCH(ACTV)                                                                                \
   {                                                                                                              \
     auto kern = experts_mfma_group_kernel<D, NT, ACTV, F16>;                                                     \
@@ -1115,21 +863,17 @@ static hipError_t launch_group_experts(const SparseArgs& A, int act, hipStream_t
     if (e != hipSuccess) return e;                                                                               \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, s, A);                                                  \
   }
-  switch (act) {
-    case D2DMOE_ACT_RELU: D2DMOE_GROUP_LAUNCH(D2DMOE_ACT_RELU) break;
-    case D2DMOE_ACT_GELU: D2DMOE_GROUP_LAUNCH(D2DMOE_ACT_GELU) break;
-    default: D2DMOE_GROUP_LAUNCH(-1) break;
+  if constexpr (RT_ACT) {
+    D2DMOE_GROUP_LAUNCH(-1)
+  } else {
+    switch (act) {
+      case D2DMOE_ACT_RELU: D2DMOE_GROUP_LAUNCH(D2DMOE_ACT_RELU) break;
+      case D2DMOE_ACT_GELU: D2DMOE_GROUP_LAUNCH(D2DMOE_ACT_GELU) break;
+      default: D2DMOE_GROUP_LAUNCH(-1) break;
+    }
   }
 #undef D2DMOE_GROUP_LAUNCH
   return hipSuccess;
-}
-
-// The wider models (D = 1024: GPT-2 medium, BERT-large, ViT-L; D = 1280: GPT-2 large): the same kernel with the
-// activation chosen at run time, at one workgroup per CU (a wave's x fragments, W2^T fragments and output accumulators
-// grow with D: 300 - 370 registers).
-template <int D, int NT, bool F16>
-static void launch_sparse_experts_wide(const SparseArgs& A, unsigned grid, hipStream_t s) {
-  hipLaunchKernelGGL((experts_mfma_sparse_kernel<D, NT, -1, F16>), dim3(grid), dim3(256), 0, s, A);
 }
 
 void launch_plan_count_scan(const void* routing, int64_t N, int E, int32_t* seg_counts, int32_t* seg_pairs,
@@ -1200,16 +944,17 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
   const unsigned grid = (unsigned)(8 * device_cu_count());
   const bool f16 = sh.dtype == D2DMOE_F16;
   if (sh.gated) { if (f16) launch_gated_sparse_experts<true>(A, sh.activation, grid, s); else launch_gated_sparse_experts<false>(A, sh.activation, grid, s); }
-  else if (sh.d_model == 1024) {
-    if (L.nt == 1) { if (f16) launch_sparse_experts_wide<1024, 1, true>(A, grid, s); else launch_sparse_experts_wide<1024, 1, false>(A, grid, s); }
-    else { if (f16) launch_sparse_experts_wide<1024, 2, true>(A, grid, s); else launch_sparse_experts_wide<1024, 2, false>(A, grid, s); }
-  } else if (sh.d_model == 1280) {
-    if (f16) launch_sparse_experts_wide<1280, 1, true>(A, grid, s); else launch_sparse_experts_wide<1280, 1, false>(A, grid, s);
-  }
-  else if (L.nt == 1) { if (f16) launch_sparse_experts<1, true>(A, sh.activation, grid, s); else launch_sparse_experts<1, false>(A, sh.activation, grid, s); }
-  else if (L.nt == 2) { if (f16) launch_sparse_experts<2, true>(A, sh.activation, grid, s); else launch_sparse_experts<2, false>(A, sh.activation, grid, s); }
   else {
-    hipError_t ge = f16 ? launch_group_experts<768, 4, true>(A, sh.activation, s) : launch_group_experts<768, 4, false>(A, sh.activation, s);
+    // D = 768 with the activation as a template argument; the wider models (D = 1024: GPT-2 medium, BERT-large, ViT-L;
+    // D = 1280: GPT-2 large) with the activation chosen at run time
+    hipError_t ge = hipErrorInvalidValue;
+#define D2DMOE_GROUP(DD, NTT, RT) (f16 ? launch_group_experts<DD, NTT, true, RT>(A, sh.activation, s) : launch_group_experts<DD, NTT, false, RT>(A, sh.activation, s))
+    if (sh.d_model == 1024) ge = (L.nt == 1) ? D2DMOE_GROUP(1024, 1, true) : D2DMOE_GROUP(1024, 2, true);
+    else if (sh.d_model == 1280) ge = D2DMOE_GROUP(1280, 1, true);
+    else if (L.nt == 1) ge = D2DMOE_GROUP(768, 1, false);
+    else if (L.nt == 2) ge = D2DMOE_GROUP(768, 2, false);
+    else ge = D2DMOE_GROUP(768, 4, false);
+#undef D2DMOE_GROUP
     if (ge != hipSuccess) return ge;
   }
   const int64_t n_threads = N * (sh.d_model / 8);
@@ -1224,3 +969,4 @@ hipError_t launch_mfma_sparse(const d2dmoe_shape& sh, const void* x, const void*
 }
 
 }  // namespace d2dmoe
+
