@@ -447,26 +447,25 @@ __global__ __launch_bounds__(256, sg_wgs_per_cu(D, NT)) void experts_mfma_group_
     uint2 bqr[NT];   // biases of the rows this wave finishes (quad w of every row tile): fetched once per group
 #pragma unroll
     for (int t = 0; t < NT; ++t) bqr[t] = *(const uint2*)(bias_e + t * 32 + 8 * w + 4 * g);
-    // x rows: one tile ahead (at three workgroups per CU, where the registers of a second set are not there, the
-    // kernel spills and runs slower than at two)
-    constexpr bool XPRE = true;
-    bf16x8 xb[KQ];
-    if constexpr (XPRE) {
+    // x rows are requested one tile ahead, into the set of registers the tile after this one computes from (two sets
+    // that swap roles: a copy at the end of the trip would be scheduled right behind each last use and wait for the
+    // read-ahead there).  At three workgroups per CU, where a second set does not fit, the kernel spills and runs
+    // slower than at two.
+    bf16x8 x0[KQ], x1[KQ];
+    {
       const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)s_tok[c32] * D) + 2 * w * KQ + g;
 #pragma unroll
-      for (int ks = 0; ks < KQ; ++ks) xb[ks] = xrow[2 * ks];
+      for (int ks = 0; ks < KQ; ++ks) x0[ks] = xrow[2 * ks];
     }
-    for (int sb = 0; sb < nsub; ++sb) {
-      bf16x8 xn[XPRE ? KQ : 1];
-      if constexpr (XPRE) {   // the next tile's x rows (the last trip re-reads its own)
+    // Everything requested so far (weights, the first tile's x rows) is waited for HERE: a wait left to the loop body
+    // would, from the second trip on, count the rows requested at the top of the trip instead.
+    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
+    auto first_product = [&](const int sb, bf16x8 (&xc)[KQ], bf16x8 (&xn)[KQ]) __attribute__((always_inline)) {
+      {   // the next tile's x rows (the last trip re-reads its own)
         const int sn = (sb + 1 < nsub) ? sb + 1 : sb;
         const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)s_tok[sn * 32 + c32] * D) + 2 * w * KQ + g;
 #pragma unroll
         for (int ks = 0; ks < KQ; ++ks) xn[ks] = xrow[2 * ks];
-      } else {
-        const bf16x8* xrow = (const bf16x8*)(A.x + (int64_t)s_tok[sb * 32 + c32] * D) + 2 * w * KQ + g;
-#pragma unroll
-        for (int ks = 0; ks < KQ; ++ks) xb[ks] = xrow[2 * ks];
       }
       f32x16 acc1[NT];
 #pragma unroll
@@ -476,7 +475,7 @@ __global__ __launch_bounds__(256, sg_wgs_per_cu(D, NT)) void experts_mfma_group_
 #pragma unroll
       for (int ks = 0; ks < KQ; ++ks)
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc1[t] = mfma_32x32x16<F16>(wr[ks * NT + t], xb[ks], acc1[t]);
+        for (int t = 0; t < NT; ++t) acc1[t] = mfma_32x32x16<F16>(wr[ks * NT + t], xc[ks], acc1[t]);
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -504,10 +503,10 @@ __global__ __launch_bounds__(256, sg_wgs_per_cu(D, NT)) void experts_mfma_group_
         ((uint2*)(hbs + (sb * 2 * NT + t * 2 + (w >> 1)) * 64 + lane))[w & 1] = pk;
       }
       __syncthreads();   // partial tiles are rewritten by the next tile; the hidden fragments are complete
-      if constexpr (XPRE) {
-#pragma unroll
-        for (int ks = 0; ks < KQ; ++ks) xb[ks] = xn[ks];
-      }
+    };
+    for (int sb = 0; sb < nsub; sb += 2) {
+      first_product(sb, x0, x1);
+      if (sb + 1 < nsub) first_product(sb + 1, x1, x0);
     }
 
     // ---- second product of every tile of the group: W2^T fragments of this wave's columns take the registers over
@@ -515,6 +514,7 @@ __global__ __launch_bounds__(256, sg_wgs_per_cu(D, NT)) void experts_mfma_group_
 #pragma unroll
     for (int i = 0; i < CTW * 2 * NT; ++i) wr[i] = w2f[i * 64];
     const int col0 = w * (D / 4) + 4 * g;
+    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): the weights; inside the loop the count would be the previous tile's row stores
     for (int sb = 0; sb < nsub; ++sb) {
       const int rows = (np - sb * SP_BT < SP_BT) ? (np - sb * SP_BT) : SP_BT;
       const int tok = s_tok[sb * 32 + c32], dst = s_dst[sb * 32 + c32];
