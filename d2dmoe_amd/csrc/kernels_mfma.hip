@@ -41,6 +41,20 @@ bool mfma_router_supported(const d2dmoe_shape& sh) {
   if ((sh.dtype != D2DMOE_BF16 && sh.dtype != D2DMOE_F16) || sh.router_width <= 0) return false;
   if (sh.router_activation != D2DMOE_ACT_RELU || sh.router_output_activation != D2DMOE_ACT_ABS) return false;
   if (sh.d_model % 64 != 0) return false;
+  // hidden widths 128 and 256; any number of experts that keeps rows of the routing matrix 16-byte aligned, up to 256
+  // (the second product works on tiles of 32 experts: the packed W2 is padded with zero rows)
+  if (sh.router_width != 128 && sh.router_width != 256) return false;
+  return sh.n_experts % 8 == 0 && sh.n_experts >= 8 && sh.n_experts <= 256;
+}
+
+// experts the router kernels compute on: a multiple of 32 they are instantiated for
+int mfma_router_padded_experts(const d2dmoe_shape& sh) {
+  if (sh.router_width == 256) return 256;
+  return sh.n_experts <= 32 ? 32 : (sh.n_experts <= 64 ? 64 : (sh.n_experts <= 128 ? 128 : 256));
+}
+
+// the shapes the resident and the split kernels are written for (the others run the one-wave-per-tile kernel)
+static bool router_shape_exact(const d2dmoe_shape& sh) {
   return (sh.router_width == 128 && sh.n_experts == 128) || (sh.router_width == 256 && sh.n_experts == 256);
 }
 
@@ -91,7 +105,7 @@ PackedLayout packed_layout(const d2dmoe_shape& sh) {
   // to a later call names the router
   L.has_router = mfma_router_supported(sh);
   L.r1_off = off;   if (L.has_router) off += (size_t)sh.router_width * sh.d_model * 2;
-  L.r2_off = off;   if (L.has_router) off += (size_t)sh.n_experts * sh.router_width * 2;
+  L.r2_off = off;   if (L.has_router) off += (size_t)mfma_router_padded_experts(sh) * sh.router_width * 2;
   L.total = (off + 255) / 256 * 256;
   return L;
 }
@@ -160,7 +174,7 @@ __global__ void pack_bias_kernel(const bf16_t* __restrict__ b1, bf16_t* __restri
 //       w = (ks2/2)*32 + (ks2%2)*16 + 8*(i/4) + 4g + (i%4)  (the k order in which the first GEMM leaves the hidden
 //       activations in registers)                                                                   value W2[e][w]
 __global__ void pack_router_kernel(const bf16_t* __restrict__ rw1, const bf16_t* __restrict__ rw2, bf16_t* __restrict__ d1,
-                                   bf16_t* __restrict__ d2, int D, int W, int E) {
+                                   bf16_t* __restrict__ d2, int D, int W, int E, int e_real) {   // E: padded to tiles of 32
   const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t n1 = (int64_t)W * D / 8, n2 = (int64_t)E * W / 8;
   const int lane = (int)(p % 64);
@@ -179,7 +193,7 @@ __global__ void pack_router_kernel(const bf16_t* __restrict__ rw1, const bf16_t*
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int wi = (ks2 / 2) * 32 + (ks2 % 2) * 16 + 8 * (i / 4) + 4 * g + (i % 4);
-      d2[pp * 8 + i] = rw2[(int64_t)(et * 32 + c) * W + wi];
+      d2[pp * 8 + i] = (et * 32 + c < e_real) ? rw2[(int64_t)(et * 32 + c) * W + wi] : (bf16_t)0;
     }
   }
 }
@@ -190,10 +204,11 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
   char* base = (char*)packed;
   if (L.has_router) {
     if (router_w1 == nullptr || router_w2 == nullptr) return hipErrorInvalidValue;
-    const int64_t n = ((int64_t)sh.router_width * sh.d_model + (int64_t)sh.n_experts * sh.router_width) / 8;
+    const int e_pad = mfma_router_padded_experts(sh);
+    const int64_t n = ((int64_t)sh.router_width * sh.d_model + (int64_t)e_pad * sh.router_width) / 8;
     hipLaunchKernelGGL(pack_router_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const bf16_t*)router_w1,
                        (const bf16_t*)router_w2, (bf16_t*)(base + L.r1_off), (bf16_t*)(base + L.r2_off), sh.d_model,
-                       sh.router_width, sh.n_experts);
+                       sh.router_width, e_pad, sh.n_experts);
   }
   if (L.has_sparse) {
     hipError_t e = launch_sparse_pack(sh, L, w1, b1, w2, w_up, packed, s);
@@ -812,7 +827,7 @@ template <int WT, int ET, int U, bool F16 = false>
 __global__ __launch_bounds__(256) void router_select_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16x8* __restrict__ w1f, const bf16x8* __restrict__ w2f,
     bf16_t* __restrict__ routing, bf16_t* __restrict__ norms_out, int32_t* __restrict__ counts, int64_t N, int D,
-    float thr_scale) {
+    float thr_scale, int e_real) {   // e_real <= ET * 32 experts exist (a multiple of 8); the rest are zero rows of W2
   constexpr uint32_t ONE = F16 ? 0x3C00u : 0x3F80u;   // 1.0 in the storage type
   constexpr int E = ET * 32;
   __shared__ __attribute__((aligned(16))) unsigned char stage_all[4 * 32 * E * 2];   // per wave: 32 rows of routing
@@ -910,7 +925,7 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
     for (int i = 0; i < 32 / RPI; ++i) {
       const int row = srow + RPI * i;
       const u32x4 v = stage[row * CH + (spc ^ (row & (CH - 1)))];
-      if (tok0 + row < N) *(u32x4*)(dst + (tok0 + row) * E + spc * 8) = v;
+      if (tok0 + row < N && spc * 8 < e_real) *(u32x4*)(dst + (tok0 + row) * e_real + spc * 8) = v;
     }
     __builtin_amdgcn_wave_barrier();
   };
@@ -949,7 +964,7 @@ __global__ __launch_bounds__(256) void router_select_mfma_kernel(
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
           const unsigned long long bal = __ballot(on[et][q * 4 + s] && valid);
-          if (lane == 0) {
+          if (lane == 0 && et * 32 + 8 * q < e_real) {   // (experts come in blocks of 8: both indices are in or out)
             const int lo = __popcll(bal & 0xffffffffull), hi = __popcll(bal >> 32);
             if (lo) atomicAdd(counts + et * 32 + 8 * q + s, lo);
             if (hi) atomicAdd(counts + et * 32 + 8 * q + 4 + s, hi);
@@ -1382,7 +1397,7 @@ __global__ __launch_bounds__(256) void routing_counts_kernel(const bf16_t* __res
 }
 
 bool mfma_router_writes_plan_counts(const d2dmoe_shape& sh) {
-  return mfma_router_supported(sh) && sh.d_model == RR_D && sh.router_width == 128 &&
+  return mfma_router_supported(sh) && router_shape_exact(sh) && sh.d_model == RR_D && sh.router_width == 128 &&
          sh.n_tokens >= (int64_t)64 * device_cu_count();
 }
 
@@ -1412,7 +1427,7 @@ static hipError_t launch_mfma_router_select_t(const d2dmoe_shape& sh, const void
                        (bf16_t*)norms_out, counts, seg_counts, seg_pairs, sh.n_tokens, thr_scale);
     return hipGetLastError();
   }
-  const bool split = (sh.n_tokens < (int64_t)128 * cus || sh.d_model >= 2048) && (sh.d_model / 16) % 4 == 0;
+  const bool split = router_shape_exact(sh) && (sh.n_tokens < (int64_t)128 * cus || sh.d_model >= 2048) && (sh.d_model / 16) % 4 == 0;
   if (split) {
     const unsigned grid = (unsigned)cdiv64(sh.n_tokens, 32);
     const bool deep = (sh.d_model / 16) % 8 == 0;
@@ -1450,17 +1465,21 @@ static hipError_t launch_mfma_router_select_t(const d2dmoe_shape& sh, const void
     return hipGetLastError();
   }
   const unsigned grid = (unsigned)cdiv64(sh.n_tokens, 128);
+  const bool deep = (sh.d_model / 16) % 8 == 0;
+#define D2DMOE_ROUTER(WT, ET, U)                                                                                         \
+  hipLaunchKernelGGL((router_select_mfma_kernel<WT, ET, U, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing, \
+                     (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale, sh.n_experts)
   if (sh.router_width == 128) {
-    if ((sh.d_model / 16) % 8 == 0)
-      hipLaunchKernelGGL((router_select_mfma_kernel<4, 4, 4, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
-                         (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
-    else
-      hipLaunchKernelGGL((router_select_mfma_kernel<4, 4, 2, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
-                         (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+    switch (mfma_router_padded_experts(sh)) {
+      case 32: if (deep) D2DMOE_ROUTER(4, 1, 4); else D2DMOE_ROUTER(4, 1, 2); break;
+      case 64: if (deep) D2DMOE_ROUTER(4, 2, 4); else D2DMOE_ROUTER(4, 2, 2); break;
+      case 128: if (deep) D2DMOE_ROUTER(4, 4, 4); else D2DMOE_ROUTER(4, 4, 2); break;
+      default: if (deep) D2DMOE_ROUTER(4, 8, 4); else D2DMOE_ROUTER(4, 8, 2); break;
+    }
   } else {
-    hipLaunchKernelGGL((router_select_mfma_kernel<8, 8, 2, F16>), dim3(grid), dim3(256), 0, s, xp, r1, r2, (bf16_t*)routing,
-                       (bf16_t*)norms_out, counts, sh.n_tokens, sh.d_model, thr_scale);
+    D2DMOE_ROUTER(8, 8, 2);
   }
+#undef D2DMOE_ROUTER
   return hipGetLastError();
 }
 

@@ -492,11 +492,15 @@ def test_router_select_resident(N, dtype):
 
 @pytest.mark.parametrize('N,D,W,E', [(197, 768, 128, 128), (1, 768, 128, 128), (33, 768, 128, 128), (1576, 768, 128, 128),
                                      (50432, 768, 128, 128), (16, 2048, 256, 256), (300, 2048, 256, 256),
-                                     (8191, 768, 128, 128), (4100, 2048, 256, 256)])
+                                     (8191, 768, 128, 128), (4100, 2048, 256, 256),
+                                     (1576, 768, 128, 24), (50432, 768, 128, 24), (300, 768, 128, 64), (700, 1024, 128, 200),
+                                     (33, 1280, 128, 160), (500, 2048, 256, 96), (1, 768, 128, 8)])
 @pytest.mark.parametrize('tau', [0.1, 0.9])
 def test_router_select_mfma(N, D, W, E, tau):
     """Fused router + selection: norms within tolerance of the float64 router, mask bit-exact for the kernel's own
-    norms (stage-wise exactness), counts exact, and few mask flips against the oracle's bf16 router."""
+    norms (stage-wise exactness), counts exact, and few mask flips against the oracle's bf16 router.  Expert counts
+    other than the router's hidden width (any multiple of 8 up to 256: the reference benchmark's 24, 64, 96, 160, 200)
+    run on zero-padded tiles of 32 experts."""
     _say('router+select mfma', N, D, W, E, tau)
     Ed = 24 if D == 768 else 8
     x, _, p = H.random_case(N, D, E, Ed, W, seed=N + D, dtype=torch.bfloat16)
