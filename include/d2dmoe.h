@@ -188,7 +188,7 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
  * expert-major: ungated at D = 768 / 1024 / 1280, gated at D = 2048; small batch: D a multiple of 256 -- and tiled
  * products: bf16, f16 or f32, D a multiple of 256) and a router
  * section (when shape.router_width > 0 and the fused router+selection kernel covers the router: bf16 or f16, ReLU/abs,
- * width = experts = 128 or 256). */
+ * hidden width 128 or 256, D a multiple of 64, and a number of experts that is a multiple of 8, at most 256). */
 size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape);
 
 /* Re-tiles expert and router weights into MFMA fragment order.  A derived, cacheable buffer: call once per
