@@ -4,9 +4,10 @@
 //   plan     routing [N,E]  ->  offsets[E+1], token_idx[P] (expert-major, tokens ascending: the canonical permutation),
 //                               tok_off[N+1] (token-major offsets), pair_dst[P] (expert-major pair -> token-major
 //                               slot, experts ascending inside a token), tile_off[E+1] (tiles of 32 pairs), flag
-//   experts  one workgroup per tile of 32 (token, expert) pairs of ONE expert: gather the 32 x rows, GEMM1 against
-//            that expert's W1 fragments, bias + activation + routing weight, GEMM2 against its W2^T fragments, store
-//            the 32 result rows (bf16, as the reference's per-expert intermediate is) at their token-major slots
+//   experts  a workgroup per group of up to 8 tiles of 32 (token, expert) pairs of ONE expert, whose weights stay in
+//            registers while the tiles pass: gather a tile's 32 x rows, GEMM1 against the expert's W1 fragments, bias
+//            + activation + routing weight, GEMM2 against its W2^T fragments, store the 32 result rows (16-bit, as the
+//            reference's per-expert intermediate is) at their token-major slots
 //   combine  out[n] = sum over the token's slots in ascending expert order, float32, one rounding, + last_bias (+ x)
 //            -- the order of the reference's merge kernel (moe_impls.py:499-514), no atomics.
 // Nothing is decided on the host: when the routed pairs exceed the provisioned capacity the flag stays 0, these
