@@ -581,8 +581,21 @@ def reference_shape_record(ops, dev, steps, warmup):
         rows.append({'k_frac': k_frac, 'ms_per_step': r['ms_layer'], 'tokens_per_s': r['tokens_per_s'],
                      'mean_active_experts': r['mean_active'], 'roofline': regime_roofline(r, N, PEAK_BF16_TFLOPS)})
     dense_ms = dense_mlp_ms(x, D, E * Ed, act, steps, warmup)
+    # float16 storage (the reference script times float32 and float16, :223-228): the same kernels on the other 16-bit type
+    p16 = {k: v.to(torch.float16) for k, v in p.items()}
+    x16 = x.to(torch.float16)
+    packed16 = ops.pack_weights(ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x16), act), p16['w1'], p16['b1'], p16['w2'],
+                                None, p16['router_w1'], p16['router_w2'])
+    rows16 = []
+    for k_frac in (1.0, 0.1):
+        g = torch.Generator().manual_seed(int(k_frac * 100))
+        norms_in = (torch.rand(N, E, generator=g) < k_frac).to(torch.float16).to(dev)
+        r = run_regime(ops, x16, p16, packed16, 0.01, act, steps, warmup, D, E, Ed, W, norms_in=norms_in)
+        rows16.append({'k_frac': k_frac, 'ms_per_step': r['ms_layer'], 'tokens_per_s': r['tokens_per_s'],
+                       'mean_active_experts': r['mean_active']})
     return {'workload': f'reference micro-benchmark shape: {B}x{T}={N} tokens, D={D}, {E} experts x {Ed}, {act}, bf16, '
-                        f'Bernoulli(k_frac) router override, tau=0.99', 'dense_mlp_ms': dense_ms, 'rows': rows}
+                        f'Bernoulli(k_frac) router override, tau=0.99', 'dense_mlp_ms': dense_ms, 'rows': rows,
+            'rows_float16': rows16}
 
 
 def main():
