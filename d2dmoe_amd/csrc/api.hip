@@ -402,13 +402,18 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   // next to it;
   // and with at most 128 tokens whatever the fraction -- the layer is bound by the weight stream there, which the tiled
   // products pay for with whole 256-token tiles;
-  // big ungated experts whatever the fraction: the dense sweep cannot skip at their granularity)
+  // big ungated experts from a lower fraction on, and whatever the fraction when the norms are handed in -- the
+  // reference benchmark's Bernoulli override, where the fraction says nothing about the density: the dense sweep
+  // cannot skip at their granularity)
   if (path == D2DMOE_PATH_AUTO && sh.n_tokens > (sh.gated && mfma_decode_supported(sh) ? 48 : 16) && packed != nullptr &&
       (thr_scale >= ((sh.gated || !mfma_dense_supported(sh)) ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128) ||
-       (!sh.gated && sh.expert_dim > 64)) &&
+       (!sh.gated && sh.expert_dim > 64 && (norms_in != nullptr || thr_scale >= 0.5f))) &&
       mfma_sparse_supported(sh) &&
       ((!sh.gated && mfma_dense_supported(sh)) || mfma_gemm_supported(sh)))
     path = D2DMOE_PATH_MFMA_SPARSE;
+  else if (path == D2DMOE_PATH_AUTO && norms_in == nullptr && !sh.gated && sh.expert_dim > 64 && packed != nullptr &&
+           sh.n_tokens > 16 && mfma_dense_supported(sh))
+    path = D2DMOE_PATH_MFMA_DENSE;   // a low fraction from a real router: d2dmoe_experts' own rule would still try the plan
   // ... and when the router kernel of this call is the one that walks the 32-token segments of that path's plan, it
   // leaves the plan's per-segment counts in the workspace on its way
   bool plan_counts_ready = false;

@@ -75,7 +75,8 @@ enum {
                                  most 32: up to 12 / 6 experts per token, tiled products as fall-back).  Gated experts at D = 2048 with at most 64
                                  neurons: up to 32 experts per token (8 beyond 16 384 tokens), else the tiled products
                                  run.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 (gated: >= 0.5); for ungated
-                                 experts of more than 64 neurons AUTO picks it whatever the threshold, in d2dmoe_experts too */
+                                 experts of more than 64 neurons AUTO picks it in d2dmoe_experts, and in d2dmoe_forward when norms_in is
+                                 given or thr_scale >= 0.5 */
   D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 or f16 MFMA for a handful of tokens: per pass of 16 tokens one workgroup per expert streams
                                  that expert's packed weights once (gated or ungated experts); at most 48 tokens (three
                                  passes).  AUTO picks it up to 16 tokens, for gated experts up to 48 */
