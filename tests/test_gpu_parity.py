@@ -266,6 +266,29 @@ def test_experts_mfma_sparse_matches_oracle(N, E, Ed, density):
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('N,D,E,Ed', [(300, 768, 24, 128), (300, 768, 128, 24), (300, 768, 16, 64), (300, 1024, 64, 32),
+                                      (300, 1280, 40, 32), (2600, 768, 3, 128), (1, 768, 1, 24)])
+def test_experts_mfma_sparse_degenerate_routings(N, D, E, Ed, dtype):
+    """Expert-major path on routings that leave the plan with empty or lopsided lists: no pair at all (the output is
+    last_bias), every token on the last expert only (one list, every token finished inside the experts kernel), one
+    token on every expert (E lists of one pair), and one expert per token round-robin with the residual added."""
+    _say('experts sparse degenerate', N, D, E, Ed, dtype)
+    x, _, p = H.random_case(N, D, E, Ed, 8, seed=N + E, dtype=dtype)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, 0, 1 if dtype == torch.bfloat16 else 2, 'relu')
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, None, None)
+    assert packed is not None
+    zeros = torch.zeros(N, E)
+    last = zeros.clone(); last[:, E - 1] = 1
+    one_token = zeros.clone(); one_token[N // 2] = 1
+    diag = zeros.clone(); diag[torch.arange(N), torch.arange(N) % E] = 1
+    for routing, residual in ((zeros, False), (last, False), (one_token, False), (diag, True)):
+        routing = routing.to(dtype)
+        got = _experts_got(x, routing, p, 'relu', residual=residual, path='mfma_sparse', packed=packed)
+        assert H.rel_err(got, _experts_want(x, routing, p, 'relu', residual)) < H.tol_for(dtype)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('N,E,Ed,density,act', [(5000, 24, 128, 0.1, 'relu'), (2000, 10, 100, 0.3, 'gelu'), (33, 24, 128, 0.2, 'relu'),
                                                 (1, 24, 128, 0.5, 'relu'), (9000, 3, 128, 0.5, 'tanh'),
                                                 (50432, 24, 128, 0.1, 'relu'), (50432, 24, 128, 0.5, 'relu')])
