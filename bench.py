@@ -562,6 +562,24 @@ def skew_record(args, ops, dev, steps, warmup):
     return rec
 
 
+def router_driven_record(args, ops, dev, name, steps, warmup):
+    """One of the other ungated layer shapes inside the default line (router-driven, both readings of the threshold)."""
+    B, T, D, E, Ed, W, act = WORKLOADS[name]
+    N = B * T
+    p = make_params(D, E, Ed, W, seed=0, dtype=torch.bfloat16, device=dev)
+    x = torch.randn(N, D, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(dev)
+    packed = ops.pack_weights(ops.make_shape(N, D, E, Ed, W, ops._dtype_code(x), act), p['w1'], p['b1'], p['w2'], None,
+                              p['router_w1'], p['router_w2'])
+    rec = {'workload': f'{name}: {B}x{T}={N} tokens, D={D}, {E} experts x {Ed}, {act}, router {D}->{W}->{E}, whole layer',
+           'dense_mlp_ms': dense_mlp_ms(x, D, E * Ed, act, steps, warmup)}
+    for key, thr in (('module_tau', 1.0 - args.tau), ('literal_rule', args.tau)):
+        r = run_regime(ops, x, p, packed, float(thr), act, steps, warmup, D, E, Ed, W)
+        rec[key] = {'keep_norm_ge_frac_of_max': round(thr, 4), 'ms_per_step': r['ms_layer'], 'tokens_per_s': r['tokens_per_s'],
+                    'mean_active_experts': r['mean_active'], 'router_select_ms': r['ms_router'],
+                    'roofline': regime_roofline(r, N, PEAK_BF16_TFLOPS)}
+    return rec
+
+
 def reference_shape_record(ops, dev, steps, warmup):
     """The shape and sweep of the reference's own micro-benchmark (scripts/test_moe_implementations.py:109-142, 214-285):
     hidden 768, 24 experts x 128 neurons, ReLU, 256 x 197 tokens; the router's output is overridden by Bernoulli(k_frac)
@@ -718,6 +736,8 @@ def main():
             args.steps, args.warmup = saved
             sub['vit_b_skew'] = skew_record(args, ops, dev, sub_steps, sub_warmup)
             sub['reference_shape'] = reference_shape_record(ops, dev, sub_steps, sub_warmup)
+            for w in ('gpt2_medium_layer', 'vit_b_24x128'):
+                sub[w] = router_driven_record(args, ops, dev, w, sub_steps, sub_warmup)
         line['sub_records'] = sub
     if not args.no_cpu_baseline:
         line['cpu_baseline'] = cpu_baseline(D, E, Ed, W, act, args.tau)
