@@ -25,7 +25,7 @@ struct SparseWorkspace {
 };
 
 // Routed pairs per token the path is provisioned for.  Ungated experts (36 KB each at the ViT-B shape): 8 -- the dense
-// sweep is as fast from about 7 on.  Gated experts at the Gemma shape (786 KB each): the tiled products cost 0.8 ms per
+// sweep is as fast from about 8 on.  Gated experts at the Gemma shape (786 KB each): the tiled products cost 0.8 ms per
 // 4096 tokens whatever the routing and the expert-major kernels stay below that up to about 40 pairs per token, so the
 // capacity is 32 -- up to 16 384 tokens, where the per-pair rows (4 KB each) take 2 GB; beyond that 8.
 int mfma_sparse_capacity_k(const d2dmoe_shape& sh) {

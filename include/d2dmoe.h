@@ -70,8 +70,7 @@ enum {
   D2DMOE_PATH_GENERIC = 1,    /* token-tile-major scalar-FMA kernel: any shape, f32, bf16 or f16 storage, f32 math */
   D2DMOE_PATH_MFMA_DENSE = 2, /* bf16 or f16 MFMA, token-tile-major, masked dense sweep over all experts */
   D2DMOE_PATH_MFMA_SPARSE = 3, /* bf16 or f16 MFMA, expert-major over the permutation, then ordered combine; taken when at most
-                                 8 experts per token are routed on average (5 for experts of 33 - 64 neurons; checked on the
-                                 device), else the dense sweep runs.  Ungated experts at D = 768 (also D = 1024 with at most 64 neurons and D = 1280 with at
+                                 8 experts per token are routed on average (checked on the device), else the dense sweep runs.  Ungated experts at D = 768 (also D = 1024 with at most 64 neurons and D = 1280 with at
                                  most 32: up to 12 / 6 experts per token, tiled products as fall-back).  Gated experts at D = 2048 with at most 64
                                  neurons: up to 32 experts per token (8 beyond 16 384 tokens), else the tiled products
                                  run.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 (gated: >= 0.5); for ungated
@@ -86,7 +85,7 @@ enum {
                                  an output-stationary second product adds every expert's contribution, in ascending expert
                                  order, to float32 token rows held in LDS.  Runs when at most 48 experts per token are
                                  routed on average (checked on the device), else the dense sweep does.  Never picked by
-                                 AUTO: it is ahead of the other paths only between about 6 and 9 experts per token */
+                                 AUTO: it is ahead of the other paths only between about 7 and 9 experts per token */
   D2DMOE_PATH_MFMA_GEMM = 5   /* bf16 or f32 MFMA, D a multiple of 256, gated or ungated experts: two tiled products over all
                                  experts with the routing value as a factor of the hidden activations, which stay in
                                  the workspace between them; AUTO picks it for more than 16 tokens when the dense sweep
