@@ -119,6 +119,21 @@ def test_packed_and_workspace_sizes_follow_the_documented_layouts():
     # ViT-B shape: dense-sweep stream (4 waves x 12 chunks x 192 fragments of 1 KB) is part of the buffer
     v = ops.make_shape(50432, 768, 128, 24, 128, abi.BF16)
     assert lib.d2dmoe_packed_bytes(ctypes.byref(v)) >= 4 * 12 * 192 * 1024
+    # router section: W2 is padded with zero rows to the next of 32 / 64 / 128 / 256 experts, so the same layer with and
+    # without a router differs by W1 + padded W2; 24 experts take one tile of 32, 100 experts have no fused router
+    for E, Ed, pad in ((24, 128, 32), (64, 48, 64), (128, 24, 128)):
+        with_r = lib.d2dmoe_packed_bytes(ctypes.byref(ops.make_shape(0, 768, E, Ed, 128, abi.BF16)))
+        without = lib.d2dmoe_packed_bytes(ctypes.byref(ops.make_shape(0, 768, E, Ed, 0, abi.BF16)))
+        assert 0 <= with_r - without - (128 * 768 + pad * 128) * 2 < 512, (E, with_r - without)
+    e100 = ops.make_shape(0, 768, 100, 30, 128, abi.BF16)
+    assert lib.d2dmoe_packed_bytes(ctypes.byref(e100)) == lib.d2dmoe_packed_bytes(
+        ctypes.byref(ops.make_shape(0, 768, 100, 30, 0, abi.BF16)))
+    # expert-major workspace at D = 768: provisioned for 8 routed experts per token whatever the expert size (rows of
+    # 768 16-bit values per pair, token and slot lists of 4 bytes each)
+    for E, Ed in ((128, 24), (48, 64), (24, 128)):
+        ws = lib.d2dmoe_workspace_bytes(ctypes.byref(ops.make_shape(50432, 768, E, Ed, 128, abi.BF16)))
+        want = 8 * 50432 * (768 * 2 + 8)
+        assert want <= ws <= want + (64 << 20), (E, Ed, ws)
 
 
 # ------------------------------------------------------------------ host-side module mirror -------------
