@@ -313,7 +313,7 @@ def gated_record(args, ops, dev, workload):
     return line
 
 
-def run_gpt2(args, dev):
+def gpt2_record(args, dev):
     """Whole-model workload: GPT-2-small (12 blocks, D = 768, 12 heads, vocab 50257) with every FFN replaced by a MoE layer
     of 128 experts x 24 neurons (GELU-erf, biases) and a 768 -> 128 -> 128 router; 16 x 1024 token ids; bf16; random
     weights.  Attention, LayerNorm, embeddings and the LM head are stock PyTorch; the MoE layers are this library."""
@@ -388,7 +388,11 @@ def run_gpt2(args, dev):
                      'achieved': active / ms_experts / 1e9, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': active / ms_experts / 1e9 / PEAK_BF16_TFLOPS, 'traffic': None, 'kernel_ms': ms_experts},
     }
-    print(json.dumps(line))
+    return line
+
+
+def run_gpt2(args, dev):
+    print(json.dumps(gpt2_record(args, dev)))
 
 
 def run_vit(args, dev):
@@ -738,6 +742,16 @@ def main():
             sub['reference_shape'] = reference_shape_record(ops, dev, sub_steps, sub_warmup)
             for w in ('gpt2_medium_layer', 'vit_b_24x128'):
                 sub[w] = router_driven_record(args, ops, dev, w, sub_steps, sub_warmup)
+            # BASELINE config 4 in short: the whole GPT-2-small forward with MoE FFNs (few steps: a step is 7 ms)
+            saved = args.steps, args.warmup
+            args.steps, args.warmup = max(saved[0] // 5, 5), 2
+            g = gpt2_record(args, dev)
+            args.steps, args.warmup = saved
+            sub['gpt2_small'] = {'workload': g['config']['workload'], 'model_ms': g['ms_per_step'], 'tokens_per_s': g['value'],
+                                 'dense_model_ms': g['dense_model_ms'], 'moe_layers_ms': g['moe_layers_ms'],
+                                 'dense_ffn_layer_ms': g['dense_ffn_layer_ms'],
+                                 'mean_active_experts': sum(r['mean_active_experts'] for r in g['per_layer']) / len(g['per_layer']),
+                                 'literal_rule': g['literal_rule'], 'roofline': g['roofline']}
         line['sub_records'] = sub
     if not args.no_cpu_baseline:
         line['cpu_baseline'] = cpu_baseline(D, E, Ed, W, act, args.tau)
