@@ -265,6 +265,40 @@ def test_experts_mfma_sparse_matches_oracle(N, E, Ed, density):
     assert torch.equal(got, _experts_got(x, routing, p, 'relu', path='mfma_sparse', packed=packed))   # deterministic
 
 
+def test_layer_big_experts_auto_paths():
+    """d2dmoe_forward under AUTO with 24 experts of 128 neurons (the reference benchmark's split): with the norms
+    handed in (the Bernoulli override of scripts/test_moe_implementations.py:136-142, tau 0.99) the expert-major path
+    runs whatever the threshold, and above its capacity the sweep takes over on the device; behind the real router a low
+    threshold fraction goes straight to the sweep and a high one to the expert-major path.  Each result must be, bit for
+    bit, what the experts entry point gives for the same routing on the path named."""
+    N, D, E, Ed, W = 3000, 768, 24, 128, 128
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=5, dtype=torch.bfloat16)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, W, 1, 'relu')
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, d['router_w1'], d['router_w2'])
+    lb = d['last_bias'].view(-1)
+    xd = x.to(DEV)
+
+    def layer(thr_scale, norms_in):
+        return _ops().forward(xd, d['router_w1'], d['router_w2'], thr_scale, d['w1'], d['b1'], d['w2'], None, lb, 'relu',
+                              False, norms_in, False, False, 'auto', packed)
+
+    def experts(routing, path):
+        return _ops().experts(xd, routing, d['w1'], d['b1'], d['w2'], None, lb, 'relu', False, path, packed)
+
+    for k_frac, path in ((0.1, 'mfma_sparse'), (0.9, 'mfma_dense')):
+        g = torch.Generator().manual_seed(int(k_frac * 10))
+        norms_in = (torch.rand(N, E, generator=g) < k_frac).to(torch.bfloat16).to(DEV)
+        out, routing, _, _ = layer(0.01, norms_in)
+        assert torch.equal(routing.cpu(), O.gate_dynk_max(norms_in.cpu(), 0.99))
+        assert torch.equal(out, experts(routing, path)), (k_frac, path)
+        assert H.rel_err(out.cpu(), _experts_want(x, routing.cpu(), p, 'relu')) < H.TOL_BF16
+    for thr_scale, path in ((0.1, 'mfma_dense'), (0.9, 'mfma_sparse')):
+        out, routing, _, _ = layer(thr_scale, None)
+        assert torch.equal(out, experts(routing, path)), (thr_scale, path)
+        assert H.rel_err(out.cpu(), _experts_want(x, routing.cpu(), p, 'relu')) < H.TOL_BF16
+
+
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('N,D,E,Ed', [(300, 768, 24, 128), (300, 768, 128, 24), (300, 768, 16, 64), (300, 1024, 64, 32),
                                       (300, 1280, 40, 32), (2600, 768, 3, 128), (1, 768, 1, 24)])
