@@ -273,6 +273,10 @@ static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* ro
       if (!packed) return D2DMOE_E_NULL;
       const size_t need = mfma_sparse_workspace_bytes(sh);
       if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
+      // the tiled products of the fall-back work behind the plan: they must fit what is left there
+      if (fb_gemm && sh.n_tokens * (int64_t)sh.n_experts > mfma_sparse_capacity_pairs(sh) &&
+          workspace_bytes < mfma_sparse_fallback_offset(sh) + mfma_gemm_workspace_bytes(sh))
+        return D2DMOE_E_WORKSPACE;
       const int* flag = nullptr;
       hipError_t e = launch_mfma_sparse(sh, x, routing, packed, last_bias, out, workspace, mfma_sparse_capacity_k(sh), &flag, s,
                                         plan_counts_ready);

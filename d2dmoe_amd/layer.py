@@ -185,8 +185,9 @@ class MoeficationMoE(MoELayer):
         if self.router is None or not (self.router.test_override_outputs_p is not None or self.router.hip_compatible()):
             return False
         if torch.is_grad_enabled() and _grad_wanted(x, *self.parameters()):
-            raise NotImplementedError("the HIP layer path has no backward; wrap the call in torch.no_grad(), or switch the "
-                                      "experts to a PyTorch forward_mode for training")
+            raise NotImplementedError(f"MoE layer {getattr(self, 'name', None)!r}: the HIP layer path has no backward; wrap the "
+                                      "call in torch.no_grad() / torch.inference_mode() or call requires_grad_(False) on "
+                                      "the layer, or switch the experts to a PyTorch forward_mode for training")
         return True
 
     def _router_operands(self):

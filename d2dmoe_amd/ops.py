@@ -272,11 +272,17 @@ class PreparedForward:
         self.shapes = {}
         # the router section is the last one of a packed buffer: a buffer packed without it serves calls that bring their
         # own predicted norms (norms_in), and only those
-        _check_packed(self.lib, make_shape(0, self.d, self.e, self.ed, 0, self.code, **self.kw), packed)
+        # (a layer whose experts have no MFMA kernel can still carry a router section only: then the router-less size is 0
+        # and the buffer is held to the size with the router)
         self.router_packed_ok = True
-        if packed is not None and self.w > 0:
-            need = self.lib.d2dmoe_packed_bytes(self.shape_for(0)[1])
-            self.router_packed_ok = packed.numel() * packed.element_size() >= need
+        if packed is not None:
+            have = packed.numel() * packed.element_size()
+            bare = self.lib.d2dmoe_packed_bytes(ctypes.byref(make_shape(0, self.d, self.e, self.ed, 0, self.code, **self.kw)))
+            full = self.lib.d2dmoe_packed_bytes(self.shape_for(0)[1]) if self.w > 0 else bare
+            if (bare == 0 and full == 0) or have < bare or (bare == 0 and have < full):
+                raise abi.D2DMoEError(f'packed buffer holds {have} bytes but this shape/dtype needs {bare if bare else full}: '
+                                      'it was packed for other weights (pack again with the shape of this call)')
+            self.router_packed_ok = have >= full
 
     def shape_for(self, n: int):
         got = self.shapes.get(n)

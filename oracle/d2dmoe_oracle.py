@@ -97,14 +97,6 @@ ACTIVATIONS: Dict[str, Callable[[torch.Tensor], torch.Tensor]] = {
 # --------------------------------------------------------------------------------------------
 
 
-def init_uniform_(p: torch.Tensor) -> torch.Tensor:
-    """U(-1/sqrt(last_dim), +1/sqrt(last_dim)) in place  (moe_layers.py:19-24)."""
-    bound = 1.0 / math.sqrt(p.size(-1))
-    with torch.no_grad():
-        p.uniform_(-bound, bound)
-    return p
-
-
 def make_layer_params(d_model: int, n_experts: int, expert_dim: int, router_width: int,
                       seed: int, gated: bool = False, bias: bool = True,
                       dtype: torch.dtype = torch.float32) -> Dict[str, torch.Tensor]:

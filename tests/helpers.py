@@ -33,6 +33,18 @@ def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
     return (got - want).abs().max().item() / denom
 
 
+def elem_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    """Element-wise companion of rel_err: max |got - want| / (|want| + max|want| / 16).  Unlike the max-norm ratio it
+    holds every element to a bound that shrinks with the element, down to a floor of a sixteenth of the largest one
+    (below that floor an element of a sum of many rounded terms carries no relative accuracy of its own)."""
+    got = got.detach().double().cpu()
+    want = want.detach().double().cpu()
+    floor = want.abs().max().item() / 16.0
+    if floor == 0.0:
+        return got.abs().max().item()
+    return ((got - want).abs() / (want.abs() + floor)).max().item()
+
+
 def tol_for(dtype) -> float:
     return {torch.float32: TOL_F32, torch.bfloat16: TOL_BF16, torch.float16: TOL_F16}[dtype]
 

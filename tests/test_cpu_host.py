@@ -136,6 +136,28 @@ def test_packed_and_workspace_sizes_follow_the_documented_layouts():
         assert want <= ws <= want + (64 << 20), (E, Ed, ws)
 
 
+def test_expert_major_workspace_covers_its_tiled_products_fallback():
+    """Ungated D = 768 layers the fused sweep does not cover (more than 256 experts, or more than 32 chunks of 256 hidden
+    neurons) fall back, behind the expert-major plan, to the tiled products, which work in the workspace BEHIND the plan:
+    the size query must cover router scratch + the plan's lists + the products' own need (hidden fragments of whole
+    256-token tiles + float32 partial sums)."""
+    from d2dmoe_amd import hip_abi as abi, ops
+    lib = abi.load()
+    for N, E, Ed in ((4096, 512, 32), (4096, 320, 32), (1000, 256, 64), (8192, 384, 24), (300, 1024, 8)):
+        for dt in (abi.BF16, abi.F16):
+            ws = lib.d2dmoe_workspace_bytes(ctypes.byref(ops.make_shape(N, 768, E, Ed, 128, dt)))
+            edp = Ed if Ed % 4 == 0 else (Ed + 31) // 32 * 32
+            hp = (E * edp + 255) // 256 * 256
+            n_ttiles = (min(N, 8192) + 255) // 256
+            tiles, ks2, ksplit = n_ttiles * 3, hp // 16, 1
+            while ksplit < 8 and tiles * ksplit < 256 and (ks2 // (ksplit * 2)) % 4 == 0:
+                ksplit *= 2
+            gemm = n_ttiles * 256 * hp * 2 + ksplit * min(N, 8192) * 768 * 4
+            plan_lists = 2 * 8 * N * 4 + (N + 1) * 4
+            router = N * (128 + E) * 2
+            assert ws >= router + plan_lists + gemm, (N, E, Ed, dt, ws, router + plan_lists + gemm)
+
+
 # ------------------------------------------------------------------ host-side module mirror -------------
 def _toy_layer(act=nn.ReLU, experts_class='hip_kernel'):
     from d2dmoe_amd import MoeficationMoE, MoeficationRouter

