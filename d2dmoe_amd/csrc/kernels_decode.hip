@@ -1,8 +1,10 @@
 // Small-batch ("decode") bf16 MFMA path: at most 16 tokens, so the layer is bound by streaming the weights of the
 // routed experts once.  One workgroup per expert pulls that expert's packed gate/up weights through
 // v_mfma_f32_16x16x32_bf16 with all tokens resident in LDS and leaves the hidden activations (256 KB for 256 experts
-// of 32 neurons) in memory; a second kernel owns 16 output columns per workgroup and sums the down projections of the
-// routed experts in ascending order.  Also here: a skinny Linear kernel (router layers for <= 16 tokens) that needs no packing.
+// of 32 neurons) in memory; a second kernel owns 32 output columns and a range of experts per workgroup, requests that
+// range's down-projection weights in one go, and sums the routed experts in ascending order (workgroups that share a
+// column block add their partial sums in range order).  Also here: a skinny Linear kernel (router layers for <= 16
+// tokens) that needs no packing.
 //
 // Fragment layouts of the 16x16x32 bf16 MFMA on a 64-lane wave (gq = lane / 16, c = lane % 16):
 //   A (16 x 32): lane holds row c,    k = 8 gq .. 8 gq + 7
@@ -48,10 +50,45 @@ bool mfma_decode_supported(const d2dmoe_shape& sh) {
 
 size_t mfma_decode_packed_bytes(const d2dmoe_shape& sh) { return mfma_decode_supported(sh) ? decode_layout(sh).total : 0; }
 
+constexpr int DO_WAVES = 8;
+constexpr int DO_COLS = 32;          // output columns per workgroup of the output kernel
+constexpr int DO_MAX_SPLIT = 16;     // expert ranges per column block at most
+
+// Expert ranges per column block of the output kernel.  A wave keeps the down-projection fragments of all its experts in
+// registers (KS2 * 12 registers per expert, 16 / KS2 experts at most), so a workgroup of 8 waves covers at most
+// 128 / KS2 experts; beyond that, and while the grid would leave CUs without a workgroup, the experts are cut into more
+// ranges.
+static int decode_split(const d2dmoe_shape& sh) {
+  const int ks2 = decode_layout(sh).nt16 / 2;
+  const int per_wg = DO_WAVES * (16 / ks2);
+  int q = (sh.n_experts + per_wg - 1) / per_wg;
+  const int col_blocks = sh.d_model / DO_COLS;
+  const int fill = (device_cu_count() + col_blocks - 1) / col_blocks;
+  if (fill > q) q = fill;
+  const int q_max = (sh.n_experts + DO_WAVES - 1) / DO_WAVES;   // at least one expert per wave
+  if (q > q_max) q = q_max;
+  if (q > DO_MAX_SPLIT) q = DO_MAX_SPLIT;
+  return q < 1 ? 1 : q;
+}
+
+struct DecodeWorkspace { size_t hfrag, active, partial, tickets, total; };
+
+static DecodeWorkspace decode_workspace(const d2dmoe_shape& sh) {
+  DecodeWorkspace W;
+  auto up = [](size_t v) { return (v + 255) / 256 * 256; };
+  size_t off = 0;
+  W.hfrag = off;   off += up((size_t)sh.n_experts * decode_layout(sh).edp * DC_MAX_TOKENS * 2);   // hidden fragments
+  W.active = off;  off += up((size_t)sh.n_experts * 4);                                           // "some token routes here"
+  // float32 partial sums [column block][range][16 tokens x 32 columns], sized for the largest split
+  W.partial = off; off += up((size_t)(sh.d_model / DO_COLS) * DO_MAX_SPLIT * DC_MAX_TOKENS * DO_COLS * 4);
+  W.tickets = off; off += up((size_t)(sh.d_model / DO_COLS) * 4);                                 // arrivals per column block
+  W.total = off;
+  return W;
+}
+
 size_t mfma_decode_workspace_bytes(const d2dmoe_shape& sh) {
   if (!mfma_decode_supported(sh)) return 0;
-  // hidden activations as bf16 fragments, then one "some token routes here" flag per expert
-  return (size_t)sh.n_experts * decode_layout(sh).edp * DC_MAX_TOKENS * 2 + (size_t)sh.n_experts * 4;
+  return decode_workspace(sh).total;
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -59,7 +96,7 @@ size_t mfma_decode_workspace_bytes(const d2dmoe_shape& sh) {
 // the two kernels below reads ONE contiguous stream.
 //   gate(/up) stream [E][block NB][kstep KS][matrix NM][tile 2][lane 64][8]:
 //                    neuron j = block*32 + tile*16 + c, d = kstep*32 + 8 gq + i                          w[e][d][j]
-//   down^T stream    [column block D/8][E][kstep2 NB][gq 4][c8 8][8]:  column = cb*8 + c8,
+//   down^T stream    [column block D/32][E][kstep2 NB][column tile 2][lane 64][8]:  column = cb*32 + tile*16 + c,
 //                    neuron j = ks2*32 + 16*(i/4) + 4 gq + (i%4)                                         w2[e][j][column]
 //   bias             [E][EdP] bf16
 // ---------------------------------------------------------------------------------------------------
@@ -70,7 +107,7 @@ __global__ void pack_decode_kernel(const bf16_t* __restrict__ w1, const bf16_t* 
   const int nm = (w_up != nullptr) ? 2 : 1;
   const int KS = D / 32, NB = edp / 32;
   const int64_t n_gu = (int64_t)E * NB * KS * nm * 2 * 64;   // 16-byte pieces
-  const int64_t n_d = (int64_t)(D / 8) * E * NB * 32;
+  const int64_t n_d = (int64_t)(D / 32) * E * NB * 2 * 64;
   if (p < n_gu) {
     int64_t q = p;
     const int lane = (int)(q % 64); q /= 64;
@@ -90,12 +127,13 @@ __global__ void pack_decode_kernel(const bf16_t* __restrict__ w1, const bf16_t* 
   } else if (p < n_gu + n_d) {
     const int64_t pp = p - n_gu;
     int64_t q = pp;
-    const int c8 = (int)(q % 8); q /= 8;
-    const int gq = (int)(q % 4); q /= 4;
+    const int lane = (int)(q % 64); q /= 64;
+    const int tile = (int)(q % 2); q /= 2;
     const int ks2 = (int)(q % NB); q /= NB;
     const int e = (int)(q % E);
     const int cb = (int)(q / E);
-    const int col = cb * 8 + c8;
+    const int gq = lane / 16;
+    const int col = cb * 32 + tile * 16 + lane % 16;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int j = ks2 * 32 + 16 * (i / 4) + 4 * gq + (i % 4);
@@ -131,11 +169,15 @@ hipError_t launch_decode_pack(const d2dmoe_shape& sh, const void* w1, const void
 //   hidden  gated: act(g) * u, else act(g + b1); times the routing weight; rounded to bf16 and stored as one B
 //           fragment of the second product: hfrag[e][block][lane]
 //
-// decode_out_kernel: workgroup = 8 output columns, 8 waves.
-//   the routed experts are listed in ascending order and cut into 8 consecutive runs, one per wave; a wave chains
-//   OUT^T += W2[e]^T . H[e]^T over its run in one float32 accumulator (rows 8..15 of the 16-row MFMA tile repeat
-//   rows 0..7 and are dropped); the 8 partial tiles are added in wave order, then last_bias and the residual, one
-//   rounding.  The summation order depends on the routing only.
+// decode_out_kernel: workgroup = (block of 32 output columns, range of experts), 8 waves, two waves per SIMD.
+//   Wave w owns a run of consecutive experts of the range.  It first requests the down-projection fragments of ALL of them
+//   (nothing it has to compute decides that), then -- whole layer only -- works out the second router layer and the
+//   selection while those loads are in flight, then requests the hidden fragments of its experts and chains
+//   OUT^T += W2[e]^T . H[e]^T over them in ascending order in two float32 accumulators (one per tile of 16 columns).  The 8
+//   partial tiles are added in wave order.  Ranges of one column block (when the experts are cut into several, so that
+//   the grid covers the machine) leave their sums in the workspace; the last of them to arrive, found by an arrival
+//   counter, adds them in range order.  Then last_bias, the residual, one rounding.  The summation order depends on the
+//   routing and the launch shape only, never on timing.
 // ---------------------------------------------------------------------------------------------------
 struct DecodeArgs {
   const bf16_t* x; const bf16_t* routing; const bf16x8* wgu; const bf16x8* wd; const bf16_t* bias;
@@ -144,7 +186,9 @@ struct DecodeArgs {
   // and its extra workgroups compute the first router layer; the output kernel derives the routing from the norms itself.
   int fused;
   const bf16_t* rw1; bf16_t* rhidden; int rwidth; int ract;     // first router layer: [rwidth, D] -> rhidden [N, rwidth]
-  const bf16_t* norms; bf16_t* routing_out; int32_t* counts; float thr_scale;
+  bf16_t* norms; bf16_t* routing_out; int32_t* counts; float thr_scale;
+  const bf16_t* rw2; int roact;           // second router layer [E, rwidth], output activation (computed by the output kernel)
+  float* partial; int* tickets; int split;   // output kernel: expert ranges per column block, their sums and arrival counters
 };
 
 // First router layer inside the hidden kernel's launch: 4 features per workgroup of 4 waves.  K is cut into the same parts
@@ -207,6 +251,9 @@ __global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) 
     decode_router_l1_block<F16>(A, (int)blockIdx.x, (float (*)[4][64])part_raw);
     return;
   }
+  // the output kernel's arrival counters start at zero (it runs after this grid)
+  if (blockIdx.x == gridDim.x - 1 && A.split > 1)
+    for (int i = threadIdx.x; i < D / DO_COLS; i += 256) A.tickets[i] = 0;
   const int hb = (int)blockIdx.x - n_router;
   const int KS = D / 32;          // K steps of GEMM1
   const int KQ = KS / 4;          // per wave
@@ -293,37 +340,171 @@ __global__ __launch_bounds__(256) void decode_hidden_kernel(const DecodeArgs A) 
   ((uint4*)A.hfrag)[((int64_t)e * KS2 + k2) * 64 + lane] = pk;
 }
 
-constexpr int DO_WAVES = 8;
+// Second router layer for NT 16-feature tiles ft[0..NT), by one wave, with the bits of linear_skinny_kernel: K is cut into
+// the same parts (16 where K is long, else 4), each accumulated on its own in K order, the parts summed in order, the sum
+// rounded to the storage type before the activation.  nb[i][r]: the lane's norms of tile i (token c16, features
+// ft[i]*16 + 4 gq + r) as storage bits.
+// KQS > 0 (K = 128 * KQS, K steps of 32 per part): every operand is requested by router_l2_request before anything else
+// of the kernel, so that these loads do not queue up behind the weight stream (a wave's loads return in order).
+template <int NT, int KQS>
+struct RouterL2Operands { bf16x8 av[KQS > 0 ? 4 * KQS : 1], bv[NT][KQS > 0 ? 4 * KQS : 1]; };
 
-// Workgroup = 8 output columns, 8 waves; wave w owns experts [w*EW, (w+1)*EW) with EW = ceil(E/8) rounded up to 64 at
-// most per pass, and walks the routed ones among them in ascending order.
-template <int KS2, bool F16 = false>
+template <int NT, int KQS>
+__device__ __forceinline__ void router_l2_request(const DecodeArgs& A, const int (&ft)[NT], int lane, RouterL2Operands<NT, KQS>& R) {
+  if constexpr (KQS > 0) {
+    const int gq = lane >> 4, c16 = lane & 15;
+    const int K = A.rwidth;
+    const int trow = (c16 < A.N) ? c16 : (A.N - 1);
+    const bf16x8* ap = (const bf16x8*)(A.rhidden + (int64_t)trow * K) + gq;
+#pragma unroll
+    for (int ks = 0; ks < 4 * KQS; ++ks) R.av[ks] = ap[ks * 4];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      const bf16x8* bp = (const bf16x8*)(A.rw2 + (int64_t)(ft[i] * 16 + c16) * K) + gq;
+#pragma unroll
+      for (int ks = 0; ks < 4 * KQS; ++ks) R.bv[i][ks] = bp[ks * 4];
+    }
+  }
+}
+
+template <bool F16, int NT, int KQS>
+__device__ __forceinline__ void router_l2_finish(const DecodeArgs& A, const int (&ft)[NT], int lane, const RouterL2Operands<NT, KQS>& R,
+                                                 uint16_t (&nb)[NT][4]) {
+  float v[NT][4];
+  if constexpr (KQS > 0) {
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < KQS; ++k) acc = mfma_16x16x32<F16>(R.bv[i][p * KQS + k], R.av[p * KQS + k], acc);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[i][r] = (p == 0) ? acc[r] : v[i][r] + acc[r];
+      }
+    }
+  } else {
+    const int gq = lane >> 4, c16 = lane & 15;
+    const int K = A.rwidth;
+    const int trow = (c16 < A.N) ? c16 : (A.N - 1);
+    const bf16x8* ap = (const bf16x8*)(A.rhidden + (int64_t)trow * K) + gq;
+    const int P = (K % 512 == 0 && K >= 1024) ? 16 : 4;
+    const int KQ = K / P;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      const bf16x8* bp = (const bf16x8*)(A.rw2 + (int64_t)(ft[i] * 16 + c16) * K) + gq;
+      for (int p = 0; p < P; ++p) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int ks = 0; ks < KQ / 32; ++ks) acc = mfma_16x16x32<F16>(bp[(p * (KQ / 32) + ks) * 4], ap[(p * (KQ / 32) + ks) * 4], acc);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[i][r] = (p == 0) ? acc[r] : v[i][r] + acc[r];
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NT; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) nb[i][r] = enc16<F16>(apply_act(A.roact, round16<F16>(v[i][r])));
+}
+
+// Workgroup = (column block cb, expert range q): blockIdx.x = cb * split + q.  KS2 = 32-neuron K steps per expert.
+// KQS: see router_l2_request (whole layer with a router of width 128 * KQS; 0 otherwise).
+template <int KS2, bool F16 = false, int KQS = 0>
 __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeArgs A) {
-  constexpr int UB = 8 / KS2;                  // experts per load batch (8 hidden fragments, half as many weight loads;
-                                               // twice as many in flight was slower: 18.7 against 16.7 us at 16 tokens)
-  __shared__ float part[DO_WAVES][4][64];
+  constexpr int ME = 16 / KS2;                 // experts a wave keeps in registers at most
+  __shared__ float part[DO_WAVES][2][4][64];
   __shared__ float s_thr[16];                  // fused: the tokens' thresholds
   __shared__ unsigned short s_bits[DO_WAVES * 64];   // fused: per expert, bit t = token t routes to it
+  __shared__ bf16_t s_norms[DC_MAX_TOKENS][DO_WAVES * 64 + 8];   // fused: the norms tile
+  __shared__ int s_last;
   const int D = A.D, N = A.N, E = A.E;
-  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  const int w = __builtin_amdgcn_readfirstlane(t >> 6);   // uniform: the branches on a wave's experts are scalar
   const int gq = lane >> 4, c16 = lane & 15;
-  const int cb = blockIdx.x;                   // 8-column block
-  const int EW = (E + DO_WAVES - 1) / DO_WAVES;
-  const int e_lo = w * EW, e_hi = (e_lo + EW < E) ? (e_lo + EW) : E;
-  if (A.fused) {
-    // Dynamic-k selection from the norms (moefication.py:80-85), by every workgroup for itself (8 KB out of L2): wave 0
-    // takes the maximum of every token's row, then a lane per expert compares its column with the thresholds.  Same
-    // arithmetic as select_kernel: m NaN-propagating, thr = round(m * thr_scale), on = norm >= thr.
-    // (E <= 512 here: one expert per thread; its column is requested before the maxima are worked out)
-    const int ecol = (t < E) ? t : (E - 1);
-    bf16_t colv[DC_MAX_TOKENS];
+  const int Q = A.split;
+  const int cb = (int)blockIdx.x / Q, q = (int)blockIdx.x % Q;
+  const int EPG = (E + Q - 1) / Q;                              // experts per range
+  const int EPW = (EPG + DO_WAVES - 1) / DO_WAVES;              // ... per wave (<= ME: the launcher's choice of Q)
+  const int g_lo = q * EPG, g_hi = (g_lo + EPG < E) ? (g_lo + EPG) : E;
+  const int e_lo = g_lo + w * EPW;
+  const int e_hi = (e_lo + EPW < g_hi) ? (e_lo + EPW) : g_hi;   // may be <= e_lo: a wave without experts
+
+  // ---- 0. whole layer: the operands of this wave's first two tiles of the second router layer, ahead of everything
+  const int E16 = E / 16;
+  int ft_first[2] = {w < E16 ? w : 0, (w + DO_WAVES < E16) ? (w + DO_WAVES) : (w < E16 ? w : 0)};
+  RouterL2Operands<2, KQS> rl2;
+  if (A.fused) router_l2_request<2, KQS>(A, ft_first, lane, rl2);
+
+  // ---- 1. the down-projection fragments of every expert of this wave (not fused: of those some token routes to; the
+  // flags of the wave's experts come in with one load and a ballot, so that the branches below are scalar and no load
+  // waits for another)
+  bf16x8 wa[ME][KS2][2];
+  unsigned umask;                              // bit j: expert e_lo + j is in use
+  {
+    const int e = e_lo + (lane < ME ? lane : 0);
+    const bool mine = lane < ME && lane < EPW && e < e_hi;
+    const int flag = (A.fused || !mine) ? 1 : A.active[e];
+    umask = (unsigned)__ballot(mine && flag != 0);
+  }
+  const bf16x8* wdf = A.wd + (int64_t)cb * E * KS2 * 2 * 64 + lane;
+  const bf16x8 zero8 = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+  auto request_weights = [&](auto j_c) __attribute__((always_inline)) {
+    constexpr int j = decltype(j_c)::value;
+    if constexpr (KQS > 0) {
+      // whole layer: every expert of the wave, without a branch (the compiler can then count the loads that follow the
+      // router's and wait for those alone); a slot past the wave's experts repeats a valid expert and is cleared later
+      const int e = (e_lo + j < E) ? (e_lo + j) : (E - 1);
 #pragma unroll
-    for (int tk = 0; tk < DC_MAX_TOKENS; ++tk) colv[tk] = A.norms[(int64_t)(tk < N ? tk : N - 1) * E + ecol];
+      for (int k2 = 0; k2 < KS2; ++k2)
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) wa[j][k2][ct] = wdf[(((int64_t)e * KS2 + k2) * 2 + ct) * 64];
+    } else if ((umask >> j) & 1u) {
+#pragma unroll
+      for (int k2 = 0; k2 < KS2; ++k2)
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) wa[j][k2][ct] = wdf[(((int64_t)(e_lo + j) * KS2 + k2) * 2 + ct) * 64];
+    } else {
+#pragma unroll
+      for (int k2 = 0; k2 < KS2; ++k2)
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) wa[j][k2][ct] = zero8;
+    }
+  };
+  // (whole layer with the router operands in registers: the last quarter of the experts is requested once those
+  // registers are free again, or the kernel spills -- and a reload from scratch would queue up behind the weight stream)
+  constexpr int ME_FIRST = (KQS > 0) ? (ME - ME / 4) : ME;
+  static_for<0, ME_FIRST>(request_weights);
+  __builtin_amdgcn_sched_barrier(0);
+
+  if (A.fused) {
+    // ---- 2. second router layer (every workgroup for itself: rwidth * E * 2 bytes out of L2) and the dynamic-k selection
+    // (moefication.py:80-85).  Wave w takes the feature tiles w, w + 8, ...; wave 0 then takes the maximum of every
+    // token's row, and a thread per expert compares its column with the thresholds.  Same arithmetic as select_kernel:
+    // m NaN-propagating, thr = round(m * thr_scale), on = norm >= thr.
+    // (two tiles at a time; the tile index of a wave without a second tile repeats its first: same values, same place)
+    for (int ft0 = w; ft0 < E16; ft0 += 2 * DO_WAVES) {
+      const int ft[2] = {ft0, (ft0 + DO_WAVES < E16) ? (ft0 + DO_WAVES) : ft0};
+      uint16_t nb[2][4];
+      if (ft0 == w) {
+        router_l2_finish<F16, 2, KQS>(A, ft, lane, rl2, nb);          // requested at the top
+      } else {
+        RouterL2Operands<2, 0> none;
+        router_l2_finish<F16, 2, 0>(A, ft, lane, none, nb);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s_norms[c16][ft[i] * 16 + 4 * gq + r] = nb[i][r];
+      }
+    }
+    static_for<ME_FIRST, ME>(request_weights);
+    __builtin_amdgcn_sched_barrier(0);
+    // (barriers of this phase order LDS traffic only: __syncthreads would wait for the weight loads in flight)
+    lds_barrier();
     if (w == 0) {
-      const int tc = (c16 < N) ? c16 : (N - 1);
       float m = -INFINITY;
       for (int e8 = gq * 8; e8 < E; e8 += 32) {          // E is a multiple of 32 here
-        const u32x4 v = *(const u32x4*)(A.norms + (int64_t)tc * E + e8);
+        const u32x4 v = *(const u32x4*)(&s_norms[c16][e8]);
         const uint32_t vw[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int i = 0; i < 8; ++i) m = nanmax(m, (i & 1) ? dec16_hi<F16>(vw[i >> 1]) : dec16<F16>(vw[i >> 1] & 0xffffu));
@@ -336,105 +517,105 @@ __global__ __launch_bounds__(DO_WAVES * 64) void decode_out_kernel(const DecodeA
       asm volatile("" : "+v"(thr_prod));
       if (gq == 0) s_thr[c16] = round16<F16>(thr_prod);
     }
-    __syncthreads();
+    lds_barrier();
     if (t < E) {
       unsigned bits = 0u;
 #pragma unroll
-      for (int tk = 0; tk < DC_MAX_TOKENS; ++tk) bits |= ((tk < N && dec16<F16>(colv[tk]) >= s_thr[tk]) ? 1u : 0u) << tk;
+      for (int tk = 0; tk < DC_MAX_TOKENS; ++tk) bits |= ((tk < N && dec16<F16>(s_norms[tk][t]) >= s_thr[tk]) ? 1u : 0u) << tk;
       s_bits[t] = (unsigned short)bits;
-      if (cb == 0) {                                      // one workgroup also leaves the routing tensor and the counts
-        for (int tk = 0; tk < N; ++tk) A.routing_out[(int64_t)tk * E + t] = ((bits >> tk) & 1u) ? (bf16_t)(F16 ? 0x3c00 : 0x3f80) : (bf16_t)0;
-        if (A.counts != nullptr) A.counts[t] = __popc(bits);
+      // The layer's other outputs as 2 N + 1 jobs dealt round-robin to the workgroups, so that none is held up: job
+      // j < N is row j of the routing tensor, job N + j row j of the norms, job 2 N the counts.
+      for (int j = (int)blockIdx.x; j <= 2 * N; j += (int)gridDim.x) {
+        if (j < N) A.routing_out[(int64_t)j * E + t] = ((bits >> j) & 1u) ? (bf16_t)(F16 ? 0x3c00 : 0x3f80) : (bf16_t)0;
+        else if (j < 2 * N) A.norms[(int64_t)(j - N) * E + t] = s_norms[j - N][t];
+        else if (A.counts != nullptr) A.counts[t] = __popc(bits);
       }
     }
-    __syncthreads();
+    lds_barrier();
   }
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  // A fragment rows 0..7 only (lanes c16 >= 8 repeat them); result rows 8..15 are dropped
-  const bf16x8* wdf = A.wd + (int64_t)cb * E * KS2 * 32 + gq * 8 + (c16 & 7);
+
+  // ---- 3. hidden fragments of all the wave's experts in one go (an expert out of use: some valid fragment, multiplied by
+  // zero weights or cleared below), then the products in ascending expert order, without a branch
   const bf16x8* hf = A.hfrag + lane;
-  constexpr int KP = (KS2 + 1) / 2;            // weight loads per expert: two K steps each
-  const int khalf = (KS2 > 1) ? (c16 >> 3) : 0;
-  bf16x8 aA[UB][KP], bA[UB][KS2], aB[UB][KP], bB[UB][KS2];
-  int esA[UB], esB[UB];
-  for (int e0 = e_lo; e0 < e_hi; e0 += 64) {   // 64 experts per pass: one flag per lane
-    const bool on = (e0 + lane < e_hi) && (A.fused ? (s_bits[e0 + lane] != 0) : (A.active[e0 + lane] != 0));
-    unsigned long long mask = __ballot(on);
-    int cntA = 0, cntB = 0;
-    // take the next up to UB routed experts off the mask and request their fragments; unused slots repeat the last one
-    auto fill = [&](bf16x8 (&a)[UB][KP], bf16x8 (&b)[UB][KS2], int (&es)[UB], int& cnt) __attribute__((always_inline)) {
-      cnt = 0;
-      int e = e0;
+  bf16x8 hb[ME][KS2];
 #pragma unroll
-      for (int j = 0; j < UB; ++j) {
-        if (mask != 0ull) {
-          e = e0 + (int)__builtin_ctzll(mask);
-          mask &= mask - 1ull;
-          ++cnt;
-        }
+  for (int j = 0; j < ME; ++j) {
+    const int e = (e_lo + j < E) ? (e_lo + j) : (E - 1);
 #pragma unroll
-        for (int k2 = 0; k2 < KS2; ++k2) b[j][k2] = hf[((int64_t)e * KS2 + k2) * 64];
-        es[j] = e;
-      }
-      // Rows 8..15 of the A tile are not needed (the result rows they produce are dropped), so their lanes fetch the
-      // fragment of the NEXT K step instead of repeating rows 0..7: one load brings two K steps, and the second one's
-      // MFMA takes the register rotated by 8 lanes inside every row of 16 (a DPP move).  No load sits under a
-      // lane-dependent branch.  (KS2 == 1: nothing to pair, the upper lanes repeat the lower ones.)
+    for (int k2 = 0; k2 < KS2; ++k2) hb[j][k2] = hf[((int64_t)e * KS2 + k2) * 64];
+  }
+  f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-      for (int j = 0; j < UB; ++j)
+  for (int j = 0; j < ME; ++j) {
+    // the columns of tokens that do not route here are cleared (fused: the hidden fragment holds every token; not fused:
+    // an expert out of use may hold anything)
+    bool keep = ((umask >> j) & 1u) != 0u;
+    if (A.fused) keep = keep && (((s_bits[(e_lo + j < E) ? (e_lo + j) : (E - 1)] >> c16) & 1u) != 0u);
 #pragma unroll
-        for (int kp = 0; kp < KP; ++kp) a[j][kp] = wdf[((int64_t)es[j] * KS2 + 2 * kp + khalf) * 32];
-    };
-    auto multiply = [&](bf16x8 (&a)[UB][KP], bf16x8 (&b)[UB][KS2], int (&es)[UB], int cnt) __attribute__((always_inline)) {
-#pragma unroll
-      for (int j = 0; j < UB; ++j) {
-        if (j < cnt) {
-          // fused: the hidden fragment holds every token; the columns of tokens that do not route here are cleared
-          const bool keep = A.fused ? (((s_bits[es[j]] >> c16) & 1u) != 0u) : true;
-#pragma unroll
-          for (int k2 = 0; k2 < KS2; ++k2) {
-            u32x4 bm = __builtin_bit_cast(u32x4, b[j][k2]);
-            bm.x = keep ? bm.x : 0u; bm.y = keep ? bm.y : 0u; bm.z = keep ? bm.z : 0u; bm.w = keep ? bm.w : 0u;
-            bf16x8 av = a[j][k2 / 2];
-            if (KS2 > 1 && (k2 & 1)) {       // the odd K step sits in the upper 8 lanes of every row: rotate it down
-              u32x4 aw = __builtin_bit_cast(u32x4, av);
-              aw.x = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)aw.x, 0x128, 0xf, 0xf, false);
-              aw.y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)aw.y, 0x128, 0xf, 0xf, false);
-              aw.z = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)aw.z, 0x128, 0xf, 0xf, false);
-              aw.w = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)aw.w, 0x128, 0xf, 0xf, false);
-              av = __builtin_bit_cast(bf16x8, aw);
-            }
-            acc = mfma_16x16x32<F16>(av, __builtin_bit_cast(bf16x8, bm), acc);
-          }
-        }
-      }
-    };
-    if (mask != 0ull) {
-      fill(aA, bA, esA, cntA);
-      while (cntA > 0) {
-        cntB = 0;
-        if (mask != 0ull) fill(aB, bB, esB, cntB);
-        multiply(aA, bA, esA, cntA);
-        cntA = 0;
-        if (mask != 0ull) fill(aA, bA, esA, cntA);
-        multiply(aB, bB, esB, cntB);
-      }
+    for (int k2 = 0; k2 < KS2; ++k2) {
+      u32x4 bm = __builtin_bit_cast(u32x4, hb[j][k2]);
+      bm.x = keep ? bm.x : 0u; bm.y = keep ? bm.y : 0u; bm.z = keep ? bm.z : 0u; bm.w = keep ? bm.w : 0u;
+      const bf16x8 bv = __builtin_bit_cast(bf16x8, bm);
+      acc[0] = mfma_16x16x32<F16>(wa[j][k2][0], bv, acc[0]);
+      acc[1] = mfma_16x16x32<F16>(wa[j][k2][1], bv, acc[1]);
     }
   }
 #pragma unroll
-  for (int r = 0; r < 4; ++r) part[w][r][lane] = acc[r];
-  __syncthreads();
-  if (w == 0 && c16 < N && gq < 2) {
-    // C layout (transposed product): lane holds token c16, rows 4 gq + r = columns cb*8 + 4 gq + r
-    float o[4];
+  for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) part[w][ct][r][lane] = acc[ct][r];
+  lds_barrier();
+
+  // ---- 4. waves in order; thread (ct, lane) of the first 128 ends with token c16 and 4 consecutive columns
+  const int ct = (t >> 6) & 1;
+  float o[4] = {0.f, 0.f, 0.f, 0.f};
+  if (t < 128) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      float sacc = part[0][r][lane];
+      float sacc = part[0][ct][r][lane];
 #pragma unroll
-      for (int ww = 1; ww < DO_WAVES; ++ww) sacc += part[ww][r][lane];
+      for (int ww = 1; ww < DO_WAVES; ++ww) sacc += part[ww][ct][r][lane];
       o[r] = sacc;
     }
-    const int col = cb * 8 + 4 * gq;
+  }
+  if (Q > 1) {
+    // Leave this range's sums and count the arrival; the last range of the column block to arrive adds all of them in range
+    // order.  Sums and counter are written and read with device-scope atomic accesses only: such a store is written
+    // through to the memory side (the ranges ran on other CUs, maybe other XCDs, whose L2 caches do not snoop each other),
+    // such a load is not served from a stale line, and the barrier ahead of the counter update has waited for every
+    // thread's stores to be acknowledged.  No release / acquire fences: a fence in every wave (an L2 write-back and
+    // invalidation each) made this kernel four times slower, and even the one pair hung on the counter update cost 2.8 us
+    // of the kernel's 15.
+    float* mine = A.partial + ((int64_t)cb * Q + q) * (DC_MAX_TOKENS * DO_COLS);
+    if (t < 128) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        __hip_atomic_store(mine + t * 4 + r, o[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (t == 0) {
+      const int arrived = __hip_atomic_fetch_add(A.tickets + cb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (arrived == Q - 1) ? 1 : 0;
+    }
+    __syncthreads();
+    if (s_last == 0) return;
+    if (t < 128) {
+      const float* all = A.partial + (int64_t)cb * Q * (DC_MAX_TOKENS * DO_COLS);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float sacc = 0.f;
+        for (int qq = 0; qq < Q; ++qq) {
+          const float v = __hip_atomic_load(all + (int64_t)qq * (DC_MAX_TOKENS * DO_COLS) + t * 4 + r, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT);
+          sacc = (qq == 0) ? v : sacc + v;
+        }
+        o[r] = sacc;
+      }
+    }
+  }
+  if (t < 128 && c16 < N) {
+    // C layout (transposed product): lane holds token c16, rows 4 gq + r = columns cb*32 + ct*16 + 4 gq + r
+    const int col = cb * DO_COLS + ct * 16 + 4 * gq;
     if (A.last_bias != nullptr) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) o[r] += dec16<F16>(A.last_bias[col + r]);
@@ -466,11 +647,17 @@ template <bool F16>
 static hipError_t launch_hidden_t(const DecodeArgs& A, bool gated, hipStream_t s) {
   return gated ? launch_hidden<true, F16>(A, s) : launch_hidden<false, F16>(A, s);
 }
+template <bool F16, int KQS>
+static void launch_out_q(const DecodeArgs& A, int nt16, unsigned grid, hipStream_t s) {
+  if (nt16 == 2) hipLaunchKernelGGL((decode_out_kernel<1, F16, KQS>), dim3(grid), dim3(DO_WAVES * 64), 0, s, A);
+  else if (nt16 == 4) hipLaunchKernelGGL((decode_out_kernel<2, F16, KQS>), dim3(grid), dim3(DO_WAVES * 64), 0, s, A);
+  else hipLaunchKernelGGL((decode_out_kernel<4, F16, KQS>), dim3(grid), dim3(DO_WAVES * 64), 0, s, A);
+}
 template <bool F16>
 static void launch_out_t(const DecodeArgs& A, int nt16, unsigned grid, hipStream_t s) {
-  if (nt16 == 2) hipLaunchKernelGGL((decode_out_kernel<1, F16>), dim3(grid), dim3(DO_WAVES * 64), 0, s, A);
-  else if (nt16 == 4) hipLaunchKernelGGL((decode_out_kernel<2, F16>), dim3(grid), dim3(DO_WAVES * 64), 0, s, A);
-  else hipLaunchKernelGGL((decode_out_kernel<4, F16>), dim3(grid), dim3(DO_WAVES * 64), 0, s, A);
+  if (A.fused && A.rwidth == 256) launch_out_q<F16, 2>(A, nt16, grid, s);
+  else if (A.fused && A.rwidth == 128) launch_out_q<F16, 1>(A, nt16, grid, s);
+  else launch_out_q<F16, 0>(A, nt16, grid, s);
 }
 
 hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed_section,
@@ -481,7 +668,10 @@ hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void*
   A.x = (const bf16_t*)x; A.routing = (const bf16_t*)routing; A.wgu = (const bf16x8*)(pk + L.gu_off);
   A.wd = (const bf16x8*)(pk + L.d_off); A.bias = (const bf16_t*)(pk + L.b_off);
   A.hfrag = (bf16x8*)workspace;
-  A.active = (int*)((char*)workspace + (size_t)sh.n_experts * L.edp * DC_MAX_TOKENS * 2);
+  const DecodeWorkspace WS = decode_workspace(sh);
+  A.active = (int*)((char*)workspace + WS.active);
+  A.partial = (float*)((char*)workspace + WS.partial); A.tickets = (int*)((char*)workspace + WS.tickets);
+  A.split = decode_split(sh); A.rw2 = nullptr; A.roact = 0;
   A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out;
   A.N = (int)sh.n_tokens; A.D = sh.d_model; A.E = sh.n_experts; A.nt16 = L.nt16; A.act = sh.activation;
   A.add_residual = sh.add_residual;
@@ -490,13 +680,14 @@ hipError_t launch_mfma_decode(const d2dmoe_shape& sh, const void* x, const void*
   const bool f16 = sh.dtype == D2DMOE_F16;
   const hipError_t e = f16 ? launch_hidden_t<true>(A, sh.gated != 0, s) : launch_hidden_t<false>(A, sh.gated != 0, s);
   if (e != hipSuccess) return e;
-  if (f16) launch_out_t<true>(A, L.nt16, (unsigned)(sh.d_model / 8), s);
-  else launch_out_t<false>(A, L.nt16, (unsigned)(sh.d_model / 8), s);
+  if (f16) launch_out_t<true>(A, L.nt16, (unsigned)(sh.d_model / DO_COLS * A.split), s);
+  else launch_out_t<false>(A, L.nt16, (unsigned)(sh.d_model / DO_COLS * A.split), s);
   return hipGetLastError();
 }
 
-// The whole layer for at most 16 tokens in three launches: hidden activations of every expert + first router layer (one
-// launch: neither waits for the other), second router layer (norms), output kernel with the selection inside.
+// The whole layer for at most 16 tokens in two launches: hidden activations of every expert + first router layer (one
+// launch: neither waits for the other), then the output kernel, which requests its weights, works out the second router
+// layer and the selection while they travel, and multiplies.
 bool mfma_decode_layer_supported(const d2dmoe_shape& sh) {
   return mfma_decode_supported(sh) && sh.n_tokens >= 1 && sh.n_tokens <= DC_MAX_TOKENS && sh.n_experts % 32 == 0 &&
          sh.n_experts <= DO_WAVES * 64 && sh.router_width > 0 && linear_skinny_supported(sh.n_tokens, sh.d_model, sh.dtype) &&
@@ -511,21 +702,21 @@ hipError_t launch_mfma_decode_layer(const d2dmoe_shape& sh, const void* x, const
   DecodeArgs A;
   A.x = (const bf16_t*)x; A.routing = nullptr; A.wgu = (const bf16x8*)(pk + L.gu_off);
   A.wd = (const bf16x8*)(pk + L.d_off); A.bias = (const bf16_t*)(pk + L.b_off);
+  const DecodeWorkspace WS = decode_workspace(sh);
   A.hfrag = (bf16x8*)workspace; A.active = nullptr;
+  A.partial = (float*)((char*)workspace + WS.partial); A.tickets = (int*)((char*)workspace + WS.tickets);
+  A.split = decode_split(sh); A.rw2 = (const bf16_t*)router_w2; A.roact = sh.router_output_activation;
   A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out;
   A.N = (int)sh.n_tokens; A.D = sh.d_model; A.E = sh.n_experts; A.nt16 = L.nt16; A.act = sh.activation;
   A.add_residual = sh.add_residual;
   A.fused = 1; A.rw1 = (const bf16_t*)router_w1; A.rhidden = (bf16_t*)router_hidden; A.rwidth = sh.router_width;
-  A.ract = sh.router_activation; A.norms = (const bf16_t*)norms; A.routing_out = (bf16_t*)routing; A.counts = counts;
+  A.ract = sh.router_activation; A.norms = (bf16_t*)norms; A.routing_out = (bf16_t*)routing; A.counts = counts;
   A.thr_scale = thr_scale;
   const bool f16 = sh.dtype == D2DMOE_F16;
   hipError_t e = f16 ? launch_hidden_t<true>(A, sh.gated != 0, s) : launch_hidden_t<false>(A, sh.gated != 0, s);
   if (e != hipSuccess) return e;
-  e = launch_linear_skinny(router_hidden, router_w2, norms, (int)sh.n_tokens, sh.router_width, sh.n_experts,
-                           sh.router_output_activation, s, sh.dtype);
-  if (e != hipSuccess) return e;
-  if (f16) launch_out_t<true>(A, L.nt16, (unsigned)(sh.d_model / 8), s);
-  else launch_out_t<false>(A, L.nt16, (unsigned)(sh.d_model / 8), s);
+  if (f16) launch_out_t<true>(A, L.nt16, (unsigned)(sh.d_model / DO_COLS * A.split), s);
+  else launch_out_t<false>(A, L.nt16, (unsigned)(sh.d_model / DO_COLS * A.split), s);
   return hipGetLastError();
 }
 
