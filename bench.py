@@ -296,7 +296,7 @@ def gated_record(args, ops, dev, workload):
         # buffer and router weights; > 2.4 GB in all, each copy's small-batch section 201 MB), so every call streams its
         # weights from HBM.  Timed over whole rotations: HIP events around eager launches, and replays of one graph that
         # holds one call per copy.
-        sets = [(rw1, rw2, packed)] + [(rw1.clone(), rw2.clone(), packed.clone()) for _ in range(COLD_SETS - 1)]
+        sets = [(rw1, rw2, packed)] + [(rw1.clone(), rw2.clone(), ops.clone_packed(packed)) for _ in range(COLD_SETS - 1)]
 
         def layer_on(k):
             r1, r2, pk = sets[k]

@@ -59,6 +59,43 @@ int check_shape(const d2dmoe_shape* sh) {
   return D2DMOE_OK;
 }
 
+// The descriptor d2dmoe_pack_weights hands out for a buffer packed for sh.
+d2dmoe_packed_desc make_packed_desc(const d2dmoe_shape& sh) {
+  d2dmoe_packed_desc d = {};
+  d.magic = D2DMOE_PACKED_MAGIC;
+  d.layout_version = D2DMOE_PACKED_LAYOUT_VERSION;
+  d.dtype = sh.dtype; d.d_model = sh.d_model; d.n_experts = sh.n_experts; d.expert_dim = sh.expert_dim;
+  d.gated = sh.gated ? 1 : 0;
+  d.router_width = mfma_router_supported(sh) ? sh.router_width : 0;
+  d.sections = mfma_packed_sections(sh);
+  d.bytes = mfma_packed_bytes(sh);
+  return d;
+}
+
+// Host-side check of a packed buffer's descriptor against the shape of the call that is about to use it.  need_router:
+// the call runs the fused router kernel out of the buffer's router section.
+int check_packed(const d2dmoe_shape& sh, const void* packed, const d2dmoe_packed_desc* d, bool need_router) {
+  if (packed == nullptr) return D2DMOE_OK;
+  if (d == nullptr) return D2DMOE_E_PACKED;
+  if (d->magic != D2DMOE_PACKED_MAGIC || d->layout_version != D2DMOE_PACKED_LAYOUT_VERSION) return D2DMOE_E_PACKED;
+  if (d->dtype != sh.dtype || d->d_model != sh.d_model || d->n_experts != sh.n_experts || d->expert_dim != sh.expert_dim ||
+      d->gated != (sh.gated ? 1 : 0))
+    return D2DMOE_E_PACKED;
+  // what a buffer packed for this layer with the router width the descriptor names looks like (the router section is
+  // the last one, so the other sections do not move with it)
+  d2dmoe_shape as_packed = sh;
+  as_packed.router_width = d->router_width;
+  if (d->router_width > 0) {   // packed with a router section: the fused router kernel's own activations
+    as_packed.router_activation = D2DMOE_ACT_RELU;
+    as_packed.router_output_activation = D2DMOE_ACT_ABS;
+  }
+  const d2dmoe_packed_desc want = make_packed_desc(as_packed);
+  if (want.bytes == 0 || d->bytes != want.bytes || d->sections != want.sections || want.router_width != d->router_width)
+    return D2DMOE_E_PACKED;
+  if (need_router && (!(d->sections & D2DMOE_SECTION_ROUTER) || d->router_width != sh.router_width)) return D2DMOE_E_PACKED;
+  return D2DMOE_OK;
+}
+
 struct ForwardWorkspace {
   size_t hidden_off, norms_off, perm_off, total;
 };
@@ -103,6 +140,7 @@ const char* d2dmoe_status_string(int status) {
     case D2DMOE_E_UNSUPPORTED: return "no kernel for this request in this build";
     case D2DMOE_E_ALIGN: return "tensor pointer not aligned to 16 bytes";
     case D2DMOE_E_STATIC_LIMIT: return "shape needs more workspace than the static array of d2dmoe_forward_static holds";
+    case D2DMOE_E_PACKED: return "packed buffer without its descriptor, or packed for another layer or layout version";
     default: break;
   }
   if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -205,28 +243,54 @@ size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape) {
   return mfma_packed_bytes(*shape);
 }
 
+int d2dmoe_packed_describe(const d2dmoe_shape* shape, d2dmoe_packed_desc* desc) {
+  const int st = check_shape(shape);
+  if (st != D2DMOE_OK) return st;
+  if (!desc) return D2DMOE_E_NULL;
+  if (mfma_packed_bytes(*shape) == 0) return D2DMOE_E_UNSUPPORTED;
+  *desc = make_packed_desc(*shape);
+  return D2DMOE_OK;
+}
+
+int d2dmoe_packed_desc_from_header(const void* host_header_64_bytes, d2dmoe_packed_desc* desc) {
+  if (!host_header_64_bytes || !desc) return D2DMOE_E_NULL;
+  d2dmoe_packed_desc d;
+  __builtin_memcpy(&d, host_header_64_bytes, sizeof(d));
+  if (d.magic != D2DMOE_PACKED_MAGIC) return D2DMOE_E_PACKED;
+  *desc = d;
+  return D2DMOE_OK;
+}
+
 int d2dmoe_pack_weights(const d2dmoe_shape* shape, const void* w1, const void* b1, const void* w2, const void* w_up,
-                        const void* router_w1, const void* router_w2, void* packed, size_t packed_bytes, void* stream) {
+                        const void* router_w1, const void* router_w2, void* packed, size_t packed_bytes,
+                        d2dmoe_packed_desc* desc_out, void* stream) {
   int st = check_shape(shape);
   if (st != D2DMOE_OK) return st;
-  if (!w1 || !w2 || !packed) return D2DMOE_E_NULL;
+  if (!w1 || !w2 || !packed || !desc_out) return D2DMOE_E_NULL;
   if (!mfma_dense_supported(*shape) && !mfma_router_supported(*shape) && !mfma_decode_supported(*shape) &&
       !mfma_gemm_supported(*shape))
     return D2DMOE_E_UNSUPPORTED;
   if (shape->gated && !w_up) return D2DMOE_E_NULL;
   if (mfma_router_supported(*shape) && (!router_w1 || !router_w2)) return D2DMOE_E_NULL;
-  if (packed_bytes < mfma_packed_bytes(*shape) || !aligned16(packed)) return D2DMOE_E_WORKSPACE;
-  return (int)launch_mfma_pack(*shape, w1, b1, w2, w_up, router_w1, router_w2, packed, (hipStream_t)stream);
+  if (packed_bytes < mfma_packed_bytes(*shape) || (((uintptr_t)packed) & 255u)) return D2DMOE_E_WORKSPACE;
+  const d2dmoe_packed_desc d = make_packed_desc(*shape);
+  hipError_t e = launch_pack_header(d, packed, (hipStream_t)stream);
+  if (e == hipSuccess) e = launch_mfma_pack(*shape, w1, b1, w2, w_up, router_w1, router_w2, packed, (hipStream_t)stream);
+  if (e == hipSuccess) *desc_out = d;
+  return (int)e;
 }
 
 // plan_counts_ready: the router kernel of this call has already left the expert-major plan's per-segment counts in
 // the workspace (d2dmoe_forward only)
 static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* routing, const void* w1, const void* b1,
-                        const void* w2, const void* w_up, const void* last_bias, const void* packed, void* out,
-                        int32_t path, void* workspace, size_t workspace_bytes, void* stream, bool plan_counts_ready) {
+                        const void* w2, const void* w_up, const void* last_bias, const void* packed,
+                        const d2dmoe_packed_desc* packed_desc, void* out, int32_t path, void* workspace,
+                        size_t workspace_bytes, void* stream, bool plan_counts_ready) {
   int st = check_shape(shape);
   if (st != D2DMOE_OK) return st;
   const d2dmoe_shape& sh = *shape;
+  st = check_packed(sh, packed, packed_desc, false);
+  if (st != D2DMOE_OK) return st;
   if (sh.n_tokens == 0) return D2DMOE_OK;
   if (!x || !routing || !w1 || !w2 || !out) return D2DMOE_E_NULL;
   if (sh.gated && !w_up) return D2DMOE_E_NULL;
@@ -334,22 +398,28 @@ static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* ro
 }
 
 int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing, const void* w1, const void* b1,
-                   const void* w2, const void* w_up, const void* last_bias, const void* packed, void* out,
-                   int32_t path, void* workspace, size_t workspace_bytes, void* stream) {
-  return experts_impl(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, workspace, workspace_bytes, stream,
-                      false);
+                   const void* w2, const void* w_up, const void* last_bias, const void* packed,
+                   const d2dmoe_packed_desc* packed_desc, void* out, int32_t path, void* workspace, size_t workspace_bytes,
+                   void* stream) {
+  return experts_impl(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, packed_desc, out, path, workspace,
+                      workspace_bytes, stream, false);
 }
 
 // seg_counts / seg_pairs: see launch_mfma_router_select
 static int router_select_impl(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
-                              const void* packed, float thr_scale, void* norms_out, void* routing, int32_t* counts,
-                              void* workspace, size_t workspace_bytes, void* stream, int32_t* seg_counts,
-                              int32_t* seg_pairs) {
+                              const void* packed, const d2dmoe_packed_desc* packed_desc, float thr_scale, void* norms_out,
+                              void* routing, int32_t* counts, void* workspace, size_t workspace_bytes, void* stream,
+                              int32_t* seg_counts, int32_t* seg_pairs) {
   int st = check_shape(shape);
   if (st != D2DMOE_OK) return st;
   const d2dmoe_shape& sh = *shape;
   if (!routing) return D2DMOE_E_NULL;
   if (sh.router_width <= 0) return D2DMOE_E_SHAPE;
+  // (a buffer packed without the router section is no error here: the call then runs the unfused router kernels)
+  st = check_packed(sh, packed, packed_desc, false);
+  if (st != D2DMOE_OK) return st;
+  if (packed != nullptr && !((packed_desc->sections & D2DMOE_SECTION_ROUTER) && packed_desc->router_width == sh.router_width))
+    packed = nullptr;
   if (sh.n_tokens == 0) return counts ? (int)launch_fill_i32(counts, sh.n_experts, 0, (hipStream_t)stream) : D2DMOE_OK;
   if (!x) return D2DMOE_E_NULL;
   if (packed != nullptr && mfma_router_supported(sh) && sh.n_tokens > 16) {
@@ -370,20 +440,23 @@ static int router_select_impl(const d2dmoe_shape* shape, const void* x, const vo
 }
 
 int d2dmoe_router_select(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
-                         const void* packed, float thr_scale, void* norms_out, void* routing, int32_t* counts,
-                         void* workspace, size_t workspace_bytes, void* stream) {
-  return router_select_impl(shape, x, router_w1, router_w2, packed, thr_scale, norms_out, routing, counts, workspace,
-                            workspace_bytes, stream, nullptr, nullptr);
+                         const void* packed, const d2dmoe_packed_desc* packed_desc, float thr_scale, void* norms_out,
+                         void* routing, int32_t* counts, void* workspace, size_t workspace_bytes, void* stream) {
+  return router_select_impl(shape, x, router_w1, router_w2, packed, packed_desc, thr_scale, norms_out, routing, counts,
+                            workspace, workspace_bytes, stream, nullptr, nullptr);
 }
 
 int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
                    float thr_scale, const void* w1, const void* b1, const void* w2, const void* w_up,
-                   const void* last_bias, const void* packed, const void* norms_in, void* norms_out, void* routing,
-                   int32_t* counts, void* out, int32_t path, void* workspace, size_t workspace_bytes, void* stream) {
+                   const void* last_bias, const void* packed, const d2dmoe_packed_desc* packed_desc, const void* norms_in,
+                   void* norms_out, void* routing, int32_t* counts, void* out, int32_t path, void* workspace,
+                   size_t workspace_bytes, void* stream) {
   int st = check_shape(shape);
   if (st != D2DMOE_OK) return st;
   const d2dmoe_shape& sh = *shape;
   if (!routing || !out) return D2DMOE_E_NULL;
+  st = check_packed(sh, packed, packed_desc, false);
+  if (st != D2DMOE_OK) return st;
   if (sh.n_tokens == 0) return counts ? (int)launch_fill_i32(counts, sh.n_experts, 0, (hipStream_t)stream) : D2DMOE_OK;
   if (!x) return D2DMOE_E_NULL;
   const ForwardWorkspace plan = plan_workspace(sh);
@@ -423,35 +496,41 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   bool plan_counts_ready = false;
   if (norms_in == nullptr) {
     int32_t *seg_counts = nullptr, *seg_pairs = nullptr;
-    if (path == D2DMOE_PATH_MFMA_SPARSE && packed != nullptr && mfma_sparse_supported(sh) && mfma_router_writes_plan_counts(sh) &&
+    // (only the fused router kernel does that: the buffer must hold this layer's router section)
+    const bool router_in_packed = packed != nullptr && (packed_desc->sections & D2DMOE_SECTION_ROUTER) != 0 &&
+                                  packed_desc->router_width == sh.router_width && sh.n_tokens > 16;
+    if (path == D2DMOE_PATH_MFMA_SPARSE && router_in_packed && mfma_sparse_supported(sh) && mfma_router_writes_plan_counts(sh) &&
         plan.total - plan.perm_off >= mfma_sparse_workspace_bytes(sh)) {
       mfma_sparse_plan_counts(sh, ws + plan.perm_off, &seg_counts, &seg_pairs);
       plan_counts_ready = true;
     }
-    st = router_select_impl(shape, x, router_w1, router_w2, packed, thr_scale, norms_out, routing, counts, workspace,
-                            workspace_bytes, stream, seg_counts, seg_pairs);
+    st = router_select_impl(shape, x, router_w1, router_w2, packed, packed_desc, thr_scale, norms_out, routing, counts,
+                            workspace, workspace_bytes, stream, seg_counts, seg_pairs);
   } else {
     st = d2dmoe_select(norms_in, routing, counts, sh.n_tokens, sh.n_experts, sh.dtype, thr_scale, stream);
   }
   if (st != D2DMOE_OK) return st;
-  return experts_impl(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, out, path, ws + plan.perm_off,
+  return experts_impl(shape, x, routing, w1, b1, w2, w_up, last_bias, packed, packed_desc, out, path, ws + plan.perm_off,
                       plan.total - plan.perm_off, stream, plan_counts_ready);
 }
 
 int d2dmoe_forward_static(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
                           float thr_scale, const void* w1, const void* b1, const void* w2, const void* w_up,
-                          const void* last_bias, const void* packed, const void* norms_in, void* norms_out, void* routing,
-                          int32_t* counts, void* out, int32_t path, void* stream) {
+                          const void* last_bias, const void* packed, const d2dmoe_packed_desc* packed_desc,
+                          const void* norms_in, void* norms_out, void* routing, int32_t* counts, void* out, int32_t path,
+                          void* stream) {
   int st = check_shape(shape);
   if (st != D2DMOE_OK) return st;
   if (plan_workspace(*shape).total > (size_t)D2DMOE_STATIC_WORKSPACE_BYTES) return D2DMOE_E_STATIC_LIMIT;
+  st = check_packed(*shape, packed, packed_desc, false);   // host-only checks first: nothing below touches a device before them
+  if (st != D2DMOE_OK) return st;
   void* ws = nullptr;
   st = static_scratch(&ws);
   if (st != D2DMOE_OK) return st;
   // Every kernel behind d2dmoe_forward initialises what it reads of its workspace (counters, flags, partial sums) on the
   // stream before use, so the contents the previous call left in the array are never seen.
-  return d2dmoe_forward(shape, x, router_w1, router_w2, thr_scale, w1, b1, w2, w_up, last_bias, packed, norms_in, norms_out,
-                        routing, counts, out, path, ws, (size_t)D2DMOE_STATIC_WORKSPACE_BYTES, stream);
+  return d2dmoe_forward(shape, x, router_w1, router_w2, thr_scale, w1, b1, w2, w_up, last_bias, packed, packed_desc, norms_in,
+                        norms_out, routing, counts, out, path, ws, (size_t)D2DMOE_STATIC_WORKSPACE_BYTES, stream);
 }
 
 size_t d2dmoe_norms_packed_bytes(const d2dmoe_shape* shape) {

@@ -77,7 +77,7 @@ PackedLayout packed_layout(const d2dmoe_shape& sh) {
   L.n_chunks = (L.hidden + MD_HC - 1) / MD_HC;
   L.hidden_pad = L.n_chunks * MD_HC;
   L.pieces = sh.d_model / 16 * 2 + MD_KS2 * (sh.d_model / 128);
-  size_t off = 0;
+  size_t off = PACKED_HEADER_BYTES;   // the buffer starts with its descriptor
   L.has_dense = mfma_dense_supported(sh);
   L.w_off = off;    if (L.has_dense) off += (size_t)MD_WAVES * L.n_chunks * L.pieces * 64 * 16;
   L.b1_off = off;   if (L.has_dense) off += (size_t)L.hidden_pad * 2;   // bf16
@@ -107,10 +107,28 @@ PackedLayout packed_layout(const d2dmoe_shape& sh) {
   L.r1_off = off;   if (L.has_router) off += (size_t)sh.router_width * sh.d_model * 2;
   L.r2_off = off;   if (L.has_router) off += (size_t)mfma_router_padded_experts(sh) * sh.router_width * 2;
   L.total = (off + 255) / 256 * 256;
+  if (!(L.has_dense || L.has_sparse || L.has_decode || L.has_gemm || L.has_mid || L.has_router)) L.total = 0;
   return L;
 }
 
 size_t mfma_packed_bytes(const d2dmoe_shape& sh) { return packed_layout(sh).total; }
+
+unsigned mfma_packed_sections(const d2dmoe_shape& sh) {
+  const PackedLayout L = packed_layout(sh);
+  return (L.has_dense ? D2DMOE_SECTION_DENSE : 0u) | (L.has_sparse ? D2DMOE_SECTION_EXPERT_MAJOR : 0u) |
+         (L.has_decode ? D2DMOE_SECTION_SMALL_BATCH : 0u) | (L.has_gemm ? D2DMOE_SECTION_TILED : 0u) |
+         (L.has_mid ? D2DMOE_SECTION_COMPACTED : 0u) | (L.has_router ? D2DMOE_SECTION_ROUTER : 0u);
+}
+
+// The descriptor's 64 bytes at the start of the buffer (for a caller that wants to recover it from the buffer).
+__global__ void pack_header_kernel(const d2dmoe_packed_desc d, d2dmoe_packed_desc* dst) {
+  if (blockIdx.x == 0 && threadIdx.x == 0) *dst = d;
+}
+
+hipError_t launch_pack_header(const d2dmoe_packed_desc& d, void* packed, hipStream_t s) {
+  hipLaunchKernelGGL(pack_header_kernel, dim3(1), dim3(64), 0, s, d, (d2dmoe_packed_desc*)packed);
+  return hipGetLastError();
+}
 size_t mfma_decode_section_offset(const d2dmoe_shape& sh) { return packed_layout(sh).dc_off; }
 size_t mfma_gemm_section_offset(const d2dmoe_shape& sh) { return packed_layout(sh).gm_off; }
 

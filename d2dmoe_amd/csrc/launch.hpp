@@ -42,6 +42,8 @@ hipError_t launch_experts_generic(const d2dmoe_shape& sh, const void* x, const v
 bool mfma_dense_supported(const d2dmoe_shape& sh);
 bool mfma_router_supported(const d2dmoe_shape& sh);
 size_t mfma_packed_bytes(const d2dmoe_shape& sh);
+unsigned mfma_packed_sections(const d2dmoe_shape& sh);   // D2DMOE_SECTION_* bits of the buffer packed for sh
+hipError_t launch_pack_header(const d2dmoe_packed_desc& d, void* packed, hipStream_t s);
 hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* b1, const void* w2, const void* w_up,
                             const void* router_w1, const void* router_w2, void* packed, hipStream_t s);
 // seg_counts / seg_pairs (optional): where the expert-major plan keeps its per-segment counts; written by the router

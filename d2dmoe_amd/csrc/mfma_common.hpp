@@ -16,6 +16,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // 16 raw bytes that stay in registers
 
+constexpr size_t PACKED_HEADER_BYTES = 256;   // a packed buffer starts with its d2dmoe_packed_desc (64 bytes, padded)
 constexpr int MD_BM = 64;       // tokens per workgroup of the dense sweep
 constexpr int MD_HC = 256;      // hidden neurons per chunk (4 waves x 64)
 constexpr int MD_WAVES = 4;

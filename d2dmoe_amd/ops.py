@@ -32,16 +32,51 @@ def _require_same_dtype(what: str, ref: torch.Tensor, **tensors: Optional[torch.
                                   'element type for activations, routing and weights')
 
 
-def _check_packed(lib, shape: 'abi.Shape', packed: Optional[torch.Tensor]) -> None:
-    """A packed buffer carries no header: its size is the one thing that can be checked, and a buffer packed for another
-    shape, dtype or without the router section has another size."""
+class PackedWeights(torch.Tensor):
+    """The buffer d2dmoe_pack_weights wrote (a uint8 tensor) together with its descriptor, `desc` (abi.PackedDesc): what it
+    was packed for.  Every call that takes the buffer hands the descriptor to the library, which refuses a buffer packed
+    for another layer.  Tensor operations return plain tensors; use clone_packed() for a copy that keeps the descriptor."""
+
+    @staticmethod
+    def wrap(buf: torch.Tensor, desc: 'abi.PackedDesc') -> 'PackedWeights':
+        out = buf.as_subclass(PackedWeights)
+        out.desc = desc
+        return out
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        with torch._C.DisableTorchFunctionSubclass():
+            return func(*args, **(kwargs or {}))
+
+
+def clone_packed(packed: 'PackedWeights') -> 'PackedWeights':
+    """A copy of a packed buffer (other memory, same contents) with the same descriptor."""
+    return PackedWeights.wrap(torch.Tensor.clone(packed), _desc_of(packed))
+
+
+def packed_from_header(buf: torch.Tensor) -> 'PackedWeights':
+    """Re-attaches the descriptor to a packed buffer that lost it (saved and loaded, copied): the buffer's first 64 bytes
+    hold it.  Copies those bytes to the host (a synchronising copy)."""
+    head = bytes(buf.view(torch.uint8)[:64].cpu().numpy())
+    desc = abi.PackedDesc()
+    abi.check(abi.load().d2dmoe_packed_desc_from_header(head, ctypes.byref(desc)), 'd2dmoe_packed_desc_from_header')
+    return PackedWeights.wrap(buf, desc)
+
+
+def _desc_of(packed: Optional[torch.Tensor]):
     if packed is None:
-        return
-    need = lib.d2dmoe_packed_bytes(ctypes.byref(shape))
-    have = packed.numel() * packed.element_size()
-    if need == 0 or have < need:
-        raise abi.D2DMoEError(f'packed buffer holds {have} bytes but this shape/dtype needs {need}: it was packed for other '
-                              'weights (pack again with the shape of this call)')
+        return None
+    desc = getattr(packed, 'desc', None)
+    if desc is None:
+        raise abi.D2DMoEError('packed buffer without its descriptor: pass what pack_weights returned (clone_packed() copies '
+                              'it, packed_from_header() recovers the descriptor from a raw buffer)')
+    return desc
+
+
+def _pd(packed: Optional[torch.Tensor]):
+    """The descriptor argument of a C call: a pointer to the buffer's descriptor, or NULL without a buffer."""
+    desc = _desc_of(packed)
+    return None if desc is None else ctypes.byref(desc)
 
 
 def _require_gpu(*tensors: Optional[torch.Tensor]) -> torch.device:
@@ -136,7 +171,7 @@ def router_select(x: torch.Tensor, router_w1: torch.Tensor, router_w2: torch.Ten
     norms = torch.empty(n, e, dtype=x.dtype, device=dev) if want_norms else None
     counts = torch.empty(e, dtype=torch.int32, device=dev) if want_counts else None
     ws = _workspace(dev, max(lib.d2dmoe_workspace_bytes(ctypes.byref(sh)), 256))
-    abi.check(lib.d2dmoe_router_select(ctypes.byref(sh), _ptr(x), _ptr(router_w1), _ptr(router_w2), _ptr(packed),
+    abi.check(lib.d2dmoe_router_select(ctypes.byref(sh), _ptr(x), _ptr(router_w1), _ptr(router_w2), _ptr(packed), _pd(packed),
                                        ctypes.c_float(thr_scale), _ptr(norms), _ptr(routing), _ptr(counts), _ptr(ws),
                                        ws.numel(), _stream()), 'd2dmoe_router_select')
     return routing, norms, counts
@@ -181,9 +216,11 @@ def pack_weights(shape: abi.Shape, w1, b1, w2, w_up=None, router_w1=None, router
     if nbytes == 0:
         return None
     packed = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    desc = abi.PackedDesc()
     abi.check(lib.d2dmoe_pack_weights(ctypes.byref(shape), _ptr(w1), _ptr(b1), _ptr(w2), _ptr(w_up), _ptr(router_w1),
-                                      _ptr(router_w2), _ptr(packed), nbytes, _stream()), 'd2dmoe_pack_weights')
-    return packed
+                                      _ptr(router_w2), _ptr(packed), nbytes, ctypes.byref(desc), _stream()),
+              'd2dmoe_pack_weights')
+    return PackedWeights.wrap(packed, desc)
 
 
 def pack_norms(shape: abi.Shape, w1, b1, w2) -> Optional[torch.Tensor]:
@@ -231,12 +268,11 @@ def experts(x: torch.Tensor, routing: torch.Tensor, w1: torch.Tensor, b1: Option
     e, _, ed = w1.shape
     assert routing.shape == (n, e) and w2.shape == (e, ed, d)
     sh = make_shape(n, d, e, ed, 0, _dtype_code(x), activation, gated=w_up is not None, add_residual=add_residual)
-    _check_packed(lib, sh, packed)
     out = torch.empty_like(x)
     need = max(lib.d2dmoe_workspace_bytes(ctypes.byref(sh)), 16)
     ws = _workspace(dev, need)
     abi.check(lib.d2dmoe_experts(ctypes.byref(sh), _ptr(x), _ptr(routing), _ptr(w1), _ptr(b1), _ptr(w2), _ptr(w_up),
-                                 _ptr(last_bias), _ptr(packed), _ptr(out), abi.PATH[path], _ptr(ws), ws.numel(),
+                                 _ptr(last_bias), _ptr(packed), _pd(packed), _ptr(out), abi.PATH[path], _ptr(ws), ws.numel(),
                                  _stream()), 'd2dmoe_experts')
     return out
 
@@ -272,17 +308,11 @@ class PreparedForward:
         self.shapes = {}
         # the router section is the last one of a packed buffer: a buffer packed without it serves calls that bring their
         # own predicted norms (norms_in), and only those
-        # (a layer whose experts have no MFMA kernel can still carry a router section only: then the router-less size is 0
-        # and the buffer is held to the size with the router)
-        self.router_packed_ok = True
-        if packed is not None:
-            have = packed.numel() * packed.element_size()
-            bare = self.lib.d2dmoe_packed_bytes(ctypes.byref(make_shape(0, self.d, self.e, self.ed, 0, self.code, **self.kw)))
-            full = self.lib.d2dmoe_packed_bytes(self.shape_for(0)[1]) if self.w > 0 else bare
-            if (bare == 0 and full == 0) or have < bare or (bare == 0 and have < full):
-                raise abi.D2DMoEError(f'packed buffer holds {have} bytes but this shape/dtype needs {bare if bare else full}: '
-                                      'it was packed for other weights (pack again with the shape of this call)')
-            self.router_packed_ok = have >= full
+        # the buffer's descriptor says what it was packed for; the library checks it against the shape of every call.  A
+        # buffer packed without the router section serves calls that bring their own predicted norms (norms_in) -- and
+        # calls that run the router on the unfused kernels.
+        self.packed_desc = _desc_of(packed)
+        self.pd = None if self.packed_desc is None else ctypes.byref(self.packed_desc)
 
     def shape_for(self, n: int):
         got = self.shapes.get(n)
@@ -300,9 +330,6 @@ class PreparedForward:
             raise abi.D2DMoEError(f'forward: the activations are {x.dtype} but the layer was prepared for {self.dtype}')
         if _require_gpu(x, norms_in, out, routing, norms, counts) != self.dev:
             raise abi.D2DMoEError('all tensors must live on the same device')
-        if norms_in is None and not self.router_packed_ok:
-            raise abi.D2DMoEError('packed buffer has no router section for this layer, but the call runs the router: it was '
-                                  'packed for other weights (pack again with the router weights)')
         n, d = x.shape
         assert d == self.d
         e = self.e
@@ -319,13 +346,13 @@ class PreparedForward:
         stream = _stream()
         if static_workspace:
             abi.check(self.lib.d2dmoe_forward_static(shref, x.data_ptr(), rw1, rw2, ctypes.c_float(thr_scale), w1, b1, w2,
-                                                     w_up, lb, pk, _ptr(norms_in), _ptr(norms), routing.data_ptr(),
+                                                     w_up, lb, pk, self.pd, _ptr(norms_in), _ptr(norms), routing.data_ptr(),
                                                      _ptr(counts), out.data_ptr(), abi.PATH[path], stream),
                       'd2dmoe_forward_static')
         else:
             ws = _workspace(dev, need, stream)
             abi.check(self.lib.d2dmoe_forward(shref, x.data_ptr(), rw1, rw2, ctypes.c_float(thr_scale), w1, b1, w2, w_up, lb,
-                                              pk, _ptr(norms_in), _ptr(norms), routing.data_ptr(), _ptr(counts),
+                                              pk, self.pd, _ptr(norms_in), _ptr(norms), routing.data_ptr(), _ptr(counts),
                                               out.data_ptr(), abi.PATH[path], ws.data_ptr(), ws.numel(), stream),
                       'd2dmoe_forward')
         return out, routing, (norms_in if norms_in is not None else norms), counts

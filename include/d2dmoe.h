@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define D2DMOE_VERSION 100 /* major*10000 + minor*100 + patch */
+#define D2DMOE_VERSION 200 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 enum {
@@ -46,7 +46,9 @@ enum {
   D2DMOE_E_WORKSPACE = -5,   /* workspace missing, misaligned or smaller than d2dmoe_workspace_bytes() */
   D2DMOE_E_UNSUPPORTED = -6, /* valid request that this build has no kernel for */
   D2DMOE_E_ALIGN = -7,       /* a tensor pointer is not aligned to 16 bytes */
-  D2DMOE_E_STATIC_LIMIT = -8 /* d2dmoe_forward_static: the shape needs more than D2DMOE_STATIC_WORKSPACE_BYTES of workspace */
+  D2DMOE_E_STATIC_LIMIT = -8, /* d2dmoe_forward_static: the shape needs more than D2DMOE_STATIC_WORKSPACE_BYTES of workspace */
+  D2DMOE_E_PACKED = -9       /* a packed buffer came without its descriptor, or the descriptor says it was packed for another
+                                layer (shape, element type, sections) or by another layout version */
 };
 
 /* element types */
@@ -108,6 +110,35 @@ typedef struct d2dmoe_shape {
   int32_t router_output_activation; /* output activation of the router MLP (D2DMoE: D2DMOE_ACT_ABS) */
 } d2dmoe_shape;
 
+/* What a buffer written by d2dmoe_pack_weights was packed for.  The pack call fills one (and writes the same 64 bytes at the
+ * start of the buffer); every call that takes `packed` takes the descriptor next to it and checks it on the host against
+ * its own `shape` before anything is launched -- device memory is never read for this.  A caller that keeps packed
+ * buffers keeps their descriptors with them (or copies the buffer's first 64 bytes back and hands them to
+ * d2dmoe_packed_desc_from_header).  No counterpart in the reference, which has no derived buffers. */
+#define D2DMOE_PACKED_MAGIC 0x4b50324du   /* "M2PK" */
+#define D2DMOE_PACKED_LAYOUT_VERSION 3u
+enum {                       /* bits of d2dmoe_packed_desc.sections */
+  D2DMOE_SECTION_DENSE = 1, D2DMOE_SECTION_EXPERT_MAJOR = 2, D2DMOE_SECTION_SMALL_BATCH = 4,
+  D2DMOE_SECTION_TILED = 8, D2DMOE_SECTION_COMPACTED = 16, D2DMOE_SECTION_ROUTER = 32
+};
+typedef struct d2dmoe_packed_desc {
+  uint32_t magic;           /* D2DMOE_PACKED_MAGIC */
+  uint32_t layout_version;  /* D2DMOE_PACKED_LAYOUT_VERSION of the library that packed it */
+  int32_t dtype, d_model, n_experts, expert_dim, gated;
+  int32_t router_width;     /* router width the buffer was packed with (0: no router section) */
+  uint32_t sections;        /* D2DMOE_SECTION_* present */
+  uint32_t reserved0;
+  uint64_t bytes;           /* size of the whole buffer, header included */
+  uint64_t reserved1[2];
+} d2dmoe_packed_desc;       /* 64 bytes */
+
+/* The descriptor d2dmoe_pack_weights writes for `shape` (host only, nothing is launched): lets a caller see sections and
+ * size ahead of packing.  D2DMOE_E_UNSUPPORTED when the shape has no packed buffer. */
+int d2dmoe_packed_describe(const d2dmoe_shape* shape, d2dmoe_packed_desc* desc);
+
+/* The descriptor found in a host copy of a packed buffer's first 64 bytes; D2DMOE_E_PACKED when they do not hold one. */
+int d2dmoe_packed_desc_from_header(const void* host_header_64_bytes, d2dmoe_packed_desc* desc);
+
 /* Library version (D2DMOE_VERSION of the build). */
 int d2dmoe_version(void);
 
@@ -145,8 +176,8 @@ int d2dmoe_select(const void* norms, void* routing, int32_t* counts, int64_t n_t
  *   norms_out optional [N,E]; routing required [N,E]; counts optional int32 [E]
  * workspace: d2dmoe_workspace_bytes(shape) (only read when the fused kernel does not apply). */
 int d2dmoe_router_select(const d2dmoe_shape* shape, const void* x, const void* router_w1, const void* router_w2,
-                         const void* packed, float thr_scale, void* norms_out, void* routing, int32_t* counts,
-                         void* workspace, size_t workspace_bytes, void* stream);
+                         const void* packed, const d2dmoe_packed_desc* packed_desc, float thr_scale, void* norms_out,
+                         void* routing, int32_t* counts, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Token -> expert permutation from a routing tensor (entry > 0 means routed).
  * Replaces CustomKernelExperts.extract_indices / extract_indices_atomic
@@ -174,14 +205,16 @@ int d2dmoe_build_permutation(const void* routing, int64_t n_tokens, int32_t n_ex
  * For 0/1 routing this equals the reference's naive and Triton modes; for weighted routing it equals its
  * 'masked' mode (forward_all, moe_layers.py:193-198).
  * packed: optional buffer written by d2dmoe_pack_weights for the same weights (required by the MFMA paths;
- * D2DMOE_PATH_AUTO without it uses the generic kernel).
+ * D2DMOE_PATH_AUTO without it uses the generic kernel), with its descriptor: a buffer packed for another shape, element
+ * type or layout version is refused with D2DMOE_E_PACKED (a buffer packed WITH a router section serves calls whose shape
+ * names no router: the router section is the last one).
  * workspace: d2dmoe_workspace_bytes() of the same shape, 256-byte aligned.  Required by the expert-major, small-batch
  * and tiled-products paths; the dense sweep uses it when given (with few tokens it deals every tile's work to several
  * workgroups through it) and runs without it otherwise. */
 int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing,
                    const void* w1, const void* b1, const void* w2, const void* w_up,
-                   const void* last_bias, const void* packed, void* out, int32_t path,
-                   void* workspace, size_t workspace_bytes, void* stream);
+                   const void* last_bias, const void* packed, const d2dmoe_packed_desc* packed_desc, void* out,
+                   int32_t path, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Bytes of the derived weight buffer for the MFMA kernels (0 when `shape` has no MFMA kernel).  The buffer has one
  * section per kernel family that covers the shape (16-bit storage, i.e. bf16 or f16 -- dense sweep: D = 768, ungated;
@@ -193,11 +226,11 @@ size_t d2dmoe_packed_bytes(const d2dmoe_shape* shape);
 
 /* Re-tiles expert and router weights into MFMA fragment order.  A derived, cacheable buffer: call once per
  * weight update, with the same `shape` fields (other than n_tokens) that later calls will carry.  router_w1 and
- * router_w2 are required when the shape has a router section.  No counterpart in the reference (its Triton
- * kernels re-read the nn.Parameter layout on every call). */
+ * router_w2 are required when the shape has a router section.  desc_out (required) receives the buffer's descriptor.
+ * No counterpart in the reference (its Triton kernels re-read the nn.Parameter layout on every call). */
 int d2dmoe_pack_weights(const d2dmoe_shape* shape, const void* w1, const void* b1, const void* w2,
                         const void* w_up, const void* router_w1, const void* router_w2,
-                        void* packed, size_t packed_bytes, void* stream);
+                        void* packed, size_t packed_bytes, d2dmoe_packed_desc* desc_out, void* stream);
 
 /* Whole layer: router -> dynamic-k select -> experts -> epilogue.
  * Replaces MoeficationMoE.forward with forward_mode == 'dynk_max'
@@ -210,7 +243,7 @@ int d2dmoe_pack_weights(const d2dmoe_shape* shape, const void* w1, const void* b
 int d2dmoe_forward(const d2dmoe_shape* shape, const void* x,
                    const void* router_w1, const void* router_w2, float thr_scale,
                    const void* w1, const void* b1, const void* w2, const void* w_up, const void* last_bias,
-                   const void* packed, const void* norms_in,
+                   const void* packed, const d2dmoe_packed_desc* packed_desc, const void* norms_in,
                    void* norms_out, void* routing, int32_t* counts, void* out, int32_t path,
                    void* workspace, size_t workspace_bytes, void* stream);
 
@@ -231,7 +264,7 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x,
 int d2dmoe_forward_static(const d2dmoe_shape* shape, const void* x,
                           const void* router_w1, const void* router_w2, float thr_scale,
                           const void* w1, const void* b1, const void* w2, const void* w_up, const void* last_bias,
-                          const void* packed, const void* norms_in,
+                          const void* packed, const d2dmoe_packed_desc* packed_desc, const void* norms_in,
                           void* norms_out, void* routing, int32_t* counts, void* out, int32_t path, void* stream);
 
 /* L2 norm of every expert's output for every token, norms[e,n] = | act(x[n,:] . w1[e] + b1[e]) . w2[e] |_2 (bf16 [E,N]):

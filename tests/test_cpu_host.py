@@ -73,10 +73,10 @@ def test_shape_struct_matches_header_and_argument_checks():
     bad = ops.make_shape(10, 768, 128, 24, 128, abi.BF16)
     bad.dtype = 9
     assert lib.d2dmoe_workspace_bytes(ctypes.byref(bad)) == 0
-    assert lib.d2dmoe_experts(ctypes.byref(bad), None, None, None, None, None, None, None, None, None, 0, None, 0,
+    assert lib.d2dmoe_experts(ctypes.byref(bad), None, None, None, None, None, None, None, None, None, None, 0, None, 0,
                               None) == -3
     ok = ops.make_shape(10, 768, 128, 24, 128, abi.BF16)
-    assert lib.d2dmoe_experts(ctypes.byref(ok), None, None, None, None, None, None, None, None, None, 0, None, 0,
+    assert lib.d2dmoe_experts(ctypes.byref(ok), None, None, None, None, None, None, None, None, None, None, 0, None, 0,
                               None) == -1
     assert lib.d2dmoe_select(None, None, None, 4, 8, 0, ctypes.c_float(0.5), None) == -1
     assert lib.d2dmoe_select(1, 1, None, 4, 5000, 0, ctypes.c_float(0.5), None) == -2
@@ -156,6 +156,74 @@ def test_expert_major_workspace_covers_its_tiled_products_fallback():
             plan_lists = 2 * 8 * N * 4 + (N + 1) * 4
             router = N * (128 + E) * 2
             assert ws >= router + plan_lists + gemm, (N, E, Ed, dt, ws, router + plan_lists + gemm)
+
+
+def test_packed_descriptor_is_checked_on_the_host_before_anything_is_launched():
+    """Every entry point that takes `packed` takes its descriptor and refuses, with D2DMOE_E_PACKED and before any other
+    argument is looked at, a buffer that comes without one or was packed for another layer, element type, router or
+    layout version.  No device is touched: the packed pointer is a dummy, and a descriptor that passes is followed by the
+    NULL-pointer error for x."""
+    from d2dmoe_amd import hip_abi as abi, ops
+    lib = abi.load()
+    dummy = 256                                    # a non-NULL "device pointer" that is never dereferenced
+    sh = ops.make_shape(100, 768, 128, 24, 128, abi.BF16)
+    good = abi.PackedDesc()
+    assert lib.d2dmoe_packed_describe(ctypes.byref(sh), ctypes.byref(good)) == 0
+    assert ctypes.sizeof(good) == 64 and good.magic == abi.PACKED_MAGIC
+    assert good.bytes == lib.d2dmoe_packed_bytes(ctypes.byref(sh)) and good.router_width == 128
+    assert good.sections & 32 and good.sections & 1        # router and dense-sweep sections
+    assert lib.d2dmoe_packed_describe(ctypes.byref(ops.make_shape(10, 700, 128, 24, 128, abi.F32)), ctypes.byref(good)) == -6
+    assert lib.d2dmoe_packed_describe(ctypes.byref(sh), ctypes.byref(good)) == 0
+
+    def experts(desc, shape=sh):
+        return lib.d2dmoe_experts(ctypes.byref(shape), None, None, None, None, None, None, None, dummy,
+                                  None if desc is None else ctypes.byref(desc), None, 0, None, 0, None)
+
+    def forward(desc, shape=sh):
+        return lib.d2dmoe_forward(ctypes.byref(shape), None, None, None, ctypes.c_float(0.1), None, None, None, None, None,
+                                  dummy, None if desc is None else ctypes.byref(desc), None, None, dummy, None, dummy, 0,
+                                  None, 0, None)
+
+    def forward_static(desc, shape=sh):
+        return lib.d2dmoe_forward_static(ctypes.byref(shape), None, None, None, ctypes.c_float(0.1), None, None, None, None,
+                                         None, dummy, None if desc is None else ctypes.byref(desc), None, None, dummy, None,
+                                         dummy, 0, None)
+
+    def router_select(desc, shape=sh):
+        return lib.d2dmoe_router_select(ctypes.byref(shape), None, None, None, dummy,
+                                        None if desc is None else ctypes.byref(desc), ctypes.c_float(0.1), None, dummy, None,
+                                        None, 0, None)
+
+    def variant(**kw):
+        d = abi.PackedDesc.from_buffer_copy(bytes(good))
+        for k, v in kw.items():
+            setattr(d, k, v)
+        return d
+
+    for call in (experts, forward, router_select):
+        assert call(good) == -1, call.__name__               # descriptor accepted: the next check is x == NULL
+        assert call(None) == abi.E_PACKED, call.__name__     # a buffer without its descriptor
+        for bad in (variant(magic=0), variant(layout_version=good.layout_version + 1), variant(dtype=abi.F16),
+                    variant(d_model=1024), variant(n_experts=64), variant(expert_dim=48), variant(gated=1),
+                    variant(bytes=good.bytes - 256), variant(sections=good.sections & ~1),
+                    variant(router_width=256)):
+            assert call(bad) == abi.E_PACKED, call.__name__
+    # the static entry point looks at the workspace limit first (this shape fits), then at the descriptor
+    assert forward_static(None) == abi.E_PACKED and forward_static(variant(dtype=abi.F16)) == abi.E_PACKED
+    # a buffer packed WITH the router serves a call whose shape names none (experts only) ...
+    assert experts(good, ops.make_shape(100, 768, 128, 24, 0, abi.BF16)) == -1
+    # ... and one packed without it passes too (the router then runs on the unfused kernels); only its size must be its own
+    bare_shape = ops.make_shape(100, 768, 128, 24, 0, abi.BF16)
+    bare = abi.PackedDesc()
+    assert lib.d2dmoe_packed_describe(ctypes.byref(bare_shape), ctypes.byref(bare)) == 0
+    assert bare.router_width == 0 and not (bare.sections & 32) and bare.bytes < good.bytes
+    assert forward(bare) == -1 and experts(bare) == -1
+    assert forward(variant(router_width=0)) == abi.E_PACKED   # claims "no router" at the size of a buffer with one
+    # the header of a buffer, copied back to the host, yields the descriptor again
+    back = abi.PackedDesc()
+    assert lib.d2dmoe_packed_desc_from_header(bytes(good), ctypes.byref(back)) == 0 and bytes(back) == bytes(good)
+    assert lib.d2dmoe_packed_desc_from_header(bytes(64), ctypes.byref(back)) == abi.E_PACKED
+    assert b'packed' in lib.d2dmoe_status_string(abi.E_PACKED)
 
 
 # ------------------------------------------------------------------ host-side module mirror -------------

@@ -258,14 +258,35 @@ def test_hip_layer_refuses_autograd():
 
 
 def test_packed_buffer_of_another_shape_is_refused():
+    """The descriptor that travels with a packed buffer is checked by the library: a buffer packed for another layer is
+    refused (status -9) before anything is launched; a buffer that lost its descriptor (a slice, a plain copy) is refused
+    by the wrapper, and packed_from_header() recovers it from the buffer's first bytes.  A buffer packed without the router
+    section still serves the layer: the router then runs on the unfused kernels, with the same mask."""
     from d2dmoe_amd import D2DMoEError
     x, routing, p = H.random_case(64, 768, 128, 24, 128, seed=1, dtype=torch.bfloat16, device=DEV)
+    _, _, q = H.random_case(64, 768, 64, 48, 128, seed=2, dtype=torch.bfloat16, device=DEV)
     ops = _ops()
-    small = ops.pack_weights(ops.make_shape(0, 768, 128, 24, 0, 1, 'relu'), p['w1'], p['b1'], p['w2'])
-    with pytest.raises(D2DMoEError, match='packed buffer'):      # no router section in this buffer
-        ops.forward(x, p['router_w1'], p['router_w2'], 0.1, p['w1'], p['b1'], p['w2'], None, None, 'relu', packed=small)
+    other = ops.pack_weights(ops.make_shape(0, 768, 64, 48, 128, 1, 'relu'), q['w1'], q['b1'], q['w2'], None, q['router_w1'],
+                             q['router_w2'])
+    with pytest.raises(D2DMoEError, match='status -9'):
+        ops.forward(x, p['router_w1'], p['router_w2'], 0.1, p['w1'], p['b1'], p['w2'], None, None, 'relu', packed=other)
+    with pytest.raises(D2DMoEError, match='status -9'):
+        ops.experts(x, routing, p['w1'], p['b1'], p['w2'], packed=other)
+    full = ops.pack_weights(ops.make_shape(0, 768, 128, 24, 128, 1, 'relu'), p['w1'], p['b1'], p['w2'], None, p['router_w1'],
+                            p['router_w2'])
     with pytest.raises(D2DMoEError, match='packed buffer'):
-        ops.experts(x, routing, p['w1'], p['b1'], p['w2'], packed=small[:1024])
+        ops.experts(x, routing, p['w1'], p['b1'], p['w2'], packed=full[:1024])
+    with pytest.raises(D2DMoEError, match='packed buffer'):
+        ops.experts(x, routing, p['w1'], p['b1'], p['w2'], packed=full.clone())
+    want = ops.experts(x, routing, p['w1'], p['b1'], p['w2'], packed=full)
+    again = ops.packed_from_header(full.clone())
+    assert bytes(again.desc) == bytes(full.desc)
+    assert torch.equal(ops.experts(x, routing, p['w1'], p['b1'], p['w2'], packed=again), want)
+    assert torch.equal(ops.experts(x, routing, p['w1'], p['b1'], p['w2'], packed=ops.clone_packed(full)), want)
+    bare = ops.pack_weights(ops.make_shape(0, 768, 128, 24, 0, 1, 'relu'), p['w1'], p['b1'], p['w2'])
+    o1, r1, _, _ = ops.forward(x, p['router_w1'], p['router_w2'], 0.1, p['w1'], p['b1'], p['w2'], None, None, 'relu', packed=bare)
+    o2, r2, _, _ = ops.forward(x, p['router_w1'], p['router_w2'], 0.1, p['w1'], p['b1'], p['w2'], None, None, 'relu', packed=full)
+    assert torch.equal(r1, r2) and torch.equal(o1, o2)
 
 
 # =================================================================== router rounding and the mask (bf16, f32) =========

@@ -1102,7 +1102,8 @@ def test_entry_points_reject_bad_workspace_alignment_and_paths():
 
     def call(xp=xg.data_ptr(), path='mfma_sparse', wsp=base, wsb=need, pk=packed.data_ptr(), shape=sh):
         return lib.d2dmoe_experts(ctypes.byref(shape), xp, rg.data_ptr(), d['w1'].data_ptr(), d['b1'].data_ptr(),
-                                  d['w2'].data_ptr(), None, None, pk, out.data_ptr(), abi.PATH[path], wsp, wsb, stream)
+                                  d['w2'].data_ptr(), None, None, pk, None if pk is None else ctypes.byref(packed.desc),
+                                  out.data_ptr(), abi.PATH[path], wsp, wsb, stream)
 
     assert call() == 0
     assert call(wsb=1024) == -5                  # workspace too small for the expert-major plan
@@ -1111,7 +1112,8 @@ def test_entry_points_reject_bad_workspace_alignment_and_paths():
     assert call(pk=None, path='mfma_dense') == -1
     assert call(path='mfma_decode') == -6        # more than 48 tokens
     f32 = ops.make_shape(N, D, E, Ed, 0, abi.F32)
-    assert call(shape=f32, path='mfma_dense') == -6
+    assert call(shape=f32, path='mfma_dense') == -9   # the buffer was packed for bf16
+    assert call(shape=f32, path='mfma_dense', pk=None) == -6
     torch.cuda.synchronize()
     # the call that went through left a correct result behind
     assert H.rel_err(out.cpu(), _experts_want(x, routing, {k: v for k, v in p.items() if k != 'last_bias'}, 'relu')) < H.TOL_BF16

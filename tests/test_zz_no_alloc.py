@@ -75,7 +75,7 @@ def test_static_workspace_limit_is_reported():
     dummy = torch.zeros(64, dtype=torch.bfloat16, device=DEV)
     ptr = dummy.data_ptr()
     st = lib.d2dmoe_forward_static(ctypes.byref(sh), ptr, ptr, ptr, ctypes.c_float(0.1), ptr, ptr, ptr, None, None, None,
-                                   None, None, ptr, None, ptr, 0, None)
+                                   None, None, None, ptr, None, ptr, 0, None)
     assert st == abi.E_STATIC_LIMIT
     assert b'static' in lib.d2dmoe_status_string(st)
     small = ops.make_shape(1576, 768, 128, 24, 128, abi.BF16)
