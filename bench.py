@@ -4,8 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vit_b_50k] [--no-cpu-baseline] [--no-sweep]
 
 One "step" is one pass of the whole layer (router MLP -> dynamic-k selection -> experts -> bias epilogue) over one
-batch of synthetic tokens that already sit in HBM; the timed steps are replays of a HIP graph holding that one layer
-call (the same steps launched eagerly from Python are reported as ms_per_step_eager_launches).  The default workload is the ViT-B-shape layer of the headline
+batch of synthetic tokens that already sit in HBM; the timed steps are replays of a HIP graph that holds up to 25
+consecutive layer calls, as a model's captured forward pass holds its layers (the same steps launched eagerly from Python
+are reported as ms_per_step_eager_launches, replays of a graph holding ONE call as ms_per_step_single_call_graph).  The default workload is the ViT-B-shape layer of the headline
 metric: 256 x 197 = 50432 tokens, D = 768, 128 experts x 24 neurons, ReLU, bf16 storage with float32 accumulation,
 module tau = 0.9 (the layer keeps expert e when norm_e >= (1 - tau) * max norm, the reference's convention).
 The literal reading "norm_e >= 0.9 * max" of the same number is measured too and reported under "literal_rule".
@@ -130,27 +131,51 @@ def time_events(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+GRAPH_CALLS_MAX = 25   # calls of fn held by one captured graph at most (each call keeps its own output buffers alive)
+
+
 def time_graph(fn, steps, warmup):
-    """Mean milliseconds per call of fn when the call is captured once into a HIP graph and replayed (the C ABI calls neither
-    allocate nor synchronise, so a whole layer captures): wall clock over `steps` replays, bracketed by synchronize."""
-    graph = torch.cuda.CUDAGraph()
+    """Mean milliseconds per call of fn when the calls are captured into a HIP graph and replayed (the C ABI calls neither
+    allocate nor synchronise, so a whole layer captures).  The graph holds up to GRAPH_CALLS_MAX consecutive calls of fn,
+    as the layers of a model follow each other in one captured forward pass: what is timed is `steps` calls, as whole
+    replays of that graph plus single-call replays for the remainder, wall clock bracketed by synchronize.  (A replay of
+    a graph that holds ONE call pays 8-9 us of replay-to-replay gap per call on this machine, which a model's graph pays
+    once per forward pass; `ms_per_step_single_call_graph` in the output keeps that figure.)"""
+    def capture(n_calls):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(n_calls):
+                fn()
+        return graph
+
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         fn()
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    with torch.cuda.graph(graph):
-        fn()
-    spin_up(graph.replay)
+    per = max(1, min(steps, GRAPH_CALLS_MAX))
+    single = capture(1)
+    many = capture(per) if per > 1 else single
+    torch.cuda.synchronize()
+    spin_up(single.replay)
     for _ in range(warmup):
-        graph.replay()
+        single.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        graph.replay()
+    for _ in range(steps // per):
+        many.replay()
+    for _ in range(steps % per):
+        single.replay()
     torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    # the same number of steps as single-call replays, for the record
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        single.replay()
+    torch.cuda.synchronize()
+    time_graph.last_single_call_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return ms
 
 
 def time_quantiles(fn, iters, warmup):
@@ -225,6 +250,7 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, pa
     ms_layer_eager = (time.perf_counter() - t0) * 1e3 / steps
     # the same step replayed from a HIP graph: removes the host's launch latency between the dependent kernels
     ms_layer = time_graph(layer, steps, warmup)
+    ms_layer_single = time_graph.last_single_call_ms
     # dominant kernel alone (same routing), HIP events on the launch stream
     # the experts call the layer makes: under AUTO d2dmoe_forward takes the expert-major path for high thresholds
     experts_path = path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 and x.dtype in (torch.bfloat16, torch.float16) else 'auto')
@@ -241,7 +267,7 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, pa
     router_flops = N * (2.0 * D * W + 2.0 * W * E)
     s = x.element_size()
     algo_bytes = N * D * s * 2 + N * E * s + (2 * E * D * Ed + E * Ed + D + W * D + E * W) * s
-    return dict(ms_layer=ms_layer, ms_layer_eager=ms_layer_eager, ms_experts=ms_experts, ms_router=ms_router, pairs=pairs, mean_active=mean_k,
+    return dict(ms_layer=ms_layer, ms_layer_eager=ms_layer_eager, ms_layer_single=ms_layer_single, ms_experts=ms_experts, ms_router=ms_router, pairs=pairs, mean_active=mean_k,
                 p99_active=p99_k, active_tflops_layer=active_flops / ms_layer / 1e9,
                 active_tflops_kernel=active_flops / ms_experts / 1e9,
                 total_tflops_layer=(active_flops + router_flops) / ms_layer / 1e9,
@@ -280,10 +306,10 @@ def gated_record(args, ops, dev, workload):
     union = int((routing.float().sum(0) > 0).sum().item())
     pairs = int(routing.float().sum().item())
     ms_layer_eager = time_events(layer, args.steps, args.warmup)
-    ms_layer_graph = time_graph(layer, args.steps, args.warmup)   # as for the headline: replays of a HIP graph of one layer call
-    # a layer of a few tens of microseconds can be quicker launched eagerly than replayed (a replay's own host cost is
-    # not hidden behind so short a graph): the step is the quicker of the two, both are reported
-    ms_layer = min(ms_layer_eager, ms_layer_graph)
+    # the step, as for the headline: replays of a HIP graph holding consecutive layer calls (eager launches are reported
+    # beside it)
+    ms_layer_graph = time_graph(layer, args.steps, args.warmup)
+    ms_layer = ms_layer_graph
     ms_experts = time_events(lambda: ops.experts(x, routing, wg, None, wd, wu, None, act, False, 'auto', packed),
                              args.steps, args.warmup)
     s = x.element_size()
@@ -313,7 +339,7 @@ def gated_record(args, ops, dev, workload):
         reps = max(args.steps // COLD_SETS, 3)
         cold_eager = time_events(rotation, reps, max(args.warmup // COLD_SETS, 1)) / COLD_SETS
         cold_graph = time_graph(rotation, reps, max(args.warmup // COLD_SETS, 1)) / COLD_SETS
-        cold_layer = min(cold_eager, cold_graph)
+        cold_layer = cold_graph
         cold_experts = time_events(experts_rotation, reps, max(args.warmup // COLD_SETS, 1)) / COLD_SETS
         kernel_bytes = union * 3 * D * Ed * s + 2 * N * D * s
         cold = {'weight_sets': COLD_SETS, 'ms_per_step': cold_layer, 'ms_per_step_eager_launches': cold_eager,
@@ -594,16 +620,18 @@ def skew_norms(N, E, dtype, dev):
     return (torch.randn(N, E, generator=g).abs() * (wts / wts.max())).to(dtype).to(dev)
 
 
-def regime_roofline(r, N, peak):
+def regime_roofline(r, N, peak, traffic_row=None):
     """The experts call of one regime against both ceilings: active-pair FLOPs over the MFMA peak and the layer's
-    algorithmic bytes over the HBM peak; the bound named is the one the larger fraction belongs to."""
+    algorithmic bytes over the HBM peak; the bound named is the one the larger fraction belongs to.  traffic_row: the row
+    of profiles/traffic_per_launch.md that holds the counter traffic of this regime's kernels, if there is one."""
     f_mfma = r['active_tflops_kernel'] / peak
     f_hbm = r['algo_bytes'] / r['ms_experts'] / 1e6 / PEAK_HBM_GBPS
+    traffic, traffic_src = measured_traffic(traffic_row) if traffic_row else (None, None)
     if f_mfma >= f_hbm:
         return {'bound': 'mfma', 'achieved': r['active_tflops_kernel'], 'peak': peak, 'unit': 'TFLOP/s', 'frac': f_mfma,
-                'kernel_ms': r['ms_experts']}
+                'traffic': traffic, 'traffic_source': traffic_src, 'kernel_ms': r['ms_experts']}
     return {'bound': 'hbm', 'achieved': r['algo_bytes'] / r['ms_experts'] / 1e6, 'peak': PEAK_HBM_GBPS, 'unit': 'GB/s',
-            'frac': f_hbm, 'kernel_ms': r['ms_experts']}
+            'frac': f_hbm, 'traffic': traffic, 'traffic_source': traffic_src, 'kernel_ms': r['ms_experts']}
 
 
 def skew_record(args, ops, dev, steps, warmup):
@@ -621,7 +649,7 @@ def skew_record(args, ops, dev, steps, warmup):
         rec[key] = {'keep_norm_ge_frac_of_max': round(thr, 4), 'ms_per_step': r['ms_layer'], 'tokens_per_s': r['tokens_per_s'],
                     'mean_active_experts': r['mean_active'], 'p99_active_experts': r['p99_active'],
                     'expert_load_max_over_mean': r['expert_load_max_over_mean'],
-                    'roofline': regime_roofline(r, N, PEAK_BF16_TFLOPS)}
+                    'roofline': regime_roofline(r, N, PEAK_BF16_TFLOPS, 'vit_b_skew' if key == 'module_tau' else 'vit_b_skew_literal')}
     return rec
 
 
@@ -639,7 +667,7 @@ def router_driven_record(args, ops, dev, name, steps, warmup):
         r = run_regime(ops, x, p, packed, float(thr), act, steps, warmup, D, E, Ed, W)
         rec[key] = {'keep_norm_ge_frac_of_max': round(thr, 4), 'ms_per_step': r['ms_layer'], 'tokens_per_s': r['tokens_per_s'],
                     'mean_active_experts': r['mean_active'], 'router_select_ms': r['ms_router'],
-                    'roofline': regime_roofline(r, N, PEAK_BF16_TFLOPS)}
+                    'roofline': regime_roofline(r, N, PEAK_BF16_TFLOPS, name if key == 'module_tau' else name + '_literal')}
     return rec
 
 
@@ -772,7 +800,8 @@ def main():
                                f'module tau={args.tau} (keep norm >= {1 - args.tau:.2f}*max), whole layer',
                    'mean_active_experts': main_r['mean_active'], 'p99_active_experts': main_r['p99_active'],
                    'mfma_kernels': packed is not None, 'experts_path': args.path},
-        'ms_per_step_eager_launches': main_r['ms_layer_eager'],
+        'ms_per_step_eager_launches': main_r['ms_layer_eager'], 'ms_per_step_single_call_graph': main_r['ms_layer_single'],
+        'graph_calls_per_replay': min(args.steps, GRAPH_CALLS_MAX),
         'active_tflops': main_r['active_tflops_layer'], 'hbm_gbps': main_r['hbm_gbps_layer'],
         'roofline': {'bound': 'mfma', 'kernel': 'experts', 'achieved': main_r['active_tflops_kernel'],
                      'peak': peak, 'unit': 'TFLOP/s', 'frac': main_r['active_tflops_kernel'] / peak,

@@ -254,13 +254,18 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x,
  * every input and output.
  *   - Limit: shapes whose d2dmoe_workspace_bytes() exceeds D2DMOE_STATIC_WORKSPACE_BYTES (256 MiB) are rejected with
  *     D2DMOE_E_STATIC_LIMIT before anything is launched (the ViT-B / GPT-2 layer fits up to 20 808 tokens, the
- *     Gemma-shape layer up to 2 027).  Each GPU the library runs on holds one such array until the process ends.
+ *     Gemma-shape layer up to 2 027).  Each GPU the library runs on holds one such array until the process ends -- the
+ *     array is part of the loaded code object, so every process that loads the library pays for it on every GPU it
+ *     uses, whether or not it calls this entry point; a deployment that never does can build the library with a
+ *     small D2DMOE_STATIC_WORKSPACE_BYTES.
  *   - Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race.  The
  *     array keeps the previous call's contents; the kernels initialise what they read of it on the stream, as they do
  *     with a caller-owned workspace.
  *   - The first call on each device looks the array's device address up (hipGetSymbolAddress); make that call outside
  *     stream capture. */
+#ifndef D2DMOE_STATIC_WORKSPACE_BYTES   /* a build may size the array otherwise: hipcc -DD2DMOE_STATIC_WORKSPACE_BYTES=... */
 #define D2DMOE_STATIC_WORKSPACE_BYTES (256u << 20)
+#endif
 int d2dmoe_forward_static(const d2dmoe_shape* shape, const void* x,
                           const void* router_w1, const void* router_w2, float thr_scale,
                           const void* w1, const void* b1, const void* w2, const void* w_up, const void* last_bias,
