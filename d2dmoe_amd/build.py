@@ -14,7 +14,7 @@ import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, 'csrc')
-SOURCES = ('api.hip', 'kernels_generic.hip', 'kernels_mfma.hip', 'kernels_sparse.hip', 'kernels_decode.hip', 'kernels_gemm.hip', 'kernels_norms.hip', 'kernels_mid.hip')
+SOURCES = ('api.hip', 'kernels_generic.hip', 'kernels_mfma.hip', 'kernels_dense_wide.hip', 'kernels_sparse.hip', 'kernels_decode.hip', 'kernels_gemm.hip', 'kernels_norms.hip', 'kernels_mid.hip')
 OUTPUT = os.path.join(HERE, 'libd2dmoe_hip.so')
 ARCH = 'gfx950'
 

@@ -306,7 +306,7 @@ static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* ro
       path = D2DMOE_PATH_MFMA_SPARSE;   // still bound by the weight stream: expert-major whatever the routing
     // big experts: the dense sweep cannot skip anything (a chunk of 256 neurons is two experts), so the expert-major
     // path is tried whatever the threshold; it hands over to the sweep on the device when the routing is dense
-    else if (packed != nullptr && !sh.gated && sh.expert_dim > 64 && mfma_sparse_supported(sh) && mfma_dense_supported(sh) &&
+    else if (packed != nullptr && !sh.gated && sh.expert_dim > 64 && mfma_sparse_supported(sh) && mfma_sparse_falls_back_to_sweep(sh) &&
              workspace != nullptr && workspace_bytes >= mfma_sparse_workspace_bytes(sh))
       path = D2DMOE_PATH_MFMA_SPARSE;
     else if (packed != nullptr && mfma_dense_supported(sh)) path = D2DMOE_PATH_MFMA_DENSE;
@@ -331,8 +331,8 @@ static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* ro
     case D2DMOE_PATH_MFMA_SPARSE: {
       // expert-major when the routed pairs fit the provisioned capacity, else the dense sweep: decided on the device
       if (!mfma_sparse_supported(sh)) return D2DMOE_E_UNSUPPORTED;
-      // the fall-back: the dense sweep where it exists (ungated, D = 768), else the tiled products
-      const bool fb_gemm = sh.gated || !mfma_dense_supported(sh);
+      // the fall-back: the dense sweep (ungated, D = 768), else the tiled products
+      const bool fb_gemm = !mfma_sparse_falls_back_to_sweep(sh);
       if (fb_gemm && !mfma_gemm_supported(sh)) return D2DMOE_E_UNSUPPORTED;
       if (!packed) return D2DMOE_E_NULL;
       const size_t need = mfma_sparse_workspace_bytes(sh);
@@ -358,7 +358,7 @@ static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* ro
     case D2DMOE_PATH_MFMA_MID: {
       // compacted two-kernel path when the routed pairs fit the provisioned capacity, else the dense sweep: decided on
       // the device
-      if (!mfma_mid_supported(sh) || !mfma_dense_supported(sh)) return D2DMOE_E_UNSUPPORTED;
+      if (!mfma_mid_supported(sh) || !mfma_sparse_falls_back_to_sweep(sh)) return D2DMOE_E_UNSUPPORTED;
       if (!packed) return D2DMOE_E_NULL;
       const size_t need = mfma_mid_workspace_bytes(sh);
       if (!workspace || workspace_bytes < need || (((uintptr_t)workspace) & 255u)) return D2DMOE_E_WORKSPACE;
@@ -483,13 +483,13 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   // reference benchmark's Bernoulli override, where the fraction says nothing about the density: the dense sweep
   // cannot skip at their granularity)
   if (path == D2DMOE_PATH_AUTO && sh.n_tokens > (sh.gated && mfma_decode_supported(sh) ? 48 : 16) && packed != nullptr &&
-      (thr_scale >= ((sh.gated || !mfma_dense_supported(sh)) ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128) ||
+      (thr_scale >= (!mfma_sparse_falls_back_to_sweep(sh) ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128) ||
        (!sh.gated && sh.expert_dim > 64 && (norms_in != nullptr || thr_scale >= 0.5f))) &&
       mfma_sparse_supported(sh) &&
-      ((!sh.gated && mfma_dense_supported(sh)) || mfma_gemm_supported(sh)))
+      (mfma_sparse_falls_back_to_sweep(sh) || mfma_gemm_supported(sh)))
     path = D2DMOE_PATH_MFMA_SPARSE;
   else if (path == D2DMOE_PATH_AUTO && norms_in == nullptr && !sh.gated && sh.expert_dim > 64 && packed != nullptr &&
-           sh.n_tokens > 16 && mfma_dense_supported(sh))
+           sh.n_tokens > 16 && mfma_sparse_falls_back_to_sweep(sh))
     path = D2DMOE_PATH_MFMA_DENSE;   // a low fraction from a real router: d2dmoe_experts' own rule would still try the plan
   // ... and when the router kernel of this call is the one that walks the 32-token segments of that path's plan, it
   // leaves the plan's per-segment counts in the workspace on its way

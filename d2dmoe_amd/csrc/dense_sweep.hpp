@@ -1,0 +1,661 @@
+// The fused experts kernel ("masked dense sweep") as a header: the tile routine, its two kernels and their launcher are
+// templates over the model width, instantiated for D = 768 in kernels_mfma.hip and for D = 1024 in
+// kernels_dense_wide.hip (two translation units so that they compile side by side).
+#pragma once
+
+#include "mfma_common.hpp"
+
+namespace d2dmoe {
+
+// ---------------------------------------------------------------------------------------------------
+// Fused experts kernel, token-tile-major ("masked dense sweep").
+// Workgroup = 4 waves (one per SIMD), a tile of 64 tokens (or 32: "half tile", used for the last partial round of
+// tiles so the machine does not idle through a mostly empty round).  LDS: the x tile as B fragments (96 KB at
+// D = 768, resident), one chunk of h as A fragments (32 KB), the routing tile, bias / expert-index tables.
+// At D = 1024 the x tile takes 128 KB: the chunk is 128 neurons (h: 16 KB) and the routing tile stays in global memory,
+// a chunk's values being requested into registers while the chunk before it is multiplied.
+// Per chunk of 256 (128) neurons:
+//   GEMM1  wave w: H^T[64 (32) neurons of w, tokens] over K = D      A = W1 fragments (stream), B = x (LDS)
+//   epilogue      + b1, activation, x routing[token, expert(neuron)], round to bf16, store as A fragments to LDS
+//   GEMM2  wave w: OUT[tokens, D/4 columns of w] += H . W2            A = h (LDS), B = W2 fragments (stream)
+// OUT stays in registers across all chunks (ascending neuron = ascending expert order, float32) and is rounded
+// once in the final epilogue (+ last_bias, + x).  Chunks none of whose experts is routed to by any token of the
+// tile are skipped (uniform branch).
+//
+// Each wave runs at one wave per SIMD, so memory latency is hidden by software: the weight stream is read MD_RING
+// fragments ahead into a register ring (compile-time indices), across phase and chunk boundaries;
+// __builtin_amdgcn_sched_barrier pins every refill where it is written.  The two workgroup barriers per chunk wait
+// on LDS traffic only, so the global loads in flight survive them; GEMM2 of one chunk and GEMM1 of the next run
+// back to back between barriers.
+// ---------------------------------------------------------------------------------------------------
+struct DenseArgs {
+  const bf16_t* x; const bf16_t* routing; const bf16x8* wp; const bf16_t* b1p; const uint8_t* eidx;
+  const bf16_t* last_bias; bf16_t* out;
+  const int* skip_flag;   // optional device flag: non-zero = the expert-major path handles this call
+  float* partial;         // [csplit][part_rows][D] float32 sums of the chunk-split tiles (tokens from part_base on)
+  int csplit; int chunks_per_split; int64_t part_base; int64_t part_rows;
+  int64_t N; int E; int expert_dim; int n_chunks; int hidden; int act_rt; int add_residual; int n_full; int n_tiles;
+};
+
+// What depends on the model width: the chunk of hidden neurons a workgroup multiplies between two barriers, and
+// whether the tile's routing rows fit in LDS next to the x tile.
+template <int D> struct SweepCfg {
+  static constexpr int HC = sweep_chunk(D);       // hidden neurons per chunk
+  static constexpr int LOG_HC = (HC == 256) ? 8 : 7;
+  static constexpr int RT = HC / 128;             // 32-neuron row tiles of GEMM1 per wave
+  static constexpr int KS2 = HC / 16;             // K = 16 steps of GEMM2 per chunk
+  static constexpr bool RLDS = (D <= 768);        // routing tile staged in LDS
+  // The output tile's accumulators fill the 256 accumulation registers at D = 1024; GEMM1's sums must then live in
+  // ordinary vector registers, which the compiler does not arrange by itself (it spills accumulator tiles instead):
+  // GEMM1's MFMAs are written as assembly statements with vector-register operands there.
+  static constexpr bool VACC = (D > 768);
+};
+
+// A wave's stream of 16-byte-per-lane fragments, indexed in units of 16 bytes.  BUFFER: read with buffer loads -- the
+// stream's base sits in a resource descriptor (scalar registers), the position in the stream is a scalar byte offset
+// plus an immediate, and the lane's 16 bytes are ONE vector register that never changes: the walk through the stream
+// costs no vector arithmetic and no vector registers for addresses (as plain pointers, each group of four fragments
+// needs a 64-bit vector add and a register pair).
+template <bool BUFFER> struct StreamPtr;
+template <> struct StreamPtr<false> {
+  const bf16x8* p;
+  __device__ __forceinline__ bf16x8 operator[](int64_t i) const { return p[i]; }
+  __device__ __forceinline__ StreamPtr operator+(int64_t n) const { return {p + n}; }
+};
+template <> struct StreamPtr<true> {
+  __amdgpu_buffer_rsrc_t rsrc; uint32_t loff; int soff;   // soff: bytes, the same in all lanes
+  __device__ __forceinline__ bf16x8 operator[](int i) const {
+    // (the whole position goes into the scalar offset: one scalar add per load, and the vector offset stays one register)
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)loff, soff + i * 16, 0);
+    return __builtin_bit_cast(bf16x8, v);
+  }
+  __device__ __forceinline__ StreamPtr operator+(int64_t n) const { return {rsrc, loff, soff + (int)n * 16}; }
+};
+
+// One MFMA with its accumulator in ordinary vector registers (first: C = 0).  The compiler does not know these are matrix
+// instructions: whoever reads the sums with another kind of instruction waits with mfma_vacc_settle() first.
+template <bool F16, bool FIRST> __device__ __forceinline__ void mfma_32x32x16_vacc(const bf16x8& a, const bf16x8& b, f32x16& c) {
+  if constexpr (FIRST) {
+    if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  } else {
+    if constexpr (F16) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+}
+// The matrix pipe writes its results some cycles after the instruction issues and the hardware does not hold back a
+// vector instruction that reads them early (11 wait states for this 8-pass instruction).
+__device__ __forceinline__ void mfma_vacc_settle(f32x16& c) { asm volatile("s_nop 15\n\ts_nop 15" : "+v"(c)); }
+
+// SPLIT: the workgroup handles only chunks [c_begin, c_end) of its tile and leaves its float32 sums, without bias or
+// residual, in A.partial[split]; a finishing kernel adds the splits in ascending order.
+template <int D, int ACT, bool ED8, int TT, bool SPLIT = false, bool F16 = false>
+__device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw,
+                                           const int c_begin = 0, const int c_end = 1 << 30, const int split = 0) {
+  constexpr int KS1 = D / 16;          // K steps of GEMM1
+  constexpr int CT = D / 128;          // 32-wide column tiles per wave in GEMM2
+  constexpr int HC = SweepCfg<D>::HC, LOG_HC = SweepCfg<D>::LOG_HC, RT = SweepCfg<D>::RT, KS2 = SweepCfg<D>::KS2;
+  constexpr bool RLDS = SweepCfg<D>::RLDS, VACC = SweepCfg<D>::VACC;
+  const int E = A.E, n_chunks = A.n_chunks;
+  const int64_t N = A.N;
+  bf16x8* xs = (bf16x8*)smem_raw;                              // [2][KS1][64]
+  bf16x8* hs = xs + 2 * KS1 * 64;                              // [2][KS2][64]
+  const int RS = E + 8;                                        // padded row stride (16-byte aligned rows)
+  const int HP = n_chunks * HC;
+  bf16_t* rs = (bf16_t*)(hs + 2 * KS2 * 64);                   // [64][E+8] routing tile (RLDS)
+  bf16_t* b1s = rs + (RLDS ? MD_BM * RS : 0);                  // [HP] first-layer bias
+  uint8_t* eis = (uint8_t*)(b1s + HP);                         // [HP] expert index of each neuron
+  uint32_t* ebits = (uint32_t*)(eis + HP);                     // [E rounded up to 8] chunks each expert's neurons lie in
+  uint32_t* cmask_lds = ebits + ((E + 7) & ~7);                // chunks some token of the tile needs (bit per chunk)
+
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  // (wave index: known to be the same in all lanes where the stream below is addressed from a scalar base)
+  const int w = SweepCfg<D>::VACC ? __builtin_amdgcn_readfirstlane(t >> 6) : (t >> 6);
+  const int g = lane >> 5, c32 = lane & 31;
+  constexpr int NW1 = RT * KS1;        // W1 fragments per (wave, chunk)
+  constexpr int NW2 = KS2 * CT;        // W2 fragments per (wave, chunk)
+  constexpr int PIECES = NW1 + NW2;
+  constexpr int R = MD_RING;
+  constexpr int BM = 32 * TT;
+  static_assert(NW1 % R == 0 && NW2 % R == 0, "every phase must start at ring slot 0");
+
+  // ---- staging.  Every global load of the tile's inputs is issued up front, in the order the data is needed:
+  // routing pieces and the two tables (short, and the active-chunk mask hangs on them), the x tile, then the weight
+  // stream of the first chunk (almost every tile starts at chunk 0; if its first active chunk turns out to be another
+  // one the ring is reloaded below).  Loads complete in order, so each stage below waits only for what precedes it.
+  //
+  // A wave stages RW consecutive rows of the tile.  Lane (r = lane & 7, c = lane >> 3) takes row r of a block of 8
+  // rows and the 16-byte pieces c, c + 8, c + 16 ... of it: 8 lanes read 128 contiguous bytes of a row, 8 lanes write
+  // 128 contiguous bytes of LDS (the rows of a fragment), and all further addresses are compile-time offsets from a
+  // handful of lane values -- this part of the kernel is bound by instruction issue, not by memory.
+  // Rows past the end of the batch are read from the last row instead (rows never mix, and their results are not
+  // stored).
+  typedef StreamPtr<VACC> Stream;
+  Stream wbase;                                                               // this wave's stream
+  if constexpr (VACC)   // (raw buffer of 32-bit words covering this wave's part of the packed stream)
+    wbase = Stream{__builtin_amdgcn_make_buffer_rsrc((void*)(A.wp + (int64_t)w * n_chunks * PIECES * 64), 0,
+                                                     n_chunks * PIECES * 1024, 0x00020000), (uint32_t)lane * 16u, 0};
+  else wbase = Stream{A.wp + (int64_t)w * n_chunks * PIECES * 64 + lane};
+  bf16x8 ring[R];
+  const int first_guess = SPLIT ? c_begin : 0;
+  const int r8 = lane & 7, c8l = lane >> 3;
+  const int last_row = (int)((N - 1 - tok0) < (int64_t)(BM - 1) ? (N - 1 - tok0) : (int64_t)(BM - 1));
+  {
+    constexpr int RW = BM / 4;                      // rows per wave
+    constexpr int RB = RW / 8;                      // blocks of 8 rows per wave
+    constexpr int XK = D / 64;                      // 16-byte pieces of a row per lane (12)
+    constexpr int RK = 4;                           // routing pieces of a row per lane (E <= 256)
+    constexpr int TB1 = MD_MAX_CHUNKS / 8, TEI = MD_MAX_CHUNKS / 16;   // table pieces per thread
+    const bool wide = (E & 7) == 0;                 // routing rows are whole 16-byte pieces
+    const int EP = E >> 3;
+    if (t == 0) *cmask_lds = 0u;
+    for (int e = t; e < E; e += 256) {
+      const int h0 = e * A.expert_dim;
+      ebits[e] = (1u << (h0 >> LOG_HC)) | (1u << ((h0 + A.expert_dim - 1) >> LOG_HC));
+    }
+    int mrow[RB];                                   // tile row of each row block, clamped to the last real row
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const int m = w * RW + rb * 8 + r8;
+      mrow[rb] = m < last_row ? m : last_row;
+    }
+    u32x4 rv[RB][RK];
+    if (wide) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const u32x4* rrow = (const u32x4*)(A.routing + (tok0 + mrow[rb]) * E);
+#pragma unroll
+        for (int kb = 0; kb < RK; ++kb)
+          if (kb * 8 < EP) rv[rb][kb] = rrow[c8l + kb * 8 < EP ? c8l + kb * 8 : 0];   // lanes past the row: piece 0
+      }
+    }
+    u32x4 tb[TB1], te[TEI];
+#pragma unroll
+    for (int k = 0; k < TB1; ++k) {
+      const int i = t + k * 256;
+      tb[k] = ((const u32x4*)A.b1p)[i < HP / 8 ? i : 0];
+    }
+#pragma unroll
+    for (int k = 0; k < TEI; ++k) {
+      const int i = t + k * 256;
+      te[k] = ((const u32x4*)A.eidx)[i < HP / 16 ? i : 0];
+    }
+    u32x4 xv[RB][XK];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const u32x4* xrow = (const u32x4*)(A.x + (tok0 + mrow[rb]) * D) + c8l;
+#pragma unroll
+      for (int kb = 0; kb < XK; ++kb) xv[rb][kb] = xrow[kb * 8];
+    }
+    lds_barrier();   // chunk bits per expert written, mask cleared
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t need = 0u;                             // chunks the rows staged by this thread need
+    if (wide) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const int m = w * RW + rb * 8 + r8;
+#pragma unroll
+        for (int kb = 0; kb < RK; ++kb) {
+          if (kb * 8 < EP && c8l + kb * 8 < EP) {
+            const int piece = c8l + kb * 8;
+            const u32x4 r4 = rv[rb][kb];
+            if constexpr (RLDS) *(u32x4*)(rs + m * RS + piece * 8) = r4;
+            const u32x4 eb0 = *(const u32x4*)(ebits + piece * 8);
+            const u32x4 eb1 = *(const u32x4*)(ebits + piece * 8 + 4);
+            const uint32_t wd[4] = {r4.x, r4.y, r4.z, r4.w};
+            const uint32_t eb[8] = {eb0.x, eb0.y, eb0.z, eb0.w, eb1.x, eb1.y, eb1.z, eb1.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              need |= (wd[i >> 1] & ((i & 1) ? 0x7fff0000u : 0x7fffu)) != 0 ? eb[i] : 0u;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < TB1; ++k) {
+      const int i = t + k * 256;
+      if (i < HP / 8) ((u32x4*)b1s)[i] = tb[k];
+    }
+#pragma unroll
+    for (int k = 0; k < TEI; ++k) {
+      const int i = t + k * 256;
+      if (i < HP / 16) ((u32x4*)eis)[i] = te[k];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < R; ++i) ring[i] = wbase[((int64_t)first_guess * PIECES + i) * 64];
+    __builtin_amdgcn_sched_barrier(0);
+    if (!wide) {
+      for (int i = t; i < BM * E; i += 256) {
+        const int m = i / E, e = i - m * E;
+        const bf16_t r1 = A.routing[(tok0 + (m < last_row ? m : last_row)) * E + e];
+        if constexpr (RLDS) rs[m * RS + e] = r1;
+        if ((r1 & 0x7fff) != 0) need |= ebits[e];
+      }
+    }
+    if (need != 0u)
+      __hip_atomic_fetch_or((__attribute__((address_space(3))) uint32_t*)cmask_lds, need, __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_WORKGROUP);
+    // x fragments: piece kk of row m goes to fragment kk / 2 (K step), slot (m & 31) + 32 * (kk & 1)
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const int m = w * RW + rb * 8 + r8;
+      u32x4* xdst = (u32x4*)xs + ((m >> 5) * KS1 + (c8l >> 1)) * 64 + (m & 31) + 32 * (c8l & 1);
+#pragma unroll
+      for (int kb = 0; kb < XK; ++kb) xdst[kb * 4 * 64] = xv[rb][kb];
+    }
+  }
+  lds_barrier();
+  // Active chunks as a bit mask, the same in every wave: the chunk loop walks its set bits.
+  uint32_t cmask = __builtin_amdgcn_readfirstlane(*cmask_lds);
+  if constexpr (SPLIT) {
+    const uint32_t below_end = (c_end >= 32) ? ~0u : ((1u << c_end) - 1u);
+    cmask &= below_end & ~((1u << c_begin) - 1u);
+  }
+  const int n_act = __popc(cmask);
+
+  f32x16 acc2[TT][CT];
+#pragma unroll
+  for (int a = 0; a < TT; ++a)
+#pragma unroll
+    for (int b = 0; b < CT; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc2[a][b][r] = 0.f;
+
+  if (n_act > 0) {
+    f32x16 acc1[RT][TT];  // GEMM1 accumulators [row-tile][token tile]
+    const int first_chunk = __builtin_ctz(cmask);
+    Stream cur = wbase + (int64_t)first_chunk * PIECES * 64;
+    if (first_chunk != first_guess) {
+#pragma unroll
+      for (int i = 0; i < R; ++i) ring[i] = cur[i * 64];
+    }
+
+    // Without the routing tile in LDS: the routing values a lane's accumulators are multiplied by (its tokens, the experts
+    // of its rows), raw 16-bit patterns, requested one chunk ahead.
+    constexpr int NRQ = ED8 ? 4 : 16;
+    uint32_t rpre[TT][RT][NRQ];
+    auto routing_request = [&](int chunk_r, int g, int c32) __attribute__((always_inline)) {
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) {
+        const int m = tt * 32 + c32;
+        const char* rtile = (const char*)(A.routing + tok0 * E);   // the same in all lanes; byte offsets from it below
+        const uint32_t rrow = (uint32_t)((m < last_row ? m : last_row) * E) * 2u;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int hb = chunk_r * HC + w * (32 * RT) + 4 * g + rt * 32 + 8 * q;
+            if (ED8) {
+              rpre[tt][rt][q] = *(const bf16_t*)(rtile + (rrow + 2u * eis[hb & ~7]));
+            } else {
+              const uint32_t e4 = *(const uint32_t*)(eis + hb);
+#pragma unroll
+              for (int i = 0; i < 4; ++i) rpre[tt][rt][q * 4 + i] = *(const bf16_t*)(rtile + (rrow + 2u * ((e4 >> (8 * i)) & 0xff)));
+            }
+          }
+        }
+      }
+    };
+
+    // This lane's 16 bytes of the first x / h fragment of each token tile.  Where the tiles span more than the 64 KB an
+    // LDS instruction's immediate offset reaches, the compiler would keep one address per fragment in registers (and
+    // spill them): the tile offsets are made opaque there, so that every fragment is one base register + an immediate.
+    // (x tile 0 starts at the lane's own offset, both h tiles lie within one immediate's reach of the first)
+    const bf16x8* xrow[TT];
+    const bf16x8* hrow[TT];
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+      uint32_t xo = (uint32_t)(tt * KS1 * 64 + lane), ho = (uint32_t)lane;
+      if constexpr (VACC) {
+        if (tt > 0) asm volatile("" : "+v"(xo));
+        if (tt == 0) asm volatile("" : "+v"(ho));
+      } else {
+        ho += (uint32_t)(tt * KS2 * 64);
+      }
+      xrow[tt] = xs + xo;
+      hrow[tt] = (VACC && tt > 0) ? hrow[0] + tt * KS2 * 64 : hs + ho;
+    }
+
+    for (int ci = 0; ci < n_act; ++ci) {
+      const int chunk = __builtin_ctz(cmask);
+      cmask &= cmask - 1;
+      const Stream nxt = (cmask != 0) ? (wbase + (int64_t)__builtin_ctz(cmask) * PIECES * 64) : cur;
+      // Where registers are short (VACC), what the epilogue derives from the lane index -- table and h-tile addresses,
+      // routing rows -- is recomputed from a fresh copy of it in every chunk instead of being kept across the products.
+      int lane_c = lane;
+      if constexpr (VACC) asm volatile("" : "+v"(lane_c));
+      const int g = lane_c >> 5, c32 = lane_c & 31;
+      const int hb0 = chunk * HC + w * (32 * RT) + 4 * g;   // first neuron of this lane's accumulator rows, row-tile 0
+
+      // epilogue state, filled and consumed in slices between MFMAs
+      uint2 e_bias[4];     // 4 bf16 biases per accumulator quad
+      uint32_t e_idx[4];   // expert index: one per quad (ED8) or four packed uint8
+      float e_rq[TT][ED8 ? 4 : 16];
+      float e_hv[TT][16];
+      auto epi_load_tables = [&](int rt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int hb = hb0 + rt * 32 + 8 * q;
+          e_bias[q] = *(const uint2*)(b1s + hb);
+          // Ed multiple of 8: the aligned block of 8 neurons a quad pair covers belongs to one expert, the same for
+          // every lane, so one routing value per (quad, token tile) serves four accumulator rows
+          e_idx[q] = ED8 ? (uint32_t)eis[hb & ~7] : *(const uint32_t*)(eis + hb);
+        }
+      };
+      auto epi_load_routing = [&](int rt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+          if constexpr (RLDS) {
+            const bf16_t* rrow = rs + (tt * 32 + c32) * RS;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              if (ED8) {
+                e_rq[tt][q] = dec16<F16>(rrow[e_idx[q]]);
+              } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) e_rq[tt][q * 4 + i] = dec16<F16>(rrow[(e_idx[q] >> (8 * i)) & 0xff]);
+              }
+            }
+          } else {
+#pragma unroll
+            for (int i = 0; i < NRQ; ++i) e_rq[tt][i] = dec16<F16>(rpre[tt][rt][i]);
+          }
+        }
+      };
+      auto epi_math = [&](int rt, int q) __attribute__((always_inline)) {
+        const float b0 = dec16<F16>(e_bias[q].x & 0xffffu), b1 = dec16_hi<F16>(e_bias[q].x);
+        const float b2 = dec16<F16>(e_bias[q].y & 0xffffu), b3 = dec16_hi<F16>(e_bias[q].y);
+        const float bias[4] = {b0, b1, b2, b3};
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int r = q * 4 + i;
+            float v = acc1[rt][tt][r] + bias[i];
+            v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(A.act_rt, v);
+            e_hv[tt][r] = v * (ED8 ? e_rq[tt][q] : e_rq[tt][r]);
+          }
+        }
+      };
+      auto epi_store = [&](int rt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            uint4 pk;
+            pk.x = enc16x2<F16>(e_hv[tt][half * 8 + 0], e_hv[tt][half * 8 + 1]);
+            pk.y = enc16x2<F16>(e_hv[tt][half * 8 + 2], e_hv[tt][half * 8 + 3]);
+            pk.z = enc16x2<F16>(e_hv[tt][half * 8 + 4], e_hv[tt][half * 8 + 5]);
+            pk.w = enc16x2<F16>(e_hv[tt][half * 8 + 6], e_hv[tt][half * 8 + 7]);
+            const int ks2 = (w * RT + rt) * 2 + half;
+            ((uint4*)hs)[(tt * KS2 + ks2) * 64 + lane_c] = pk;
+          }
+        }
+      };
+      // GEMM1 of the chunk whose stream starts at `pre` (its W1 fragments; the refills run on into its W2 fragments)
+      auto gemm1 = [&](const Stream pre) __attribute__((always_inline)) {
+        if constexpr (!VACC) {
+#pragma unroll
+          for (int a = 0; a < RT; ++a)
+#pragma unroll
+            for (int b = 0; b < TT; ++b)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) acc1[a][b][r] = 0.f;
+        }
+        bf16x8 xb[TT];
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) xb[tt] = xrow[tt][0];
+        static_for<0, KS1>([&](auto ks_c) __attribute__((always_inline)) {
+          constexpr int ks = decltype(ks_c)::value;
+          bf16x8 a[RT];
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) a[rt] = ring[(RT * ks + rt) % R];
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) ring[(RT * ks + rt) % R] = pre[(RT * ks + rt + R) * 64];
+          constexpr int kn = (ks + 1 < KS1) ? ks + 1 : ks;      // x fragments of the next step, read one step ahead
+          bf16x8 nxb[TT];
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) nxb[tt] = xrow[tt][kn * 64];
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+              if constexpr (VACC) mfma_32x32x16_vacc<F16, ks == 0>(a[rt], xb[tt], acc1[rt][tt]);
+              else acc1[rt][tt] = mfma_32x32x16<F16>(a[rt], xb[tt], acc1[rt][tt]);
+            }
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) xb[tt] = nxb[tt];
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        if constexpr (VACC) {
+#pragma unroll
+          for (int a = 0; a < RT; ++a)
+#pragma unroll
+            for (int b = 0; b < TT; ++b) mfma_vacc_settle(acc1[a][b]);
+        }
+      };
+      // GEMM2 of the current chunk; refills run on into the next chunk's W1 fragments
+      auto gemm2 = [&]() __attribute__((always_inline)) {
+        bf16x8 ha[TT];
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) ha[tt] = hrow[tt][0];
+        static_for<0, KS2>([&](auto j_c) __attribute__((always_inline)) {
+          constexpr int j = decltype(j_c)::value;
+          constexpr int jn = (j + 1 < KS2) ? j + 1 : j;         // h fragments of the next step, read one step ahead
+          bf16x8 nha[TT];
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) nha[tt] = hrow[tt][jn * 64];
+          static_for<0, CT>([&](auto ct_c) __attribute__((always_inline)) {
+            constexpr int ct = decltype(ct_c)::value;
+            constexpr int s = j * CT + ct;      // position in this phase; refill position s + R
+            const bf16x8 b = ring[s % R];
+            ring[s % R] = (s + R < NW2) ? cur[(NW1 + s + R) * 64] : nxt[(s + R - NW2) * 64];
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt)
+              acc2[tt][ct] = mfma_32x32x16<F16>(ha[tt], b, acc2[tt][ct]);
+          });
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) ha[tt] = nha[tt];
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      };
+
+      if (ci == 0) {
+        if constexpr (!RLDS) routing_request(chunk, g, c32);
+        gemm1(cur);
+      }
+      lds_barrier();   // every wave has finished reading the previous h tile
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        epi_load_tables(rt);
+        epi_load_routing(rt);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) epi_math(rt, q);
+        epi_store(rt);
+      }
+      lds_barrier();   // h tile complete
+      // (the values of the last chunk are requested once more instead of branching round the loads)
+      if constexpr (!RLDS) routing_request(cmask != 0 ? __builtin_ctz(cmask) : chunk, g, c32);
+      gemm2();
+      if (ci + 1 < n_act) gemm1(nxt);
+      cur = nxt;
+    }
+  }
+
+  // ---- final epilogue: the accumulators are rounded to bf16 once, AFTER + last_bias (+ x) in float32, and leave as
+  // whole rows.  One pass per 32-token tile: every wave writes its D/4 columns of the pass's rows to LDS as float
+  // [32][D + 4] (bias added on the way: a lane's accumulators share CT columns), then wave w takes rows 8w .. 8w + 7
+  // with the lane mapping of the staging above -- lane (r, c) reads 8 consecutive columns c, c + 8, ... of row r, adds
+  // the residual, rounds, stores 16 bytes; 8 lanes cover 128 contiguous bytes of an output row.  The residual rows
+  // are requested before the pass's LDS traffic; the read loop has no branches and no address arithmetic.
+  {
+    constexpr int OS = D + 4;                       // row stride in floats (+16 bytes: rows shift by 4 banks, so the
+    float* ot = (float*)smem_raw;                   // 8 rows a wave reads at once cover all 32); fits in x + h regions
+    static_assert((size_t)32 * OS * 4 <= (size_t)(2 * KS1 * 64 + 2 * KS2 * 64) * 16, "out staging fits");
+    constexpr int OP = D / 64;                      // 8-column pieces per thread and pass
+    const bool with_bias = !SPLIT && A.last_bias != nullptr;
+    const bool with_res = !SPLIT && A.add_residual != 0;
+    float lb[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+      lb[ct] = with_bias ? dec16<F16>(A.last_bias[w * (D / 4) + ct * 32 + c32]) : 0.f;
+    const int row = w * 8 + r8;                     // row of the pass this thread finishes
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+      const int64_t n = tok0 + tt * 32 + row;
+      const bool live = n < N;
+      u32x4 xr[OP];
+      if (with_res) {
+        const u32x4* xrow = (const u32x4*)(A.x + (live ? n : N - 1) * D) + c8l;
+#pragma unroll
+        for (int k = 0; k < OP; ++k) xr[k] = xrow[k * 8];
+      }
+      lds_barrier();                                // previous readers of this LDS region are done
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        const int col = w * (D / 4) + ct * 32 + c32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          ot[(8 * (r / 4) + 4 * g + (r % 4)) * OS + col] = with_bias ? acc2[tt][ct][r] + lb[ct] : acc2[tt][ct][r];
+      }
+      lds_barrier();
+      const float* orow = ot + row * OS + c8l * 8;
+      u32x4 o[OP];
+      float4 pv0[OP], pv1[OP];
+#pragma unroll
+      for (int k = 0; k < OP; ++k) {
+        pv0[k] = *(const float4*)(orow + k * 64);
+        pv1[k] = *(const float4*)(orow + k * 64 + 4);
+        if constexpr (!SPLIT) {
+          float v[8] = {pv0[k].x, pv0[k].y, pv0[k].z, pv0[k].w, pv1[k].x, pv1[k].y, pv1[k].z, pv1[k].w};
+          if (with_res) {
+            const uint32_t xw[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] += (i & 1) ? dec16_hi<F16>(xw[i >> 1]) : dec16<F16>(xw[i >> 1] & 0xffffu);
+          }
+          o[k].x = enc16x2<F16>(v[0], v[1]); o[k].y = enc16x2<F16>(v[2], v[3]);
+          o[k].z = enc16x2<F16>(v[4], v[5]); o[k].w = enc16x2<F16>(v[6], v[7]);
+        }
+      }
+      if (live) {
+        if constexpr (SPLIT) {
+          float* prow = A.partial + ((int64_t)split * A.part_rows + (n - A.part_base)) * D + c8l * 8;
+#pragma unroll
+          for (int k = 0; k < OP; ++k) {
+            *(float4*)(prow + k * 64) = pv0[k];
+            *(float4*)(prow + k * 64 + 4) = pv1[k];
+          }
+        } else {
+          u32x4* grow = (u32x4*)(A.out + n * D) + c8l;
+#pragma unroll
+          for (int k = 0; k < OP; ++k) grow[k * 8] = o[k];
+        }
+      }
+    }
+  }
+}
+
+// Out-of-line copy of the tile routine for the variant below (keeps its register allocation apart from the loop).
+template <int D, int ACT, bool ED8, int TT, bool F16>
+__device__ __attribute__((noinline)) void dense_tile_call(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw) {
+  dense_tile<D, ACT, ED8, TT, false, F16>(A, tok0, smem_raw);
+}
+
+// The same sweep launched as one workgroup per CU that walks the tiles in launch order.  Used where the launch is
+// usually a no-op (the fall-back behind the expert-major path): a skipped call then retires after one round of empty
+// workgroups instead of one per tile.
+template <int D, int ACT, bool ED8, bool F16 = false>
+__global__ __launch_bounds__(256, 1) void experts_mfma_dense_walk_kernel(const DenseArgs A) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
+  for (int b = blockIdx.x; b < A.n_tiles; b += gridDim.x) {
+    if (b < A.n_full)
+      dense_tile_call<D, ACT, ED8, 2, F16>(A, (int64_t)b * 64, smem_raw);
+    else
+      dense_tile_call<D, ACT, ED8, 1, F16>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
+    __syncthreads();   // the next tile's staging overwrites the LDS the final epilogue just read
+  }
+}
+
+// Workgroups [0, n_full) take tiles of 64 tokens.  The tokens left over after the last full round of the machine go to
+// tiles of 32; if those would still leave most CUs idle, each of them is dealt to csplit workgroups by chunk ranges,
+// which leave float32 sums in A.partial for the finishing kernel.
+template <int D, int ACT, bool ED8, bool F16 = false>
+__global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
+  const int b = blockIdx.x;
+  if (b < A.n_full) {
+    dense_tile<D, ACT, ED8, 2, false, F16>(A, (int64_t)b * 64, smem_raw);
+  } else if (A.csplit <= 1) {
+    dense_tile<D, ACT, ED8, 1, false, F16>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
+  } else {
+    const int idx = b - A.n_full;
+    const int tile = idx / A.csplit, split = idx % A.csplit;
+    const int c_begin = split * A.chunks_per_split;
+    dense_tile<D, ACT, ED8, 1, true, F16>(A, (int64_t)A.n_full * 64 + (int64_t)tile * 32, smem_raw, c_begin,
+                                     c_begin + A.chunks_per_split, split);
+  }
+}
+
+struct DenseTiling {
+  int64_t n_full, n_half;   // tiles of 64 and of 32 tokens
+  int csplit, per;          // workgroups per tile of 32 and chunks per workgroup (1, n_chunks: not split)
+  int64_t part_base, part_rows;   // tokens covered by split tiles
+};
+DenseTiling dense_tiling(const d2dmoe_shape& sh, bool allow_split);
+size_t dense_lds_bytes(const d2dmoe_shape& sh);
+
+template <int D, int ACT, bool ED8, bool F16>
+static inline hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
+                                   const void* last_bias, void* out, const int* skip_flag, void* workspace,
+                                   size_t workspace_bytes, hipStream_t s) {
+  const PackedLayout L = packed_layout(sh);
+  const char* base = (const char*)packed;
+  const size_t lds = dense_lds_bytes(sh);
+  if (lds > 160 * 1024) return hipErrorInvalidValue;
+  const int cus = device_cu_count();
+  // Behind the expert-major path the launch is usually a no-op: one workgroup per CU walks the tiles, so a skipped call
+  // retires after one round of empty workgroups.  With big experts (the reference's benchmark shape, swept over
+  // densities) the fall-back runs as often as not, and the walk costs 15 % per tile: the ordinary grid there.
+  const bool walk = skip_flag != nullptr && sh.expert_dim <= 64;
+  const bool allow_split = !walk && workspace != nullptr && workspace_bytes >= mfma_dense_workspace_bytes(sh);
+  const DenseTiling T = dense_tiling(sh, allow_split);
+  auto kern = walk ? experts_mfma_dense_walk_kernel<D, ACT, ED8, F16> : experts_mfma_dense_kernel<D, ACT, ED8, F16>;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return e;
+  DenseArgs A;
+  A.x = (const bf16_t*)x; A.routing = (const bf16_t*)routing; A.wp = (const bf16x8*)(base + L.w_off);
+  A.b1p = (const bf16_t*)(base + L.b1_off); A.eidx = (const uint8_t*)(base + L.eidx_off);
+  A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.N = sh.n_tokens; A.E = sh.n_experts; A.expert_dim = sh.expert_dim;
+  A.n_chunks = L.n_chunks; A.hidden = L.hidden; A.act_rt = sh.activation; A.add_residual = sh.add_residual;
+  A.n_full = (int)T.n_full; A.n_tiles = (int)(T.n_full + T.n_half); A.skip_flag = skip_flag;
+  A.partial = (float*)workspace; A.csplit = T.csplit; A.chunks_per_split = T.per;
+  A.part_base = T.part_base; A.part_rows = T.part_rows;
+  int64_t grid = T.n_full + T.n_half * T.csplit;
+  if (walk && A.n_tiles > cus) grid = cus;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, s, A);
+  e = hipGetLastError();
+  if (e != hipSuccess || T.csplit <= 1) return e;
+  return launch_sum_partials(A.partial, last_bias, (const bf16_t*)x + T.part_base * sh.d_model,
+                             (bf16_t*)out + T.part_base * sh.d_model, T.part_rows, sh.d_model, T.csplit, sh.add_residual, s,
+                             sh.dtype, skip_flag);
+}
+
+template <int D, int ACT>
+static inline hipError_t launch_dense_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
+                                   const void* last_bias, void* out, const int* skip_flag, void* workspace,
+                                   size_t workspace_bytes, hipStream_t s) {
+  if (sh.dtype == D2DMOE_F16) {
+    if (sh.expert_dim % 8 == 0)
+      return launch_dense_cfg<D, ACT, true, true>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+    return launch_dense_cfg<D, ACT, false, true>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+  }
+  if (sh.expert_dim % 8 == 0)
+    return launch_dense_cfg<D, ACT, true, false>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+  return launch_dense_cfg<D, ACT, false, false>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
+}
+
+}  // namespace d2dmoe

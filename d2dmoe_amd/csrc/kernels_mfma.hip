@@ -11,29 +11,36 @@
 // registers are already in place: r = 0..7 feed one K=16 step, r = 8..15 the next.  The k-slot -> hidden-neuron
 // map this implies (slot (g, i) of a step <-> neuron 8*(i/4) + 4g + (i%4) of a 16-block) is baked into the
 // packed W2 fragments, so no shuffle is needed between the two GEMMs.
-#include "mfma_common.hpp"
+#include "dense_sweep.hpp"
 
 namespace d2dmoe {
 
-static size_t dense_lds_bytes(const d2dmoe_shape& sh) {
+size_t dense_lds_bytes(const d2dmoe_shape& sh) {
+  const int hc = sweep_chunk(sh.d_model);
   const int hidden = sh.n_experts * sh.expert_dim;
-  const int n_chunks = (hidden + MD_HC - 1) / MD_HC;
+  const int n_chunks = (hidden + hc - 1) / hc;
   const int KS1 = sh.d_model / 16;
-  return (size_t)(2 * KS1 * 64 + 2 * MD_KS2 * 64) * 16            // x fragments, h fragments
-         + (size_t)MD_BM * (sh.n_experts + 8) * 2                  // routing tile, rows padded by 8 elements
-         + (size_t)n_chunks * MD_HC * 3                            // b1 (bf16) and expert index (uint8) per neuron
+  return (size_t)(2 * KS1 * 64 + 2 * (hc / 16) * 64) * 16         // x fragments, h fragments
+         + (sh.d_model <= 768 ? (size_t)MD_BM * (sh.n_experts + 8) * 2 : 0)   // routing tile, rows padded by 8 elements
+         + (size_t)n_chunks * hc * 3                               // b1 (bf16) and expert index (uint8) per neuron
          + (size_t)((sh.n_experts + 7) / 8 * 8 + 4) * sizeof(uint32_t);   // chunk bits per expert, active-chunk mask
 }
 
-// The fused experts kernel is instantiated for D = 768 (ViT-B, GPT-2 small, BERT-base), ungated experts, bf16.
+// The fused experts kernel is instantiated for D = 768 (ViT-B, GPT-2 small, BERT-base) and D = 1024 (GPT-2 medium,
+// BERT-large, ViT-L), ungated experts, bf16 and float16.
 bool mfma_dense_supported(const d2dmoe_shape& sh) {
   if ((sh.dtype != D2DMOE_BF16 && sh.dtype != D2DMOE_F16) || sh.gated) return false;
-  if (sh.d_model != 768) return false;
+  if (sh.d_model != 768 && sh.d_model != 1024) return false;
+  const int hc = sweep_chunk(sh.d_model);
   if (sh.n_experts > 256) return false;          // expert indices are staged as uint8
-  if (sh.expert_dim > MD_HC) return false;       // an expert spans at most two chunks
-  if ((sh.n_experts * sh.expert_dim + MD_HC - 1) / MD_HC > MD_MAX_CHUNKS) return false;   // staging registers, chunk mask
-  return dense_lds_bytes(sh) <= 160 * 1024;      // x tile + h tile + routing tile + bias/expert-index tables
+  if (sh.expert_dim > hc) return false;          // an expert spans at most two chunks
+  if ((sh.n_experts * sh.expert_dim + hc - 1) / hc > MD_MAX_CHUNKS) return false;   // staging registers, chunk mask
+  return dense_lds_bytes(sh) <= 160 * 1024;      // x tile + h tile (+ routing tile) + bias/expert-index tables
 }
+
+// The expert-major path hands over to the sweep on the device where the sweep is the faster dense alternative it was
+// measured against (D = 768); at the other widths to the tiled products.
+bool mfma_sparse_falls_back_to_sweep(const d2dmoe_shape& sh) { return !sh.gated && sh.d_model == 768 && mfma_dense_supported(sh); }
 
 // The fused router+select kernel covers the D2DMoE router: bf16, depth 2, ReLU hidden / abs output activation,
 // width and expert count both 128 or both 256, D a multiple of 64.
@@ -74,9 +81,10 @@ bool mfma_sparse_supported(const d2dmoe_shape& sh) {
 PackedLayout packed_layout(const d2dmoe_shape& sh) {
   PackedLayout L;
   L.hidden = sh.n_experts * sh.expert_dim;
-  L.n_chunks = (L.hidden + MD_HC - 1) / MD_HC;
-  L.hidden_pad = L.n_chunks * MD_HC;
-  L.pieces = sh.d_model / 16 * 2 + MD_KS2 * (sh.d_model / 128);
+  const int hc = sweep_chunk(sh.d_model);
+  L.n_chunks = (L.hidden + hc - 1) / hc;
+  L.hidden_pad = L.n_chunks * hc;
+  L.pieces = sh.d_model / 16 * (hc / 128) + (hc / 16) * (sh.d_model / 128);
   size_t off = PACKED_HEADER_BYTES;   // the buffer starts with its descriptor
   L.has_dense = mfma_dense_supported(sh);
   L.w_off = off;    if (L.has_dense) off += (size_t)MD_WAVES * L.n_chunks * L.pieces * 64 * 16;
@@ -135,11 +143,11 @@ size_t mfma_gemm_section_offset(const d2dmoe_shape& sh) { return packed_layout(s
 // ---------------------------------------------------------------------------------------------------
 // Packing.  Each wave of the fused kernel reads ONE linear stream of 1 KB fragments (16 bytes per lane), in the
 // order the kernel consumes them:
-//   stream[wave][chunk][piece][lane][8 bf16],   KS1 = D/16, CT = D/128
-//   pieces [0, 2 KS1)          W1 fragments, piece = kstep*2 + rt:
-//       neuron h = chunk*256 + wave*64 + rt*32 + c,  d = kstep*16 + 8g + i        value w1[h/Ed][d][h%Ed]
-//   pieces [2 KS1, 2 KS1+16 CT) W2 fragments, piece = 2 KS1 + ks2*CT + ct:
-//       neuron h = chunk*256 + (ks2/2)*32 + (ks2%2)*16 + 8*(i/4) + 4g + (i%4)
+//   stream[wave][chunk][piece][lane][8 bf16],   KS1 = D/16, CT = D/128, HC = neurons per chunk, RT = HC/128, KS2 = HC/16
+//   pieces [0, RT KS1)         W1 fragments, piece = kstep*RT + rt:
+//       neuron h = chunk*HC + wave*32*RT + rt*32 + c,  d = kstep*16 + 8g + i      value w1[h/Ed][d][h%Ed]
+//   pieces [RT KS1, RT KS1 + KS2 CT) W2 fragments, piece = RT KS1 + ks2*CT + ct:
+//       neuron h = chunk*HC + (ks2/2)*32 + (ks2%2)*16 + 8*(i/4) + 4g + (i%4)
 //       column   = wave*(D/4) + ct*32 + c                                         value w2[h/Ed][h%Ed][column]
 // plus b1 as bf16 [hidden_pad] and the expert index of every neuron as uint8 [hidden_pad]; padding neurons
 // (beyond E*Ed) carry zero weights and zero bias.  One thread per 16-byte piece.
@@ -155,22 +163,23 @@ __global__ void pack_stream_kernel(const bf16_t* __restrict__ w1, const bf16_t* 
   const int wave = (int)(q / n_chunks);
   const int g = lane / 32, c = lane % 32;
   const int KS1 = D / 16, CT = D / 128;
+  const int HC = sweep_chunk(D), RT = HC / 128;
   bf16_t v[8];
-  if (piece < 2 * KS1) {
-    const int ks = piece / 2, rt = piece % 2;
-    const int h = chunk * MD_HC + wave * 64 + rt * 32 + c;
+  if (piece < RT * KS1) {
+    const int ks = piece / RT, rt = piece % RT;
+    const int h = chunk * HC + wave * 32 * RT + rt * 32 + c;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int d = ks * 16 + 8 * g + i;
       v[i] = (h < hidden) ? w1[((int64_t)(h / Ed) * D + d) * Ed + (h % Ed)] : (bf16_t)0;
     }
   } else {
-    const int r = piece - 2 * KS1;
+    const int r = piece - RT * KS1;
     const int ks2 = r / CT, ct = r % CT;
     const int col = wave * (D / 4) + ct * 32 + c;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int h = chunk * MD_HC + (ks2 / 2) * 32 + (ks2 % 2) * 16 + 8 * (i / 4) + 4 * g + (i % 4);
+      const int h = chunk * HC + (ks2 / 2) * 32 + (ks2 % 2) * 16 + 8 * (i / 4) + 4 * g + (i % 4);
       v[i] = (h < hidden) ? w2[((int64_t)(h / Ed) * Ed + (h % Ed)) * D + col] : (bf16_t)0;
     }
   }
@@ -255,466 +264,9 @@ hipError_t launch_mfma_pack(const d2dmoe_shape& sh, const void* w1, const void* 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Fused experts kernel, token-tile-major ("masked dense sweep").
-// Workgroup = 4 waves (one per SIMD), a tile of 64 tokens (or 32: "half tile", used for the last partial round of
-// tiles so the machine does not idle through a mostly empty round).  LDS: the x tile as B fragments (96 KB at
-// D = 768, resident), one chunk of h as A fragments (32 KB), the routing tile, bias / expert-index tables.
-// Per chunk of 256 neurons:
-//   GEMM1  wave w: H^T[64 neurons of w, tokens] over K = D           A = W1 fragments (stream), B = x (LDS)
-//   epilogue      + b1, activation, x routing[token, expert(neuron)], round to bf16, store as A fragments to LDS
-//   GEMM2  wave w: OUT[tokens, D/4 columns of w] += H . W2            A = h (LDS), B = W2 fragments (stream)
-// OUT stays in registers across all chunks (ascending neuron = ascending expert order, float32) and is rounded
-// once in the final epilogue (+ last_bias, + x).  Chunks none of whose experts is routed to by any token of the
-// tile are skipped (uniform branch).
-//
-// Each wave runs at one wave per SIMD, so memory latency is hidden by software: the weight stream is read MD_RING
-// fragments ahead into a register ring (compile-time indices), across phase and chunk boundaries;
-// __builtin_amdgcn_sched_barrier pins every refill where it is written.  The two workgroup barriers per chunk wait
-// on LDS traffic only, so the global loads in flight survive them; GEMM2 of one chunk and GEMM1 of the next run
-// back to back between barriers.
+// Fused experts kernel, token-tile-major ("masked dense sweep"): the kernels are templates in dense_sweep.hpp; here
+// their tiling and the D = 768 instances.
 // ---------------------------------------------------------------------------------------------------
-struct DenseArgs {
-  const bf16_t* x; const bf16_t* routing; const bf16x8* wp; const bf16_t* b1p; const uint8_t* eidx;
-  const bf16_t* last_bias; bf16_t* out;
-  const int* skip_flag;   // optional device flag: non-zero = the expert-major path handles this call
-  float* partial;         // [csplit][part_rows][D] float32 sums of the chunk-split tiles (tokens from part_base on)
-  int csplit; int chunks_per_split; int64_t part_base; int64_t part_rows;
-  int64_t N; int E; int expert_dim; int n_chunks; int hidden; int act_rt; int add_residual; int n_full; int n_tiles;
-};
-
-// SPLIT: the workgroup handles only chunks [c_begin, c_end) of its tile and leaves its float32 sums, without bias or
-// residual, in A.partial[split]; a finishing kernel adds the splits in ascending order.
-template <int D, int ACT, bool ED8, int TT, bool SPLIT = false, bool F16 = false>
-__device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw,
-                                           const int c_begin = 0, const int c_end = 1 << 30, const int split = 0) {
-  constexpr int KS1 = D / 16;          // K steps of GEMM1
-  constexpr int CT = D / 128;          // 32-wide column tiles per wave in GEMM2
-  const int E = A.E, n_chunks = A.n_chunks;
-  const int64_t N = A.N;
-  bf16x8* xs = (bf16x8*)smem_raw;                              // [2][KS1][64]
-  bf16x8* hs = xs + 2 * KS1 * 64;                              // [2][MD_KS2][64]
-  const int RS = E + 8;                                        // padded row stride (16-byte aligned rows)
-  const int HP = n_chunks * MD_HC;
-  bf16_t* rs = (bf16_t*)(hs + 2 * MD_KS2 * 64);                // [64][E+8] routing tile
-  bf16_t* b1s = rs + MD_BM * RS;                               // [HP] first-layer bias
-  uint8_t* eis = (uint8_t*)(b1s + HP);                         // [HP] expert index of each neuron
-  uint32_t* ebits = (uint32_t*)(eis + HP);                     // [E rounded up to 8] chunks each expert's neurons lie in
-  uint32_t* cmask_lds = ebits + ((E + 7) & ~7);                // chunks some token of the tile needs (bit per chunk)
-
-  const int t = threadIdx.x;
-  const int lane = t & 63;
-  const int w = t >> 6;
-  const int g = lane >> 5, c32 = lane & 31;
-  constexpr int NW1 = 2 * KS1;         // W1 fragments per (wave, chunk)
-  constexpr int NW2 = MD_KS2 * CT;     // W2 fragments per (wave, chunk)
-  constexpr int PIECES = NW1 + NW2;
-  constexpr int R = MD_RING;
-  constexpr int BM = 32 * TT;
-  static_assert(NW1 % R == 0 && NW2 % R == 0, "every phase must start at ring slot 0");
-
-  // ---- staging.  Every global load of the tile's inputs is issued up front, in the order the data is needed:
-  // routing pieces and the two tables (short, and the active-chunk mask hangs on them), the x tile, then the weight
-  // stream of the first chunk (almost every tile starts at chunk 0; if its first active chunk turns out to be another
-  // one the ring is reloaded below).  Loads complete in order, so each stage below waits only for what precedes it.
-  //
-  // A wave stages RW consecutive rows of the tile.  Lane (r = lane & 7, c = lane >> 3) takes row r of a block of 8
-  // rows and the 16-byte pieces c, c + 8, c + 16 ... of it: 8 lanes read 128 contiguous bytes of a row, 8 lanes write
-  // 128 contiguous bytes of LDS (the rows of a fragment), and all further addresses are compile-time offsets from a
-  // handful of lane values -- this part of the kernel is bound by instruction issue, not by memory.
-  // Rows past the end of the batch are read from the last row instead (rows never mix, and their results are not
-  // stored).
-  const bf16x8* wbase = A.wp + (int64_t)w * n_chunks * PIECES * 64 + lane;   // this wave's stream
-  bf16x8 ring[R];
-  const int first_guess = SPLIT ? c_begin : 0;
-  const int r8 = lane & 7, c8l = lane >> 3;
-  const int last_row = (int)((N - 1 - tok0) < (int64_t)(BM - 1) ? (N - 1 - tok0) : (int64_t)(BM - 1));
-  {
-    constexpr int RW = BM / 4;                      // rows per wave
-    constexpr int RB = RW / 8;                      // blocks of 8 rows per wave
-    constexpr int XK = D / 64;                      // 16-byte pieces of a row per lane (12)
-    constexpr int RK = 4;                           // routing pieces of a row per lane (E <= 256)
-    constexpr int TB1 = MD_MAX_CHUNKS / 8, TEI = MD_MAX_CHUNKS / 16;   // table pieces per thread
-    const bool wide = (E & 7) == 0;                 // routing rows are whole 16-byte pieces
-    const int EP = E >> 3;
-    if (t == 0) *cmask_lds = 0u;
-    for (int e = t; e < E; e += 256) {
-      const int h0 = e * A.expert_dim;
-      ebits[e] = (1u << (h0 >> 8)) | (1u << ((h0 + A.expert_dim - 1) >> 8));
-    }
-    int mrow[RB];                                   // tile row of each row block, clamped to the last real row
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      const int m = w * RW + rb * 8 + r8;
-      mrow[rb] = m < last_row ? m : last_row;
-    }
-    u32x4 rv[RB][RK];
-    if (wide) {
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        const u32x4* rrow = (const u32x4*)(A.routing + (tok0 + mrow[rb]) * E);
-#pragma unroll
-        for (int kb = 0; kb < RK; ++kb)
-          if (kb * 8 < EP) rv[rb][kb] = rrow[c8l + kb * 8 < EP ? c8l + kb * 8 : 0];   // lanes past the row: piece 0
-      }
-    }
-    u32x4 tb[TB1], te[TEI];
-#pragma unroll
-    for (int k = 0; k < TB1; ++k) {
-      const int i = t + k * 256;
-      tb[k] = ((const u32x4*)A.b1p)[i < HP / 8 ? i : 0];
-    }
-#pragma unroll
-    for (int k = 0; k < TEI; ++k) {
-      const int i = t + k * 256;
-      te[k] = ((const u32x4*)A.eidx)[i < HP / 16 ? i : 0];
-    }
-    u32x4 xv[RB][XK];
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      const u32x4* xrow = (const u32x4*)(A.x + (tok0 + mrow[rb]) * D) + c8l;
-#pragma unroll
-      for (int kb = 0; kb < XK; ++kb) xv[rb][kb] = xrow[kb * 8];
-    }
-    lds_barrier();   // chunk bits per expert written, mask cleared
-    __builtin_amdgcn_sched_barrier(0);
-    uint32_t need = 0u;                             // chunks the rows staged by this thread need
-    if (wide) {
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        const int m = w * RW + rb * 8 + r8;
-#pragma unroll
-        for (int kb = 0; kb < RK; ++kb) {
-          if (kb * 8 < EP && c8l + kb * 8 < EP) {
-            const int piece = c8l + kb * 8;
-            const u32x4 r4 = rv[rb][kb];
-            *(u32x4*)(rs + m * RS + piece * 8) = r4;
-            const u32x4 eb0 = *(const u32x4*)(ebits + piece * 8);
-            const u32x4 eb1 = *(const u32x4*)(ebits + piece * 8 + 4);
-            const uint32_t wd[4] = {r4.x, r4.y, r4.z, r4.w};
-            const uint32_t eb[8] = {eb0.x, eb0.y, eb0.z, eb0.w, eb1.x, eb1.y, eb1.z, eb1.w};
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-              need |= (wd[i >> 1] & ((i & 1) ? 0x7fff0000u : 0x7fffu)) != 0 ? eb[i] : 0u;
-          }
-        }
-      }
-    }
-#pragma unroll
-    for (int k = 0; k < TB1; ++k) {
-      const int i = t + k * 256;
-      if (i < HP / 8) ((u32x4*)b1s)[i] = tb[k];
-    }
-#pragma unroll
-    for (int k = 0; k < TEI; ++k) {
-      const int i = t + k * 256;
-      if (i < HP / 16) ((u32x4*)eis)[i] = te[k];
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < R; ++i) ring[i] = wbase[((int64_t)first_guess * PIECES + i) * 64];
-    __builtin_amdgcn_sched_barrier(0);
-    if (!wide) {
-      for (int i = t; i < BM * E; i += 256) {
-        const int m = i / E, e = i - m * E;
-        const bf16_t r1 = A.routing[(tok0 + (m < last_row ? m : last_row)) * E + e];
-        rs[m * RS + e] = r1;
-        if ((r1 & 0x7fff) != 0) need |= ebits[e];
-      }
-    }
-    if (need != 0u)
-      __hip_atomic_fetch_or((__attribute__((address_space(3))) uint32_t*)cmask_lds, need, __ATOMIC_RELAXED,
-                            __HIP_MEMORY_SCOPE_WORKGROUP);
-    // x fragments: piece kk of row m goes to fragment kk / 2 (K step), slot (m & 31) + 32 * (kk & 1)
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      const int m = w * RW + rb * 8 + r8;
-      u32x4* xdst = (u32x4*)xs + ((m >> 5) * KS1 + (c8l >> 1)) * 64 + (m & 31) + 32 * (c8l & 1);
-#pragma unroll
-      for (int kb = 0; kb < XK; ++kb) xdst[kb * 4 * 64] = xv[rb][kb];
-    }
-  }
-  lds_barrier();
-  // Active chunks as a bit mask, the same in every wave: the chunk loop walks its set bits.
-  uint32_t cmask = __builtin_amdgcn_readfirstlane(*cmask_lds);
-  if constexpr (SPLIT) {
-    const uint32_t below_end = (c_end >= 32) ? ~0u : ((1u << c_end) - 1u);
-    cmask &= below_end & ~((1u << c_begin) - 1u);
-  }
-  const int n_act = __popc(cmask);
-
-  f32x16 acc2[TT][CT];
-#pragma unroll
-  for (int a = 0; a < TT; ++a)
-#pragma unroll
-    for (int b = 0; b < CT; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc2[a][b][r] = 0.f;
-
-  if (n_act > 0) {
-    f32x16 acc1[2][TT];   // GEMM1 accumulators [row-tile][token tile]
-    const int first_chunk = __builtin_ctz(cmask);
-    const bf16x8* cur = wbase + (int64_t)first_chunk * PIECES * 64;
-    if (first_chunk != first_guess) {
-#pragma unroll
-      for (int i = 0; i < R; ++i) ring[i] = cur[i * 64];
-    }
-
-    for (int ci = 0; ci < n_act; ++ci) {
-      const int chunk = __builtin_ctz(cmask);
-      cmask &= cmask - 1;
-      const bf16x8* nxt = (cmask != 0) ? (wbase + (int64_t)__builtin_ctz(cmask) * PIECES * 64) : cur;
-      const int hb0 = chunk * MD_HC + w * 64 + 4 * g;   // first neuron of this lane's accumulator rows, row-tile 0
-
-      // epilogue state, filled and consumed in slices between MFMAs
-      uint2 e_bias[4];     // 4 bf16 biases per accumulator quad
-      uint32_t e_idx[4];   // expert index: one per quad (ED8) or four packed uint8
-      float e_rq[TT][ED8 ? 4 : 16];
-      float e_hv[TT][16];
-      auto epi_load_tables = [&](int rt) __attribute__((always_inline)) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int hb = hb0 + rt * 32 + 8 * q;
-          e_bias[q] = *(const uint2*)(b1s + hb);
-          // Ed multiple of 8: the aligned block of 8 neurons a quad pair covers belongs to one expert, the same for
-          // every lane, so one routing value per (quad, token tile) serves four accumulator rows
-          e_idx[q] = ED8 ? (uint32_t)eis[hb & ~7] : *(const uint32_t*)(eis + hb);
-        }
-      };
-      auto epi_load_routing = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-          const bf16_t* rrow = rs + (tt * 32 + c32) * RS;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            if (ED8) {
-              e_rq[tt][q] = dec16<F16>(rrow[e_idx[q]]);
-            } else {
-#pragma unroll
-              for (int i = 0; i < 4; ++i) e_rq[tt][q * 4 + i] = dec16<F16>(rrow[(e_idx[q] >> (8 * i)) & 0xff]);
-            }
-          }
-        }
-      };
-      auto epi_math = [&](int rt, int q) __attribute__((always_inline)) {
-        const float b0 = dec16<F16>(e_bias[q].x & 0xffffu), b1 = dec16_hi<F16>(e_bias[q].x);
-        const float b2 = dec16<F16>(e_bias[q].y & 0xffffu), b3 = dec16_hi<F16>(e_bias[q].y);
-        const float bias[4] = {b0, b1, b2, b3};
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int r = q * 4 + i;
-            float v = acc1[rt][tt][r] + bias[i];
-            v = (ACT >= 0) ? act_fn<ACT>(v) : apply_act(A.act_rt, v);
-            e_hv[tt][r] = v * (ED8 ? e_rq[tt][q] : e_rq[tt][r]);
-          }
-        }
-      };
-      auto epi_store = [&](int rt) __attribute__((always_inline)) {
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            uint4 pk;
-            pk.x = enc16x2<F16>(e_hv[tt][half * 8 + 0], e_hv[tt][half * 8 + 1]);
-            pk.y = enc16x2<F16>(e_hv[tt][half * 8 + 2], e_hv[tt][half * 8 + 3]);
-            pk.z = enc16x2<F16>(e_hv[tt][half * 8 + 4], e_hv[tt][half * 8 + 5]);
-            pk.w = enc16x2<F16>(e_hv[tt][half * 8 + 6], e_hv[tt][half * 8 + 7]);
-            const int ks2 = (w * 2 + rt) * 2 + half;
-            ((uint4*)hs)[(tt * MD_KS2 + ks2) * 64 + lane] = pk;
-          }
-        }
-      };
-      // GEMM1 of the chunk whose stream starts at `pre` (its W1 fragments; the refills run on into its W2 fragments)
-      auto gemm1 = [&](const bf16x8* pre) __attribute__((always_inline)) {
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-#pragma unroll
-          for (int b = 0; b < TT; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc1[a][b][r] = 0.f;
-        bf16x8 xb[TT];
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) xb[tt] = xs[tt * KS1 * 64 + lane];
-        static_for<0, KS1>([&](auto ks_c) __attribute__((always_inline)) {
-          constexpr int ks = decltype(ks_c)::value;
-          const bf16x8 a0 = ring[(2 * ks) % R];
-          const bf16x8 a1 = ring[(2 * ks + 1) % R];
-          ring[(2 * ks) % R] = pre[(2 * ks + R) * 64];
-          ring[(2 * ks + 1) % R] = pre[(2 * ks + 1 + R) * 64];
-          constexpr int kn = (ks + 1 < KS1) ? ks + 1 : ks;      // x fragments of the next step, read one step ahead
-          bf16x8 nxb[TT];
-#pragma unroll
-          for (int tt = 0; tt < TT; ++tt) nxb[tt] = xs[(tt * KS1 + kn) * 64 + lane];
-#pragma unroll
-          for (int tt = 0; tt < TT; ++tt) {
-            acc1[0][tt] = mfma_32x32x16<F16>(a0, xb[tt], acc1[0][tt]);
-            acc1[1][tt] = mfma_32x32x16<F16>(a1, xb[tt], acc1[1][tt]);
-          }
-#pragma unroll
-          for (int tt = 0; tt < TT; ++tt) xb[tt] = nxb[tt];
-          __builtin_amdgcn_sched_barrier(0);
-        });
-      };
-      // GEMM2 of the current chunk; refills run on into the next chunk's W1 fragments
-      auto gemm2 = [&]() __attribute__((always_inline)) {
-        bf16x8 ha[TT];
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) ha[tt] = hs[tt * MD_KS2 * 64 + lane];
-        static_for<0, MD_KS2>([&](auto j_c) __attribute__((always_inline)) {
-          constexpr int j = decltype(j_c)::value;
-          constexpr int jn = (j + 1 < MD_KS2) ? j + 1 : j;      // h fragments of the next step, read one step ahead
-          bf16x8 nha[TT];
-#pragma unroll
-          for (int tt = 0; tt < TT; ++tt) nha[tt] = hs[(tt * MD_KS2 + jn) * 64 + lane];
-          static_for<0, CT>([&](auto ct_c) __attribute__((always_inline)) {
-            constexpr int ct = decltype(ct_c)::value;
-            constexpr int s = j * CT + ct;      // position in this phase; refill position s + R
-            const bf16x8 b = ring[s % R];
-            ring[s % R] = (s + R < NW2) ? cur[(NW1 + s + R) * 64] : nxt[(s + R - NW2) * 64];
-#pragma unroll
-            for (int tt = 0; tt < TT; ++tt)
-              acc2[tt][ct] = mfma_32x32x16<F16>(ha[tt], b, acc2[tt][ct]);
-          });
-#pragma unroll
-          for (int tt = 0; tt < TT; ++tt) ha[tt] = nha[tt];
-          __builtin_amdgcn_sched_barrier(0);
-        });
-      };
-
-      if (ci == 0) gemm1(cur);
-      lds_barrier();   // every wave has finished reading the previous h tile
-#pragma unroll
-      for (int rt = 0; rt < 2; ++rt) {
-        epi_load_tables(rt);
-        epi_load_routing();
-#pragma unroll
-        for (int q = 0; q < 4; ++q) epi_math(rt, q);
-        epi_store(rt);
-      }
-      lds_barrier();   // h tile complete
-      gemm2();
-      if (ci + 1 < n_act) gemm1(nxt);
-      cur = nxt;
-    }
-  }
-
-  // ---- final epilogue: the accumulators are rounded to bf16 once, AFTER + last_bias (+ x) in float32, and leave as
-  // whole rows.  One pass per 32-token tile: every wave writes its D/4 columns of the pass's rows to LDS as float
-  // [32][D + 4] (bias added on the way: a lane's accumulators share CT columns), then wave w takes rows 8w .. 8w + 7
-  // with the lane mapping of the staging above -- lane (r, c) reads 8 consecutive columns c, c + 8, ... of row r, adds
-  // the residual, rounds, stores 16 bytes; 8 lanes cover 128 contiguous bytes of an output row.  The residual rows
-  // are requested before the pass's LDS traffic; the read loop has no branches and no address arithmetic.
-  {
-    constexpr int OS = D + 4;                       // row stride in floats (+16 bytes: rows shift by 4 banks, so the
-    float* ot = (float*)smem_raw;                   // 8 rows a wave reads at once cover all 32); fits in x + h regions
-    static_assert((size_t)32 * OS * 4 <= (size_t)(2 * KS1 * 64 + 2 * MD_KS2 * 64) * 16, "out staging fits");
-    constexpr int OP = D / 64;                      // 8-column pieces per thread and pass
-    const bool with_bias = !SPLIT && A.last_bias != nullptr;
-    const bool with_res = !SPLIT && A.add_residual != 0;
-    float lb[CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
-      lb[ct] = with_bias ? dec16<F16>(A.last_bias[w * (D / 4) + ct * 32 + c32]) : 0.f;
-    const int row = w * 8 + r8;                     // row of the pass this thread finishes
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-      const int64_t n = tok0 + tt * 32 + row;
-      const bool live = n < N;
-      u32x4 xr[OP];
-      if (with_res) {
-        const u32x4* xrow = (const u32x4*)(A.x + (live ? n : N - 1) * D) + c8l;
-#pragma unroll
-        for (int k = 0; k < OP; ++k) xr[k] = xrow[k * 8];
-      }
-      lds_barrier();                                // previous readers of this LDS region are done
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) {
-        const int col = w * (D / 4) + ct * 32 + c32;
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          ot[(8 * (r / 4) + 4 * g + (r % 4)) * OS + col] = with_bias ? acc2[tt][ct][r] + lb[ct] : acc2[tt][ct][r];
-      }
-      lds_barrier();
-      const float* orow = ot + row * OS + c8l * 8;
-      u32x4 o[OP];
-      float4 pv0[OP], pv1[OP];
-#pragma unroll
-      for (int k = 0; k < OP; ++k) {
-        pv0[k] = *(const float4*)(orow + k * 64);
-        pv1[k] = *(const float4*)(orow + k * 64 + 4);
-        if constexpr (!SPLIT) {
-          float v[8] = {pv0[k].x, pv0[k].y, pv0[k].z, pv0[k].w, pv1[k].x, pv1[k].y, pv1[k].z, pv1[k].w};
-          if (with_res) {
-            const uint32_t xw[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] += (i & 1) ? dec16_hi<F16>(xw[i >> 1]) : dec16<F16>(xw[i >> 1] & 0xffffu);
-          }
-          o[k].x = enc16x2<F16>(v[0], v[1]); o[k].y = enc16x2<F16>(v[2], v[3]);
-          o[k].z = enc16x2<F16>(v[4], v[5]); o[k].w = enc16x2<F16>(v[6], v[7]);
-        }
-      }
-      if (live) {
-        if constexpr (SPLIT) {
-          float* prow = A.partial + ((int64_t)split * A.part_rows + (n - A.part_base)) * D + c8l * 8;
-#pragma unroll
-          for (int k = 0; k < OP; ++k) {
-            *(float4*)(prow + k * 64) = pv0[k];
-            *(float4*)(prow + k * 64 + 4) = pv1[k];
-          }
-        } else {
-          u32x4* grow = (u32x4*)(A.out + n * D) + c8l;
-#pragma unroll
-          for (int k = 0; k < OP; ++k) grow[k * 8] = o[k];
-        }
-      }
-    }
-  }
-}
-
-// Out-of-line copy of the tile routine for the variant below (keeps its register allocation apart from the loop).
-template <int D, int ACT, bool ED8, int TT, bool F16>
-__device__ __attribute__((noinline)) void dense_tile_call(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw) {
-  dense_tile<D, ACT, ED8, TT, false, F16>(A, tok0, smem_raw);
-}
-
-// The same sweep launched as one workgroup per CU that walks the tiles in launch order.  Used where the launch is
-// usually a no-op (the fall-back behind the expert-major path): a skipped call then retires after one round of empty
-// workgroups instead of one per tile.
-template <int D, int ACT, bool ED8, bool F16 = false>
-__global__ __launch_bounds__(256, 1) void experts_mfma_dense_walk_kernel(const DenseArgs A) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
-  for (int b = blockIdx.x; b < A.n_tiles; b += gridDim.x) {
-    if (b < A.n_full)
-      dense_tile_call<D, ACT, ED8, 2, F16>(A, (int64_t)b * 64, smem_raw);
-    else
-      dense_tile_call<D, ACT, ED8, 1, F16>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
-    __syncthreads();   // the next tile's staging overwrites the LDS the final epilogue just read
-  }
-}
-
-// Workgroups [0, n_full) take tiles of 64 tokens.  The tokens left over after the last full round of the machine go to
-// tiles of 32; if those would still leave most CUs idle, each of them is dealt to csplit workgroups by chunk ranges,
-// which leave float32 sums in A.partial for the finishing kernel.
-template <int D, int ACT, bool ED8, bool F16 = false>
-__global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
-  const int b = blockIdx.x;
-  if (b < A.n_full) {
-    dense_tile<D, ACT, ED8, 2, false, F16>(A, (int64_t)b * 64, smem_raw);
-  } else if (A.csplit <= 1) {
-    dense_tile<D, ACT, ED8, 1, false, F16>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
-  } else {
-    const int idx = b - A.n_full;
-    const int tile = idx / A.csplit, split = idx % A.csplit;
-    const int c_begin = split * A.chunks_per_split;
-    dense_tile<D, ACT, ED8, 1, true, F16>(A, (int64_t)A.n_full * 64 + (int64_t)tile * 32, smem_raw, c_begin,
-                                     c_begin + A.chunks_per_split, split);
-  }
-}
-
 int device_cu_count() {
   static const int n = [] {
     int dev = 0, cus = 0;
@@ -725,18 +277,14 @@ int device_cu_count() {
   return n;
 }
 
-struct DenseTiling {
-  int64_t n_full, n_half;   // tiles of 64 and of 32 tokens
-  int csplit, per;          // workgroups per tile of 32 and chunks per workgroup (1, n_chunks: not split)
-  int64_t part_base, part_rows;   // tokens covered by split tiles
-};
 
 // Tiles of 64 tokens fill whole rounds of one workgroup per CU.  When the last round would be at most half full its
 // tokens go to tiles of 32 instead, and if those still leave CUs idle each of them is dealt to several workgroups by
 // chunk ranges -- so the tail of the launch (or, with few tokens, the whole launch) spreads over the machine.
-static DenseTiling dense_tiling(const d2dmoe_shape& sh, bool allow_split) {
+DenseTiling dense_tiling(const d2dmoe_shape& sh, bool allow_split) {
   const int cus = device_cu_count();
-  const int n_chunks = (sh.n_experts * sh.expert_dim + MD_HC - 1) / MD_HC;
+  const int hc = sweep_chunk(sh.d_model);
+  const int n_chunks = (sh.n_experts * sh.expert_dim + hc - 1) / hc;
   DenseTiling T;
   const int64_t t64 = cdiv64(sh.n_tokens, 64);
   const int64_t leftover = t64 % cus;
@@ -767,59 +315,10 @@ size_t mfma_dense_workspace_bytes(const d2dmoe_shape& sh) {
   return T.csplit > 1 ? (size_t)T.csplit * T.part_rows * sh.d_model * 4 : 0;
 }
 
-template <int D, int ACT, bool ED8, bool F16>
-static hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
-                                   const void* last_bias, void* out, const int* skip_flag, void* workspace,
-                                   size_t workspace_bytes, hipStream_t s) {
-  const PackedLayout L = packed_layout(sh);
-  const char* base = (const char*)packed;
-  const size_t lds = dense_lds_bytes(sh);
-  if (lds > 160 * 1024) return hipErrorInvalidValue;
-  const int cus = device_cu_count();
-  // Behind the expert-major path the launch is usually a no-op: one workgroup per CU walks the tiles, so a skipped call
-  // retires after one round of empty workgroups.  With big experts (the reference's benchmark shape, swept over
-  // densities) the fall-back runs as often as not, and the walk costs 15 % per tile: the ordinary grid there.
-  const bool walk = skip_flag != nullptr && sh.expert_dim <= 64;
-  const bool allow_split = !walk && workspace != nullptr && workspace_bytes >= mfma_dense_workspace_bytes(sh);
-  const DenseTiling T = dense_tiling(sh, allow_split);
-  auto kern = walk ? experts_mfma_dense_walk_kernel<D, ACT, ED8, F16> : experts_mfma_dense_kernel<D, ACT, ED8, F16>;
-  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) return e;
-  DenseArgs A;
-  A.x = (const bf16_t*)x; A.routing = (const bf16_t*)routing; A.wp = (const bf16x8*)(base + L.w_off);
-  A.b1p = (const bf16_t*)(base + L.b1_off); A.eidx = (const uint8_t*)(base + L.eidx_off);
-  A.last_bias = (const bf16_t*)last_bias; A.out = (bf16_t*)out; A.N = sh.n_tokens; A.E = sh.n_experts; A.expert_dim = sh.expert_dim;
-  A.n_chunks = L.n_chunks; A.hidden = L.hidden; A.act_rt = sh.activation; A.add_residual = sh.add_residual;
-  A.n_full = (int)T.n_full; A.n_tiles = (int)(T.n_full + T.n_half); A.skip_flag = skip_flag;
-  A.partial = (float*)workspace; A.csplit = T.csplit; A.chunks_per_split = T.per;
-  A.part_base = T.part_base; A.part_rows = T.part_rows;
-  int64_t grid = T.n_full + T.n_half * T.csplit;
-  if (walk && A.n_tiles > cus) grid = cus;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, s, A);
-  e = hipGetLastError();
-  if (e != hipSuccess || T.csplit <= 1) return e;
-  return launch_sum_partials(A.partial, last_bias, (const bf16_t*)x + T.part_base * sh.d_model,
-                             (bf16_t*)out + T.part_base * sh.d_model, T.part_rows, sh.d_model, T.csplit, sh.add_residual, s,
-                             sh.dtype, skip_flag);
-}
-
-template <int D, int ACT>
-static hipError_t launch_dense_act(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
-                                   const void* last_bias, void* out, const int* skip_flag, void* workspace,
-                                   size_t workspace_bytes, hipStream_t s) {
-  if (sh.dtype == D2DMOE_F16) {
-    if (sh.expert_dim % 8 == 0)
-      return launch_dense_cfg<D, ACT, true, true>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
-    return launch_dense_cfg<D, ACT, false, true>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
-  }
-  if (sh.expert_dim % 8 == 0)
-    return launch_dense_cfg<D, ACT, true, false>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
-  return launch_dense_cfg<D, ACT, false, false>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
-}
-
 hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                              const void* last_bias, void* out, const int* skip_flag, void* workspace, size_t workspace_bytes,
                              hipStream_t s) {
+  if (sh.d_model != 768) return launch_mfma_dense_wide(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);
   switch (sh.activation) {
     case D2DMOE_ACT_RELU:
       return launch_dense_act<768, D2DMOE_ACT_RELU>(sh, x, routing, packed, last_bias, out, skip_flag, workspace, workspace_bytes, s);

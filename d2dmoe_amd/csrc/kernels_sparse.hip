@@ -58,7 +58,7 @@ static SparseWorkspace sparse_workspace(const d2dmoe_shape& sh, int max_mean_k) 
   W.token_idx = take((size_t)W.cap * 4);
   W.pair_dst = take((size_t)W.cap * 4);
   size_t ybytes = (size_t)W.cap * sh.d_model * 2;
-  if (sh.gated || !mfma_dense_supported(sh)) {   // where the fall-back is the tiled products, they work in the same region
+  if (!mfma_sparse_falls_back_to_sweep(sh)) {   // where the fall-back is the tiled products, they work in the same region
     const size_t g = mfma_gemm_workspace_bytes(sh);
     if (g > ybytes) ybytes = g;
   }

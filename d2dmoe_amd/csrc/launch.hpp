@@ -40,6 +40,7 @@ hipError_t launch_experts_generic(const d2dmoe_shape& sh, const void* x, const v
 
 // ---- bf16 MFMA kernels (kernels_mfma.hip) ----
 bool mfma_dense_supported(const d2dmoe_shape& sh);
+bool mfma_sparse_falls_back_to_sweep(const d2dmoe_shape& sh);   // else: to the tiled products
 bool mfma_router_supported(const d2dmoe_shape& sh);
 size_t mfma_packed_bytes(const d2dmoe_shape& sh);
 unsigned mfma_packed_sections(const d2dmoe_shape& sh);   // D2DMOE_SECTION_* bits of the buffer packed for sh
@@ -58,6 +59,10 @@ size_t mfma_dense_workspace_bytes(const d2dmoe_shape& sh);
 hipError_t launch_mfma_dense(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
                              const void* last_bias, void* out, const int* skip_flag, void* workspace, size_t workspace_bytes,
                              hipStream_t s);
+// the D = 1024 instances of the same sweep (kernels_dense_wide.hip)
+hipError_t launch_mfma_dense_wide(const d2dmoe_shape& sh, const void* x, const void* routing, const void* packed,
+                                  const void* last_bias, void* out, const int* skip_flag, void* workspace,
+                                  size_t workspace_bytes, hipStream_t s);
 // out = round(sum over splits (ascending) of partial[split] + last_bias (+ x)); partial is [n_splits][N][D] float32
 hipError_t launch_sum_partials(const float* partial, const void* last_bias, const void* x, void* out, int64_t N, int D,
                                int n_splits, int add_residual, hipStream_t s, int dtype = D2DMOE_BF16, const int* skip_flag = nullptr);

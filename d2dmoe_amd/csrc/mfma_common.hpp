@@ -18,7 +18,9 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // 16 raw byte
 
 constexpr size_t PACKED_HEADER_BYTES = 256;   // a packed buffer starts with its d2dmoe_packed_desc (64 bytes, padded)
 constexpr int MD_BM = 64;       // tokens per workgroup of the dense sweep
-constexpr int MD_HC = 256;      // hidden neurons per chunk (4 waves x 64)
+constexpr int MD_HC = 256;      // hidden neurons per chunk (4 waves x 64) at D = 768
+// ... and at any width the sweep is built for: 128 where the x tile leaves no room for a 256-neuron h tile
+__host__ __device__ constexpr int sweep_chunk(int d_model) { return d_model <= 768 ? 256 : 128; }
 constexpr int MD_WAVES = 4;
 constexpr int MD_KS2 = MD_HC / 16;  // K=16 steps of the second GEMM per chunk
 constexpr int MD_MAX_CHUNKS = 32;   // chunks per layer the dense sweep stages tables for (hidden <= 8192)
@@ -33,8 +35,8 @@ constexpr int MID_HROW = 32;        // hidden values kept per routed pair (exper
 // Sections of the buffer d2dmoe_pack_weights writes.  A section is present when its kernel covers the shape.
 struct PackedLayout {
   int hidden;      // E * Ed
-  int n_chunks;    // ceil(hidden / MD_HC)
-  int hidden_pad;  // n_chunks * MD_HC
+  int n_chunks;    // ceil(hidden / sweep_chunk(D))
+  int hidden_pad;  // n_chunks * sweep_chunk(D)
   int pieces;      // weight fragments per (wave, chunk) of the dense stream
   int nt;          // 32-neuron row tiles per expert in the expert-major section: ceil(Ed / 32)
   size_t w_off, b1_off, eidx_off;        // dense sweep: weight stream, bias (bf16), expert index per neuron (uint8)

@@ -231,6 +231,75 @@ def test_experts_mfma_dense_activations_bias_residual_weights(act):
     assert torch.equal(got, p['last_bias'].expand(200, -1))
 
 
+@pytest.mark.parametrize('N,E,Ed,density,act', [(197, 128, 32, 0.8, 'gelu'), (197, 128, 32, 0.02, 'gelu'), (1600, 128, 32, 0.79, 'gelu'),
+                                                (64, 64, 64, 1.0, 'relu'), (65, 128, 24, 0.5, 'relu'), (1, 128, 32, 0.5, 'gelu'),
+                                                (300, 24, 128, 0.5, 'relu'), (130, 100, 30, 0.5, 'tanh'), (100, 7, 5, 0.5, 'relu'),
+                                                (96, 160, 16, 0.3, 'leaky_relu'), (4200, 16, 256, 0.6, 'gelu')])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_experts_mfma_dense_at_width_1024(N, E, Ed, density, act, dtype):
+    """The fused sweep at D = 1024 (GPT-2 medium, BERT-large, ViT-L; hidden size up to 4096): chunks of 128 neurons,
+    routing values fetched from global memory one chunk ahead, first product accumulated in vector registers.  Against
+    the float64 oracle, the tiled products (the path these widths took before) and the generic kernel; nothing routed,
+    weighted routing with residual, run-to-run bits; the last shape (experts of 256 neurons) has no sweep and must
+    still take the tiled products under AUTO."""
+    _say('experts mfma D=1024', N, E, Ed, density, act, dtype)
+    tol = H.TOL_BF16 if dtype == torch.bfloat16 else 4e-3
+    x, routing, p = H.random_case(N, 1024, E, Ed, 8, seed=N + E, dtype=dtype, density=density)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, 1024, E, Ed, 0, _ops()._dtype_code(x), act)
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, None, None)
+    assert packed is not None
+    want = _experts_want(x, routing, p, act)
+    if Ed > 128:
+        got = _experts_got(x, routing, p, act, path='auto', packed=packed)
+        assert torch.equal(got, _experts_got(x, routing, p, act, path='mfma_gemm', packed=packed))
+        assert H.rel_err(got, want) < tol
+        return
+    got = _experts_got(x, routing, p, act, path='mfma_dense', packed=packed)
+    assert H.rel_err(got, want) < tol
+    assert H.elem_err(got, want) < tol
+    assert H.rel_err(got, _experts_got(x, routing, p, act, path='mfma_gemm', packed=packed)) < (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    if N > 16:
+        assert torch.equal(got, _experts_got(x, routing, p, act, path='auto', packed=packed))
+    assert torch.equal(got, _experts_got(x, routing, p, act, path='mfma_dense', packed=packed))
+    zero = _experts_got(x, torch.zeros_like(routing), p, act, path='mfma_dense', packed=packed)
+    assert torch.equal(zero, p['last_bias'].expand(N, -1))
+    g = torch.Generator().manual_seed(5)
+    weights = (routing.float() * (torch.rand(N, E, generator=g) + 0.5)).to(dtype)
+    got = _experts_got(x, weights, p, act, residual=True, path='mfma_dense', packed=packed)
+    assert H.rel_err(got, _experts_want(x, weights, p, act, True)) < tol
+    q = {k: v for k, v in p.items() if k not in ('b1', 'last_bias')}
+    dq = H.to_dev(q, DEV)
+    packed_q = _ops().pack_weights(sh, dq['w1'], None, dq['w2'], None, None, None)
+    got = _experts_got(x, routing, q, act, path='mfma_dense', packed=packed_q)
+    assert H.rel_err(got, _experts_want(x, routing, q, act)) < tol
+
+
+def test_experts_mfma_dense_at_width_1024_full_size_properties():
+    """GPT-2-medium layer at 16 384 tokens (128 experts x 32, GELU): oracle on a slice of rows, the tiled products on all
+    rows, two runs give identical bits, and permuting the tokens permutes the output rows bit for bit."""
+    N = 16384
+    x, routing, p = H.random_case(N, 1024, 128, 32, 8, seed=41, dtype=torch.bfloat16, density=0.79)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, 1024, 128, 32, 0, 1, 'gelu')
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, None, None)
+    xg, rg = x.to(DEV), routing.to(DEV)
+    lb = d['last_bias'].view(-1)
+    a = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, 'gelu', True, 'mfma_dense', packed)
+    b = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, 'gelu', True, 'mfma_dense', packed)
+    assert torch.equal(a, b)
+    t = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, 'gelu', True, 'mfma_gemm', packed)
+    assert H.rel_err(a, t) < 1e-2
+    perm = torch.randperm(N, generator=torch.Generator().manual_seed(9)).to(DEV)
+    c = _ops().experts(xg[perm].contiguous(), rg[perm].contiguous(), d['w1'], d['b1'], d['w2'], None, lb, 'gelu', True,
+                       'mfma_dense', packed)
+    assert torch.equal(c, a[perm])
+    rows = torch.cat([torch.arange(0, 128), torch.arange(8000, 8064), torch.arange(N - 64, N)])
+    want = _experts_want(x[rows], routing[rows], p, 'gelu', True)
+    assert H.rel_err(a.cpu()[rows], want) < H.TOL_BF16
+    assert H.elem_err(a.cpu()[rows], want) < H.TOL_BF16
+
+
 def test_experts_mfma_dense_full_size_properties():
     """50432 tokens (the headline workload): oracle on a slice of rows, the generic HIP kernel on all rows, and
     determinism (two runs give identical bits)."""
@@ -695,9 +764,9 @@ def test_decode_path_matches_oracle(N, D, E, Ed, W, gated, act):
 @pytest.mark.parametrize('D,E,Ed,W,gated,act', [(2048, 256, 64, 256, True, 'gelu_tanh'), (768, 128, 24, 128, False, 'relu')])
 @pytest.mark.parametrize('tau', [0.9, 0.1])
 def test_small_batch_layer_equals_staged_calls(N, D, E, Ed, W, gated, act, tau):
-    """d2dmoe_forward runs a layer of at most 16 tokens as three launches (first router layer beside the experts' first
-    layer, selection inside the output kernel).  Norms, routing, counts and outputs must be the bits the stand-alone
-    entry points produce: router -> select -> experts."""
+    """d2dmoe_forward runs a layer of at most 16 tokens as two launches (first router layer beside the experts' first
+    layer; second router layer and selection inside the output kernel).  Norms, routing, counts and outputs must be the
+    bits the stand-alone entry points produce: router -> select -> experts."""
     _say('small batch layer vs staged', N, D, E, gated, tau)
     x, _, p = H.random_case(N, D, E, Ed, W, seed=3 * N + E, dtype=torch.bfloat16, gated=gated, bias=not gated)
     d = H.to_dev(p, DEV)
@@ -716,6 +785,45 @@ def test_small_batch_layer_equals_staged_calls(N, D, E, Ed, W, gated, act, tau):
     out2 = _experts_got(x, routing2.cpu(), p, act, residual=True, path='mfma_decode', packed=packed)
     assert torch.equal(out.cpu(), out2)
     assert torch.equal(routing.cpu(), O.gate_dynk_max(norms.cpu(), tau))
+
+
+@pytest.mark.parametrize('N,D,E,Ed,W,gated,act', [(16, 2048, 256, 64, 256, True, 'gelu_tanh'), (3, 2048, 256, 64, 256, True, 'gelu_tanh'),
+                                                  (16, 768, 128, 24, 128, False, 'relu')])
+def test_small_batch_layer_back_to_back_calls_keep_their_bits(N, D, E, Ed, W, gated, act):
+    """The output kernel's workgroups each sum a range of experts and the last to arrive adds the ranges; the arrival
+    counters and the partial sums live in the workspace and are reused by the next call.  150 calls on two alternating
+    inputs with no host synchronisation in between: every result must be the bits of the first call on that input (a sum
+    that picked up another call's partials, or a counter left over, would show)."""
+    _say('small batch back to back', N, D, E, gated)
+    xa, _, p = H.random_case(N, D, E, Ed, W, seed=11 + N, dtype=torch.bfloat16, gated=gated, bias=not gated)
+    xb = torch.roll(xa, 1, dims=1).contiguous()
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, W, 1, act, gated=gated)
+    if gated:
+        packed = _ops().pack_weights(sh, d['w_gate'], None, d['w_down'], d['w_up'], d['router_w1'], d['router_w2'])
+    else:
+        packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, d['router_w1'], d['router_w2'])
+    lb = d['last_bias'].view(-1) if 'last_bias' in d else None
+
+    def layer(x):
+        if gated:
+            return _ops().forward(x, d['router_w1'], d['router_w2'], 0.1, d['w_gate'], None, d['w_down'], d['w_up'], lb, act,
+                                  True, None, True, True, 'auto', packed)
+        return _ops().forward(x, d['router_w1'], d['router_w2'], 0.1, d['w1'], d['b1'], d['w2'], None, lb, act, True, None,
+                              True, True, 'auto', packed)
+
+    xs = {'a': xa.to(DEV), 'b': xb.to(DEV)}
+    first = {name: layer(x) for name, x in xs.items()}
+    torch.cuda.synchronize()
+    assert not torch.equal(first['a'][0], first['b'][0])
+    for name, x in (('a', xa), ('b', xb)):
+        want = O.layer_from_routing(x.double(), O.upcast(p), first[name][1].cpu().double(), act, 'all', True)
+        assert H.rel_err(first[name][0].cpu(), want) < H.TOL_BF16
+    got = [('ab'[i & 1], layer(xs['ab'[i & 1]])) for i in range(150)]
+    torch.cuda.synchronize()
+    for name, res in got:
+        for a, b in zip(res, first[name]):
+            assert torch.equal(a, b)
 
 
 # =================================================================== tiled products (gated, or ungated at other widths) ===
@@ -743,7 +851,7 @@ def test_tiled_products_path_matches_oracle(N, D, E, Ed, W, act, gated, dtype):
     rows = torch.arange(N) if N * E * D * Ed < 2e10 else torch.cat([torch.arange(40), torch.arange(N - 40, N)])
     got = _experts_got(x, routing, p, act, path='mfma_gemm', packed=packed)
     assert H.rel_err(got[rows], _experts_want(x[rows], routing[rows], p, act)) < tol
-    if D != 768 or dtype == torch.float32:   # AUTO picks it for N > 16 unless the fused sweep covers the shape
+    if dtype == torch.float32 or gated or D not in (768, 1024):   # AUTO picks it for N > 16 unless the fused sweep covers the shape
         assert torch.equal(got, _experts_got(x, routing, p, act, path='auto', packed=packed))
     if N <= 1100 and D <= 1280:
         assert H.rel_err(got, _experts_got(x, routing, p, act, path='generic')) < (1e-2 if dtype == torch.bfloat16 else 1e-5)
