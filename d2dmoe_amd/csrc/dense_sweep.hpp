@@ -51,18 +51,12 @@ template <int D> struct SweepCfg {
   static constexpr bool VACC = (D > 768);
 };
 
-// A wave's stream of 16-byte-per-lane fragments, indexed in units of 16 bytes.  BUFFER: read with buffer loads -- the
-// stream's base sits in a resource descriptor (scalar registers), the position in the stream is a scalar byte offset
-// plus an immediate, and the lane's 16 bytes are ONE vector register that never changes: the walk through the stream
-// costs no vector arithmetic and no vector registers for addresses (as plain pointers, each group of four fragments
-// needs a 64-bit vector add and a register pair).
-template <bool BUFFER> struct StreamPtr;
-template <> struct StreamPtr<false> {
-  const bf16x8* p;
-  __device__ __forceinline__ bf16x8 operator[](int64_t i) const { return p[i]; }
-  __device__ __forceinline__ StreamPtr operator+(int64_t n) const { return {p + n}; }
-};
-template <> struct StreamPtr<true> {
+// A wave's stream of 16-byte-per-lane fragments, indexed in units of 16 bytes and read with buffer loads: the stream's
+// base sits in a resource descriptor (scalar registers), the position in the stream is a scalar byte offset, and the
+// lane's 16 bytes are ONE vector register that never changes -- the walk through the stream costs no vector
+// arithmetic and no vector registers for addresses (with plain pointers each group of four fragments takes a 64-bit
+// vector add and a register pair; measured at D = 768: 1.6 % of the kernel).
+struct StreamPtr {
   __amdgpu_buffer_rsrc_t rsrc; uint32_t loff; int soff;   // soff: bytes, the same in all lanes
   __device__ __forceinline__ bf16x8 operator[](int i) const {
     // (the whole position goes into the scalar offset: one scalar add per load, and the vector offset stays one register)
@@ -110,8 +104,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
 
   const int t = threadIdx.x;
   const int lane = t & 63;
-  // (wave index: known to be the same in all lanes where the stream below is addressed from a scalar base)
-  const int w = SweepCfg<D>::VACC ? __builtin_amdgcn_readfirstlane(t >> 6) : (t >> 6);
+  const int w = __builtin_amdgcn_readfirstlane(t >> 6);   // wave index, known to the compiler to be the same in all lanes
   const int g = lane >> 5, c32 = lane & 31;
   constexpr int NW1 = RT * KS1;        // W1 fragments per (wave, chunk)
   constexpr int NW2 = KS2 * CT;        // W2 fragments per (wave, chunk)
@@ -131,12 +124,10 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   // handful of lane values -- this part of the kernel is bound by instruction issue, not by memory.
   // Rows past the end of the batch are read from the last row instead (rows never mix, and their results are not
   // stored).
-  typedef StreamPtr<VACC> Stream;
-  Stream wbase;                                                               // this wave's stream
-  if constexpr (VACC)   // (raw buffer of 32-bit words covering this wave's part of the packed stream)
-    wbase = Stream{__builtin_amdgcn_make_buffer_rsrc((void*)(A.wp + (int64_t)w * n_chunks * PIECES * 64), 0,
-                                                     n_chunks * PIECES * 1024, 0x00020000), (uint32_t)lane * 16u, 0};
-  else wbase = Stream{A.wp + (int64_t)w * n_chunks * PIECES * 64 + lane};
+  typedef StreamPtr Stream;
+  // this wave's stream: a raw buffer of 32-bit words covering the wave's part of the packed weights
+  const Stream wbase{__builtin_amdgcn_make_buffer_rsrc((void*)(A.wp + (int64_t)w * n_chunks * PIECES * 64), 0,
+                                                       n_chunks * PIECES * 1024, 0x00020000), (uint32_t)lane * 16u, 0};
   bf16x8 ring[R];
   const int first_guess = SPLIT ? c_begin : 0;
   const int r8 = lane & 7, c8l = lane >> 3;
