@@ -331,7 +331,7 @@ static int experts_impl(const d2dmoe_shape* shape, const void* x, const void* ro
     case D2DMOE_PATH_MFMA_SPARSE: {
       // expert-major when the routed pairs fit the provisioned capacity, else the dense sweep: decided on the device
       if (!mfma_sparse_supported(sh)) return D2DMOE_E_UNSUPPORTED;
-      // the fall-back: the dense sweep (ungated, D = 768), else the tiled products
+      // the fall-back: the dense sweep (ungated, D = 768 or 1024, up to 256 experts), else the tiled products
       const bool fb_gemm = !mfma_sparse_falls_back_to_sweep(sh);
       if (fb_gemm && !mfma_gemm_supported(sh)) return D2DMOE_E_UNSUPPORTED;
       if (!packed) return D2DMOE_E_NULL;
@@ -474,16 +474,16 @@ int d2dmoe_forward(const d2dmoe_shape* shape, const void* x, const void* router_
   }
   // A high threshold fraction keeps few experts per token: take the expert-major path (it falls back to the dense
   // sweep on the device if the routing turns out dense after all).
-  // (gated experts, and ungated ones at the widths without a fused sweep: from a lower fraction on -- their dense
-  // alternative costs several times the expert-major path at few experts per token and the device-side switch is cheap
-  // next to it;
+  // (gated experts, and ungated ones at widths other than 768: from a lower fraction on -- their capacity is 12 or 32
+  // routed experts per token instead of 8, their dense alternative costs several times the expert-major path at few
+  // experts per token, and the device-side switch is cheap next to it;
   // and with at most 128 tokens whatever the fraction -- the layer is bound by the weight stream there, which the tiled
   // products pay for with whole 256-token tiles;
   // big ungated experts from a lower fraction on, and whatever the fraction when the norms are handed in -- the
   // reference benchmark's Bernoulli override, where the fraction says nothing about the density: the dense sweep
   // cannot skip at their granularity)
   if (path == D2DMOE_PATH_AUTO && sh.n_tokens > (sh.gated && mfma_decode_supported(sh) ? 48 : 16) && packed != nullptr &&
-      (thr_scale >= (!mfma_sparse_falls_back_to_sweep(sh) ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128) ||
+      (thr_scale >= ((sh.d_model != 768 || !mfma_sparse_falls_back_to_sweep(sh)) ? 0.5f : 0.75f) || (sh.gated && sh.n_tokens <= 128) ||
        (!sh.gated && sh.expert_dim > 64 && (norms_in != nullptr || thr_scale >= 0.5f))) &&
       mfma_sparse_supported(sh) &&
       (mfma_sparse_falls_back_to_sweep(sh) || mfma_gemm_supported(sh)))

@@ -548,10 +548,28 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   }
 }
 
+// Values that are the same in every lane but reach a device function in vector registers (its arguments do): moved to
+// scalar registers, so that what is derived from them -- buffer resources, loop bounds, branch conditions -- is scalar
+// again.
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ int64_t uniform(int64_t v) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+template <typename T> __device__ __forceinline__ T* uniform(T* p) { return (T*)(uintptr_t)uniform((int64_t)(uintptr_t)p); }
+
 // Out-of-line copy of the tile routine for the variant below (keeps its register allocation apart from the loop).
 template <int D, int ACT, bool ED8, int TT, bool F16>
 __device__ __attribute__((noinline)) void dense_tile_call(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw) {
-  dense_tile<D, ACT, ED8, TT, false, F16>(A, tok0, smem_raw);
+  DenseArgs U;
+  U.x = uniform(A.x); U.routing = uniform(A.routing); U.wp = uniform(A.wp); U.b1p = uniform(A.b1p); U.eidx = uniform(A.eidx);
+  U.last_bias = uniform(A.last_bias); U.out = uniform(A.out); U.skip_flag = nullptr; U.partial = nullptr;
+  U.csplit = 1; U.chunks_per_split = 0; U.part_base = 0; U.part_rows = 0;
+  U.N = uniform(A.N); U.E = uniform(A.E); U.expert_dim = uniform(A.expert_dim); U.n_chunks = uniform(A.n_chunks);
+  U.hidden = uniform(A.hidden); U.act_rt = uniform(A.act_rt); U.add_residual = uniform(A.add_residual);
+  U.n_full = 0; U.n_tiles = 0;
+  dense_tile<D, ACT, ED8, TT, false, F16>(U, uniform(tok0), smem_raw);
 }
 
 // The same sweep launched as one workgroup per CU that walks the tiles in launch order.  Used where the launch is

@@ -38,9 +38,8 @@ bool mfma_dense_supported(const d2dmoe_shape& sh) {
   return dense_lds_bytes(sh) <= 160 * 1024;      // x tile + h tile (+ routing tile) + bias/expert-index tables
 }
 
-// The expert-major path hands over to the sweep on the device where the sweep is the faster dense alternative it was
-// measured against (D = 768); at the other widths to the tiled products.
-bool mfma_sparse_falls_back_to_sweep(const d2dmoe_shape& sh) { return !sh.gated && sh.d_model == 768 && mfma_dense_supported(sh); }
+// The expert-major path hands over to the sweep on the device wherever there is one; else to the tiled products.
+bool mfma_sparse_falls_back_to_sweep(const d2dmoe_shape& sh) { return !sh.gated && mfma_dense_supported(sh); }
 
 // The fused router+select kernel covers the D2DMoE router: bf16, depth 2, ReLU hidden / abs output activation,
 // width and expert count both 128 or both 256, D a multiple of 64.

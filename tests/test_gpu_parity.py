@@ -239,9 +239,8 @@ def test_experts_mfma_dense_activations_bias_residual_weights(act):
 def test_experts_mfma_dense_at_width_1024(N, E, Ed, density, act, dtype):
     """The fused sweep at D = 1024 (GPT-2 medium, BERT-large, ViT-L; hidden size up to 4096): chunks of 128 neurons,
     routing values fetched from global memory one chunk ahead, first product accumulated in vector registers.  Against
-    the float64 oracle, the tiled products (the path these widths took before) and the generic kernel; nothing routed,
-    weighted routing with residual, run-to-run bits; the last shape (experts of 256 neurons) has no sweep and must
-    still take the tiled products under AUTO."""
+    the float64 oracle and the tiled products; nothing routed, weighted routing with residual, no biases, run-to-run
+    bits; the last shape (experts of 256 neurons) has no sweep and must still take the tiled products under AUTO."""
     _say('experts mfma D=1024', N, E, Ed, density, act, dtype)
     tol = H.TOL_BF16 if dtype == torch.bfloat16 else 4e-3
     x, routing, p = H.random_case(N, 1024, E, Ed, 8, seed=N + E, dtype=dtype, density=density)
@@ -273,6 +272,34 @@ def test_experts_mfma_dense_at_width_1024(N, E, Ed, density, act, dtype):
     packed_q = _ops().pack_weights(sh, dq['w1'], None, dq['w2'], None, None, None)
     got = _experts_got(x, routing, q, act, path='mfma_dense', packed=packed_q)
     assert H.rel_err(got, _experts_want(x, routing, q, act)) < tol
+
+
+@pytest.mark.parametrize('E,Ed,act,dtype', [(128, 32, 'gelu', torch.float16), (128, 30, 'relu', torch.bfloat16),
+                                            (100, 30, 'gelu', torch.float16), (128, 24, 'tanh', torch.bfloat16),
+                                            (64, 64, 'relu', torch.float16), (96, 20, 'leaky_relu', torch.float16)])
+def test_experts_mfma_dense_at_width_1024_whole_tiles(E, Ed, act, dtype):
+    """8320 tokens are 130 whole tiles of 64: the two-token-tile form of every instance of the D = 1024 sweep (storage type
+    x compiled-in or run-time activation x expert sizes that are / are not multiples of 8), against the tiled products on
+    all rows and the float64 oracle on a slice; and the same instances as the expert-major path's device-side fall-back
+    (one workgroup per CU walking the tiles), which must give the same bits."""
+    _say('experts mfma D=1024 whole tiles', E, Ed, act, dtype)
+    N = 8320
+    tol = H.TOL_BF16 if dtype == torch.bfloat16 else 4e-3
+    x, routing, p = H.random_case(N, 1024, E, Ed, 8, seed=E + Ed, dtype=dtype, density=0.7)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, 1024, E, Ed, 0, _ops()._dtype_code(x), act)
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, None, None)
+    xg, rg, lb = x.to(DEV), routing.to(DEV), d['last_bias'].view(-1)
+    a = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, act, True, 'mfma_dense', packed)
+    t = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, act, True, 'mfma_gemm', packed)
+    assert H.rel_err(a, t) < (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    rows = torch.cat([torch.arange(0, 96), torch.arange(N - 64, N)])
+    want = _experts_want(x[rows], routing[rows], p, act, True)
+    assert H.rel_err(a.cpu()[rows], want) < tol
+    assert H.elem_err(a.cpu()[rows], want) < tol
+    if Ed <= 64:   # the expert-major path exists; 0.7 * E experts per token are far beyond its capacity
+        f = _ops().experts(xg, rg, d['w1'], d['b1'], d['w2'], None, lb, act, True, 'mfma_sparse', packed)
+        assert torch.equal(f, a)
 
 
 def test_experts_mfma_dense_at_width_1024_full_size_properties():
