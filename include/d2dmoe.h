@@ -70,12 +70,14 @@ enum {
 enum {
   D2DMOE_PATH_AUTO = 0,       /* MFMA kernels when the shape and dtype have one, else the generic kernel */
   D2DMOE_PATH_GENERIC = 1,    /* token-tile-major scalar-FMA kernel: any shape, f32, bf16 or f16 storage, f32 math */
-  D2DMOE_PATH_MFMA_DENSE = 2, /* bf16 or f16 MFMA, token-tile-major, masked dense sweep over all experts */
+  D2DMOE_PATH_MFMA_DENSE = 2, /* bf16 or f16 MFMA, token-tile-major, masked dense sweep over all experts: ungated experts at
+                                 D = 768 (hidden size up to 8192) or D = 1024 (up to 4096), at most 256 experts */
   D2DMOE_PATH_MFMA_SPARSE = 3, /* bf16 or f16 MFMA, expert-major over the permutation, then ordered combine; taken when at most
                                  8 experts per token are routed on average (checked on the device), else the dense sweep runs.  Ungated experts at D = 768 (also D = 1024 with at most 64 neurons and D = 1280 with at
-                                 most 32: up to 12 / 6 experts per token, tiled products as fall-back).  Gated experts at D = 2048 with at most 64
+                                 most 32: up to 12 / 6 experts per token; fall-back: the dense sweep at D = 1024, the tiled
+                                 products at D = 1280 and wherever the sweep does not cover the layer).  Gated experts at D = 2048 with at most 64
                                  neurons: up to 32 experts per token (8 beyond 16 384 tokens), else the tiled products
-                                 run.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 (gated: >= 0.5); for ungated
+                                 run.  d2dmoe_forward picks it under AUTO when thr_scale >= 0.75 (gated, or D other than 768: >= 0.5); for ungated
                                  experts of more than 64 neurons AUTO picks it in d2dmoe_experts, and in d2dmoe_forward when norms_in is
                                  given or thr_scale >= 0.5 */
   D2DMOE_PATH_MFMA_DECODE = 4, /* bf16 or f16 MFMA for a handful of tokens: per pass of 16 tokens one workgroup per expert streams
@@ -217,7 +219,7 @@ int d2dmoe_experts(const d2dmoe_shape* shape, const void* x, const void* routing
                    int32_t path, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Bytes of the derived weight buffer for the MFMA kernels (0 when `shape` has no MFMA kernel).  The buffer has one
- * section per kernel family that covers the shape (16-bit storage, i.e. bf16 or f16 -- dense sweep: D = 768, ungated;
+ * section per kernel family that covers the shape (16-bit storage, i.e. bf16 or f16 -- dense sweep: D = 768 or 1024, ungated;
  * expert-major: ungated at D = 768 / 1024 / 1280, gated at D = 2048; small batch: D a multiple of 256 -- and tiled
  * products: bf16, f16 or f32, D a multiple of 256) and a router
  * section (when shape.router_width > 0 and the fused router+selection kernel covers the router: bf16 or f16, ReLU/abs,
