@@ -78,18 +78,26 @@ template <bool F16, bool FIRST> __device__ __forceinline__ void mfma_32x32x16_va
   }
 }
 // The matrix pipe writes its results some cycles after the instruction issues and the hardware does not hold back a
-// vector instruction that reads them early (11 wait states for this 8-pass instruction).
-__device__ __forceinline__ void mfma_vacc_settle(f32x16& c) { asm volatile("s_nop 15\n\ts_nop 15" : "+v"(c)); }
+// vector instruction that reads them early (11 wait states for this 8-pass instruction; 18 are spent).  One wait
+// serves every tile: volatile statements keep their order, so a reader of any tile comes after the first statement.
+__device__ __forceinline__ void mfma_vacc_settle(f32x16& last) { asm volatile("s_nop 15\n\ts_nop 1" : "+v"(last)); }
+__device__ __forceinline__ void mfma_vacc_settled(f32x16& other) { asm volatile("" : "+v"(other)); }
 
 // SPLIT: the workgroup handles only chunks [c_begin, c_end) of its tile and leaves its float32 sums, without bias or
 // residual, in A.partial[split]; a finishing kernel adds the splits in ascending order.
-template <int D, int ACT, bool ED8, int TT, bool SPLIT = false, bool F16 = false>
+// NW: waves per workgroup.  4 = one per SIMD, each with a quarter of the chunk's neurons (GEMM1) and of the output columns
+// (GEMM2).  8 = two per SIMD, each with an eighth: wave w works on half sub = w % 2 of what wave w / 2 of the 4-wave form
+// does and reads the same packed stream (every second W1 fragment, three of every six W2 fragments).
+template <int D, int ACT, bool ED8, int TT, bool SPLIT = false, bool F16 = false, int NW = 4>
 __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw,
                                            const int c_begin = 0, const int c_end = 1 << 30, const int split = 0) {
+  constexpr int WS = NW / 4;           // waves that share one packed stream
+  constexpr int NT = 64 * NW;          // threads
   constexpr int KS1 = D / 16;          // K steps of GEMM1
-  constexpr int CT = D / 128;          // 32-wide column tiles per wave in GEMM2
-  constexpr int HC = SweepCfg<D>::HC, LOG_HC = SweepCfg<D>::LOG_HC, RT = SweepCfg<D>::RT, KS2 = SweepCfg<D>::KS2;
+  constexpr int CT = D / 128 / WS;     // 32-wide column tiles per wave in GEMM2
+  constexpr int HC = SweepCfg<D>::HC, LOG_HC = SweepCfg<D>::LOG_HC, RT = SweepCfg<D>::RT / WS, KS2 = SweepCfg<D>::KS2;
   constexpr bool RLDS = SweepCfg<D>::RLDS, VACC = SweepCfg<D>::VACC;
+  static_assert(NW == 4 || (NW == 8 && !VACC && SweepCfg<D>::RT == 2 && (D / 128) % 2 == 0), "8 waves: the D = 768 form only");
   const int E = A.E, n_chunks = A.n_chunks;
   const int64_t N = A.N;
   bf16x8* xs = (bf16x8*)smem_raw;                              // [2][KS1][64]
@@ -108,10 +116,13 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   const int g = lane >> 5, c32 = lane & 31;
   constexpr int NW1 = RT * KS1;        // W1 fragments per (wave, chunk)
   constexpr int NW2 = KS2 * CT;        // W2 fragments per (wave, chunk)
-  constexpr int PIECES = NW1 + NW2;
-  constexpr int R = MD_RING;
+  constexpr int PIECES = WS * (NW1 + NW2);   // fragments per chunk of a packed stream
+  constexpr int R = MD_RING / WS;      // fragments in flight per wave (the same bytes per CU in both forms)
   constexpr int BM = 32 * TT;
   static_assert(NW1 % R == 0 && NW2 % R == 0, "every phase must start at ring slot 0");
+  // position in a chunk of the packed stream of this wave's s-th W1 / W2 fragment, less what depends on sub
+  auto P1 = [](int s) constexpr { return (s / RT) * (RT * WS) + s % RT; };
+  auto P2 = [](int s) constexpr { return (s / CT) * (CT * WS) + s % CT; };
 
   // ---- staging.  Every global load of the tile's inputs is issued up front, in the order the data is needed:
   // routing pieces and the two tables (short, and the active-chunk mask hangs on them), the x tile, then the weight
@@ -126,29 +137,35 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   // stored).
   typedef StreamPtr Stream;
   // this wave's stream: a raw buffer of 32-bit words covering the wave's part of the packed weights
-  const Stream wbase{__builtin_amdgcn_make_buffer_rsrc((void*)(A.wp + (int64_t)w * n_chunks * PIECES * 64), 0,
+  const int wb = w / WS, sub = w % WS;
+  const Stream wbase{__builtin_amdgcn_make_buffer_rsrc((void*)(A.wp + (int64_t)wb * n_chunks * PIECES * 64), 0,
                                                        n_chunks * PIECES * 1024, 0x00020000), (uint32_t)lane * 16u, 0};
+  // a chunk's W1 fragments of this wave start at chunkA(c), its W2 fragments at chunkA(c) + W2OFF (units of 16 bytes)
+  auto chunkA = [&](int c) __attribute__((always_inline)) { return wbase + ((int64_t)c * PIECES + sub * RT) * 64; };
+  const int W2OFF = (WS * NW1 + sub * CT - sub * RT) * 64;
   bf16x8 ring[R];
   const int first_guess = SPLIT ? c_begin : 0;
-  const int r8 = lane & 7, c8l = lane >> 3;
   const int last_row = (int)((N - 1 - tok0) < (int64_t)(BM - 1) ? (N - 1 - tok0) : (int64_t)(BM - 1));
   {
-    constexpr int RW = BM / 4;                      // rows per wave
-    constexpr int RB = RW / 8;                      // blocks of 8 rows per wave
-    constexpr int XK = D / 64;                      // 16-byte pieces of a row per lane (12)
-    constexpr int RK = 4;                           // routing pieces of a row per lane (E <= 256)
-    constexpr int TB1 = MD_MAX_CHUNKS / 8, TEI = MD_MAX_CHUNKS / 16;   // table pieces per thread
+    constexpr int RW = BM / NW;                     // rows per wave
+    constexpr int RR = RW < 8 ? RW : 8;             // rows per block (8; 4 where a wave has only 4 rows)
+    constexpr int RB = RW / RR;                     // row blocks per wave
+    constexpr int LPR = 64 / RR;                    // lanes per row
+    constexpr int XK = D / 8 / LPR;                 // 16-byte pieces of a row per lane (12 with 8 lanes per row)
+    constexpr int RK = 32 / LPR;                    // routing pieces of a row per lane (E <= 256)
+    constexpr int TB1 = MD_MAX_CHUNKS * 32 / NT, TEI = MD_MAX_CHUNKS * 16 / NT;   // table pieces per thread
+    const int r8 = lane % RR, c8l = lane / RR;
     const bool wide = (E & 7) == 0;                 // routing rows are whole 16-byte pieces
     const int EP = E >> 3;
     if (t == 0) *cmask_lds = 0u;
-    for (int e = t; e < E; e += 256) {
+    for (int e = t; e < E; e += NT) {
       const int h0 = e * A.expert_dim;
       ebits[e] = (1u << (h0 >> LOG_HC)) | (1u << ((h0 + A.expert_dim - 1) >> LOG_HC));
     }
     int mrow[RB];                                   // tile row of each row block, clamped to the last real row
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      const int m = w * RW + rb * 8 + r8;
+      const int m = w * RW + rb * RR + r8;
       mrow[rb] = m < last_row ? m : last_row;
     }
     u32x4 rv[RB][RK];
@@ -158,18 +175,18 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
         const u32x4* rrow = (const u32x4*)(A.routing + (tok0 + mrow[rb]) * E);
 #pragma unroll
         for (int kb = 0; kb < RK; ++kb)
-          if (kb * 8 < EP) rv[rb][kb] = rrow[c8l + kb * 8 < EP ? c8l + kb * 8 : 0];   // lanes past the row: piece 0
+          if (kb * LPR < EP) rv[rb][kb] = rrow[c8l + kb * LPR < EP ? c8l + kb * LPR : 0];   // lanes past the row: piece 0
       }
     }
     u32x4 tb[TB1], te[TEI];
 #pragma unroll
     for (int k = 0; k < TB1; ++k) {
-      const int i = t + k * 256;
+      const int i = t + k * NT;
       tb[k] = ((const u32x4*)A.b1p)[i < HP / 8 ? i : 0];
     }
 #pragma unroll
     for (int k = 0; k < TEI; ++k) {
-      const int i = t + k * 256;
+      const int i = t + k * NT;
       te[k] = ((const u32x4*)A.eidx)[i < HP / 16 ? i : 0];
     }
     u32x4 xv[RB][XK];
@@ -177,7 +194,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     for (int rb = 0; rb < RB; ++rb) {
       const u32x4* xrow = (const u32x4*)(A.x + (tok0 + mrow[rb]) * D) + c8l;
 #pragma unroll
-      for (int kb = 0; kb < XK; ++kb) xv[rb][kb] = xrow[kb * 8];
+      for (int kb = 0; kb < XK; ++kb) xv[rb][kb] = xrow[kb * LPR];
     }
     lds_barrier();   // chunk bits per expert written, mask cleared
     __builtin_amdgcn_sched_barrier(0);
@@ -185,11 +202,11 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     if (wide) {
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        const int m = w * RW + rb * 8 + r8;
+        const int m = w * RW + rb * RR + r8;
 #pragma unroll
         for (int kb = 0; kb < RK; ++kb) {
-          if (kb * 8 < EP && c8l + kb * 8 < EP) {
-            const int piece = c8l + kb * 8;
+          if (kb * LPR < EP && c8l + kb * LPR < EP) {
+            const int piece = c8l + kb * LPR;
             const u32x4 r4 = rv[rb][kb];
             if constexpr (RLDS) *(u32x4*)(rs + m * RS + piece * 8) = r4;
             const u32x4 eb0 = *(const u32x4*)(ebits + piece * 8);
@@ -205,20 +222,23 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     }
 #pragma unroll
     for (int k = 0; k < TB1; ++k) {
-      const int i = t + k * 256;
+      const int i = t + k * NT;
       if (i < HP / 8) ((u32x4*)b1s)[i] = tb[k];
     }
 #pragma unroll
     for (int k = 0; k < TEI; ++k) {
-      const int i = t + k * 256;
+      const int i = t + k * NT;
       if (i < HP / 16) ((u32x4*)eis)[i] = te[k];
     }
     __builtin_amdgcn_sched_barrier(0);
+    {
+      const Stream first = chunkA(first_guess);
 #pragma unroll
-    for (int i = 0; i < R; ++i) ring[i] = wbase[((int64_t)first_guess * PIECES + i) * 64];
+      for (int i = 0; i < R; ++i) ring[i] = first[P1(i) * 64];
+    }
     __builtin_amdgcn_sched_barrier(0);
     if (!wide) {
-      for (int i = t; i < BM * E; i += 256) {
+      for (int i = t; i < BM * E; i += NT) {
         const int m = i / E, e = i - m * E;
         const bf16_t r1 = A.routing[(tok0 + (m < last_row ? m : last_row)) * E + e];
         if constexpr (RLDS) rs[m * RS + e] = r1;
@@ -231,10 +251,10 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     // x fragments: piece kk of row m goes to fragment kk / 2 (K step), slot (m & 31) + 32 * (kk & 1)
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      const int m = w * RW + rb * 8 + r8;
+      const int m = w * RW + rb * RR + r8;
       u32x4* xdst = (u32x4*)xs + ((m >> 5) * KS1 + (c8l >> 1)) * 64 + (m & 31) + 32 * (c8l & 1);
 #pragma unroll
-      for (int kb = 0; kb < XK; ++kb) xdst[kb * 4 * 64] = xv[rb][kb];
+      for (int kb = 0; kb < XK; ++kb) xdst[kb * (LPR / 2) * 64] = xv[rb][kb];
     }
   }
   lds_barrier();
@@ -257,10 +277,10 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   if (n_act > 0) {
     f32x16 acc1[RT][TT];  // GEMM1 accumulators [row-tile][token tile]
     const int first_chunk = __builtin_ctz(cmask);
-    Stream cur = wbase + (int64_t)first_chunk * PIECES * 64;
+    Stream cur = chunkA(first_chunk);
     if (first_chunk != first_guess) {
 #pragma unroll
-      for (int i = 0; i < R; ++i) ring[i] = cur[i * 64];
+      for (int i = 0; i < R; ++i) ring[i] = cur[P1(i) * 64];
     }
 
     // Without the routing tile in LDS: the routing values a lane's accumulators are multiplied by (its tokens, the experts
@@ -312,7 +332,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     for (int ci = 0; ci < n_act; ++ci) {
       const int chunk = __builtin_ctz(cmask);
       cmask &= cmask - 1;
-      const Stream nxt = (cmask != 0) ? (wbase + (int64_t)__builtin_ctz(cmask) * PIECES * 64) : cur;
+      const Stream nxt = (cmask != 0) ? chunkA(__builtin_ctz(cmask)) : cur;
       // Where registers are short (VACC), what the epilogue derives from the lane index -- table and h-tile addresses,
       // routing rows -- is recomputed from a fresh copy of it in every chunk instead of being kept across the products.
       int lane_c = lane;
@@ -404,7 +424,10 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt) a[rt] = ring[(RT * ks + rt) % R];
 #pragma unroll
-          for (int rt = 0; rt < RT; ++rt) ring[(RT * ks + rt) % R] = pre[(RT * ks + rt + R) * 64];
+          for (int rt = 0; rt < RT; ++rt) {   // the refills run on into the chunk's own W2 fragments
+            constexpr int s = RT * ks, sr = s + R;
+            ring[(s + rt) % R] = (sr + rt < NW1) ? pre[P1(sr + rt) * 64] : pre[W2OFF + P2(sr + rt - NW1) * 64];
+          }
           constexpr int kn = (ks + 1 < KS1) ? ks + 1 : ks;      // x fragments of the next step, read one step ahead
           bf16x8 nxb[TT];
 #pragma unroll
@@ -421,10 +444,12 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
           __builtin_amdgcn_sched_barrier(0);
         });
         if constexpr (VACC) {
+          mfma_vacc_settle(acc1[RT - 1][TT - 1]);
 #pragma unroll
           for (int a = 0; a < RT; ++a)
 #pragma unroll
-            for (int b = 0; b < TT; ++b) mfma_vacc_settle(acc1[a][b]);
+            for (int b = 0; b < TT; ++b)
+              if (a != RT - 1 || b != TT - 1) mfma_vacc_settled(acc1[a][b]);
         }
       };
       // GEMM2 of the current chunk; refills run on into the next chunk's W1 fragments
@@ -442,7 +467,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
             constexpr int ct = decltype(ct_c)::value;
             constexpr int s = j * CT + ct;      // position in this phase; refill position s + R
             const bf16x8 b = ring[s % R];
-            ring[s % R] = (s + R < NW2) ? cur[(NW1 + s + R) * 64] : nxt[(s + R - NW2) * 64];
+            ring[s % R] = (s + R < NW2) ? cur[W2OFF + P2(s + R) * 64] : nxt[P1(s + R - NW2) * 64];
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt)
               acc2[tt][ct] = mfma_32x32x16<F16>(ha[tt], b, acc2[tt][ct]);
@@ -476,23 +501,27 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   }
 
   // ---- final epilogue: the accumulators are rounded to bf16 once, AFTER + last_bias (+ x) in float32, and leave as
-  // whole rows.  One pass per 32-token tile: every wave writes its D/4 columns of the pass's rows to LDS as float
+  // whole rows.  One pass per 32-token tile: every wave writes its D/NW columns of the pass's rows to LDS as float
   // [32][D + 4] (bias added on the way: a lane's accumulators share CT columns), then wave w takes rows 8w .. 8w + 7
-  // with the lane mapping of the staging above -- lane (r, c) reads 8 consecutive columns c, c + 8, ... of row r, adds
-  // the residual, rounds, stores 16 bytes; 8 lanes cover 128 contiguous bytes of an output row.  The residual rows
-  // are requested before the pass's LDS traffic; the read loop has no branches and no address arithmetic.
+  // (4w .. 4w + 3 with 8 waves) with the lane mapping of the staging above -- lane (r, c) reads 8 consecutive columns
+  // c, c + 8, ... of row r, adds the residual, rounds, stores 16 bytes; 8 lanes cover 128 contiguous bytes of an output
+  // row.  The residual rows are requested before the pass's LDS traffic; the read loop has no branches and no address
+  // arithmetic.
   {
     constexpr int OS = D + 4;                       // row stride in floats (+16 bytes: rows shift by 4 banks, so the
     float* ot = (float*)smem_raw;                   // 8 rows a wave reads at once cover all 32); fits in x + h regions
     static_assert((size_t)32 * OS * 4 <= (size_t)(2 * KS1 * 64 + 2 * KS2 * 64) * 16, "out staging fits");
-    constexpr int OP = D / 64;                      // 8-column pieces per thread and pass
+    constexpr int FR = 32 / NW;                     // rows of a pass per wave
+    constexpr int FL = 64 / FR;                     // lanes per row
+    constexpr int OP = D / 8 / FL;                  // 8-column pieces per thread and pass
+    const int r8 = lane % FR, c8l = lane / FR;
     const bool with_bias = !SPLIT && A.last_bias != nullptr;
     const bool with_res = !SPLIT && A.add_residual != 0;
     float lb[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
-      lb[ct] = with_bias ? dec16<F16>(A.last_bias[w * (D / 4) + ct * 32 + c32]) : 0.f;
-    const int row = w * 8 + r8;                     // row of the pass this thread finishes
+      lb[ct] = with_bias ? dec16<F16>(A.last_bias[w * (D / NW) + ct * 32 + c32]) : 0.f;
+    const int row = w * FR + r8;                    // row of the pass this thread finishes
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
       const int64_t n = tok0 + tt * 32 + row;
@@ -501,12 +530,12 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
       if (with_res) {
         const u32x4* xrow = (const u32x4*)(A.x + (live ? n : N - 1) * D) + c8l;
 #pragma unroll
-        for (int k = 0; k < OP; ++k) xr[k] = xrow[k * 8];
+        for (int k = 0; k < OP; ++k) xr[k] = xrow[k * FL];
       }
       lds_barrier();                                // previous readers of this LDS region are done
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) {
-        const int col = w * (D / 4) + ct * 32 + c32;
+        const int col = w * (D / NW) + ct * 32 + c32;
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           ot[(8 * (r / 4) + 4 * g + (r % 4)) * OS + col] = with_bias ? acc2[tt][ct][r] + lb[ct] : acc2[tt][ct][r];
@@ -517,8 +546,8 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
       float4 pv0[OP], pv1[OP];
 #pragma unroll
       for (int k = 0; k < OP; ++k) {
-        pv0[k] = *(const float4*)(orow + k * 64);
-        pv1[k] = *(const float4*)(orow + k * 64 + 4);
+        pv0[k] = *(const float4*)(orow + k * FL * 8);
+        pv1[k] = *(const float4*)(orow + k * FL * 8 + 4);
         if constexpr (!SPLIT) {
           float v[8] = {pv0[k].x, pv0[k].y, pv0[k].z, pv0[k].w, pv1[k].x, pv1[k].y, pv1[k].z, pv1[k].w};
           if (with_res) {
@@ -535,13 +564,13 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
           float* prow = A.partial + ((int64_t)split * A.part_rows + (n - A.part_base)) * D + c8l * 8;
 #pragma unroll
           for (int k = 0; k < OP; ++k) {
-            *(float4*)(prow + k * 64) = pv0[k];
-            *(float4*)(prow + k * 64 + 4) = pv1[k];
+            *(float4*)(prow + k * FL * 8) = pv0[k];
+            *(float4*)(prow + k * FL * 8 + 4) = pv1[k];
           }
         } else {
           u32x4* grow = (u32x4*)(A.out + n * D) + c8l;
 #pragma unroll
-          for (int k = 0; k < OP; ++k) grow[k * 8] = o[k];
+          for (int k = 0; k < OP; ++k) grow[k * FL] = o[k];
         }
       }
     }
@@ -591,21 +620,21 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_dense_walk_kernel(const D
 // Workgroups [0, n_full) take tiles of 64 tokens.  The tokens left over after the last full round of the machine go to
 // tiles of 32; if those would still leave most CUs idle, each of them is dealt to csplit workgroups by chunk ranges,
 // which leave float32 sums in A.partial for the finishing kernel.
-template <int D, int ACT, bool ED8, bool F16 = false>
-__global__ __launch_bounds__(256, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
+template <int D, int ACT, bool ED8, bool F16 = false, int NW = 4>
+__global__ __launch_bounds__(64 * NW, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
   const int b = blockIdx.x;
   if (b < A.n_full) {
-    dense_tile<D, ACT, ED8, 2, false, F16>(A, (int64_t)b * 64, smem_raw);
+    dense_tile<D, ACT, ED8, 2, false, F16, NW>(A, (int64_t)b * 64, smem_raw);
   } else if (A.csplit <= 1) {
-    dense_tile<D, ACT, ED8, 1, false, F16>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
+    dense_tile<D, ACT, ED8, 1, false, F16, NW>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
   } else {
     const int idx = b - A.n_full;
     const int tile = idx / A.csplit, split = idx % A.csplit;
     const int c_begin = split * A.chunks_per_split;
-    dense_tile<D, ACT, ED8, 1, true, F16>(A, (int64_t)A.n_full * 64 + (int64_t)tile * 32, smem_raw, c_begin,
-                                     c_begin + A.chunks_per_split, split);
+    dense_tile<D, ACT, ED8, 1, true, F16, NW>(A, (int64_t)A.n_full * 64 + (int64_t)tile * 32, smem_raw, c_begin,
+                                         c_begin + A.chunks_per_split, split);
   }
 }
 
@@ -632,7 +661,11 @@ static inline hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x,
   const bool walk = skip_flag != nullptr && sh.expert_dim <= 64;
   const bool allow_split = !walk && workspace != nullptr && workspace_bytes >= mfma_dense_workspace_bytes(sh);
   const DenseTiling T = dense_tiling(sh, allow_split);
-  auto kern = walk ? experts_mfma_dense_walk_kernel<D, ACT, ED8, F16> : experts_mfma_dense_kernel<D, ACT, ED8, F16>;
+#ifndef D2DMOE_SWEEP_NW
+#define D2DMOE_SWEEP_NW 4
+#endif
+  constexpr int NW = (D == 768) ? D2DMOE_SWEEP_NW : 4;   // waves per workgroup of the ordinary grid
+  auto kern = walk ? experts_mfma_dense_walk_kernel<D, ACT, ED8, F16> : experts_mfma_dense_kernel<D, ACT, ED8, F16, NW>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   DenseArgs A;
@@ -645,7 +678,7 @@ static inline hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x,
   A.part_base = T.part_base; A.part_rows = T.part_rows;
   int64_t grid = T.n_full + T.n_half * T.csplit;
   if (walk && A.n_tiles > cus) grid = cus;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, s, A);
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(walk ? 256 : 64 * NW), lds, s, A);
   e = hipGetLastError();
   if (e != hipSuccess || T.csplit <= 1) return e;
   return launch_sum_partials(A.partial, last_bias, (const bf16_t*)x + T.part_base * sh.d_model,
