@@ -50,7 +50,7 @@ WORKLOADS = {
     # float16 storage (the reference benches float32 and float16): same kernel families as bf16
     'vit_b_50k_f16': (256, 197, 768, 128, 24, 128, 'relu'),
     # one FFN layer of a GPT-2-medium-sized model (D = 1024, d_ff = 4096 as 128 experts x 32, GELU), 16 x 1024 tokens:
-    # tiled products under module tau 0.9, expert-major kernels under the literal rule
+    # the D = 1024 sweep under module tau 0.9, expert-major kernels under the literal rule
     'gpt2_medium_layer': (16, 1024, 1024, 128, 32, 128, 'gelu'),
     # the expert split of the reference's own micro-benchmark (scripts/test_moe_implementations.py:109-126: 24 experts of
     # 128 neurons) behind a real router: the sweep under module tau 0.9, the expert-major kernel for big experts under
