@@ -834,7 +834,7 @@ def main():
             sub['reference_shape'] = reference_shape_record(ops, dev, sub_steps, sub_warmup)
             for w in ('gpt2_medium_layer', 'vit_b_24x128'):
                 sub[w] = router_driven_record(args, ops, dev, w, sub_steps, sub_warmup)
-            # BASELINE config 4 in short: the whole GPT-2-small forward with MoE FFNs (few steps: a step is 7 ms)
+            # the GPT-2-small configuration in short: the whole GPT-2-small forward with MoE FFNs (few steps: a step is 7 ms)
             saved = args.steps, args.warmup
             args.steps, args.warmup = max(saved[0] // 5, 5), 2
             g = gpt2_record(args, dev)

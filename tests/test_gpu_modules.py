@@ -1,5 +1,5 @@
 """GPU parity of the module-level drop-in: every experts container of the registry on the HIP kernels, the gates other
-than dynk_max feeding them, the gated (Gemma-shape) module on the product kernels, and the BASELINE configurations at
+than dynk_max feeding them, the gated (Gemma-shape) module on the product kernels, and the benchmark configurations at
 their full sizes (GPT-2-small forward, skewed routing at 50 432 tokens).
 
 Bars as in test_gpu_parity.py: masks bit-exact given the same predicted norms; outputs within 1e-5 (float32) / 2e-2
@@ -328,7 +328,7 @@ def test_mask_flips_sit_on_the_threshold(N, tau, dtype):
     assert n_flips <= (1e-5 if dtype == torch.bfloat16 else 2e-6) * N * E
 
 
-# =================================================================== BASELINE config 4 at its size ===================
+# =================================================================== GPT-2-small configuration at its size ===================
 @pytest.mark.parametrize('tau', [0.9, 0.1])
 def test_gpt2_layer_at_full_size(tau):
     """One converted GPT-2-small FFN (GELU, biases, 128 x 24) on 16 x 1024 tokens: mask from the oracle gate on the GPU's
@@ -356,7 +356,7 @@ def test_gpt2_layer_at_full_size(tau):
 
 
 def test_gpt2_small_forward_at_full_size():
-    """BASELINE config 4 as named: 12 layers, d_model 768, 12 heads, vocabulary 50257, every FFN converted to 128 experts of
+    """The GPT-2-small benchmark configuration as named: 12 layers, d_model 768, 12 heads, vocabulary 50257, every FFN converted to 128 experts of
     24 neurons with its own 768->128->128 router, batch 16 x 1024, bf16, module tau 0.9.  The model returns finite logits
     and one routing tensor per layer; each layer's mask is a valid dynamic-k mask (at least one expert per token); the
     last layer's output is checked against the float64 oracle on the layer's own input rows."""
@@ -398,7 +398,7 @@ def test_gpt2_small_forward_at_full_size():
     assert H.rel_err(captured['out'].reshape(-1, 768).cpu()[rows], want) < H.TOL_BF16
 
 
-# =================================================================== BASELINE config 3 at its size ===================
+# =================================================================== skewed-routing configuration at its size ===================
 @pytest.mark.parametrize('tau', [0.9, 0.1])
 def test_skewed_routing_at_full_size(tau):
     """50 432 tokens, router bypassed by |N(0,1)| x Zipf(1.2) predicted norms: mask bit-exact with the oracle gate, counts
