@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define D2DMOE_VERSION 200 /* major*10000 + minor*100 + patch */
+#define D2DMOE_VERSION 210 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 enum {
@@ -118,7 +118,7 @@ typedef struct d2dmoe_shape {
  * buffers keeps their descriptors with them (or copies the buffer's first 64 bytes back and hands them to
  * d2dmoe_packed_desc_from_header).  No counterpart in the reference, which has no derived buffers. */
 #define D2DMOE_PACKED_MAGIC 0x4b50324du   /* "M2PK" */
-#define D2DMOE_PACKED_LAYOUT_VERSION 3u
+#define D2DMOE_PACKED_LAYOUT_VERSION 4u
 enum {                       /* bits of d2dmoe_packed_desc.sections */
   D2DMOE_SECTION_DENSE = 1, D2DMOE_SECTION_EXPERT_MAJOR = 2, D2DMOE_SECTION_SMALL_BATCH = 4,
   D2DMOE_SECTION_TILED = 8, D2DMOE_SECTION_COMPACTED = 16, D2DMOE_SECTION_ROUTER = 32
