@@ -5,6 +5,17 @@
 
 #include "mfma_common.hpp"
 
+// Build-time forms of the sweep (for comparison runs; the defaults are the product):
+//   D2DMOE_SWEEP_DYN  1: a tile works through the blocks of hidden neurons its tokens use (gathered chunks)
+//                     0: through every chunk of the packed stream that holds a used expert (fixed chunks)
+//   D2DMOE_SWEEP_NW   4: one wave per SIMD; 8: two (D = 768, fixed chunks only)
+#ifndef D2DMOE_SWEEP_DYN
+#define D2DMOE_SWEEP_DYN 1
+#endif
+#ifndef D2DMOE_SWEEP_NW
+#define D2DMOE_SWEEP_NW 4
+#endif
+
 namespace d2dmoe {
 
 // ---------------------------------------------------------------------------------------------------
@@ -88,9 +99,19 @@ __device__ __forceinline__ void mfma_vacc_settled(f32x16& other) { asm volatile(
 // NW: waves per workgroup.  4 = one per SIMD, each with a quarter of the chunk's neurons (GEMM1) and of the output columns
 // (GEMM2).  8 = two per SIMD, each with an eighth: wave w works on half sub = w % 2 of what wave w / 2 of the 4-wave form
 // does and reads the same packed stream (every second W1 fragment, three of every six W2 fragments).
-template <int D, int ACT, bool ED8, int TT, bool SPLIT = false, bool F16 = false, int NW = 4>
+// DYN: the chunks the tile works through are gathered, not the fixed ones of the packed stream.  The unit is a block of
+// 32 hidden neurons (a wave's GEMM1 row tile, two K steps of GEMM2).  At staging the tile finds the blocks that hold a
+// neuron of any expert some token of the tile routes to, and lists them -- active ones first, ascending, then the
+// rest.  "Chunk" v is then blocks list[v * BPC .. v * BPC + BPC) (BPC = blocks per chunk), and the tile stops after the
+// last chunk that holds an active block (the inactive blocks that fill it up multiply hidden activations that are all
+// zero).  Everything else -- ring, barriers, LDS layout, summation order over ascending neurons -- is as in the fixed
+// form, whose chunks are the case list = 0, 1, 2, ...: for a routing that uses every block the two forms run the same
+// instructions on the same addresses, and for any routing they give the same bits (the blocks left out would have
+// added zeros).  The time of a tile follows the number of distinct experts its 64 tokens use.
+template <int D, int ACT, bool ED8, int TT, bool SPLIT = false, bool F16 = false, int NW = 4, bool DYN = false>
 __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw,
                                            const int c_begin = 0, const int c_end = 1 << 30, const int split = 0) {
+  static_assert(!DYN || NW == 4, "gathered chunks: the four-wave form only");
   constexpr int WS = NW / 4;           // waves that share one packed stream
   constexpr int NT = 64 * NW;          // threads
   constexpr int KS1 = D / 16;          // K steps of GEMM1
@@ -109,11 +130,17 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   uint8_t* eis = (uint8_t*)(b1s + HP);                         // [HP] expert index of each neuron
   uint32_t* ebits = (uint32_t*)(eis + HP);                     // [E rounded up to 8] chunks each expert's neurons lie in
   uint32_t* cmask_lds = ebits + ((E + 7) & ~7);                // chunks some token of the tile needs (bit per chunk)
+  // DYN: experts some token routes to (bit per expert, in the first 8 words of ebits, which it does not use otherwise),
+  // the waves' ballots of active blocks, and the list of blocks
+  uint32_t* emask = ebits;
+  constexpr int BPC = HC / 32;                                 // blocks per chunk
+  constexpr int MAXB = MD_MAX_CHUNKS * 8;                      // most blocks a layer can have (256: block numbers are bytes)
 
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int w = __builtin_amdgcn_readfirstlane(t >> 6);   // wave index, known to the compiler to be the same in all lanes
   const int g = lane >> 5, c32 = lane & 31;
+  uint8_t* blist = (uint8_t*)(cmask_lds + 2) + w * MAXB;  // DYN: this wave's own copy of the block list
   constexpr int NW1 = RT * KS1;        // W1 fragments per (wave, chunk)
   constexpr int NW2 = KS2 * CT;        // W2 fragments per (wave, chunk)
   constexpr int PIECES = WS * (NW1 + NW2);   // fragments per chunk of a packed stream
@@ -143,6 +170,50 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   // a chunk's W1 fragments of this wave start at chunkA(c), its W2 fragments at chunkA(c) + W2OFF (units of 16 bytes)
   auto chunkA = [&](int c) __attribute__((always_inline)) { return wbase + ((int64_t)c * PIECES + sub * RT) * 64; };
   const int W2OFF = (WS * NW1 + sub * CT - sub * RT) * 64;
+  // Where a chunk's fragments are.  Fixed chunks: `a` (above).  Gathered chunks (DYN): per block, in units of 16 bytes
+  // from the start of ALL waves' streams -- oA[rt]: the W1 fragments of this wave's row tile rt (K step ks at
+  // + ks * RT * 64), oB[p]: this wave's W2 fragments of the chunk's p-th block (half h, column tile ct at
+  // + (h * CT + ct) * 64); blk[rt]: the block itself (for the bias / expert-index tables).
+  struct ChunkSrc { Stream a; int oA[RT]; int oB[DYN ? BPC : 1]; int blk[RT]; uint32_t lo, hi; };
+  const Stream wall{__builtin_amdgcn_make_buffer_rsrc((void*)A.wp, 0, MD_WAVES * n_chunks * PIECES * 1024, 0x00020000),
+                    (uint32_t)lane * 16u, 0};
+  // lo / hi: the chunk's block numbers, one byte each (BPC = 4: lo only)
+  auto src_of_blocks = [&](uint32_t lo, uint32_t hi) __attribute__((always_inline)) {
+    ChunkSrc c;
+    c.a = wbase; c.lo = lo; c.hi = hi;
+#pragma unroll
+    for (int p = 0; p < BPC; ++p) {
+      const int b = (int)(((p < 4 ? lo : hi) >> ((p & 3) * 8)) & 0xffu);
+      c.oB[DYN ? p : 0] = ((w * n_chunks + b / BPC) * PIECES + NW1 + 2 * (b % BPC) * CT) * 64;
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int pos = w * RT + rt;
+      const int b = (int)(((pos < 4 ? lo : hi) >> ((pos & 3) * 8)) & 0xffu);
+      const int q = b % BPC;
+      c.blk[rt] = b;
+      c.oA[rt] = (((q / RT) * n_chunks + b / BPC) * PIECES + q % RT) * 64;
+    }
+    return c;
+  };
+  auto blocks_of_fixed = [&](int c, uint32_t& lo, uint32_t& hi) __attribute__((always_inline)) {   // chunk c as it is packed
+    lo = (uint32_t)(c * BPC) * 0x01010101u + 0x03020100u;
+    hi = (uint32_t)(c * BPC) * 0x01010101u + 0x07060504u;
+  };
+  auto blocks_of_listed = [&](int v, uint32_t& lo, uint32_t& hi) __attribute__((always_inline)) {  // chunk v of the list
+    const uint32_t* bl = (const uint32_t*)blist + v * (BPC / 4);
+    lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)bl[0]);
+    hi = (BPC > 4) ? (uint32_t)__builtin_amdgcn_readfirstlane((int)bl[BPC > 4 ? 1 : 0]) : 0u;
+  };
+  // the s-th W1 / W2 fragment of a chunk (s: position in this wave's sequence)
+  auto w1_frag = [&](const ChunkSrc& c, int s) __attribute__((always_inline)) {
+    if constexpr (DYN) return wall[c.oA[s % RT] + (s / RT) * (RT * 64)];
+    else return c.a[P1(s) * 64];
+  };
+  auto w2_frag = [&](const ChunkSrc& c, int s) __attribute__((always_inline)) {
+    if constexpr (DYN) return wall[c.oB[(s / CT) / 2] + (((s / CT) % 2) * CT + s % CT) * 64];
+    else return c.a[W2OFF + P2(s) * 64];
+  };
   bf16x8 ring[R];
   const int first_guess = SPLIT ? c_begin : 0;
   const int last_row = (int)((N - 1 - tok0) < (int64_t)(BM - 1) ? (N - 1 - tok0) : (int64_t)(BM - 1));
@@ -158,9 +229,13 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     const bool wide = (E & 7) == 0;                 // routing rows are whole 16-byte pieces
     const int EP = E >> 3;
     if (t == 0) *cmask_lds = 0u;
-    for (int e = t; e < E; e += NT) {
-      const int h0 = e * A.expert_dim;
-      ebits[e] = (1u << (h0 >> LOG_HC)) | (1u << ((h0 + A.expert_dim - 1) >> LOG_HC));
+    if constexpr (DYN) {
+      if (t < 8) emask[t] = 0u;
+    } else {
+      for (int e = t; e < E; e += NT) {
+        const int h0 = e * A.expert_dim;
+        ebits[e] = (1u << (h0 >> LOG_HC)) | (1u << ((h0 + A.expert_dim - 1) >> LOG_HC));
+      }
     }
     int mrow[RB];                                   // tile row of each row block, clamped to the last real row
 #pragma unroll
@@ -199,6 +274,9 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     lds_barrier();   // chunk bits per expert written, mask cleared
     __builtin_amdgcn_sched_barrier(0);
     uint32_t need = 0u;                             // chunks the rows staged by this thread need
+    uint32_t ebyte[RK];                             // DYN: which of the 8 experts of each of its pieces they route to
+#pragma unroll
+    for (int kb = 0; kb < RK; ++kb) ebyte[kb] = 0u;
     if (wide) {
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
@@ -209,14 +287,29 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
             const int piece = c8l + kb * LPR;
             const u32x4 r4 = rv[rb][kb];
             if constexpr (RLDS) *(u32x4*)(rs + m * RS + piece * 8) = r4;
-            const u32x4 eb0 = *(const u32x4*)(ebits + piece * 8);
-            const u32x4 eb1 = *(const u32x4*)(ebits + piece * 8 + 4);
             const uint32_t wd[4] = {r4.x, r4.y, r4.z, r4.w};
-            const uint32_t eb[8] = {eb0.x, eb0.y, eb0.z, eb0.w, eb1.x, eb1.y, eb1.z, eb1.w};
+            if constexpr (DYN) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-              need |= (wd[i >> 1] & ((i & 1) ? 0x7fff0000u : 0x7fffu)) != 0 ? eb[i] : 0u;
+              for (int i = 0; i < 8; ++i)
+                ebyte[kb] |= (wd[i >> 1] & ((i & 1) ? 0x7fff0000u : 0x7fffu)) != 0 ? (1u << i) : 0u;
+            } else {
+              const u32x4 eb0 = *(const u32x4*)(ebits + piece * 8);
+              const u32x4 eb1 = *(const u32x4*)(ebits + piece * 8 + 4);
+              const uint32_t eb[8] = {eb0.x, eb0.y, eb0.z, eb0.w, eb1.x, eb1.y, eb1.z, eb1.w};
+#pragma unroll
+              for (int i = 0; i < 8; ++i)
+                need |= (wd[i >> 1] & ((i & 1) ? 0x7fff0000u : 0x7fffu)) != 0 ? eb[i] : 0u;
+            }
           }
+        }
+      }
+      if constexpr (DYN) {
+#pragma unroll
+        for (int kb = 0; kb < RK; ++kb) {
+          const int piece = c8l + kb * LPR;
+          if (ebyte[kb] != 0u)
+            __hip_atomic_fetch_or((__attribute__((address_space(3))) uint32_t*)(emask + (piece >> 2)),
+                                  ebyte[kb] << ((piece & 3) * 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
       }
     }
@@ -232,9 +325,16 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     }
     __builtin_amdgcn_sched_barrier(0);
     {
-      const Stream first = chunkA(first_guess);
+      ChunkSrc first;
+      if constexpr (DYN) {
+        uint32_t lo, hi;
+        blocks_of_fixed(first_guess, lo, hi);
+        first = src_of_blocks(lo, hi);
+      } else {
+        first.a = chunkA(first_guess);
+      }
 #pragma unroll
-      for (int i = 0; i < R; ++i) ring[i] = first[P1(i) * 64];
+      for (int i = 0; i < R; ++i) ring[i] = w1_frag(first, i);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (!wide) {
@@ -242,10 +342,16 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
         const int m = i / E, e = i - m * E;
         const bf16_t r1 = A.routing[(tok0 + (m < last_row ? m : last_row)) * E + e];
         if constexpr (RLDS) rs[m * RS + e] = r1;
-        if ((r1 & 0x7fff) != 0) need |= ebits[e];
+        if constexpr (DYN) {
+          if ((r1 & 0x7fff) != 0)
+            __hip_atomic_fetch_or((__attribute__((address_space(3))) uint32_t*)(emask + (e >> 5)), 1u << (e & 31),
+                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        } else {
+          if ((r1 & 0x7fff) != 0) need |= ebits[e];
+        }
       }
     }
-    if (need != 0u)
+    if (!DYN && need != 0u)
       __hip_atomic_fetch_or((__attribute__((address_space(3))) uint32_t*)cmask_lds, need, __ATOMIC_RELAXED,
                             __HIP_MEMORY_SCOPE_WORKGROUP);
     // x fragments: piece kk of row m goes to fragment kk / 2 (K step), slot (m & 31) + 32 * (kk & 1)
@@ -259,7 +365,49 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   }
   lds_barrier();
   // Active chunks as a bit mask, the same in every wave: the chunk loop walks its set bits.
-  uint32_t cmask = __builtin_amdgcn_readfirstlane(*cmask_lds);
+  // (DYN: a mask of the chunks of the list that hold an active block -- the first ceil(active blocks / BPC))
+  uint32_t cmask;
+  if constexpr (DYN) {
+    // Block b is active iff one of the experts with a neuron in it is routed to by some token of the tile.  Every wave
+    // works the list out for itself (lane l looks at blocks l, l + 64, ...) and keeps its own copy in LDS: no exchange
+    // between the waves, no further barrier.
+    const int n_blocks = n_chunks * BPC;
+    const int Ed = A.expert_dim;
+    unsigned long long bal[MAXB / 64];
+    bool on[MAXB / 64];
+    int total = 0;
+#pragma unroll
+    for (int k = 0; k < MAXB / 64; ++k) {
+      const int b = lane + 64 * k;
+      on[k] = false;
+      bal[k] = 0ull;
+      if (64 * k < n_blocks) {                       // uniform
+        if (b < n_blocks) {
+          const int e_lo = (32 * b) / Ed;
+          int e_hi = (32 * b + 31) / Ed;
+          e_hi = e_hi < E - 1 ? e_hi : E - 1;
+          for (int e = e_lo; e <= e_hi; ++e) on[k] |= ((emask[e >> 5] >> (e & 31)) & 1u) != 0;
+        }
+        bal[k] = __ballot(on[k]);
+        total += __popcll(bal[k]);
+      }
+    }
+    int before = 0;                                  // active blocks in the passes before this one
+#pragma unroll
+    for (int k = 0; k < MAXB / 64; ++k) {
+      const int b = lane + 64 * k;
+      if (64 * k < n_blocks) {
+        const int below = before + __popcll(bal[k] & ((1ull << lane) - 1ull));
+        if (b < n_blocks) blist[on[k] ? below : total + (b - below)] = (uint8_t)b;
+        before += __popcll(bal[k]);
+      }
+    }
+    const int n_vc = (total + BPC - 1) / BPC;
+    cmask = (n_vc >= 32) ? ~0u : ((1u << n_vc) - 1u);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the list is read back below by the wave that wrote it
+  } else {
+    cmask = __builtin_amdgcn_readfirstlane(*cmask_lds);
+  }
   if constexpr (SPLIT) {
     const uint32_t below_end = (c_end >= 32) ? ~0u : ((1u << c_end) - 1u);
     cmask &= below_end & ~((1u << c_begin) - 1u);
@@ -277,17 +425,34 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
   if (n_act > 0) {
     f32x16 acc1[RT][TT];  // GEMM1 accumulators [row-tile][token tile]
     const int first_chunk = __builtin_ctz(cmask);
-    Stream cur = chunkA(first_chunk);
-    if (first_chunk != first_guess) {
+    auto src_of_chunk = [&](int c) __attribute__((always_inline)) {
+      if constexpr (DYN) {
+        uint32_t lo, hi;
+        blocks_of_listed(c, lo, hi);
+        return src_of_blocks(lo, hi);
+      } else {
+        ChunkSrc r;
+        r.a = chunkA(c);
+        return r;
+      }
+    };
+    ChunkSrc cur = src_of_chunk(first_chunk);
+    bool guessed = first_chunk == first_guess;
+    if constexpr (DYN) {
+      uint32_t glo, ghi;
+      blocks_of_fixed(first_guess, glo, ghi);
+      guessed = cur.lo == glo && (BPC <= 4 || cur.hi == ghi);
+    }
+    if (!guessed) {
 #pragma unroll
-      for (int i = 0; i < R; ++i) ring[i] = cur[P1(i) * 64];
+      for (int i = 0; i < R; ++i) ring[i] = w1_frag(cur, i);
     }
 
     // Without the routing tile in LDS: the routing values a lane's accumulators are multiplied by (its tokens, the experts
     // of its rows), raw 16-bit patterns, requested one chunk ahead.
     constexpr int NRQ = ED8 ? 4 : 16;
     uint32_t rpre[TT][RT][NRQ];
-    auto routing_request = [&](int chunk_r, int g, int c32) __attribute__((always_inline)) {
+    auto routing_request = [&](const ChunkSrc& src_r, int chunk_r, int g, int c32) __attribute__((always_inline)) {
 #pragma unroll
       for (int tt = 0; tt < TT; ++tt) {
         const int m = tt * 32 + c32;
@@ -297,7 +462,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
         for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const int hb = chunk_r * HC + w * (32 * RT) + 4 * g + rt * 32 + 8 * q;
+            const int hb = (DYN ? src_r.blk[rt] * 32 : chunk_r * HC + w * (32 * RT) + rt * 32) + 4 * g + 8 * q;
             if (ED8) {
               rpre[tt][rt][q] = *(const bf16_t*)(rtile + (rrow + 2u * eis[hb & ~7]));
             } else {
@@ -332,13 +497,17 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
     for (int ci = 0; ci < n_act; ++ci) {
       const int chunk = __builtin_ctz(cmask);
       cmask &= cmask - 1;
-      const Stream nxt = (cmask != 0) ? chunkA(__builtin_ctz(cmask)) : cur;
+      const ChunkSrc nxt = (cmask != 0) ? src_of_chunk(__builtin_ctz(cmask)) : cur;
       // Where registers are short (VACC), what the epilogue derives from the lane index -- table and h-tile addresses,
       // routing rows -- is recomputed from a fresh copy of it in every chunk instead of being kept across the products.
       int lane_c = lane;
       if constexpr (VACC) asm volatile("" : "+v"(lane_c));
       const int g = lane_c >> 5, c32 = lane_c & 31;
-      const int hb0 = chunk * HC + w * (32 * RT) + 4 * g;   // first neuron of this lane's accumulator rows, row-tile 0
+      // first neuron of this lane's accumulator rows in row tile rt
+      auto hb_of = [&](const ChunkSrc& c, int chunk_c, int rt) __attribute__((always_inline)) {
+        if constexpr (DYN) return c.blk[rt] * 32 + 4 * g;
+        else return chunk_c * HC + w * (32 * RT) + rt * 32 + 4 * g;
+      };
 
       // epilogue state, filled and consumed in slices between MFMAs
       uint2 e_bias[4];     // 4 bf16 biases per accumulator quad
@@ -348,7 +517,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
       auto epi_load_tables = [&](int rt) __attribute__((always_inline)) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int hb = hb0 + rt * 32 + 8 * q;
+          const int hb = hb_of(cur, chunk, rt) + 8 * q;
           e_bias[q] = *(const uint2*)(b1s + hb);
           // Ed multiple of 8: the aligned block of 8 neurons a quad pair covers belongs to one expert, the same for
           // every lane, so one routing value per (quad, token tile) serves four accumulator rows
@@ -406,7 +575,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
         }
       };
       // GEMM1 of the chunk whose stream starts at `pre` (its W1 fragments; the refills run on into its W2 fragments)
-      auto gemm1 = [&](const Stream pre) __attribute__((always_inline)) {
+      auto gemm1 = [&](const ChunkSrc& pre) __attribute__((always_inline)) {
         if constexpr (!VACC) {
 #pragma unroll
           for (int a = 0; a < RT; ++a)
@@ -426,7 +595,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt) {   // the refills run on into the chunk's own W2 fragments
             constexpr int s = RT * ks, sr = s + R;
-            ring[(s + rt) % R] = (sr + rt < NW1) ? pre[P1(sr + rt) * 64] : pre[W2OFF + P2(sr + rt - NW1) * 64];
+            ring[(s + rt) % R] = (sr + rt < NW1) ? w1_frag(pre, sr + rt) : w2_frag(pre, sr + rt - NW1);
           }
           constexpr int kn = (ks + 1 < KS1) ? ks + 1 : ks;      // x fragments of the next step, read one step ahead
           bf16x8 nxb[TT];
@@ -467,7 +636,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
             constexpr int ct = decltype(ct_c)::value;
             constexpr int s = j * CT + ct;      // position in this phase; refill position s + R
             const bf16x8 b = ring[s % R];
-            ring[s % R] = (s + R < NW2) ? cur[W2OFF + P2(s + R) * 64] : nxt[P1(s + R - NW2) * 64];
+            ring[s % R] = (s + R < NW2) ? w2_frag(cur, s + R) : w1_frag(nxt, s + R - NW2);
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt)
               acc2[tt][ct] = mfma_32x32x16<F16>(ha[tt], b, acc2[tt][ct]);
@@ -479,7 +648,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
       };
 
       if (ci == 0) {
-        if constexpr (!RLDS) routing_request(chunk, g, c32);
+        if constexpr (!RLDS) routing_request(cur, chunk, g, c32);
         gemm1(cur);
       }
       lds_barrier();   // every wave has finished reading the previous h tile
@@ -493,7 +662,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
       }
       lds_barrier();   // h tile complete
       // (the values of the last chunk are requested once more instead of branching round the loads)
-      if constexpr (!RLDS) routing_request(cmask != 0 ? __builtin_ctz(cmask) : chunk, g, c32);
+      if constexpr (!RLDS) routing_request(nxt, cmask != 0 ? __builtin_ctz(cmask) : chunk, g, c32);
       gemm2();
       if (ci + 1 < n_act) gemm1(nxt);
       cur = nxt;
@@ -591,6 +760,7 @@ template <typename T> __device__ __forceinline__ T* uniform(T* p) { return (T*)(
 // Out-of-line copy of the tile routine for the variant below (keeps its register allocation apart from the loop).
 template <int D, int ACT, bool ED8, int TT, bool F16>
 __device__ __attribute__((noinline)) void dense_tile_call(const DenseArgs& A, const int64_t tok0, unsigned char* smem_raw) {
+  constexpr bool DYN = D2DMOE_SWEEP_DYN != 0;
   DenseArgs U;
   U.x = uniform(A.x); U.routing = uniform(A.routing); U.wp = uniform(A.wp); U.b1p = uniform(A.b1p); U.eidx = uniform(A.eidx);
   U.last_bias = uniform(A.last_bias); U.out = uniform(A.out); U.skip_flag = nullptr; U.partial = nullptr;
@@ -598,7 +768,7 @@ __device__ __attribute__((noinline)) void dense_tile_call(const DenseArgs& A, co
   U.N = uniform(A.N); U.E = uniform(A.E); U.expert_dim = uniform(A.expert_dim); U.n_chunks = uniform(A.n_chunks);
   U.hidden = uniform(A.hidden); U.act_rt = uniform(A.act_rt); U.add_residual = uniform(A.add_residual);
   U.n_full = 0; U.n_tiles = 0;
-  dense_tile<D, ACT, ED8, TT, false, F16>(U, uniform(tok0), smem_raw);
+  dense_tile<D, ACT, ED8, TT, false, F16, 4, DYN>(U, uniform(tok0), smem_raw);
 }
 
 // The same sweep launched as one workgroup per CU that walks the tiles in launch order.  Used where the launch is
@@ -620,21 +790,21 @@ __global__ __launch_bounds__(256, 1) void experts_mfma_dense_walk_kernel(const D
 // Workgroups [0, n_full) take tiles of 64 tokens.  The tokens left over after the last full round of the machine go to
 // tiles of 32; if those would still leave most CUs idle, each of them is dealt to csplit workgroups by chunk ranges,
 // which leave float32 sums in A.partial for the finishing kernel.
-template <int D, int ACT, bool ED8, bool F16 = false, int NW = 4>
+template <int D, int ACT, bool ED8, bool F16 = false, int NW = 4, bool DYN = false>
 __global__ __launch_bounds__(64 * NW, 1) void experts_mfma_dense_kernel(const DenseArgs A) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   if (A.skip_flag != nullptr && *A.skip_flag != 0) return;   // uniform over the whole grid
   const int b = blockIdx.x;
   if (b < A.n_full) {
-    dense_tile<D, ACT, ED8, 2, false, F16, NW>(A, (int64_t)b * 64, smem_raw);
+    dense_tile<D, ACT, ED8, 2, false, F16, NW, DYN>(A, (int64_t)b * 64, smem_raw);
   } else if (A.csplit <= 1) {
-    dense_tile<D, ACT, ED8, 1, false, F16, NW>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
+    dense_tile<D, ACT, ED8, 1, false, F16, NW, DYN>(A, (int64_t)A.n_full * 64 + (int64_t)(b - A.n_full) * 32, smem_raw);
   } else {
     const int idx = b - A.n_full;
     const int tile = idx / A.csplit, split = idx % A.csplit;
     const int c_begin = split * A.chunks_per_split;
-    dense_tile<D, ACT, ED8, 1, true, F16, NW>(A, (int64_t)A.n_full * 64 + (int64_t)tile * 32, smem_raw, c_begin,
-                                         c_begin + A.chunks_per_split, split);
+    dense_tile<D, ACT, ED8, 1, true, F16, NW, DYN>(A, (int64_t)A.n_full * 64 + (int64_t)tile * 32, smem_raw, c_begin,
+                                              c_begin + A.chunks_per_split, split);
   }
 }
 
@@ -661,11 +831,9 @@ static inline hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x,
   const bool walk = skip_flag != nullptr && sh.expert_dim <= 64;
   const bool allow_split = !walk && workspace != nullptr && workspace_bytes >= mfma_dense_workspace_bytes(sh);
   const DenseTiling T = dense_tiling(sh, allow_split);
-#ifndef D2DMOE_SWEEP_NW
-#define D2DMOE_SWEEP_NW 4
-#endif
   constexpr int NW = (D == 768) ? D2DMOE_SWEEP_NW : 4;   // waves per workgroup of the ordinary grid
-  auto kern = walk ? experts_mfma_dense_walk_kernel<D, ACT, ED8, F16> : experts_mfma_dense_kernel<D, ACT, ED8, F16, NW>;
+  constexpr bool DYN = D2DMOE_SWEEP_DYN && NW == 4;
+  auto kern = walk ? experts_mfma_dense_walk_kernel<D, ACT, ED8, F16> : experts_mfma_dense_kernel<D, ACT, ED8, F16, NW, DYN>;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
   DenseArgs A;

@@ -327,6 +327,65 @@ def test_experts_mfma_dense_at_width_1024_full_size_properties():
     assert H.elem_err(a.cpu()[rows], want) < H.TOL_BF16
 
 
+def _structured_routing(kind, N, E, seed):
+    """Routings whose experts are used unevenly, the cases in which a tile of the sweep works through fewer blocks of
+    hidden neurons than the layer has."""
+    g = torch.Generator().manual_seed(seed)
+    r = torch.zeros(N, E)
+    if kind == 'hot':            # every token picks 2 of the same 5 experts
+        hot = torch.randperm(E, generator=g)[:5]
+        pick = torch.stack([hot[torch.randperm(5, generator=g)[:2]] for _ in range(N)])
+        r.scatter_(1, pick, 1.0)
+    elif kind == 'one_dense':    # a few hot experts, and one token in a hundred routes to half of all experts
+        hot = torch.randperm(E, generator=g)[:3]
+        r[:, hot] = (torch.rand(N, 3, generator=g) < 0.7).float()
+        dense = torch.rand(N, generator=g) < 0.01
+        r[dense] = (torch.rand(int(dense.sum()), E, generator=g) < 0.5).float()
+    elif kind == 'by_tile':      # tokens of one 64-token tile share a window of experts that moves from tile to tile
+        for t0 in range(0, N, 64):
+            e0 = (t0 // 64 * 7) % E
+            idx = (e0 + torch.arange(6)) % E
+            r[t0:t0 + 64, idx] = (torch.rand(min(64, N - t0), 6, generator=g) < 0.6).float()
+    elif kind == 'last_only':    # only the last expert (the last block, partly padding when hidden % 32 != 0)
+        r[:, E - 1] = 1.0
+    elif kind == 'zipf':         # norms |randn| * rank^-1.2 under the 0.1 * max rule
+        w = (torch.randperm(E, generator=g).float() + 1.0) ** -1.2
+        n = torch.randn(N, E, generator=g).abs() * w
+        r = (n >= 0.1 * n.max(1, keepdim=True).values).float()
+    return r
+
+
+@pytest.mark.parametrize('kind', ['hot', 'one_dense', 'by_tile', 'last_only', 'zipf'])
+@pytest.mark.parametrize('N,D,E,Ed,act,dtype', [(1000, 768, 128, 24, 'relu', torch.bfloat16), (8320, 768, 128, 24, 'gelu', torch.bfloat16),
+                                                (700, 768, 100, 30, 'relu', torch.float16), (900, 768, 24, 128, 'relu', torch.bfloat16),
+                                                (1000, 1024, 128, 32, 'gelu', torch.bfloat16), (8320, 1024, 100, 30, 'relu', torch.float16),
+                                                (300, 768, 7, 5, 'relu', torch.bfloat16)])
+def test_experts_mfma_dense_uneven_expert_use(kind, N, D, E, Ed, act, dtype):
+    """The sweep gathers its chunks from the blocks of 32 hidden neurons that a tile's tokens use.  Routings with hot
+    experts, a rare dense token, expert windows that move from tile to tile, a single expert at the end of the layer, and
+    Zipf-weighted norms: against the float64 oracle and the generic kernel (small cases).  Where every tile is a whole
+    one (8320 tokens), a random permutation of the tokens -- tiles then hold other tokens and gather other blocks -- must
+    permute the output rows bit for bit: a block a tile works through for its other tokens adds exact zeros to a row."""
+    _say('experts mfma uneven use', kind, N, D, E, Ed, act, dtype)
+    tol = H.TOL_BF16 if dtype == torch.bfloat16 else 4e-3
+    x, _, p = H.random_case(N, D, E, Ed, 8, seed=N + E, dtype=dtype, density=0.5)
+    routing = _structured_routing(kind, N, E, seed=E + Ed).to(dtype)
+    d = H.to_dev(p, DEV)
+    sh = _ops().make_shape(0, D, E, Ed, 0, _ops()._dtype_code(x), act)
+    packed = _ops().pack_weights(sh, d['w1'], d['b1'], d['w2'], None, None, None)
+    got = _experts_got(x, routing, p, act, residual=True, path='mfma_dense', packed=packed)
+    rows = torch.arange(N) if N <= 1000 else torch.cat([torch.arange(0, 200), torch.arange(N - 200, N)])
+    want = _experts_want(x[rows], routing[rows], p, act, True)
+    assert H.rel_err(got[rows], want) < tol
+    assert H.elem_err(got[rows], want) < tol
+    if N <= 1000 and D == 768:
+        assert H.rel_err(got, _experts_got(x, routing, p, act, residual=True, path='generic')) < (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    if N == 8320:     # whole tiles only (the tail tiles sum their chunk ranges in a second step)
+        perm = torch.randperm(N, generator=torch.Generator().manual_seed(4))
+        got_p = _experts_got(x[perm].contiguous(), routing[perm].contiguous(), p, act, residual=True, path='mfma_dense', packed=packed)
+        assert torch.equal(got_p, got[perm])
+
+
 def test_experts_mfma_dense_full_size_properties():
     """50432 tokens (the headline workload): oracle on a slice of rows, the generic HIP kernel on all rows, and
     determinism (two runs give identical bits)."""
