@@ -185,8 +185,9 @@ class HipKernelExperts(_HipContainer):
     def output_norms(self, x):
         """L2 norm of every expert's output for every token, [E,N]: the router-training targets the reference reads off
         a forward hook on `output_activation_extraction_stub` in 'masked' mode (train_routers.py:49-86,
-        utils.py:353-369).  On a ROCm device in bf16 with D = 768 and experts of at most 32 neurons one HIP kernel computes
-        them without forming the [E,N,D] outputs; anything else takes the reference's own route through the stubs."""
+        utils.py:353-369).  On a ROCm device in bf16 or float16, with D a multiple of 256 up to 2048 and experts of at most
+        64 neurons, one HIP kernel computes them without forming the [E,N,D] outputs; anything else (float32, other
+        widths) takes the reference's own route through the stubs."""
         assert x.dim() == 2, f'{x.size()=}'
         if x.is_cuda and not (torch.is_grad_enabled() and (x.requires_grad or self.w1.requires_grad)):
             sh = ops.make_shape(0, self.hidden_dim, self.num_experts, self.expert_dim, 0, ops._dtype_code(x),

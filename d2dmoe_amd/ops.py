@@ -240,7 +240,8 @@ def pack_norms(shape: abi.Shape, w1, b1, w2) -> Optional[torch.Tensor]:
 
 def expert_output_norms(x: torch.Tensor, w1: torch.Tensor, b1: Optional[torch.Tensor], w2: torch.Tensor,
                         activation: str = 'relu', packed: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """norms [E,N] = | act(x w1[e] + b1[e]) w2[e] |_2 through d2dmoe_expert_output_norms (bf16, D = 768, Ed <= 32)."""
+    """norms [E,N] = | act(x w1[e] + b1[e]) w2[e] |_2 through d2dmoe_expert_output_norms (bf16 or float16, D a multiple of
+    256 up to 2048, ungated experts of at most 64 neurons)."""
     _require_same_dtype('expert_output_norms', x, w1=w1, b1=b1, w2=w2)
     dev = _require_gpu(x, w1, b1, w2, packed)
     lib = abi.load()
@@ -250,7 +251,8 @@ def expert_output_norms(x: torch.Tensor, w1: torch.Tensor, b1: Optional[torch.Te
     if packed is None:
         packed = pack_norms(sh, w1, b1, w2)
     if packed is None:
-        raise abi.D2DMoEError('d2dmoe_expert_output_norms does not cover this shape (bf16, D = 768, experts of <= 32 neurons)')
+        raise abi.D2DMoEError('d2dmoe_expert_output_norms does not cover this shape (bf16 / float16, D a multiple of 256 up to 2048, '
+                              'ungated experts of <= 64 neurons)')
     out = torch.empty(e, n, dtype=x.dtype, device=dev)
     abi.check(lib.d2dmoe_expert_output_norms(ctypes.byref(sh), _ptr(x), _ptr(packed), _ptr(out), _stream()),
               'd2dmoe_expert_output_norms')

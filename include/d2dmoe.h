@@ -274,13 +274,14 @@ int d2dmoe_forward_static(const d2dmoe_shape* shape, const void* x,
                           const void* packed, const d2dmoe_packed_desc* packed_desc, const void* norms_in,
                           void* norms_out, void* routing, int32_t* counts, void* out, int32_t path, void* stream);
 
-/* L2 norm of every expert's output for every token, norms[e,n] = | act(x[n,:] . w1[e] + b1[e]) . w2[e] |_2 (bf16 [E,N]):
+/* L2 norm of every expert's output for every token, norms[e,n] = | act(x[n,:] . w1[e] + b1[e]) . w2[e] |_2 ([E,N]):
  * the regression targets of router training.  Replaces running the layer in 'masked' mode with a forward hook on
  * output_activation_extraction_stub that takes torch.linalg.vector_norm(output, ord=2, dim=-1) of the [E,N,D] expert
  * outputs (architectures/moe/moe_layers.py:125-133, 193-198; utils.py:353-369;
  * methods/dynamic_sparsification/train_routers.py:49-86).  The outputs are never formed: the second layer enters as
- * each expert's Ed x Ed Gram matrix.  bf16, D = 768, ungated experts of at most 32 neurons; D2DMOE_E_UNSUPPORTED
- * otherwise (d2dmoe_norms_packed_bytes then returns 0).
+ * each expert's Ed x Ed Gram matrix.  bf16 or float16 (norms in the same type), D a multiple of 256 up to 2048, ungated
+ * experts of at most 64 neurons, any activation; D2DMOE_E_UNSUPPORTED otherwise (d2dmoe_norms_packed_bytes then
+ * returns 0).
  *   packed: d2dmoe_norms_packed_bytes(shape) bytes written by d2dmoe_pack_norms for the same weights (a derived,
  *           cacheable buffer of its own, separate from d2dmoe_pack_weights'); no workspace. */
 size_t d2dmoe_norms_packed_bytes(const d2dmoe_shape* shape);

@@ -136,6 +136,29 @@ def test_packed_and_workspace_sizes_follow_the_documented_layouts():
         assert want <= ws <= want + (64 << 20), (E, Ed, ws)
 
 
+def test_norms_buffer_size_follows_the_documented_layout():
+    """d2dmoe_norms_packed_bytes: four wave streams of first-layer fragments (16 bytes per lane; experts padded to 32
+    neurons, to 64 from 33 neurons on, 8 such slots of 32 per chunk, one ring of 32 fragments of padding per wave), bias,
+    Gram fragments in two 16-bit parts (one 32 x 32 block per small expert, 2 x 2 per big one), one scale per slot; 0 for
+    what the kernel does not cover."""
+    from d2dmoe_amd import hip_abi as abi, ops
+    lib = abi.load()
+    for D, E, Ed in ((768, 128, 24), (768, 100, 30), (1024, 128, 32), (768, 24, 64), (2048, 9, 33), (256, 7, 5), (1280, 160, 32)):
+        for dt in (abi.BF16, abi.F16):
+            got = lib.d2dmoe_norms_packed_bytes(ctypes.byref(ops.make_shape(0, D, E, Ed, 0, dt)))
+            slots = E * (2 if Ed > 32 else 1)
+            chunks = (slots + 7) // 8
+            stream = 4 * (chunks * 2 * (D // 16) + 32) * 64 * 16
+            bias = chunks * 8 * 32 * 2
+            gram = chunks * 8 * (8 if Ed > 32 else 4) * 64 * 16
+            scale = chunks * 8 * 4
+            assert stream + bias + gram + scale <= got < stream + bias + gram + scale + 768, (D, E, Ed, dt)
+    for D, E, Ed, dt, gated in ((768, 128, 24, abi.F32, False), (800, 128, 24, abi.BF16, False), (2304, 16, 24, abi.BF16, False),
+                                (768, 16, 65, abi.BF16, False), (2048, 256, 64, abi.BF16, True)):
+        sh = ops.make_shape(0, D, E, Ed, 0, dt, 'gelu_tanh' if gated else 'relu', gated=gated)
+        assert lib.d2dmoe_norms_packed_bytes(ctypes.byref(sh)) == 0, (D, E, Ed, dt, gated)
+
+
 def test_expert_major_workspace_covers_its_tiled_products_fallback():
     """Ungated D = 768 layers the fused sweep does not cover (more than 256 experts, or more than 32 chunks of 256 hidden
     neurons) fall back, behind the expert-major plan, to the tiled products, which work in the workspace BEHIND the plan:

@@ -1317,24 +1317,59 @@ def test_entry_points_reject_bad_workspace_alignment_and_paths():
 # Router-training targets: per-expert output norms (reference: train_routers.py:49-86, utils.py:353-369)
 # ---------------------------------------------------------------------------------------------------------------------
 @pytest.mark.gpu
-@pytest.mark.parametrize('N,E,Ed,act', [(197, 128, 24, 'relu'), (65, 100, 30, 'gelu'), (1, 7, 5, 'relu'),
-                                        (300, 16, 32, 'tanh'), (130, 9, 24, 'leaky_relu')])
-def test_expert_output_norms_match_oracle(N, E, Ed, act):
-    _say('expert output norms', N, E, Ed, act)
-    x, _, p = H.random_case(N, 768, E, Ed, 8, seed=N + E + 5, dtype=torch.bfloat16)
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16], ids=['bf16', 'f16'])
+@pytest.mark.parametrize('N,D,E,Ed,act', [(197, 768, 128, 24, 'relu'), (65, 768, 100, 30, 'gelu'), (1, 768, 7, 5, 'relu'),
+                                          (300, 768, 16, 32, 'tanh'), (130, 768, 9, 24, 'leaky_relu'),
+                                          # experts of 33-64 neurons (two slots of 32 each), other widths, 32-token tiles
+                                          (150, 768, 24, 64, 'relu'), (70, 768, 5, 33, 'gelu'), (129, 1024, 128, 32, 'gelu'),
+                                          (200, 1024, 19, 48, 'relu'), (97, 256, 11, 8, 'relu'), (64, 512, 16, 64, 'gelu'),
+                                          (100, 1280, 40, 32, 'gelu'), (33, 2048, 12, 40, 'relu'), (31, 1536, 9, 16, 'tanh')])
+def test_expert_output_norms_match_oracle(N, D, E, Ed, act, dtype):
+    _say('expert output norms', N, D, E, Ed, act, dtype)
+    tol = H.tol_for(dtype)
+    x, _, p = H.random_case(N, D, E, Ed, 8, seed=N + E + 5, dtype=dtype)
     d = H.to_dev(p, DEV)
     got = _ops().expert_output_norms(x.to(DEV), d['w1'], d['b1'], d['w2'], act)
-    assert got.shape == (E, N) and got.dtype == torch.bfloat16
+    assert got.shape == (E, N) and got.dtype == dtype
     q = O.upcast(p)
     want = O.expert_output_norms(x.double(), q['w1'], q['b1'], q['w2'], act)
-    assert H.rel_err(got.cpu(), want) < H.TOL_BF16
+    assert H.rel_err(got.cpu(), want) < tol
     # element-wise as well: a norm is a sum of squares, there is no cancellation to hide behind
-    rel = ((got.cpu().double() - want).abs() / want.clamp_min(1e-3)).max().item()
-    assert rel < 2e-2, rel
+    rel = ((got.cpu().double() - want).abs() / want.clamp_min(1e-3 * want.max().item())).max().item()
+    assert rel < tol, rel
     # without the first-layer bias
     got = _ops().expert_output_norms(x.to(DEV), d['w1'], None, d['w2'], act)
     want = O.expert_output_norms(x.double(), q['w1'], None, q['w2'], act)
-    assert H.rel_err(got.cpu(), want) < H.TOL_BF16
+    assert H.rel_err(got.cpu(), want) < tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('Ed', [24, 64])
+def test_expert_output_norms_float16_second_layer_of_any_magnitude(Ed):
+    """The Gram matrix of the second layer is stored in float16 scaled by a power of two per expert: second-layer
+    weights whose squared row norms leave the float16 range at either end (the outputs themselves do not) give the norms
+    of the oracle, each expert with a magnitude of its own."""
+    N, D, E = 130, 768, 12
+    _say('expert output norms, float16, scaled second layers', Ed)
+    x, _, p = H.random_case(N, D, E, Ed, 8, seed=77, dtype=torch.float16)
+    scale = torch.tensor([2.0 ** k for k in (-14, -10, -6, -2, 0, 1, 3, 5, 7, 9, 10, 11)]).view(E, 1, 1)
+    w2 = p['w2'].float()
+    w2 = w2 / w2.abs().amax(dim=(1, 2), keepdim=True) * scale     # largest entry of expert e: 2^k
+    p['w2'] = w2.half()
+    assert torch.isfinite(p['w2']).all()
+    assert (p['w2'][-1].float().pow(2).sum(-1) > 65504).any() and (p['w2'][0].float().pow(2).sum(-1) < 6.1e-5).all()
+    p['w1'] = (p['w1'].float() * 0.05).half()      # hidden activations small enough for the outputs to stay finite
+    d = H.to_dev(p, DEV)
+    got = _ops().expert_output_norms(x.to(DEV), d['w1'], d['b1'], d['w2'], 'relu').cpu()
+    q = O.upcast(p)
+    want = O.expert_output_norms(x.double(), q['w1'], q['b1'], q['w2'], 'relu')
+    assert torch.isfinite(want.half()).all(), 'the case is meant to stay inside the float16 range'
+    for e in range(E):    # per expert: every magnitude on its own scale
+        big = want[e] > 6.2e-5        # normal float16 results
+        assert big.any() or e < 2
+        rel = ((got[e].double() - want[e]).abs()[big] / want[e][big]).max().item() if big.any() else 0.0
+        assert rel < H.TOL_F16, (e, rel)
+        assert ((got[e].double() - want[e]).abs()[~big] <= 2.0 ** -24 + H.TOL_F16 * want[e][~big]).all()
 
 
 @pytest.mark.gpu
