@@ -30,8 +30,9 @@ namespace d2dmoe {
 //   epilogue      + b1, activation, x routing[token, expert(neuron)], round to bf16, store as A fragments to LDS
 //   GEMM2  wave w: OUT[tokens, D/4 columns of w] += H . W2            A = h (LDS), B = W2 fragments (stream)
 // OUT stays in registers across all chunks (ascending neuron = ascending expert order, float32) and is rounded
-// once in the final epilogue (+ last_bias, + x).  Chunks none of whose experts is routed to by any token of the
-// tile are skipped (uniform branch).
+// once in the final epilogue (+ last_bias, + x).  A tile leaves out what none of its tokens routes to: by blocks of
+// 32 neurons gathered into chunks of its own (the default, described at dense_tile below), or by whole chunks of the
+// packed stream (uniform branch).
 //
 // Each wave runs at one wave per SIMD, so memory latency is hidden by software: the weight stream is read MD_RING
 // fragments ahead into a register ring (compile-time indices), across phase and chunk boundaries;

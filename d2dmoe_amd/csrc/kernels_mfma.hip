@@ -23,7 +23,7 @@ size_t dense_lds_bytes(const d2dmoe_shape& sh) {
   return (size_t)(2 * KS1 * 64 + 2 * (hc / 16) * 64) * 16         // x fragments, h fragments
          + (sh.d_model <= 768 ? (size_t)MD_BM * (sh.n_experts + 8) * 2 : 0)   // routing tile, rows padded by 8 elements
          + (size_t)n_chunks * hc * 3                               // b1 (bf16) and expert index (uint8) per neuron
-         + (size_t)((sh.n_experts + 7) / 8 * 8 + 4) * sizeof(uint32_t)    // chunk bits per expert, active-chunk mask
+         + (size_t)((sh.n_experts + 7) / 8 * 8 + 4) * sizeof(uint32_t)    // per expert: chunk bits (fixed chunks) or one bit per expert (gathered); the active-chunk mask
          + (size_t)MD_WAVES * MD_MAX_CHUNKS * 8;                            // every wave's list of blocks
 }
 
