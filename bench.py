@@ -551,6 +551,7 @@ def run_norms(args, ops, dev):
     ms_stubs = time_events(stubs, 3, 1)
     executed = N * E * 2.0 * D * 32          # first product with experts padded to 32 neurons
     useful = N * E * 2.0 * D * Ed
+    traffic, traffic_src = measured_traffic('vit_b_50k_norms')
     line = {
         'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
         'value': N / ms * 1e3, 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'spin_up_ms': SPIN_UP_MS,
@@ -560,8 +561,8 @@ def run_norms(args, ops, dev):
                                f'D={D}, {E} experts x {Ed}, relu; one step = norms [E,N] of one batch'},
         'reference_route_ms': ms_stubs,
         'roofline': {'bound': 'mfma', 'kernel': 'expert_norms_kernel', 'achieved': useful / ms / 1e9, 'peak': PEAK_BF16_TFLOPS,
-                     'unit': 'TFLOP/s', 'frac': useful / ms / 1e9 / PEAK_BF16_TFLOPS, 'traffic': None, 'kernel_ms': ms,
-                     'executed_tflops': executed / ms / 1e9},
+                     'unit': 'TFLOP/s', 'frac': useful / ms / 1e9 / PEAK_BF16_TFLOPS, 'traffic': traffic, 'traffic_source': traffic_src,
+                     'kernel_ms': ms, 'executed_tflops': executed / ms / 1e9},
     }
     print(json.dumps(line))
 
