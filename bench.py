@@ -723,7 +723,7 @@ def main():
     ap.add_argument('--path', default='auto', choices=['auto', 'mfma_dense', 'mfma_sparse', 'mfma_mid', 'generic'],
                     help='force the experts path of the ungated workloads (default: the library chooses)')
     ap.add_argument('--quantile-iters', type=int, default=200,
-                    help='per-call timed launches of the experts kernel for median / 2.5 % / 97.5 % (0 = skip)')
+                    help='per-call timed launches of the experts kernel for median / 2.5 %% / 97.5 %% (0 = skip)')
     ap.add_argument('--spin-up-ms', type=float, default=SPIN_UP_MS,
                     help='milliseconds of untimed load ahead of every timed region, before its warm-up steps (0 = none)')
     ap.add_argument('--copy-probe', action='store_true',

@@ -566,6 +566,9 @@ def test_bench_refuses_more_than_one_gpu():
     res = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--gpus', '2'], capture_output=True, text=True, timeout=120)
     assert res.returncode != 0
     assert 'single-GPU' in (res.stderr + res.stdout)
+    # ... and its usage text prints (argparse formats every help string with %)
+    res = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--help'], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0 and '--workload' in res.stdout, res.stderr[-400:]
 
 
 # ------------------------------------------------------------------ every experts container of the registry ----
