@@ -197,19 +197,22 @@ def time_quantiles(fn, iters, warmup):
 
 
 def measured_ceilings(dev):
-    """What this very GPU sustains on plain library work: a large bf16 GEMM (hipBLASLt through torch.matmul) and a
-    streaming copy.  Printed next to the published peaks; the roofline fractions stay relative to the published ones."""
+    """What this very GPU sustains on plain library work: a large bf16 GEMM (hipBLASLt through torch, in both layouts of
+    the second operand; the faster one is the figure quoted) and a streaming copy.  Printed next to the published peaks; the roofline fractions stay relative to the published ones."""
     a = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
     b = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
-    ms = time_events(lambda: torch.matmul(a, b), 10, 3)
-    gemm = 2 * 8192 ** 3 / ms / 1e9
+    ms_nn = time_events(lambda: torch.matmul(a, b), 10, 3)
+    ms_nt = time_events(lambda: torch.nn.functional.linear(a, b), 10, 3)   # the weight operand row-major in K: nn.Linear's layout
+    gemm_nn, gemm_nt = 2 * 8192 ** 3 / ms_nn / 1e9, 2 * 8192 ** 3 / ms_nt / 1e9
+    gemm = max(gemm_nn, gemm_nt)
     del a, b
     src = torch.zeros(64 << 20, dtype=torch.float32, device=dev)   # 256 MiB read + 256 MiB written per call
     dst = torch.empty_like(src)
     ms = time_events(lambda: dst.copy_(src), 10, 3)
     copy = 2 * src.numel() * 4 / ms / 1e6
     del src, dst
-    return {'library_gemm_bf16_8192_tflops': gemm, 'copy_gbps': copy}
+    return {'library_gemm_bf16_8192_tflops': gemm, 'library_gemm_bf16_8192_nn_tflops': gemm_nn,
+            'library_gemm_bf16_8192_nt_tflops': gemm_nt, 'copy_gbps': copy}
 
 
 def dense_mlp_ms(x, D, hidden, act, steps, warmup):
