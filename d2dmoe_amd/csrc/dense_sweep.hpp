@@ -47,6 +47,7 @@ struct DenseArgs {
   float* partial;         // [csplit][part_rows][D] float32 sums of the chunk-split tiles (tokens from part_base on)
   int csplit; int chunks_per_split; int64_t part_base; int64_t part_rows;
   int64_t N; int E; int expert_dim; int n_chunks; int hidden; int act_rt; int add_residual; int n_full; int n_tiles;
+  int pf_lines;           // 128-byte lines of the whole weight stream, for the warming reads
 };
 
 // What depends on the model width: the chunk of hidden neurons a workgroup multiplies between two barriers, and
@@ -265,6 +266,21 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
       const int i = t + k * NT;
       te[k] = ((const u32x4*)A.eidx)[i < HP / 16 ? i : 0];
     }
+    // Warming reads of the weight stream: workgroup b touches lines 2 NT b .. 2 NT b + 2 NT - 1 (one 4-byte load per
+    // 128-byte line, two per thread; past the end: line 0).  All workgroups of a round walk the stream in step, a ring of
+    // MD_RING fragments ahead of the MFMAs -- enough for lines that wait in an L2 or in the memory-side cache, not for
+    // lines that come from memory, which is where a layer's weights are when other layers' work has gone through the
+    // caches since its last call.  The first round's workgroups between them touch the whole stream while they stage
+    // their tiles; by the time the stream gets there, the lines are on the near side of memory.
+    uint32_t pf[2];
+    {
+      const uint32_t* wl = (const uint32_t*)A.wp;
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int l = ((int)blockIdx.x * 2 + k) * NT + t;
+        pf[k] = wl[(int64_t)(l < A.pf_lines ? l : 0) * 32];
+      }
+    }
     u32x4 xv[RB][XK];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
@@ -363,6 +379,7 @@ __device__ __forceinline__ void dense_tile(const DenseArgs& A, const int64_t tok
 #pragma unroll
       for (int kb = 0; kb < XK; ++kb) xdst[kb * (LPR / 2) * 64] = xv[rb][kb];
     }
+    asm volatile("" :: "v"(pf[0]), "v"(pf[1]));      // the warming reads' registers are theirs until they have landed
   }
   lds_barrier();
   // Active chunks as a bit mask, the same in every wave: the chunk loop walks its set bits.
@@ -768,6 +785,7 @@ __device__ __attribute__((noinline)) void dense_tile_call(const DenseArgs& A, co
   U.csplit = 1; U.chunks_per_split = 0; U.part_base = 0; U.part_rows = 0;
   U.N = uniform(A.N); U.E = uniform(A.E); U.expert_dim = uniform(A.expert_dim); U.n_chunks = uniform(A.n_chunks);
   U.hidden = uniform(A.hidden); U.act_rt = uniform(A.act_rt); U.add_residual = uniform(A.add_residual);
+  U.pf_lines = uniform(A.pf_lines);
   U.n_full = 0; U.n_tiles = 0;
   dense_tile<D, ACT, ED8, TT, false, F16, 4, DYN>(U, uniform(tok0), smem_raw);
 }
@@ -845,6 +863,7 @@ static inline hipError_t launch_dense_cfg(const d2dmoe_shape& sh, const void* x,
   A.n_full = (int)T.n_full; A.n_tiles = (int)(T.n_full + T.n_half); A.skip_flag = skip_flag;
   A.partial = (float*)workspace; A.csplit = T.csplit; A.chunks_per_split = T.per;
   A.part_base = T.part_base; A.part_rows = T.part_rows;
+  A.pf_lines = (int)((size_t)MD_WAVES * L.n_chunks * L.pieces * 64 * 16 / 128);
   int64_t grid = T.n_full + T.n_half * T.csplit;
   if (walk && A.n_tiles > cus) grid = cus;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(walk ? 256 : 64 * NW), lds, s, A);
