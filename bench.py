@@ -279,6 +279,40 @@ def run_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, W, pa
                 expert_load_max_over_mean=(tokens_per_expert.max() / tokens_per_expert.mean().clamp_min(1e-9)).item())
 
 
+def cold_regime(ops, x, p, packed, thr_scale, act, steps, warmup, D, E, Ed, path='auto'):
+    """The layer with cold operands, as it runs inside a model: the step rotates over COLD_SETS sets of inputs, weights
+    and packed buffers (> 256 MB in all from 16 384 tokens on, the size of the memory-side cache), so that a call finds
+    none of its weights in a cache -- other layers' work has gone through them since.  The reference's timer clears the
+    cache between repetitions too (triton do_bench, scripts/test_moe_implementations.py:171-175).  Returns the whole-layer
+    time (replays of a graph holding whole rotations) and the experts kernel's (HIP events around a rotation)."""
+    sets = [(x, p, packed)]
+    for k in range(1, COLD_SETS):
+        g = torch.Generator().manual_seed(100 + k)
+        xk = torch.randn(x.shape, generator=g).to(x.dtype).to(x.device)
+        pk = {name: v.clone() for name, v in p.items()}
+        sets.append((xk, pk, ops.clone_packed(packed)))
+    routings = []
+    for xk, pk, pkd in sets:
+        routings.append(ops.forward(xk, pk['router_w1'], pk['router_w2'], thr_scale, pk['w1'], pk['b1'], pk['w2'], None,
+                                    pk['last_bias'], act, False, None, False, False, path, pkd)[1])
+    experts_path = path if path != 'auto' else ('mfma_sparse' if thr_scale >= 0.75 and x.dtype in (torch.bfloat16, torch.float16) else 'auto')
+
+    def rotation():
+        for xk, pk, pkd in sets:
+            ops.forward(xk, pk['router_w1'], pk['router_w2'], thr_scale, pk['w1'], pk['b1'], pk['w2'], None, pk['last_bias'],
+                        act, False, None, False, False, path, pkd)
+
+    def experts_rotation():
+        for (xk, pk, pkd), r in zip(sets, routings):
+            ops.experts(xk, r, pk['w1'], pk['b1'], pk['w2'], None, pk['last_bias'], act, False, experts_path, pkd)
+
+    reps, wreps = max(steps // COLD_SETS, 3), max(warmup // COLD_SETS, 1)
+    ms_layer = time_graph(rotation, reps, wreps) / COLD_SETS
+    ms_experts = time_events(experts_rotation, reps, wreps) / COLD_SETS
+    pairs = sum(r.float().sum().item() for r in routings) / COLD_SETS
+    return {'operand_sets': COLD_SETS, 'ms_per_step': ms_layer, 'kernel_ms': ms_experts, 'mean_pairs': pairs}
+
+
 def run_gated(args, ops, dev):
     print(json.dumps(gated_record(args, ops, dev, args.workload)))
 
@@ -795,6 +829,9 @@ def main():
                                   'p99_active_experts': r['p99_active'], 'active_tflops': r['active_tflops_layer']})
         dense_ms = dense_mlp_ms(x, D, E * Ed, act, args.steps, args.warmup)
         ceil = measured_ceilings(dev)
+        cold = None
+        if norms_in is None and not f32:
+            cold = cold_regime(ops, x, p, packed, float(1.0 - args.tau), act, args.steps, args.warmup, D, E, Ed, path=args.path)
     line = {
         'metric': 'MoE-FFN tokens/s + active TFLOP/s & HBM GB/s vs roofline, ViT-B layer tau=0.9',
         'value': main_r['tokens_per_s'], 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'spin_up_ms': SPIN_UP_MS,
@@ -823,6 +860,12 @@ def main():
                                       'algorithmic_bytes': lit_r['algo_bytes'], 'kernel_ms': lit_r['ms_experts']}},
         'sweep': sweep,
     }
+    if cold is not None:
+        # warm = the figures above (one set of operands, which the caches keep between steps)
+        pairs_flops = cold['mean_pairs'] * 4.0 * D * Ed
+        cold['tokens_per_s'] = N / cold['ms_per_step'] * 1e3
+        cold['frac'] = pairs_flops / cold['kernel_ms'] / 1e9 / peak
+        line['roofline']['cold'] = cold
     if args.workload == 'vit_b_50k' and args.path == 'auto' and not args.no_sub_records:
         # the other workloads this library is measured on, each with its own roofline, so that one run shows them all
         del x, p, packed
