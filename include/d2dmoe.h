@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define D2DMOE_VERSION 210 /* major*10000 + minor*100 + patch */
+#define D2DMOE_VERSION 211 /* major*10000 + minor*100 + patch */
 
 /* status codes */
 enum {
